@@ -1,0 +1,29 @@
+"""CPU oracle for the single-GPU MoE expert path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing under ``halo_amd/`` imports this package; only ``tests/``,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` do, and there only as the checker or as the
+timed CPU baseline, never as the product.
+
+Every function restates, on the CPU in numpy (integer work) or torch fp32/fp64 (floating point), what the reference
+computes for this path, and cites the reference file:line it follows (paths relative to the reference checkout).
+
+How each function is pinned (tests/test_oracle_*.py):
+
+* ``route_sort.argsort_routing`` / ``build_inv_map`` -- brute-force slot-by-slot sort on tiny inputs, the literal
+  receive ``[[0,-1,2],[2,0,3],[-1,3,-1],[-1,-1,0]]`` of ``tests/cpu/parallelism/test_ep_receive_counts.py:65-70``,
+  the twelve routing cases of ``tests/common/route_sort_reference.py:46-59`` through their invariants, and the
+  ``inv_map`` invariants of ``tests/cpu/parallelism/test_moe_permute_equivalence.py:79-106``.
+* ``permute.*`` -- fp64 ``index_select`` / ``index_add`` (library routines) and the literal sentinel example of
+  ``tests/gpu/kernels/test_moe_permute.py:93-97``.
+* ``glu.*`` -- torch autograd through ``F.silu`` / ``F.gelu`` / ``clamp`` in fp64 (library routines), the identity
+  ``gptoss(alpha=1) - clamped_silu = silu(min(g, L))`` and bound sub-gradients.
+* ``grouped_mm.*`` -- ``torch.matmul`` per group with autograd, and the empty-group counts ``(7,33,0,1,64,0)`` and
+  ``(0,0,0,0,105,0)`` of ``tests/gpu/kernels/test_grouped_mm_empty_groups.py``.
+* ``router.*`` -- ``torch.softmax`` / ``torch.topk`` on tie-free rows, autograd for the backward, and the tie rule
+  (lower expert index wins) by brute force.  The order ``torch.topk`` gives tied scores is implementation-defined in
+  the reference's third-party router: for tied rows the reference's own order is "parity unpinned"; this build fixes
+  it to the lower index.
+* ``block_fp8.*`` -- the ``exp2(ceil(log2(amax/448)))`` diagnostic formula, the ``448*4`` boundary case, padded
+  shapes and the zero block of ``tests/cpu/weight_sync/test_block_fp8.py``.
+* ``moe_layer.*`` -- the dense formula ``out[t] = sum_k w[t,k] * FFN_e(x[t])`` over valid slots.
+"""

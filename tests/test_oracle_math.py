@@ -1,0 +1,244 @@
+"""Pins ``oracle.glu``, ``oracle.grouped_mm``, ``oracle.router``, ``oracle.block_fp8`` and ``oracle.moe_layer`` against
+library routines (torch autograd, matmul, softmax, topk, the float8 cast), identities and brute force."""
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import block_fp8, glu, grouped_mm, moe_layer, router
+
+PROBE = (-64.0, -8.0, -1.0, -0.5, -1e-3, 0.0, 1e-3, 0.5, 1.0, 8.0, 64.0)  # fused_glu.py:33 of the reference
+
+VARIANTS = {
+    "silu": (dict(activation=glu.SILU), lambda g, u: F.silu(g) * u),
+    "gelu_tanh": (dict(activation=glu.GELU_TANH), lambda g, u: F.gelu(g, approximate="tanh") * u),
+    "clamped_silu": (dict(activation=glu.CLAMPED_SILU, limit=2.5),
+                     lambda g, u: F.silu(g.clamp(max=2.5)) * u.clamp(-2.5, 2.5)),
+    "silu_then_clamp": (dict(activation=glu.CLAMPED_SILU, limit=2.5, clamp_activated=True),
+                        lambda g, u: F.silu(g).clamp(max=2.5) * u.clamp(-2.5, 2.5)),
+    "gptoss": (dict(activation=glu.CLAMPED_SILU, alpha=1.702, limit=7.0, up_plus_one=True),
+               lambda g, u: (u.clamp(-7, 7) + 1) * (g.clamp(max=7) * torch.sigmoid(g.clamp(max=7) * 1.702))),
+}
+
+
+@pytest.mark.parametrize("name", VARIANTS)
+def test_glu_forward_and_gradients_match_autograd(name):
+    kwargs, eager = VARIANTS[name]
+    g = torch.Generator().manual_seed(0)
+    gate = torch.cat([torch.randn(500, generator=g) * 4, torch.tensor(PROBE)]).double()
+    up = torch.cat([torch.randn(500, generator=g) * 4, torch.tensor(PROBE[::-1])]).double()
+    dout = torch.randn(gate.shape, generator=g).double()
+    gl, ul = gate.clone().requires_grad_(True), up.clone().requires_grad_(True)
+    want = eager(gl, ul)
+    want.backward(dout)
+    assert torch.allclose(glu.glu_forward(gate, up, **kwargs), want.detach(), rtol=1e-13, atol=1e-13)
+    dgate, dup = glu.glu_backward(gate, up, dout, **kwargs)
+    assert torch.allclose(dgate, gl.grad, rtol=1e-12, atol=1e-12)
+    assert torch.allclose(dup, ul.grad, rtol=1e-12, atol=1e-12)
+
+
+def test_glu_clamp_gradient_passes_at_the_bound():
+    # torch's clamp passes the gradient on the closed interval; so must the closed forms
+    limit = 2.0
+    gate = torch.tensor([limit, limit, -limit, 0.5], dtype=torch.float64)
+    up = torch.tensor([limit, -limit, limit, limit], dtype=torch.float64)
+    dout = torch.ones(4, dtype=torch.float64)
+    dgate, dup = glu.glu_backward(gate, up, dout, glu.CLAMPED_SILU, limit=limit)
+    assert (dgate != 0).all() and (dup != 0).all()
+    dgate_hi, dup_hi = glu.glu_backward(gate + 1e-9, up * (1 + 1e-9), dout, glu.CLAMPED_SILU, limit=limit)
+    assert dgate_hi[0] == 0 and dup_hi[0] == 0  # just past the bound the gradient is cut
+
+
+def test_glu_identity_gptoss_alpha1_minus_clamped_silu_is_silu_of_clamped_gate():
+    g = torch.Generator().manual_seed(1)
+    gate, up = torch.randn(300, generator=g).double() * 5, torch.randn(300, generator=g).double() * 5
+    a = glu.glu_forward(gate, up, glu.CLAMPED_SILU, alpha=1.0, limit=3.0, up_plus_one=True)
+    b = glu.glu_forward(gate, up, glu.CLAMPED_SILU, limit=3.0)
+    assert torch.allclose(a - b, F.silu(gate.clamp(max=3.0)), atol=1e-12)
+
+
+def test_glu_bf16_is_fp32_math_rounded_once():
+    g = torch.Generator().manual_seed(2)
+    gate, up = torch.randn(256, generator=g).bfloat16(), torch.randn(256, generator=g).bfloat16()
+    want = (F.silu(gate.float()) * up.float()).bfloat16()
+    assert torch.equal(glu.glu_forward(gate, up, glu.SILU), want)
+
+
+# ------------------------------------------------------------------------------------------------ grouped GEMM
+
+@pytest.mark.parametrize("counts", ((7, 33, 0, 1, 64, 0), (0, 0, 0, 0, 105, 0), (5, 5, 5)))
+def test_grouped_mm_matches_matmul_and_autograd(counts):
+    torch.manual_seed(0)
+    total, k, n = sum(counts), 24, 20
+    a = torch.randn(total, k, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(len(counts), k, n, dtype=torch.float64, requires_grad=True)
+    offs = np.cumsum(counts).astype(np.int32)
+    pieces, start = [], 0
+    for e, c in enumerate(counts):
+        pieces.append(a[start:start + c] @ b[e])
+        start += c
+    want = torch.cat(pieces)
+    dout = torch.randn(total, n, dtype=torch.float64)
+    want.backward(dout)
+    kw = dict(acc_dtype=torch.float64)
+    assert torch.allclose(grouped_mm.grouped_mm(a.detach(), b.detach(), offs, **kw), want.detach(), atol=1e-12)
+    assert torch.allclose(grouped_mm.grouped_mm_dgrad(dout, b.detach(), offs, **kw), a.grad, atol=1e-12)
+    wgrad = grouped_mm.grouped_mm_wgrad(a.detach(), dout, offs, **kw)
+    assert torch.allclose(wgrad, b.grad, atol=1e-12)
+    for e, c in enumerate(counts):
+        assert (c == 0) == (not wgrad[e].any())
+
+
+# ------------------------------------------------------------------------------------------------------ router
+
+def test_router_selection_ties_go_to_the_lower_index():
+    logits = torch.tensor([[1.0, 1.0, 0.5, 1.0], [0.0, 2.0, 2.0, -1.0], [3.0, 3.0, 3.0, 3.0]])
+    assert router.select_topk(logits, 2).tolist() == [[0, 1], [1, 2], [0, 1]]
+    assert router.select_topk(logits, 3).tolist() == [[0, 1, 3], [1, 2, 0], [0, 1, 2]]
+
+
+def test_router_matches_torch_topk_on_tie_free_rows_and_in_bf16_ties():
+    g = torch.Generator().manual_seed(0)
+    logits = torch.randn(512, 64, generator=g)
+    idx, w = router.route(logits, 8, router.SOFTMAX_ALL, normalize=True, eps=0.0)
+    probs = torch.softmax(logits, dtype=torch.float, dim=-1)
+    top_v, top_i = torch.topk(probs, 8, dim=-1)
+    assert torch.equal(idx, top_i)
+    assert torch.equal(w, top_v / top_v.sum(-1, keepdim=True))
+    # bf16 logits tie often: selection must still be descending, lower index first among equals
+    lb = (torch.randn(2048, 128, generator=g) * 0.9).bfloat16()
+    idx_b, w_b = router.route(lb, 8)
+    picked = lb.float().gather(-1, idx_b)
+    assert (picked[:, :-1] >= picked[:, 1:]).all()
+    same = picked[:, :-1] == picked[:, 1:]
+    assert same.any(), "the case should contain ties"
+    assert (idx_b[:, :-1][same] < idx_b[:, 1:][same]).all()
+    kth = picked[:, -1:]
+    rest = lb.float().scatter(-1, idx_b, float("-inf"))
+    assert (rest <= kth).all()
+    tied_out = (rest == kth)
+    cols = torch.arange(128).expand_as(rest)
+    last_in = torch.where(picked == kth, idx_b, -1).max(-1, keepdim=True).values
+    assert (cols[tied_out] > last_in.expand_as(rest)[tied_out]).all()  # an excluded equal score sits at a higher index
+    assert w_b.dtype == torch.float32 and torch.equal(w_b, w_b.bfloat16().float())  # bf16 values stored in fp32
+
+
+def test_router_gptoss_mode_and_backward():
+    g = torch.Generator().manual_seed(1)
+    logits = torch.randn(64, 32, generator=g)
+    idx, w = router.route(logits, 4, router.SOFTMAX_TOPK)
+    top_v, top_i = torch.topk(logits, 4, dim=-1)
+    assert torch.equal(idx, top_i) and torch.allclose(w, torch.softmax(top_v, dim=-1))
+    gw = torch.randn(64, 4, generator=g)
+    for mode, norm in ((router.SOFTMAX_ALL, True), (router.SOFTMAX_ALL, False), (router.SOFTMAX_TOPK, False)):
+        leaf = logits.clone().requires_grad_(True)
+        if mode == router.SOFTMAX_TOPK:
+            ww = torch.softmax(leaf.gather(-1, idx), dim=-1)
+        else:
+            ww = torch.softmax(leaf, dim=-1).gather(-1, idx)
+            if norm:
+                ww = ww / ww.sum(-1, keepdim=True)
+        ww.backward(gw)
+        got = router.route_backward(logits, idx, gw, mode, norm, 0.0)
+        assert torch.allclose(got, leaf.grad, rtol=1e-4, atol=1e-6)
+
+
+# ------------------------------------------------------------------------------------------------- block fp8
+
+def test_e4m3_encoder_matches_torch_cast_on_every_code_and_on_random_values():
+    codes = np.arange(256, dtype=np.uint8)
+    finite = (codes & 0x7F) != 0x7F
+    decoded = block_fp8.decode_e4m3fn(codes[finite])
+    want = torch.from_numpy(codes[finite]).view(torch.float8_e4m3fn).float().numpy()
+    assert np.array_equal(decoded, want)
+    assert np.array_equal(block_fp8.encode_e4m3fn(decoded) & 0x7F, codes[finite] & 0x7F)
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(20000, generator=g) * torch.rand(20000, generator=g) * 300).clamp(-448, 448)
+    x = torch.cat([x, torch.tensor([0.0, 2.0**-9, 2.0**-10, 3 * 2.0**-10, 448.0, -448.0, 0.0009765625 * 1.5])])
+    got = block_fp8.encode_e4m3fn(x.numpy())
+    want = x.to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    nz = (want & 0x7F) != 0
+    assert np.array_equal(got[nz], want[nz]) and not (got[~nz] & 0x7F).any()
+
+
+def _diagnostic(w):
+    # the formula the reference's own test holds (tests/cpu/weight_sync/test_block_fp8.py:13-21)
+    n, k = w.shape
+    x = F.pad(w.float(), (0, (-k) % 128, 0, (-n) % 128))
+    xb = x.reshape(x.shape[0] // 128, 128, x.shape[1] // 128, 128)
+    amax = xb.abs().amax(dim=(1, 3), keepdim=True).clamp_min(1e-12)
+    scale = torch.exp2(torch.ceil(torch.log2(amax / 448.0)))
+    q = (xb / scale).clamp(-448, 448).to(torch.float8_e4m3fn).reshape(x.shape)[:n, :k].contiguous()
+    return q.view(torch.uint8).numpy(), scale[:, 0, :, 0].numpy()
+
+
+@pytest.mark.parametrize("shape", [(128, 128), (256, 384), (200, 130), (5, 7), (512, 64)])
+def test_block_quantiser_matches_the_diagnostic_formula(shape):
+    torch.manual_seed(0)
+    weight = (torch.randn(shape) * torch.rand(shape).mul(4)).bfloat16()
+    q, scale = block_fp8.quantize_block_fp8(weight.float().numpy())
+    ref_q, ref_scale = _diagnostic(weight)
+    assert np.array_equal(scale, ref_scale)
+    same = (q & 0x7F) == (ref_q & 0x7F)
+    assert same.all() and np.array_equal(q[(q & 0x7F) != 0], ref_q[(q & 0x7F) != 0])
+
+
+def test_block_quantiser_boundary_zero_block_and_leading_dims():
+    w = np.zeros((128, 256), dtype=np.float32)
+    w[0, 0] = 448.0 * 4
+    w[0, 128] = 448.0 * 4 * 1.0001
+    q, scale = block_fp8.quantize_block_fp8(w)
+    assert scale.tolist() == [[4.0, 8.0]]
+    q0, s0 = block_fp8.quantize_block_fp8(np.zeros((128, 128), dtype=np.float32))
+    assert np.isfinite(s0).all() and (s0 > 0).all() and not (q0 & 0x7F).any()
+    rng = np.random.default_rng(2)
+    bank = rng.standard_normal((3, 130, 129)).astype(np.float32)
+    qb, sb = block_fp8.quantize_block_fp8(bank)
+    assert qb.shape == bank.shape and sb.shape == (3, 2, 2)
+    for e in range(3):
+        q1, s1 = block_fp8.quantize_block_fp8(bank[e])
+        assert np.array_equal(qb[e], q1) and np.array_equal(sb[e], s1)
+    restored = block_fp8.dequantize_block_fp8(qb, sb)
+    assert (np.abs(restored - bank) <= np.abs(bank) * 0.0625 + sb.max() * 2.0**-9).all()
+
+
+# --------------------------------------------------------------------------------------------------- MoE layer
+
+@pytest.mark.parametrize("fused", (True, False))
+@pytest.mark.parametrize("kind", ("silu", "gptoss"))
+def test_layer_loop_matches_the_dense_formula(fused, kind):
+    g = torch.Generator().manual_seed(3)
+    T, H, E, K, Fw = 11, 8, 3, 2, 6
+    x = torch.randn(T, H, dtype=torch.float64, generator=g)
+    experts = torch.randint(-1, 5, (T, K), generator=g)  # -1 padding, 3..4 not local
+    weights = torch.rand(T, K, dtype=torch.float64, generator=g)
+    params = {"down_proj": torch.randn(E, Fw, H, dtype=torch.float64, generator=g)}
+    if fused:
+        params["gate_up_proj"] = torch.randn(E, H, 2 * Fw, dtype=torch.float64, generator=g)
+    else:
+        params["gate_proj"] = torch.randn(E, H, Fw, dtype=torch.float64, generator=g)
+        params["up_proj"] = torch.randn(E, H, Fw, dtype=torch.float64, generator=g)
+        params["gate_proj_bias"] = torch.randn(E, Fw, dtype=torch.float64, generator=g)
+        params["down_proj_bias"] = torch.randn(E, H, dtype=torch.float64, generator=g)
+    combine = moe_layer.Glu(kind, 1.702, 7.0) if kind == "gptoss" else moe_layer.Glu(kind)
+    got = moe_layer.compute_experts_loop(x, experts, weights, params, combine, E)
+    want = moe_layer.dense_formula(x, experts, weights, params, combine, E)
+    assert torch.allclose(got, want, atol=1e-10)
+
+
+def test_layer_forward_routes_and_adds_the_shared_expert():
+    g = torch.Generator().manual_seed(4)
+    T, H, E, K, Fw = 16, 8, 4, 2, 6
+    x = torch.randn(T, H, generator=g)
+    wr = torch.randn(E, H, generator=g)
+    params = {"gate_up_proj": torch.randn(E, H, 2 * Fw, generator=g) * 0.1,
+              "down_proj": torch.randn(E, Fw, H, generator=g) * 0.1}
+    shared = {"gate_proj": torch.randn(Fw, H, generator=g), "up_proj": torch.randn(Fw, H, generator=g),
+              "down_proj": torch.randn(H, Fw, generator=g), "shared_expert_gate": torch.randn(1, H, generator=g)}
+    out, logits, idx, w = moe_layer.moe_layer_forward(x, wr, params, moe_layer.Glu(), K, shared=shared)
+    routed, *_ = moe_layer.moe_layer_forward(x, wr, params, moe_layer.Glu(), K)
+    mlp = F.linear(F.silu(F.linear(x, shared["gate_proj"])) * F.linear(x, shared["up_proj"]), shared["down_proj"])
+    assert torch.allclose(out - routed, mlp * torch.sigmoid(x @ shared["shared_expert_gate"].t()), atol=1e-5)
+    assert torch.equal(idx, torch.topk(torch.softmax(logits, -1), K).indices)
+    assert torch.allclose(w.sum(-1), torch.ones(T))
