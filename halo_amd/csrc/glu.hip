@@ -1,0 +1,225 @@
+// Fused GLU combines and their gradients for gfx950: SiLU, tanh-GELU and the clamped SwiGLU family, over row-strided
+// gate / up operands so a packed [gate | up] projection is read in place and its gradient written as one buffer.
+// fp32 math, 16-byte accesses, one thread per 16 bytes of output.
+//
+// Replaces _glu_fwd_kernel / _glu_bwd_kernel (halo/kernels/fused_glu.py:118-205) of the reference.
+#include "common.h"
+
+namespace hmoe {
+namespace {
+
+constexpr int kThreads = 256;
+
+struct GluParams {
+  float alpha;
+  float limit;
+};
+
+__device__ __forceinline__ float fast_sigmoid(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+__device__ __forceinline__ float fast_tanh(float x) { return 1.0f - 2.0f * __builtin_amdgcn_rcpf(__expf(2.0f * x) + 1.0f); }
+
+constexpr float kSqrt2OverPi = 0.7978845608028654f;
+constexpr float kGeluCoeff = 0.044715f;
+
+// kAct: hmoe_glu_activation.  kClampAct / kPlusOne only matter for the clamped family.
+template <int kAct, bool kClampAct, bool kPlusOne>
+__device__ __forceinline__ float glu_value(float g, float u, GluParams p) {
+  if constexpr (kAct == HMOE_GLU_SILU) {
+    return g * fast_sigmoid(g) * u;
+  } else if constexpr (kAct == HMOE_GLU_GELU_TANH) {
+    const float t = fast_tanh(kSqrt2OverPi * (g + kGeluCoeff * g * g * g));
+    return 0.5f * g * (1.0f + t) * u;
+  } else {
+    float ug = fminf(fmaxf(u, -p.limit), p.limit);
+    if constexpr (kPlusOne) ug += 1.0f;
+    const float ga = kClampAct ? g : fminf(g, p.limit);
+    const float glu = ga * fast_sigmoid(ga * p.alpha);
+    const float act = kClampAct ? fminf(glu, p.limit) : glu;
+    return act * ug;
+  }
+}
+
+template <int kAct, bool kClampAct, bool kPlusOne>
+__device__ __forceinline__ void glu_grad(float g, float u, float d, GluParams p, float& dg, float& du) {
+  if constexpr (kAct == HMOE_GLU_SILU) {
+    const float s = fast_sigmoid(g);
+    dg = d * u * (s * (1.0f + g * (1.0f - s)));
+    du = d * (g * s);
+  } else if constexpr (kAct == HMOE_GLU_GELU_TANH) {
+    const float t = fast_tanh(kSqrt2OverPi * (g + kGeluCoeff * g * g * g));
+    const float inner = kSqrt2OverPi * (1.0f + 3.0f * kGeluCoeff * (g * g));
+    dg = d * u * (0.5f * (1.0f + t) + 0.5f * g * (1.0f - t * t) * inner);
+    du = d * (0.5f * g * (1.0f + t));
+  } else {
+    float ug = fminf(fmaxf(u, -p.limit), p.limit);
+    if constexpr (kPlusOne) ug += 1.0f;
+    const float ga = kClampAct ? g : fminf(g, p.limit);
+    const float s = fast_sigmoid(ga * p.alpha);
+    const float glu = ga * s;
+    const float act = kClampAct ? fminf(glu, p.limit) : glu;
+    const float dglu = s + ga * p.alpha * s * (1.0f - s);
+    // a clamp passes its gradient on the closed interval, the bound included
+    const float up_in = (u >= -p.limit && u <= p.limit) ? 1.0f : 0.0f;
+    const float gate_in = (kClampAct ? (glu <= p.limit) : (g <= p.limit)) ? 1.0f : 0.0f;
+    dg = d * ug * dglu * gate_in;
+    du = d * act * up_in;
+  }
+}
+
+template <typename T, int W>
+struct Chunk {
+  float v[W];
+  __device__ __forceinline__ void load(const T* p) {
+    if constexpr (W == 1) {
+      v[0] = Elem<T>::load(p);
+    } else {
+      Vec16<T> t;
+      t.load(p);
+#pragma unroll
+      for (int i = 0; i < W; ++i) v[i] = t.v[i];
+    }
+  }
+  __device__ __forceinline__ void store(T* p) const {
+    if constexpr (W == 1) {
+      Elem<T>::store(p, v[0]);
+    } else {
+      Vec16<T> t;
+#pragma unroll
+      for (int i = 0; i < W; ++i) t.v[i] = v[i];
+      t.store(p);
+    }
+  }
+};
+
+template <typename T, int W, int kAct, bool kClampAct, bool kPlusOne>
+__global__ void __launch_bounds__(kThreads)
+glu_fwd_kernel(const T* __restrict__ gate, const T* __restrict__ up, T* __restrict__ out, int64_t stride_gate,
+               int64_t stride_up, int64_t n_rows, int64_t chunks_per_row, int64_t width, GluParams p) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t row = i / chunks_per_row;
+  if (row >= n_rows) return;
+  const int64_t col = (i - row * chunks_per_row) * W;
+  Chunk<T, W> g, u, o;
+  g.load(gate + row * stride_gate + col);
+  u.load(up + row * stride_up + col);
+#pragma unroll
+  for (int k = 0; k < W; ++k) o.v[k] = glu_value<kAct, kClampAct, kPlusOne>(g.v[k], u.v[k], p);
+  o.store(out + row * width + col);
+}
+
+template <typename T, int W, int kAct, bool kClampAct, bool kPlusOne>
+__global__ void __launch_bounds__(kThreads)
+glu_bwd_kernel(const T* __restrict__ gate, const T* __restrict__ up, const T* __restrict__ grad_out,
+               T* __restrict__ dgate, T* __restrict__ dup, int64_t stride_gate, int64_t stride_up,
+               int64_t stride_dgate, int64_t stride_dup, int64_t n_rows, int64_t chunks_per_row, int64_t width,
+               GluParams p) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t row = i / chunks_per_row;
+  if (row >= n_rows) return;
+  const int64_t col = (i - row * chunks_per_row) * W;
+  Chunk<T, W> g, u, d, dg, du;
+  g.load(gate + row * stride_gate + col);
+  u.load(up + row * stride_up + col);
+  d.load(grad_out + row * width + col);
+#pragma unroll
+  for (int k = 0; k < W; ++k) glu_grad<kAct, kClampAct, kPlusOne>(g.v[k], u.v[k], d.v[k], p, dg.v[k], du.v[k]);
+  dg.store(dgate + row * stride_dgate + col);
+  du.store(dup + row * stride_dup + col);
+}
+
+struct GluArgs {
+  const void *gate, *up, *grad_out;
+  void *out, *dgate, *dup;
+  int64_t stride_gate, stride_up, stride_dgate, stride_dup, n_rows, width;
+  GluParams p;
+  bool backward;
+  hipStream_t stream;
+};
+
+template <typename T, int W, int kAct, bool kClampAct, bool kPlusOne>
+void launch(const GluArgs& a) {
+  const int64_t chunks = a.width / W;
+  const int64_t total = chunks * a.n_rows;
+  const dim3 grid(static_cast<unsigned>((total + kThreads - 1) / kThreads)), block(kThreads);
+  if (!a.backward)
+    glu_fwd_kernel<T, W, kAct, kClampAct, kPlusOne><<<grid, block, 0, a.stream>>>(
+        static_cast<const T*>(a.gate), static_cast<const T*>(a.up), static_cast<T*>(a.out), a.stride_gate,
+        a.stride_up, a.n_rows, chunks, a.width, a.p);
+  else
+    glu_bwd_kernel<T, W, kAct, kClampAct, kPlusOne><<<grid, block, 0, a.stream>>>(
+        static_cast<const T*>(a.gate), static_cast<const T*>(a.up), static_cast<const T*>(a.grad_out),
+        static_cast<T*>(a.dgate), static_cast<T*>(a.dup), a.stride_gate, a.stride_up, a.stride_dgate, a.stride_dup,
+        a.n_rows, chunks, a.width, a.p);
+}
+
+template <typename T, int W>
+int launch_activation(const GluArgs& a, int activation, int clamp_activated, int up_plus_one) {
+  if (activation == HMOE_GLU_SILU) launch<T, W, HMOE_GLU_SILU, false, false>(a);
+  else if (activation == HMOE_GLU_GELU_TANH) launch<T, W, HMOE_GLU_GELU_TANH, false, false>(a);
+  else if (activation == HMOE_GLU_CLAMPED_SILU) {
+    if (clamp_activated && up_plus_one) launch<T, W, HMOE_GLU_CLAMPED_SILU, true, true>(a);
+    else if (clamp_activated) launch<T, W, HMOE_GLU_CLAMPED_SILU, true, false>(a);
+    else if (up_plus_one) launch<T, W, HMOE_GLU_CLAMPED_SILU, false, true>(a);
+    else launch<T, W, HMOE_GLU_CLAMPED_SILU, false, false>(a);
+  } else {
+    return HMOE_INVALID_ARGUMENT;
+  }
+  if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
+  return HMOE_OK;
+}
+
+int run(const GluArgs& a, int dtype, int activation, int clamp_activated, int up_plus_one) {
+  if (a.n_rows < 0 || a.width < 0) return HMOE_INVALID_ARGUMENT;
+  if (a.n_rows == 0 || a.width == 0) return HMOE_OK;
+  if (!a.gate || !a.up) return HMOE_INVALID_ARGUMENT;
+  if (a.backward ? (!a.grad_out || !a.dgate || !a.dup) : !a.out) return HMOE_INVALID_ARGUMENT;
+  if (a.n_rows * a.width / 1 >= (int64_t(1) << 40)) return HMOE_UNSUPPORTED;
+  const int64_t w = dtype == HMOE_BF16 ? 8 : 4;
+  bool vec = a.width % w == 0 && a.stride_gate % w == 0 && a.stride_up % w == 0 && aligned16(a.gate) &&
+             aligned16(a.up);
+  if (a.backward)
+    vec = vec && a.stride_dgate % w == 0 && a.stride_dup % w == 0 && aligned16(a.grad_out) && aligned16(a.dgate) &&
+          aligned16(a.dup);
+  else
+    vec = vec && aligned16(a.out);
+  if (dtype == HMOE_BF16)
+    return vec ? launch_activation<bf16_t, 8>(a, activation, clamp_activated, up_plus_one)
+               : launch_activation<bf16_t, 1>(a, activation, clamp_activated, up_plus_one);
+  if (dtype == HMOE_F32)
+    return vec ? launch_activation<float, 4>(a, activation, clamp_activated, up_plus_one)
+               : launch_activation<float, 1>(a, activation, clamp_activated, up_plus_one);
+  return HMOE_UNSUPPORTED;
+}
+
+}  // namespace
+}  // namespace hmoe
+
+extern "C" {
+
+int hmoe_glu_fwd(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up, int64_t n_rows,
+                 int64_t width, int dtype, int activation, float alpha, float limit, int clamp_activated,
+                 int up_plus_one, void* out, void* stream) {
+  hmoe::GluArgs a{};
+  a.gate = gate; a.up = up; a.out = out;
+  a.stride_gate = stride_gate; a.stride_up = stride_up; a.n_rows = n_rows; a.width = width;
+  a.p = {alpha, limit};
+  a.backward = false;
+  a.stream = static_cast<hipStream_t>(stream);
+  return hmoe::run(a, dtype, activation, clamp_activated, up_plus_one);
+}
+
+int hmoe_glu_bwd(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up, const void* grad_out,
+                 int64_t n_rows, int64_t width, int dtype, int activation, float alpha, float limit,
+                 int clamp_activated, int up_plus_one, void* dgate, void* dup, int64_t stride_dgate,
+                 int64_t stride_dup, void* stream) {
+  hmoe::GluArgs a{};
+  a.gate = gate; a.up = up; a.grad_out = grad_out; a.dgate = dgate; a.dup = dup;
+  a.stride_gate = stride_gate; a.stride_up = stride_up; a.stride_dgate = stride_dgate; a.stride_dup = stride_dup;
+  a.n_rows = n_rows; a.width = width;
+  a.p = {alpha, limit};
+  a.backward = true;
+  a.stream = static_cast<hipStream_t>(stream);
+  return hmoe::run(a, dtype, activation, clamp_activated, up_plus_one);
+}
+
+}  // extern "C"

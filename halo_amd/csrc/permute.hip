@@ -1,0 +1,295 @@
+// Token permute / weighted unpermute (combine) / expert-bias gradient for gfx950.  All four kernels stream rows:
+// one wavefront per row, 16-byte accesses per lane, fp32 accumulation, one rounding.  No atomics.
+//
+// Replaces of the reference: tokens.index_select (halo/kernels/moe_permute.py:133-136), _gather_reduce_kernel
+// (:17-41), _weighted_unpermute_bwd_kernel (:44-72) and MoEExpertBiasGather.backward's one-hot GEMM (:202-208).
+#include "common.h"
+
+namespace hmoe {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kRowsPerBlock = kThreads / HMOE_WAVE;
+
+// W consecutive elements of T held as floats; W is 16 bytes' worth when rows are 16-byte aligned, else 1.
+template <typename T, int W>
+struct Pack {
+  float v[W];
+  __device__ __forceinline__ void load(const T* p) {
+    if constexpr (W == 1) {
+      v[0] = Elem<T>::load(p);
+    } else {
+      Vec16<T> t;
+      t.load(p);
+#pragma unroll
+      for (int i = 0; i < W; ++i) v[i] = t.v[i];
+    }
+  }
+  __device__ __forceinline__ void store(T* p) const {
+    if constexpr (W == 1) {
+      Elem<T>::store(p, v[0]);
+    } else {
+      Vec16<T> t;
+#pragma unroll
+      for (int i = 0; i < W; ++i) t.v[i] = v[i];
+      t.store(p);
+    }
+  }
+};
+
+// Raw 16-byte (or one-element) copy chunk: a gather moves bits, it never converts.
+template <typename T, int W>
+struct Raw {
+  using V = typename std::conditional<W == 1, T, uint4>::type;
+  V bits;
+  __device__ __forceinline__ void load(const T* p) { bits = *reinterpret_cast<const V*>(p); }
+  __device__ __forceinline__ void store(T* p) const { *reinterpret_cast<V*>(p) = bits; }
+};
+
+template <typename T, int W>
+__global__ void __launch_bounds__(kThreads)
+gather_rows_kernel(const T* __restrict__ src, int64_t src_stride, const int64_t* __restrict__ index,
+                   T* __restrict__ out, int64_t n_out, int64_t hidden) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / HMOE_WAVE;
+  if (row >= n_out) return;
+  const T* from = src + index[row] * src_stride;
+  T* to = out + row * hidden;
+  const int64_t step = static_cast<int64_t>(HMOE_WAVE) * W;
+  int64_t c = static_cast<int64_t>(lane_id()) * W;
+  for (; c + 3 * step < hidden; c += 4 * step) {  // four loads in flight per lane
+    Raw<T, W> a, b, d, e;
+    a.load(from + c);
+    b.load(from + c + step);
+    d.load(from + c + 2 * step);
+    e.load(from + c + 3 * step);
+    a.store(to + c);
+    b.store(to + c + step);
+    d.store(to + c + 2 * step);
+    e.store(to + c + 3 * step);
+  }
+  for (; c < hidden; c += step) {
+    Raw<T, W> a;
+    a.load(from + c);
+    a.store(to + c);
+  }
+}
+
+template <typename T, int W, bool kWeighted>
+__global__ void __launch_bounds__(kThreads)
+gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, const int64_t* __restrict__ inv_map,
+                     T* __restrict__ out, int64_t n_out, int top_k, int64_t n_src, int64_t hidden) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / HMOE_WAVE;
+  if (row >= n_out) return;
+  const int64_t* map = inv_map + row * top_k;
+  T* to = out + row * hidden;
+  const int64_t step = static_cast<int64_t>(HMOE_WAVE) * W;
+  for (int64_t c = static_cast<int64_t>(lane_id()) * W; c < hidden; c += step) {
+    Pack<T, W> acc;
+#pragma unroll
+    for (int i = 0; i < W; ++i) acc.v[i] = 0.f;
+    for (int k = 0; k < top_k; ++k) {
+      const int64_t j = map[k];
+      if (j >= 0 && j < n_src) {
+        Pack<T, W> x;
+        x.load(src + j * hidden + c);
+        if constexpr (kWeighted) {
+          const float w = Elem<T>::load(weight + j);
+#pragma unroll
+          for (int i = 0; i < W; ++i) acc.v[i] += x.v[i] * w;
+        } else {
+#pragma unroll
+          for (int i = 0; i < W; ++i) acc.v[i] += x.v[i];
+        }
+      }
+    }
+    acc.store(to + c);
+  }
+}
+
+template <typename T, int W>
+__global__ void __launch_bounds__(kThreads)
+unpermute_bwd_kernel(const T* __restrict__ grad_out, int64_t grad_stride, const T* __restrict__ expert_out,
+                     const T* __restrict__ weights, const int64_t* __restrict__ token_idx,
+                     T* __restrict__ grad_expert, float* __restrict__ grad_weights, int64_t n_sorted,
+                     int64_t hidden) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / HMOE_WAVE;
+  if (row >= n_sorted) return;
+  const T* g = grad_out + token_idx[row] * grad_stride;
+  const float w = Elem<T>::load(weights + row);
+  const bool want_dot = expert_out != nullptr && grad_weights != nullptr;
+  const T* y = want_dot ? expert_out + row * hidden : nullptr;
+  T* to = grad_expert + row * hidden;
+  float dot = 0.f;
+  const int64_t step = static_cast<int64_t>(HMOE_WAVE) * W;
+  for (int64_t c = static_cast<int64_t>(lane_id()) * W; c < hidden; c += step) {
+    Pack<T, W> gv, ov;
+    gv.load(g + c);
+    if (want_dot) {
+      Pack<T, W> yv;
+      yv.load(y + c);
+#pragma unroll
+      for (int i = 0; i < W; ++i) dot += gv.v[i] * yv.v[i];
+    }
+#pragma unroll
+    for (int i = 0; i < W; ++i) ov.v[i] = gv.v[i] * w;
+    ov.store(to + c);
+  }
+  if (want_dot) {
+    dot = wave_sum(dot);
+    if (lane_id() == 0) grad_weights[row] = dot;
+  }
+}
+
+// grid (num_experts, column chunks).  The four wavefronts of a workgroup take every fourth row of the expert's
+// contiguous row range (found by bisection on the sorted ids) and their partial sums meet in LDS.
+template <typename T, int W>
+__global__ void __launch_bounds__(kThreads)
+expert_colsum_kernel(const T* __restrict__ grad_out, const int64_t* __restrict__ eids, T* __restrict__ grad_bias,
+                     int64_t n_rows, int64_t width) {
+  __shared__ float partial[kRowsPerBlock][HMOE_WAVE * W];
+  const int e = blockIdx.x;
+  auto lower_bound = [&](int64_t key) {
+    int64_t lo = 0, hi = n_rows;
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) >> 1;
+      if (eids[mid] < key) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+  };
+  const int64_t begin = lower_bound(e), end = lower_bound(static_cast<int64_t>(e) + 1);
+  const int wave = threadIdx.x / HMOE_WAVE;
+  const int64_t c = (static_cast<int64_t>(blockIdx.y) * HMOE_WAVE + lane_id()) * W;
+  Pack<T, W> acc;
+#pragma unroll
+  for (int i = 0; i < W; ++i) acc.v[i] = 0.f;
+  if (c < width) {
+    for (int64_t r = begin + wave; r < end; r += kRowsPerBlock) {
+      Pack<T, W> x;
+      x.load(grad_out + r * width + c);
+#pragma unroll
+      for (int i = 0; i < W; ++i) acc.v[i] += x.v[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < W; ++i) partial[wave][lane_id() * W + i] = acc.v[i];
+  __syncthreads();
+  if (wave == 0 && c < width) {
+    Pack<T, W> sum;
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+      const int at = lane_id() * W + i;
+      sum.v[i] = (partial[0][at] + partial[1][at]) + (partial[2][at] + partial[3][at]);
+    }
+    sum.store(grad_bias + static_cast<int64_t>(e) * width + c);
+  }
+}
+
+template <typename T>
+bool rows_vectorizable(int64_t hidden, std::initializer_list<int64_t> strides, std::initializer_list<const void*> ptrs) {
+  constexpr int W = 16 / sizeof(T);
+  if (hidden % W) return false;
+  for (int64_t s : strides)
+    if (s % W) return false;
+  for (const void* p : ptrs)
+    if (p && !aligned16(p)) return false;
+  return true;
+}
+
+dim3 row_grid(int64_t rows) { return dim3(static_cast<unsigned>((rows + kRowsPerBlock - 1) / kRowsPerBlock)); }
+
+}  // namespace
+}  // namespace hmoe
+
+using namespace hmoe;
+
+#define HMOE_DISPATCH_ROWS(DTYPE, VEC_OK, CALL)                      \
+  if ((DTYPE) == HMOE_BF16) {                                        \
+    using T = bf16_t;                                                \
+    if (VEC_OK) { constexpr int W = 8; CALL; } else { constexpr int W = 1; CALL; } \
+  } else if ((DTYPE) == HMOE_F32) {                                  \
+    using T = float;                                                 \
+    if (VEC_OK) { constexpr int W = 4; CALL; } else { constexpr int W = 1; CALL; } \
+  } else {                                                           \
+    return HMOE_UNSUPPORTED;                                         \
+  }
+
+extern "C" {
+
+int hmoe_gather_rows(const void* src, int64_t src_row_stride, const int64_t* index, int64_t n_out, int64_t hidden,
+                     int dtype, void* out, void* stream) {
+  if (n_out < 0 || hidden < 0 || src_row_stride < 0) return HMOE_INVALID_ARGUMENT;
+  if (n_out == 0 || hidden == 0) return HMOE_OK;
+  if (!src || !index || !out) return HMOE_INVALID_ARGUMENT;
+  if (n_out > (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool vec = dtype == HMOE_BF16 ? rows_vectorizable<bf16_t>(hidden, {src_row_stride}, {src, out})
+                                      : rows_vectorizable<float>(hidden, {src_row_stride}, {src, out});
+  HMOE_DISPATCH_ROWS(dtype, vec,
+                     (gather_rows_kernel<T, W><<<row_grid(n_out), dim3(kThreads), 0, s>>>(
+                         static_cast<const T*>(src), src_row_stride, index, static_cast<T*>(out), n_out, hidden)));
+  HMOE_CHECK_LAUNCH();
+  return HMOE_OK;
+}
+
+int hmoe_gather_reduce(const void* src, const void* weight, const int64_t* inv_map, int64_t n_out, int top_k,
+                       int64_t n_src, int64_t hidden, int dtype, void* out, void* stream) {
+  if (n_out < 0 || hidden < 0 || n_src < 0 || top_k < 0) return HMOE_INVALID_ARGUMENT;
+  if (n_out == 0 || hidden == 0) return HMOE_OK;
+  if (!out || (top_k > 0 && !inv_map) || (n_src > 0 && !src)) return HMOE_INVALID_ARGUMENT;
+  if (n_out > (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool vec = dtype == HMOE_BF16 ? rows_vectorizable<bf16_t>(hidden, {}, {src, out})
+                                      : rows_vectorizable<float>(hidden, {}, {src, out});
+  if (weight) {
+    HMOE_DISPATCH_ROWS(dtype, vec,
+                       (gather_reduce_kernel<T, W, true><<<row_grid(n_out), dim3(kThreads), 0, s>>>(
+                           static_cast<const T*>(src), static_cast<const T*>(weight), inv_map, static_cast<T*>(out),
+                           n_out, top_k, n_src, hidden)));
+  } else {
+    HMOE_DISPATCH_ROWS(dtype, vec,
+                       (gather_reduce_kernel<T, W, false><<<row_grid(n_out), dim3(kThreads), 0, s>>>(
+                           static_cast<const T*>(src), nullptr, inv_map, static_cast<T*>(out), n_out, top_k, n_src,
+                           hidden)));
+  }
+  HMOE_CHECK_LAUNCH();
+  return HMOE_OK;
+}
+
+int hmoe_unpermute_bwd(const void* grad_out, int64_t grad_out_row_stride, const void* expert_out,
+                       const void* weights, const int64_t* token_idx, int64_t n_sorted, int64_t hidden, int dtype,
+                       void* grad_expert, float* grad_weights, void* stream) {
+  if (n_sorted < 0 || hidden < 0 || grad_out_row_stride < 0) return HMOE_INVALID_ARGUMENT;
+  if (n_sorted == 0) return HMOE_OK;
+  if (!grad_out || !weights || !token_idx || !grad_expert) return HMOE_INVALID_ARGUMENT;
+  if ((expert_out == nullptr) != (grad_weights == nullptr)) return HMOE_INVALID_ARGUMENT;
+  if (n_sorted > (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool vec = dtype == HMOE_BF16
+                       ? rows_vectorizable<bf16_t>(hidden, {grad_out_row_stride}, {grad_out, expert_out, grad_expert})
+                       : rows_vectorizable<float>(hidden, {grad_out_row_stride}, {grad_out, expert_out, grad_expert});
+  HMOE_DISPATCH_ROWS(dtype, vec,
+                     (unpermute_bwd_kernel<T, W><<<row_grid(n_sorted), dim3(kThreads), 0, s>>>(
+                         static_cast<const T*>(grad_out), grad_out_row_stride, static_cast<const T*>(expert_out),
+                         static_cast<const T*>(weights), token_idx, static_cast<T*>(grad_expert), grad_weights,
+                         n_sorted, hidden)));
+  HMOE_CHECK_LAUNCH();
+  return HMOE_OK;
+}
+
+int hmoe_expert_colsum(const void* grad_out, const int64_t* eids, int64_t n_rows, int64_t width, int num_experts,
+                       int dtype, void* grad_bias, void* stream) {
+  if (n_rows < 0 || width < 0 || num_experts < 0) return HMOE_INVALID_ARGUMENT;
+  if (num_experts == 0 || width == 0) return HMOE_OK;
+  if (!grad_bias || (n_rows > 0 && (!grad_out || !eids))) return HMOE_INVALID_ARGUMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool vec = dtype == HMOE_BF16 ? rows_vectorizable<bf16_t>(width, {}, {grad_out, grad_bias})
+                                      : rows_vectorizable<float>(width, {}, {grad_out, grad_bias});
+  HMOE_DISPATCH_ROWS(dtype, vec,
+                     (expert_colsum_kernel<T, W><<<dim3(num_experts, (width + HMOE_WAVE * W - 1) / (HMOE_WAVE * W)),
+                                                  dim3(kThreads), 0, s>>>(
+                         static_cast<const T*>(grad_out), eids, static_cast<T*>(grad_bias), n_rows, width)));
+  HMOE_CHECK_LAUNCH();
+  return HMOE_OK;
+}
+
+}  // extern "C"

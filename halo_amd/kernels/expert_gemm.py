@@ -1,0 +1,73 @@
+"""Grouped GEMM for MoE expert FFNs, by weight format: bf16/fp32 (the training path), or block-fp8 weights (the
+quantised-weight serving configuration, forward only).
+
+Mirrors the dispatch seam of the reference's ``halo/kernels/expert_gemm.py:14-38``.  The reference's other
+``quant_format`` values name its fake-quant QAT formats (mxfp8 / mxfp4 / nvfp4), which are not part of this path.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from halo_amd import _lib
+from halo_amd.kernels.grouped_mm import _offs_arg, _rows, grouped_mm
+
+
+class BlockFp8Weight:
+    """Expert weights ``[G, K, N]`` as float8_e4m3fn with one fp32 power-of-two scale per 128x128 block
+    (``halo_amd.kernels.lowp.block_fp8.quantize_block_fp8`` of the matmul-convention weight)."""
+
+    def __init__(self, q: torch.Tensor, scale_inv: torch.Tensor):
+        if q.dim() != 3 or scale_inv.dim() != 3:
+            raise ValueError("expected q [G, K, N] and scale_inv [G, ceil(K/128), ceil(N/128)]")
+        g, k, n = q.shape
+        if tuple(scale_inv.shape) != (g, -(-k // 128), -(-n // 128)):
+            raise ValueError(f"scale grid {tuple(scale_inv.shape)} does not match weight {tuple(q.shape)}")
+        self.q = q.contiguous()
+        self.scale_inv = scale_inv.float().contiguous()
+
+    @property
+    def shape(self):
+        return self.q.shape
+
+
+def expert_gemm(
+    mat_a: torch.Tensor,
+    mat_b,
+    *,
+    offs: torch.Tensor | None = None,
+    quant_format=None,
+    weight_cacheable: bool = True,
+) -> torch.Tensor:
+    """``[total_tokens, K]`` activations stacked by expert times ``[num_experts, K, N]`` weights.  ``mat_b`` may be a
+    :class:`BlockFp8Weight` (or ``quant_format == "block_fp8"`` with ``mat_b = (q, scale_inv)``): bf16 activations
+    against fp8 weights dequantised on their way into the MFMA tiles, forward only."""
+    if isinstance(mat_b, BlockFp8Weight) or quant_format == "block_fp8":
+        weight = mat_b if isinstance(mat_b, BlockFp8Weight) else BlockFp8Weight(*mat_b)
+        return _fp8w_forward(mat_a, weight, offs)
+    if quant_format is not None:
+        raise NotImplementedError(
+            f"quant_format={quant_format!r}: the reference's fake-quant QAT formats are not part of the expert path"
+        )
+    return grouped_mm(mat_a, mat_b, offs=offs)
+
+
+def _fp8w_forward(mat_a: torch.Tensor, weight: BlockFp8Weight, offs: torch.Tensor | None) -> torch.Tensor:
+    device = _lib.require_device(mat_a, weight.q, weight.scale_inv, offs)
+    if mat_a.dtype != torch.bfloat16:
+        raise TypeError(f"block-fp8 expert GEMM takes bf16 activations, got {mat_a.dtype}")
+    if mat_a.requires_grad and torch.is_grad_enabled():
+        raise RuntimeError("the block-fp8 expert GEMM is forward only")
+    groups, k, n = weight.shape
+    rows = mat_a.shape[0]
+    out = torch.empty((rows, n), dtype=torch.bfloat16, device=device)
+    if rows == 0 or n == 0:
+        return out
+    mat_a = _rows(mat_a)
+    offs32 = _offs_arg(offs, groups)
+    q = weight.q.view(torch.uint8)
+    with _lib.on_device(device):
+        _lib.call("hmoe_grouped_gemm_fwd_fp8w", _lib.ptr(mat_a), mat_a.stride(0), _lib.ptr(q),
+                  _lib.ptr(weight.scale_inv), _lib.ptr(offs32), rows, groups, k, n, _lib.ptr(out), out.stride(0),
+                  _lib.stream_ptr(device))
+    return out

@@ -1,0 +1,35 @@
+"""Sync-free histograms for MoE routing (no host readback, no atomics on global memory).
+
+Mirrors the reference's ``halo/kernels/histogram.py:9-26``; the kernel is ``hmoe_bincount`` in
+``csrc/route_sort.hip`` (one workgroup, LDS counters).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from halo_amd import _lib
+
+
+def sync_free_bincount(
+    indices: torch.Tensor, size: int, *, dtype: torch.dtype = torch.float32, weights: torch.Tensor | None = None
+) -> torch.Tensor:
+    """Counts (or weight sums) of each value in ``[0, size)``; values outside the range are ignored.  ``dtype`` is
+    fp32 where counts feed metric math, int64 where they become offsets."""
+    device = _lib.require_device(indices, weights)
+    flat = indices.flatten().long().contiguous()
+    native = torch.int64 if (weights is None and not dtype.is_floating_point) else torch.float32
+    w = None if weights is None else weights.flatten().float().contiguous()
+    out = torch.empty(size, dtype=native, device=device)
+    with _lib.on_device(device):
+        _lib.call("hmoe_bincount", _lib.ptr(flat), _lib.ptr(w), flat.numel(), size, int(native == torch.int64),
+                  _lib.ptr(out), _lib.stream_ptr(device))
+    return out if out.dtype == dtype else out.to(dtype)
+
+
+def accumulate_bincount(
+    counter: torch.Tensor | None, indices: torch.Tensor, size: int, *, weights: torch.Tensor | None = None
+) -> torch.Tensor:
+    """``counter`` is ``None`` until the first forward that routes and is added into in place afterwards."""
+    counts = sync_free_bincount(indices, size, weights=weights)
+    return counts if counter is None else counter.add_(counts)

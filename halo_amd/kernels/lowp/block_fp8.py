@@ -1,0 +1,69 @@
+"""DeepSeek-style block FP8 for served weights: float8_e4m3fn values with one fp32 power-of-two scale per 128x128
+block, stored beside the weight as ``<weight>_scale_inv``.
+
+Mirrors the reference's ``halo/kernels/lowp/block_fp8.py:16-34`` and the dequantiser of
+``halo/checkpoint/tools/fp8_dequant.py:153-170``; the kernels are ``csrc/quant.hip``.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from halo_amd import _lib
+
+BLOCK = 128
+SCALE_SUFFIX = "_scale_inv"
+E4M3_MAX = 448.0
+
+
+def quantize_block_fp8(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(q, scale_inv)`` for ``weight`` ``[..., N, K]``: ``q`` has its shape in float8_e4m3fn, ``scale_inv`` is fp32
+    ``[..., ceil(N/128), ceil(K/128)]`` and ``q * scale_inv`` (broadcast over blocks) reconstructs the weight."""
+    device = _lib.require_device(weight)
+    if weight.dim() < 2:
+        raise ValueError("quantize_block_fp8 expects at least a 2-D weight")
+    if weight.dtype not in (torch.float32, torch.bfloat16):
+        weight = weight.float()
+    weight = weight.contiguous()
+    n, k = weight.shape[-2:]
+    lead = weight.shape[:-2]
+    batch = 1
+    for d in lead:
+        batch *= d
+    q = torch.empty(weight.shape, dtype=torch.uint8, device=device)
+    scale = torch.empty((*lead, -(-n // BLOCK), -(-k // BLOCK)), dtype=torch.float32, device=device)
+    with _lib.on_device(device):
+        _lib.call("hmoe_quantize_block_fp8", _lib.ptr(weight), _lib.dtype_id(weight.dtype), batch, n, k, _lib.ptr(q),
+                  _lib.ptr(scale), _lib.stream_ptr(device))
+    return q.view(torch.float8_e4m3fn), scale
+
+
+def dequantize_block_fp8(weight: torch.Tensor, scale_inv: torch.Tensor, dtype: torch.dtype = torch.bfloat16
+                         ) -> torch.Tensor:
+    """``weight * scale_inv`` per 128x128 block in fp32, rounded once to ``dtype``."""
+    device = _lib.require_device(weight, scale_inv)
+    weight = weight.contiguous()
+    n, k = weight.shape[-2:]
+    lead = weight.shape[:-2]
+    batch = 1
+    for d in lead:
+        batch *= d
+    if tuple(scale_inv.shape) != (*lead, -(-n // BLOCK), -(-k // BLOCK)):
+        raise ValueError(f"scale grid {tuple(scale_inv.shape)} does not match weight {tuple(weight.shape)}")
+    out = torch.empty(weight.shape, dtype=dtype, device=device)
+    scale_inv = scale_inv.float().contiguous()
+    with _lib.on_device(device):
+        _lib.call("hmoe_dequantize_block_fp8", _lib.ptr(weight.view(torch.uint8)), _lib.ptr(scale_inv), batch, n, k,
+                  _lib.dtype_id(dtype), _lib.ptr(out), _lib.stream_ptr(device))
+    return out
+
+
+def block_fp8_quantization_config(modules_to_not_convert: list[str]) -> dict:
+    """The ``config.json`` ``quantization_config`` serving engines read for such a checkpoint."""
+    return {
+        "quant_method": "fp8",
+        "fmt": "e4m3",
+        "activation_scheme": "dynamic",
+        "weight_block_size": [BLOCK, BLOCK],
+        "modules_to_not_convert": sorted(modules_to_not_convert),
+    }

@@ -1,0 +1,152 @@
+"""Atomic-free token permute/unpermute and per-expert bias gather for the grouped-GEMM MoE expert compute.  Both
+directions reduce through ``inv_map`` in fp32 and round once.
+
+Mirrors the reference's ``halo/kernels/moe_permute.py`` (``build_inv_map`` ``:75-89``, ``gather_reduce_rows``
+``:123-127``, ``MoEGatherPermute`` ``:130-141``, ``MoEWeightedUnpermute`` ``:144-189``, ``MoEExpertBiasGather``
+``:192-208``); the kernels are ``csrc/permute.hip``.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from halo_amd import _lib
+
+
+def _gather_rows(src: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+    """``src[index]`` for a 2-D ``src`` whose rows may be strided (a ``[:, :H]`` view of a padded buffer)."""
+    device = _lib.require_device(src, index)
+    if src.dim() != 2:
+        raise ValueError(f"expected [rows, hidden], got {tuple(src.shape)}")
+    if src.stride(1) != 1:
+        src = src.contiguous()
+    index = index.long().contiguous()
+    hidden = src.shape[1]
+    out = torch.empty((index.shape[0], hidden), dtype=src.dtype, device=device)
+    if out.numel():
+        with _lib.on_device(device):
+            _lib.call("hmoe_gather_rows", _lib.ptr(src), src.stride(0), _lib.ptr(index), index.shape[0], hidden,
+                      _lib.dtype_id(src.dtype), _lib.ptr(out), _lib.stream_ptr(device))
+    return out
+
+
+def gather_reduce_rows(src: torch.Tensor, inv_map: torch.Tensor, weight: torch.Tensor | None = None) -> torch.Tensor:
+    """``out[r] = sum_k w[j] * src[j]`` over ``j = inv_map[r, k] < len(src)``; ``w = 1`` without a weight.  The sum is
+    taken in fp32 and rounded once to ``src``'s dtype."""
+    device = _lib.require_device(src, inv_map, weight)
+    n_out, top_k = inv_map.shape
+    hidden = src.shape[-1]
+    out = torch.empty((n_out, hidden), device=device, dtype=src.dtype)
+    if n_out == 0 or hidden == 0:
+        return out
+    src = src.contiguous()
+    if weight is not None:
+        weight = weight.to(src.dtype).contiguous()
+    inv_map = inv_map.long().contiguous()
+    with _lib.on_device(device):
+        _lib.call("hmoe_gather_reduce", _lib.ptr(src), _lib.ptr(weight), _lib.ptr(inv_map), n_out, top_k,
+                  src.shape[0], hidden, _lib.dtype_id(src.dtype), _lib.ptr(out), _lib.stream_ptr(device))
+    return out
+
+
+def padded_gather_reduce(src: torch.Tensor, inv_map: torch.Tensor, weight: torch.Tensor | None = None) -> torch.Tensor:
+    """The reference keeps this name for its CPU twin (``moe_permute.py:115-120``); here it is the same kernel."""
+    return gather_reduce_rows(src, inv_map, weight)
+
+
+def build_inv_map(sorted_token_idx: torch.Tensor, recv_N: int, width: int) -> torch.Tensor:
+    """``inv_map[r, j]`` = the j-th sorted position whose recv token is ``r``, padded to ``width`` columns with the
+    sentinel ``len(sorted_token_idx)``.  Auxiliary: the routing sort already returns this map, so the expert path
+    never calls this; it serves callers holding only ``sorted_token_idx`` and is a handful of device-side torch ops
+    with no host readback (stable argsort, counts, exclusive cumsum, one scatter)."""
+    device = _lib.require_device(sorted_token_idx)
+    sorted_token_idx = sorted_token_idx.long()
+    n_sorted = sorted_token_idx.shape[0]
+    inv_map = torch.full((recv_N, width), n_sorted, dtype=torch.long, device=device)
+    if n_sorted == 0:
+        return inv_map
+    order = torch.argsort(sorted_token_idx, stable=True)
+    tokens = sorted_token_idx.index_select(0, order)
+    counts = torch.zeros(recv_N, dtype=torch.long, device=device)
+    counts.scatter_add_(0, sorted_token_idx, torch.ones_like(sorted_token_idx))
+    starts = torch.cumsum(counts, 0) - counts
+    column = torch.arange(n_sorted, device=device) - starts.index_select(0, tokens)
+    inv_map[tokens, column] = order
+    return inv_map
+
+
+class MoEGatherPermute(torch.autograd.Function):
+    """``sorted = tokens[sorted_token_idx]`` with an atomic-free gather-reduce backward over ``inv_map``."""
+
+    @staticmethod
+    def forward(ctx, tokens: torch.Tensor, sorted_token_idx: torch.Tensor, inv_map: torch.Tensor):
+        ctx.save_for_backward(inv_map)
+        return _gather_rows(tokens, sorted_token_idx)
+
+    @staticmethod
+    def backward(ctx, grad_sorted):
+        (inv_map,) = ctx.saved_tensors
+        return gather_reduce_rows(grad_sorted, inv_map), None, None
+
+
+class MoEWeightedUnpermute(torch.autograd.Function):
+    """``out[r] = sum_k w[j] * expert_out[j]`` for ``j = inv_map[r, k]``, the weighted rows summed in fp32 without an
+    intermediate rounding.  ``expert_out`` is saved only when ``weights`` needs a gradient, the one gradient that
+    reads it."""
+
+    @staticmethod
+    def forward(ctx, expert_out, weights, sorted_token_idx, inv_map):
+        expert_out, weights = expert_out.contiguous(), weights.contiguous()
+        ctx.weight_grad = ctx.needs_input_grad[1]
+        ctx.save_for_backward(expert_out if ctx.weight_grad else None, weights, sorted_token_idx.contiguous())
+        return gather_reduce_rows(expert_out, inv_map, weights)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        expert_out, weights, sorted_token_idx = ctx.saved_tensors
+        device = _lib.require_device(grad_out, weights, sorted_token_idx)
+        n_sorted, hidden = sorted_token_idx.shape[0], grad_out.shape[-1]
+        # Under EP the gradient arrives as a row-strided view of the padded transport buffer, read in place.
+        if grad_out.stride(-1) != 1:
+            grad_out = grad_out.contiguous()
+        grad_expert = torch.empty((n_sorted, hidden), device=device, dtype=grad_out.dtype)
+        grad_weights = torch.empty(n_sorted if ctx.weight_grad else 0, device=device, dtype=torch.float32)
+        if n_sorted:
+            w = weights if weights.dtype == grad_out.dtype else weights.to(grad_out.dtype)
+            y = None
+            if ctx.weight_grad:
+                y = expert_out if expert_out.dtype == grad_out.dtype else expert_out.to(grad_out.dtype)
+            with _lib.on_device(device):
+                _lib.call("hmoe_unpermute_bwd", _lib.ptr(grad_out), grad_out.stride(0), _lib.ptr(y), _lib.ptr(w),
+                          _lib.ptr(sorted_token_idx), n_sorted, hidden, _lib.dtype_id(grad_out.dtype),
+                          _lib.ptr(grad_expert), _lib.ptr(grad_weights) if ctx.weight_grad else None,
+                          _lib.stream_ptr(device))
+        return grad_expert, grad_weights.to(weights.dtype) if ctx.weight_grad else None, None, None
+
+
+class MoEExpertBiasGather(torch.autograd.Function):
+    """``bias[eids]`` to expert-sorted tokens; ``grad_bias`` is the per-expert column sum of the incoming gradient,
+    accumulated in fp32 in row order (no atomics).  ``eids`` must be non-decreasing, as the routing sort emits them."""
+
+    @staticmethod
+    def forward(ctx, bias: torch.Tensor, eids: torch.Tensor):
+        ctx.save_for_backward(eids)
+        ctx.num_experts = bias.shape[0]
+        return _gather_rows(bias, eids)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (eids,) = ctx.saved_tensors
+        device = _lib.require_device(grad_out, eids)
+        grad_out = grad_out.contiguous()
+        eids = eids.long().contiguous()
+        grad_bias = torch.empty((ctx.num_experts, grad_out.shape[1]), dtype=grad_out.dtype, device=device)
+        with _lib.on_device(device):
+            _lib.call("hmoe_expert_colsum", _lib.ptr(grad_out), _lib.ptr(eids), grad_out.shape[0], grad_out.shape[1],
+                      ctx.num_experts, _lib.dtype_id(grad_out.dtype), _lib.ptr(grad_bias), _lib.stream_ptr(device))
+        return grad_bias, None
+
+
+def warm_permute_kernels(num_tokens: int, hidden: int, top_k: int, device: torch.device, dtype: torch.dtype) -> None:
+    """Ahead-of-time binaries need no warm-up; kept for API parity (``moe_permute.py:211-227``)."""
+    _lib.load()

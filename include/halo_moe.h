@@ -1,0 +1,156 @@
+/*
+ * halo_moe.h -- C ABI of the MI355X (gfx950) MoE expert-path kernels.
+ *
+ * The reference has no FFI on this path: its boundary is the Python API of the halo/kernels ops and of the MoE block's
+ * _compute_experts.  Each entry point below names the reference function whose device work it replaces
+ * (paths relative to the reference checkout).  The Python package halo_amd binds these with ctypes.
+ *
+ * Conventions
+ *   - every pointer is a device pointer owned by the caller (outputs and workspaces included); nothing is
+ *     allocated, nothing is read back to the host, no call synchronises;
+ *   - `stream` is a hipStream_t passed as void*; all work is enqueued on it;
+ *   - row strides are in elements; `dtype` is an hmoe_dtype;
+ *   - return value: 0 on success, a negative hmoe_status otherwise (hmoe_status_string names it);
+ *   - re-entrant: no mutable global state, safe to call from autograd's backward thread.
+ */
+#ifndef HALO_MOE_H
+#define HALO_MOE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { HMOE_F32 = 0, HMOE_BF16 = 1 } hmoe_dtype;
+
+typedef enum {
+  HMOE_OK = 0,
+  HMOE_INVALID_ARGUMENT = -1, /* a null pointer, a negative size, an unknown enum */
+  HMOE_UNSUPPORTED = -2,      /* a shape or dtype no kernel covers (alignment, top_k or expert count too large) */
+  HMOE_LAUNCH_FAILED = -3     /* hipGetLastError() after the launch was not hipSuccess */
+} hmoe_status;
+
+/* GLU activation ids, as halo/kernels/fused_glu.py:23-25. */
+typedef enum { HMOE_GLU_SILU = 0, HMOE_GLU_GELU_TANH = 1, HMOE_GLU_CLAMPED_SILU = 2 } hmoe_glu_activation;
+
+/* Router gate-weight rules. */
+typedef enum {
+  HMOE_ROUTER_SOFTMAX_ALL = 0, /* softmax over all experts, gather, optional renormalise (Qwen3 family) */
+  HMOE_ROUTER_SOFTMAX_TOPK = 1 /* softmax over the k selected logits (gpt-oss) */
+} hmoe_router_mode;
+
+int hmoe_abi_version(void);
+const char* hmoe_status_string(int status);
+
+/* ------------------------------------------------------------------------------------------------ routing sort
+ * Replaces _CountingSort.forward: halo/kernels/moe_route_sort.py:128-179 (kernels :40-125).
+ * Stable counting sort of the valid slots (0 <= expert < num_local_experts) of experts[n_rows, top_k] by expert;
+ * slot = row * top_k + k.  Outputs: sorted_token_idx i64[n_valid], sorted_weights[n_valid] (same element size as
+ * weights), sorted_expert_ids[n_valid] (same integer type as experts), offs i32[num_local_experts] inclusive group
+ * ends, inv_map i64[n_rows, top_k] (each row's sorted positions ascending, padded with n_valid), dest
+ * i32[n_rows*top_k] (each slot's sorted position, n_valid for a dropped slot), ok i32[1] = (number of valid slots ==
+ * n_valid).  When ok is 0 nothing past n_valid is written.  experts_elem_bytes is 4 or 8, weight_elem_bytes 2, 4 or 8.
+ * Workspace: hmoe_route_sort_workspace_bytes(...) bytes, 16-byte aligned.  Three launches, no atomics on global
+ * memory.
+ */
+int64_t hmoe_route_sort_workspace_bytes(int64_t n_rows, int top_k, int num_local_experts);
+int hmoe_route_sort(const void* experts, int experts_elem_bytes, const void* weights, int weight_elem_bytes,
+                    int64_t n_rows, int top_k, int num_local_experts, int64_t n_valid, int64_t* sorted_token_idx,
+                    void* sorted_weights, void* sorted_expert_ids, int32_t* offs, int64_t* inv_map, int32_t* dest,
+                    int32_t* ok, void* workspace, void* stream);
+
+/* Replaces _CountingSort.backward: halo/kernels/moe_route_sort.py:181-189.
+ * grad_weights[slot] = dest[slot] < n_valid ? grad_sorted[dest[slot]] : 0. */
+int hmoe_route_sort_bwd(const void* grad_sorted, const int32_t* dest, int64_t n_slots, int64_t n_valid,
+                        int elem_bytes, void* grad_weights, void* stream);
+
+/* Replaces sync_free_bincount: halo/kernels/histogram.py:9-18.
+ * out[v] = number of indices equal to v (weights null) or the sum of their f32 weights, for 0 <= v < size; out is
+ * f32 (out_is_i64 == 0) or i64 (counts only).  Indices outside [0, size) are ignored.  One workgroup, counters in
+ * LDS; counts are exact, a weighted sum's order is not fixed (as the reference's scatter_add_). */
+int hmoe_bincount(const int64_t* indices, const float* weights, int64_t n, int size, int out_is_i64, void* out,
+                  void* stream);
+
+/* ------------------------------------------------------------------------------------------- permute / combine
+ * Replaces MoEGatherPermute.forward (tokens.index_select): halo/kernels/moe_permute.py:133-136, and
+ * MoEExpertBiasGather.forward: :197-200.  out[j, :] = src[index[j], :]. */
+int hmoe_gather_rows(const void* src, int64_t src_row_stride, const int64_t* index, int64_t n_out, int64_t hidden,
+                     int dtype, void* out, void* stream);
+
+/* Replaces _gather_reduce_kernel: halo/kernels/moe_permute.py:17-41, 92-112 (permute backward without a weight,
+ * weighted unpermute forward with one).  out[r] = sum_k w[j] * src[j], j = inv_map[r, k] < n_src; fp32 multiply and
+ * accumulate in slot order k = 0..top_k-1, one rounding to dtype.  weight may be null; it has src's dtype. */
+int hmoe_gather_reduce(const void* src, const void* weight, const int64_t* inv_map, int64_t n_out, int top_k,
+                       int64_t n_src, int64_t hidden, int dtype, void* out, void* stream);
+
+/* Replaces _weighted_unpermute_bwd_kernel: halo/kernels/moe_permute.py:44-72, 158-189.
+ * grad_expert[j] = w[j] * grad_out[tok[j]];  grad_weights[j] = <grad_out[tok[j]], expert_out[j]> in fp32 when
+ * expert_out and grad_weights are non-null. */
+int hmoe_unpermute_bwd(const void* grad_out, int64_t grad_out_row_stride, const void* expert_out,
+                       const void* weights, const int64_t* token_idx, int64_t n_sorted, int64_t hidden, int dtype,
+                       void* grad_expert, float* grad_weights, void* stream);
+
+/* Replaces MoEExpertBiasGather.backward (one-hot GEMM): halo/kernels/moe_permute.py:202-208.
+ * grad_bias[e, :] = sum of grad_out rows j with eids[j] == e, fp32 accumulate in row order, one rounding.
+ * eids must be non-decreasing (expert-sorted rows, the only order the expert path produces). */
+int hmoe_expert_colsum(const void* grad_out, const int64_t* eids, int64_t n_rows, int64_t width, int num_experts,
+                       int dtype, void* grad_bias, void* stream);
+
+/* --------------------------------------------------------------------------------------------------- fused GLU
+ * Replaces _glu_fwd_kernel / _glu_bwd_kernel: halo/kernels/fused_glu.py:118-205.  gate/up (and dgate/dup) are
+ * row-strided so a packed [gate | up] buffer is read and its gradient written in place.  fp32 math. */
+int hmoe_glu_fwd(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up, int64_t n_rows,
+                 int64_t width, int dtype, int activation, float alpha, float limit, int clamp_activated,
+                 int up_plus_one, void* out, void* stream);
+int hmoe_glu_bwd(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up, const void* grad_out,
+                 int64_t n_rows, int64_t width, int dtype, int activation, float alpha, float limit,
+                 int clamp_activated, int up_plus_one, void* dgate, void* dup, int64_t stride_dgate,
+                 int64_t stride_dup, void* stream);
+
+/* ------------------------------------------------------------------------------------------------------ router
+ * Replaces the softmax / top-k / renormalise / cast sequence of the family routers the layer calls
+ * (halo/distributed/expert_parallel/moe_layer/shared_experts_layer.py:44-56; weights as routing.py:110-122 and
+ * families/gpt_oss.py:82-84).  One wavefront per token.  indices i64[n_tokens, top_k] in descending score, equal
+ * scores in ascending expert index; weights f32[n_tokens, top_k] hold values rounded to the logits' dtype. */
+int hmoe_router_topk_fwd(const void* logits, int dtype, int64_t n_tokens, int num_experts, int top_k, int mode,
+                         int normalize, float eps, int64_t* indices, float* weights, void* stream);
+/* Gradient of the gate weights with respect to the logits (the router's softmax/renorm backward, aten in the
+ * reference).  grad_logits[n_tokens, num_experts] in the logits' dtype. */
+int hmoe_router_topk_bwd(const void* logits, int dtype, const int64_t* indices, const float* grad_weights,
+                         int64_t n_tokens, int num_experts, int top_k, int mode, int normalize, float eps,
+                         void* grad_logits, void* stream);
+
+/* ------------------------------------------------------------------------------------------------ grouped GEMM
+ * Replace F.grouped_mm as called by halo/kernels/grouped_mm.py:16-47 (forward :39, dgrad :25, wgrad :26).
+ * offs i32[num_groups] are inclusive row ends (null: one group holding every row).  b is [num_groups, K, N]
+ * contiguous.  fp32 accumulate, one rounding to dtype.  Rows past offs[num_groups-1] are not written by
+ * fwd/dgrad.  An empty group's wgrad is exact zeros.  Deterministic (no split accumulation across workgroups).
+ */
+int hmoe_grouped_gemm_fwd(const void* a, int64_t lda, const void* b, const int32_t* offs, int64_t total_rows,
+                          int num_groups, int64_t k, int64_t n, int dtype, void* out, int64_t ldo, void* stream);
+int hmoe_grouped_gemm_dgrad(const void* grad_out, int64_t ldg, const void* b, const int32_t* offs,
+                            int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype, void* grad_a,
+                            int64_t lda, void* stream);
+int hmoe_grouped_gemm_wgrad(const void* a, int64_t lda, const void* grad_out, int64_t ldg, const int32_t* offs,
+                            int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype, void* grad_b,
+                            void* stream);
+
+/* ------------------------------------------------------------------------------------------------- block fp8
+ * Replaces quantize_block_fp8: halo/kernels/lowp/block_fp8.py:23-34.  w is [batch, rows, cols]; q (e4m3fn bytes)
+ * has its shape; scale is f32 [batch, ceil(rows/128), ceil(cols/128)], a power of two per 128x128 block. */
+int hmoe_quantize_block_fp8(const void* w, int dtype, int64_t batch, int64_t rows, int64_t cols, uint8_t* q,
+                            float* scale, void* stream);
+/* Inverse (halo/checkpoint/tools/fp8_dequant.py:153-170): out = q * scale, one rounding to dtype. */
+int hmoe_dequantize_block_fp8(const uint8_t* q, const float* scale, int64_t batch, int64_t rows, int64_t cols,
+                              int dtype, void* out, void* stream);
+/* Forward grouped GEMM with block-fp8 weights (the quantised-weight configuration): a bf16 [total_rows, K],
+ * bq e4m3fn [num_groups, K, N] with b_scale f32 [num_groups, ceil(K/128), ceil(N/128)]; out bf16. */
+int hmoe_grouped_gemm_fwd_fp8w(const void* a, int64_t lda, const uint8_t* bq, const float* b_scale,
+                               const int32_t* offs, int64_t total_rows, int num_groups, int64_t k, int64_t n,
+                               void* out, int64_t ldo, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HALO_MOE_H */

@@ -1,0 +1,535 @@
+"""GPU parity tests, op by op: every HIP kernel through the C ABI (via the ``halo_amd.kernels`` ops) against the CPU
+oracle on the same seeded inputs.  Integer outputs are compared bit for bit; floating-point outputs within the
+tolerance written next to each check."""
+
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from tests.cases import ROUTING_CASES, make_receive
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def max_rel(actual, reference):
+    """Largest elementwise error relative to the reference's peak."""
+    a, r = actual.detach().double().cpu(), reference.detach().double().cpu()
+    return ((a - r).abs().max() / r.abs().max().clamp(min=1e-30)).item()
+
+
+def fro_rel(actual, reference):
+    a, r = actual.detach().double().cpu(), reference.detach().double().cpu()
+    return ((a - r).norm() / r.norm()).item()
+
+
+def cosine(actual, reference):
+    a, r = actual.detach().double().cpu().flatten(), reference.detach().double().cpu().flatten()
+    return (torch.dot(a, r) / (a.norm() * r.norm())).item()
+
+
+# ------------------------------------------------------------------------------------------------- routing sort
+
+@pytest.mark.parametrize("case", ROUTING_CASES, ids=lambda c: c.name)
+def test_route_sort_matches_oracle_bit_for_bit(device, case):
+    from halo_amd.kernels.moe_route_sort import sort_routing_by_expert
+    from oracle import route_sort as oracle
+
+    experts, weights, counts = make_receive(case, seed=ROUTING_CASES.index(case))
+    want = oracle.argsort_routing(experts.numpy(), weights.numpy(), case.local_experts, counts)
+    leaf = weights.to(device).requires_grad_(True)
+    got = sort_routing_by_expert(experts.to(device), leaf, case.local_experts, counts)
+    names = ("sorted_token_idx", "sorted_weights", "sorted_expert_ids", "offs", "inv_map")
+    for name, g, w in zip(names, got, want):
+        g = g.detach().cpu().numpy()
+        assert g.dtype == w.dtype and g.shape == w.shape, f"{case.name}: {name} {g.dtype}{g.shape} vs {w.dtype}{w.shape}"
+        if g.dtype == np.float32:
+            g, w = g.view(np.int32), w.view(np.int32)
+        assert np.array_equal(g, w), f"{case.name}: {name}"
+    # gate-weight gradient: each slot reads its sorted position's gradient, dropped slots read zero
+    upstream = torch.randn(got[1].shape, generator=torch.Generator().manual_seed(1))
+    (grad,) = torch.autograd.grad(got[1], leaf, upstream.to(device))
+    want_grad = oracle.sort_backward(upstream.numpy(), want[5], tuple(experts.shape))
+    assert np.array_equal(grad.cpu().numpy().view(np.int32), want_grad.view(np.int32))
+
+
+def test_route_sort_literal_known_answer(device):
+    from halo_amd.kernels.moe_route_sort import sort_routing_by_expert
+
+    with open(os.path.join(GOLDEN, "route_sort_literal.json")) as f:
+        gold = json.load(f)
+    experts = torch.tensor(gold["experts"], device=device)
+    weights = torch.tensor(gold["weights"], device=device)
+    got = sort_routing_by_expert(experts, weights, gold["num_local_experts"], tuple(gold["counts"]))
+    for name, g in zip(("sorted_token_idx", "sorted_weights", "sorted_expert_ids", "offs", "inv_map"), got):
+        assert g.cpu().tolist() == gold[name], name
+
+
+def test_route_sort_count_flag_and_int32_ids_and_bf16_weights(device):
+    """The device flag the async assert reads: 1 when the local slots number the host count (only the sum is read),
+    0 when they do not -- checked on the flag itself, so no assert ever fires on the GPU."""
+    from halo_amd.kernels.moe_route_sort import counting_sort_raw, sort_routing_by_expert
+    from oracle import route_sort as oracle
+
+    case = ROUTING_CASES[1]
+    experts, weights, counts = make_receive(case, seed=1)
+    e, w = experts.to(device), weights.to(device)
+    for n_valid, expect in ((sum(counts), 1), (sum(counts) - 1, 0), (sum(counts) + 1, 0)):
+        *_, ok = counting_sort_raw(e, w, case.local_experts, n_valid)
+        assert int(ok.item()) == expect
+    moved = (counts[0] - 1, counts[1] + 1, *counts[2:])
+    a = sort_routing_by_expert(e, w, case.local_experts, moved)
+    b = sort_routing_by_expert(e, w, case.local_experts, counts)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    with pytest.raises(ValueError, match="2 receive counts for 4 local experts"):
+        sort_routing_by_expert(torch.zeros(2, 2, dtype=torch.long, device=device),
+                               torch.rand(2, 2, device=device), 4, (3, 1))
+    # int32 ids and bf16 weights are copied bit for bit too
+    want = oracle.argsort_routing(experts.numpy().astype(np.int32), weights.bfloat16().view(torch.int16).numpy(),
+                                  case.local_experts, counts)
+    got = sort_routing_by_expert(e.int(), w.bfloat16(), case.local_experts, counts)
+    assert got[2].dtype == torch.int32 and got[1].dtype == torch.bfloat16
+    assert np.array_equal(got[1].view(torch.int16).cpu().numpy(), want[1])
+    assert np.array_equal(got[2].cpu().numpy(), want[2])
+
+
+def test_route_sort_is_bit_reproducible(device):
+    from halo_amd.kernels.moe_route_sort import sort_routing_by_expert
+
+    case = ROUTING_CASES[-1]
+    experts, weights, counts = make_receive(case, seed=5)
+    e, w = experts.to(device), weights.to(device)
+    first = sort_routing_by_expert(e, w, case.local_experts, counts)
+    for _ in range(3):
+        again = sort_routing_by_expert(e, w, case.local_experts, counts)
+        assert all(torch.equal(x, y) for x, y in zip(first, again))
+
+
+def test_bincount(device):
+    from halo_amd.kernels.histogram import accumulate_bincount, sync_free_bincount
+
+    g = torch.Generator().manual_seed(0)
+    idx = torch.randint(0, 128, (8192, 8), generator=g)
+    want = torch.bincount(idx.flatten(), minlength=128)
+    assert torch.equal(sync_free_bincount(idx.to(device), 128, dtype=torch.long).cpu(), want)
+    got = sync_free_bincount(idx.to(device), 128)
+    assert got.dtype == torch.float32 and torch.equal(got.cpu(), want.float())
+    w = torch.rand(idx.shape, generator=g)
+    want_w = torch.zeros(128, dtype=torch.float64).scatter_add_(0, idx.flatten(), w.flatten().double())
+    got_w = sync_free_bincount(idx.to(device), 128, weights=w.to(device))
+    assert max_rel(got_w, want_w) < 1e-5  # fp32 sums of ~512 terms each, order not fixed
+    counter = accumulate_bincount(None, idx.to(device), 128)
+    counter = accumulate_bincount(counter, idx.to(device), 128)
+    assert torch.equal(counter.cpu(), 2 * want.float())
+
+
+# -------------------------------------------------------------------------------------------- permute / combine
+
+DTYPE_TOLS = ((torch.float32, 1e-5), (torch.bfloat16, 2e-2))
+ROUTINGS = ((517, 8, 2816, 0.5), (64, 4, 100, 1.0), (33, 8, 1025, 0.1), (300, 8, 2048, 1.0))
+
+
+def _routing(n_tokens, top_k, n_sorted, seed):
+    from oracle import route_sort as oracle
+
+    g = torch.Generator().manual_seed(seed)
+    slots = torch.arange(n_tokens).repeat_interleave(top_k)
+    token_idx = slots[torch.randperm(slots.numel(), generator=g)[:n_sorted]]
+    return token_idx, torch.from_numpy(oracle.build_inv_map(token_idx.numpy(), n_tokens, top_k))
+
+
+@pytest.mark.parametrize(("dtype", "tol"), DTYPE_TOLS, ids=("fp32", "bf16"))
+@pytest.mark.parametrize(("n_tokens", "top_k", "hidden", "fill"), ROUTINGS)
+def test_weighted_unpermute_and_permute_match_oracle(device, dtype, tol, n_tokens, top_k, hidden, fill):
+    from halo_amd.kernels.moe_permute import MoEGatherPermute, MoEWeightedUnpermute
+    from oracle import permute as oracle
+
+    n_sorted = int(n_tokens * top_k * fill)
+    token_idx, inv_map = _routing(n_tokens, top_k, n_sorted, seed=n_tokens)
+    g = torch.Generator().manual_seed(n_tokens + 1)
+    y = torch.randn(n_sorted, hidden, generator=g).to(dtype)
+    w = torch.rand(n_sorted, generator=g).to(dtype)
+    grad = torch.randn(n_tokens, hidden, generator=g).to(dtype)
+    yd, wd = y.to(device).requires_grad_(True), w.to(device).requires_grad_(True)
+    out = MoEWeightedUnpermute.apply(yd, wd, token_idx.to(device), inv_map.to(device))
+    out.backward(grad.to(device))
+    want_out = oracle.gather_reduce(y, inv_map, w, out_dtype=torch.float64)
+    want_gy, want_gw = oracle.weighted_unpermute_backward(grad.double(), y.double(), w.double(), token_idx)
+    for name, got, want in (("out", out, want_out), ("grad_expert", yd.grad, want_gy), ("grad_w", wd.grad, want_gw)):
+        assert got.dtype == dtype
+        assert max_rel(got, want) < tol, f"{name}: {max_rel(got, want):.3e}"
+        if dtype == torch.bfloat16:
+            # a result accumulated in fp32 is the exact result rounded once: within 1.1x of the bf16 rounding floor
+            floor = fro_rel(want.to(torch.bfloat16), want)
+            assert fro_rel(got, want) <= 1.1 * floor + 1e-12, (name, fro_rel(got, want), floor)
+    # permute forward (bit copy) and backward (unweighted gather-sum)
+    tokens = torch.randn(n_tokens, hidden, generator=g).to(dtype)
+    td = tokens.to(device).requires_grad_(True)
+    sorted_tokens = MoEGatherPermute.apply(td, token_idx.to(device), inv_map.to(device))
+    assert torch.equal(sorted_tokens.cpu(), oracle.gather_rows(tokens, token_idx))
+    gs = torch.randn(n_sorted, hidden, generator=g).to(dtype)
+    sorted_tokens.backward(gs.to(device))
+    want_b = oracle.gather_reduce(gs, inv_map, out_dtype=torch.float64)
+    assert max_rel(td.grad, want_b) < tol
+    if dtype == torch.bfloat16:
+        assert torch.equal(td.grad.cpu(), want_b.to(torch.bfloat16))  # sums of <= 8 bf16 values: fp32 is exact
+
+
+def test_gather_reduce_sentinel_known_answer_and_strided_inputs(device):
+    from halo_amd.kernels.moe_permute import MoEGatherPermute, MoEWeightedUnpermute, gather_reduce_rows
+    from oracle import permute as oracle
+
+    src = torch.arange(1, 7, device=device, dtype=torch.float32).unsqueeze(-1).expand(6, 3).contiguous()
+    inv_map = torch.tensor([[0, 3], [5, 6], [6, 6]], device=device)  # 6 == len(src): sentinel
+    assert gather_reduce_rows(src, inv_map)[:, 0].tolist() == [5.0, 6.0, 0.0]
+    # strided operands: expert_out / weights as views, grad_out and tokens as [:, :H] views of padded buffers
+    n_tokens, top_k, hidden = 257, 8, 704
+    n_sorted = n_tokens * top_k // 2
+    token_idx, inv_map = _routing(n_tokens, top_k, n_sorted, seed=0)
+    g = torch.Generator().manual_seed(0)
+    wide_out = torch.randn(n_sorted, 2 * hidden, generator=g)
+    wide_w = torch.rand(n_sorted, 2, generator=g)
+    wide_grad = torch.randn(n_tokens, hidden + 64, generator=g)
+    yd = wide_out.to(device).requires_grad_(True)
+    wd = wide_w.to(device).requires_grad_(True)
+    y_view, w_view = yd[:, :hidden], wd[:, 0]
+    grad_view = wide_grad.to(device)[:, :hidden]
+    assert not y_view.is_contiguous() and grad_view.stride() == (hidden + 64, 1)
+    out = MoEWeightedUnpermute.apply(y_view, w_view, token_idx.to(device), inv_map.to(device))
+    out.backward(grad_view)
+    y, w, grad = wide_out[:, :hidden], wide_w[:, 0], wide_grad[:, :hidden]
+    assert max_rel(out, oracle.gather_reduce(y, inv_map, w, out_dtype=torch.float64)) < 1e-5
+    want_gy, want_gw = oracle.weighted_unpermute_backward(grad.double(), y.double(), w.double(), token_idx)
+    assert max_rel(yd.grad[:, :hidden], want_gy) < 1e-5 and max_rel(wd.grad[:, 0], want_gw) < 1e-5
+    padded = torch.randn(n_tokens, 768, generator=g).bfloat16().to(device)  # 704 columns of a 768-wide buffer
+    got = MoEGatherPermute.apply(padded[:, :hidden], token_idx.to(device), inv_map.to(device))
+    assert torch.equal(got, padded[:, :hidden][token_idx.to(device)])
+
+
+def test_empty_dispatch_and_no_weight_grad(device):
+    from halo_amd.kernels.moe_permute import MoEWeightedUnpermute, build_inv_map
+
+    out = MoEWeightedUnpermute.apply(torch.zeros(0, 16, device=device), torch.zeros(0, device=device),
+                                     torch.zeros(0, dtype=torch.long, device=device),
+                                     torch.zeros(0, 8, dtype=torch.long, device=device))
+    assert out.shape == (0, 16)
+    inv = build_inv_map(torch.empty(0, dtype=torch.long, device=device), 8, 4)
+    assert inv.shape == (8, 4) and bool((inv == 0).all())
+    got = MoEWeightedUnpermute.apply(torch.empty(0, 5, device=device), torch.empty(0, device=device),
+                                     torch.empty(0, dtype=torch.long, device=device), inv)
+    assert got.shape == (8, 5) and not got.any()
+    # weights needing no gradient: expert_out is not kept, the expert gradient is the same bit for bit
+    token_idx, inv_map = _routing(129, 8, 516, seed=1)
+    g = torch.Generator().manual_seed(2)
+    y = torch.randn(516, 1100, generator=g).bfloat16().to(device)
+    w = torch.rand(516, generator=g).bfloat16().to(device)
+    grad = torch.randn(129, 1100, generator=g).bfloat16().to(device)
+    grads = {}
+    for need in (True, False):
+        yy, ww = y.clone().requires_grad_(True), w.clone().requires_grad_(need)
+        saved = []
+        with torch.autograd.graph.saved_tensors_hooks(lambda t: saved.append(t) or t, lambda t: t):
+            o = MoEWeightedUnpermute.apply(yy, ww, token_idx.to(device), inv_map.to(device))
+        o.backward(grad)
+        grads[need] = yy.grad
+        assert any(t.shape == y.shape for t in saved) == need
+    assert torch.equal(grads[True], grads[False])
+
+
+def test_build_inv_map_matches_oracle(device):
+    from halo_amd.kernels.moe_permute import build_inv_map
+    from oracle import route_sort as oracle
+
+    token_idx, inv_map = _routing(2000, 8, 9000, seed=7)
+    assert torch.equal(build_inv_map(token_idx.to(device), 2000, 8).cpu(), inv_map)
+
+
+def test_expert_bias_gather(device):
+    from halo_amd.kernels.moe_permute import MoEExpertBiasGather
+    from oracle import permute as oracle
+
+    g = torch.Generator().manual_seed(3)
+    for dtype, tol in DTYPE_TOLS:
+        eids = torch.sort(torch.randint(0, 32, (5000,), generator=g)).values
+        eids = eids[(eids != 7) & (eids != 31)]  # two idle experts, one of them last
+        bias = torch.randn(32, 2880, generator=g).to(dtype)
+        grad = torch.randn(eids.numel(), 2880, generator=g).to(dtype)
+        bd = bias.to(device).requires_grad_(True)
+        out = MoEExpertBiasGather.apply(bd, eids.to(device))
+        assert torch.equal(out.cpu(), oracle.bias_gather(bias, eids))
+        out.backward(grad.to(device))
+        want = oracle.bias_gather_backward(grad.double(), eids, 32)
+        assert max_rel(bd.grad, want) < tol
+        assert not bd.grad[7].any() and not bd.grad[31].any()
+
+
+# ---------------------------------------------------------------------------------------------------- fused GLU
+
+def _combines():
+    from halo_amd.kernels.fused_glu import GluCombine
+
+    return {
+        "silu": GluCombine.silu(),
+        "gelu_tanh": GluCombine.gelu_tanh(),
+        "clamped_silu": GluCombine.clamped_silu(2.5),
+        "silu_then_clamp": GluCombine.clamped_silu(2.5, clamp_activated=True),
+        "gptoss": GluCombine.gptoss(1.702, 7.0),
+    }
+
+
+@pytest.mark.parametrize("name", ("silu", "gelu_tanh", "clamped_silu", "silu_then_clamp", "gptoss"))
+@pytest.mark.parametrize(("dtype", "tol"), ((torch.float32, 1e-5), (torch.bfloat16, 2e-2)), ids=("fp32", "bf16"))
+@pytest.mark.parametrize(("rows", "width"), ((300, 768), (17, 100), (64, 2880), (5, 1025)))
+def test_glu_matches_oracle_packed_and_separate(device, name, dtype, tol, rows, width):
+    from oracle import glu as oracle
+
+    combine = _combines()[name]
+    kw = dict(activation=combine.activation, alpha=combine.alpha, limit=combine.limit,
+              clamp_activated=combine.clamp_activated, up_plus_one=combine.up_plus_one)
+    g = torch.Generator().manual_seed(rows * 7 + width)
+    gate_up = (torch.randn(rows, 2 * width, generator=g) * 3).to(dtype)
+    dout = torch.randn(rows, width, generator=g).to(dtype)
+    gate, up = gate_up[:, :width], gate_up[:, width:]
+    want = oracle.glu_forward(gate.double(), up.double(), **kw)
+    want_dg, want_du = oracle.glu_backward(gate.double(), up.double(), dout.double(), **kw)
+    # separate operands
+    gd, ud = gate.contiguous().to(device).requires_grad_(True), up.contiguous().to(device).requires_grad_(True)
+    out = combine(gd, ud)
+    out.backward(dout.to(device))
+    assert out.dtype == dtype
+    assert max_rel(out, want) < tol and max_rel(gd.grad, want_dg) < tol and max_rel(ud.grad, want_du) < tol
+    # packed [gate | up], read in place; the gradient comes back as one buffer and equals the separate form's bits
+    pd = gate_up.to(device).requires_grad_(True)
+    out_p = combine.packed(pd)
+    out_p.backward(dout.to(device))
+    assert torch.equal(out_p, out)
+    assert torch.equal(pd.grad[:, :width], gd.grad) and torch.equal(pd.grad[:, width:], ud.grad)
+
+
+def test_glu_subgradient_at_the_clamp_bound_and_probe_vector(device):
+    from halo_amd.kernels.fused_glu import (GluCombine, is_gelu_tanh_activation, is_silu_activation,
+                                            resolve_clamped_glu_mul, resolve_fused_glu_mul)
+    from oracle import glu as oracle
+
+    limit = 2.0
+    gate = torch.tensor([[limit, limit, -limit, 0.5, limit + 1e-3, 0.0, 0.0, 0.0]], device=device)
+    up = torch.tensor([[limit, -limit, limit, limit, 1.0, limit + 1e-3, -limit - 1e-3, 1.0]], device=device)
+    gd, ud = gate.clone().requires_grad_(True), up.clone().requires_grad_(True)
+    GluCombine.clamped_silu(limit)(gd, ud).backward(torch.ones_like(gate))
+    want_dg, want_du = oracle.glu_backward(gate.cpu().double(), up.cpu().double(), torch.ones(1, 8).double(),
+                                           oracle.CLAMPED_SILU, limit=limit)
+    assert ((gd.grad.cpu() != 0) == (want_dg != 0)).all() and ((ud.grad.cpu() != 0) == (want_du != 0)).all()
+    assert bool((gd.grad[0, :4] != 0).all()) and gd.grad[0, 4] == 0  # at the bound passes, past it is cut
+    assert ud.grad[0, 5] == 0 and ud.grad[0, 6] == 0
+    probe = torch.tensor([[-64.0, -8.0, -1.0, -0.5, -1e-3, 0.0, 1e-3, 0.5, 1.0, 8.0, 64.0, 0.0]], device=device)
+    out = GluCombine.silu()(probe, torch.ones_like(probe))
+    assert torch.isfinite(out).all() and max_rel(out, torch.nn.functional.silu(probe.cpu().double())) < 1e-6
+    assert is_silu_activation(torch.nn.SiLU()) and not is_silu_activation(torch.nn.GELU())
+    assert is_gelu_tanh_activation(torch.nn.GELU(approximate="tanh")) and not is_gelu_tanh_activation(torch.nn.GELU())
+    assert resolve_fused_glu_mul(torch.nn.functional.silu) == GluCombine.silu()
+    assert resolve_fused_glu_mul(torch.relu) is None
+    assert resolve_clamped_glu_mul(torch.nn.functional.silu, 3.0, clamp_activated=True) == \
+        GluCombine.clamped_silu(3.0, clamp_activated=True)
+    assert [c.name for c in _combines().values()] == list(_combines())
+
+
+# ------------------------------------------------------------------------------------------------------- router
+
+@pytest.mark.parametrize(("tokens", "experts", "top_k"), ((512, 8, 2), (2048, 128, 8), (300, 32, 4), (64, 512, 10),
+                                                         (100, 1000, 8), (7, 64, 64)))
+@pytest.mark.parametrize("dtype", (torch.float32, torch.bfloat16), ids=("fp32", "bf16"))
+def test_router_selection_is_bit_exact_and_weights_close(device, tokens, experts, top_k, dtype):
+    from halo_amd.kernels.router import SOFTMAX_ALL, SOFTMAX_TOPK, fused_topk_gate
+    from oracle import router as oracle
+
+    g = torch.Generator().manual_seed(tokens + experts)
+    logits = (torch.randn(tokens, experts, generator=g) * 0.9).to(dtype)
+    if dtype == torch.bfloat16:
+        assert (logits.float().sort(-1).values.diff(dim=-1) == 0).any(), "bf16 logits should tie"
+    for mode, normalize, eps in ((SOFTMAX_ALL, True, 0.0), (SOFTMAX_ALL, False, 0.0), (SOFTMAX_ALL, True, 1e-20),
+                                 (SOFTMAX_TOPK, False, 0.0)):
+        want_idx, want_w = oracle.route(logits, top_k, mode, normalize, eps)
+        ld = logits.to(device).requires_grad_(True)
+        idx, w = fused_topk_gate(ld, top_k, mode=mode, normalize=normalize, eps=eps)
+        assert idx.dtype == torch.int64 and w.dtype == torch.float32
+        assert torch.equal(idx.cpu(), want_idx), f"selection differs (mode {mode})"
+        # weights: fp32 math (a few fp32 ulps from the oracle's), then one rounding to the logits' dtype, which can
+        # land on the neighbouring bf16 value: at most one bf16 ulp (2^-7 relative) there, 1e-6 relative in fp32
+        ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 1e-6
+        assert ((w.detach().cpu() - want_w).abs() <= ulp * want_w.abs() + 1e-30).all()
+        if dtype == torch.bfloat16:
+            assert torch.equal(w, w.bfloat16().float())
+        gw = torch.randn(tokens, top_k, generator=g)
+        (grad,) = torch.autograd.grad(w, ld, gw.to(device))
+        want_grad = oracle.route_backward(logits.double(), want_idx, gw, mode, normalize, eps)
+        assert grad.dtype == dtype
+        assert max_rel(grad, want_grad) < (2e-2 if dtype == torch.bfloat16 else 1e-5)
+
+
+def test_router_ties_go_to_the_lower_index(device):
+    from halo_amd.kernels.router import fused_topk_gate
+
+    logits = torch.tensor([[1.0, 1.0, 0.5, 1.0], [0.0, 2.0, 2.0, -1.0], [3.0, 3.0, 3.0, 3.0]], device=device)
+    assert fused_topk_gate(logits, 2)[0].tolist() == [[0, 1], [1, 2], [0, 1]]
+    assert fused_topk_gate(logits, 3)[0].tolist() == [[0, 1, 3], [1, 2, 0], [0, 1, 2]]
+    wide = torch.zeros(2, 200, device=device)  # every score equal, experts spread over several lanes and registers
+    assert fused_topk_gate(wide, 5)[0].tolist() == [[0, 1, 2, 3, 4]] * 2
+    wide[0, 130], wide[0, 65], wide[0, 199] = 1.0, 1.0, 1.0
+    assert fused_topk_gate(wide, 5)[0][0].tolist() == [65, 130, 199, 0, 1]
+
+
+# ------------------------------------------------------------------------------------------------- grouped GEMM
+
+def _offsets(counts, device):
+    return torch.cumsum(torch.tensor(counts), 0).to(torch.int32).to(device)
+
+
+GEMM_CASES = (
+    # counts per group, K, N
+    ((7, 33, 0, 1, 64, 0), 128, 96),       # the reference's empty-group roster
+    ((0, 0, 0, 0, 105, 0), 128, 96),       # one live expert
+    ((130, 1, 255, 128, 129), 256, 384),   # ragged around the 128-row tile
+    ((300, 0, 45), 2880, 360),             # widths off the tile size (2880 = 22.5 x 128)
+    ((64,) * 16, 512, 1536),
+)
+
+
+@pytest.mark.parametrize(("counts", "k", "n"), GEMM_CASES)
+@pytest.mark.parametrize(("dtype", "tol"), ((torch.bfloat16, 2e-2), (torch.float32, 1e-5)), ids=("bf16", "fp32"))
+def test_grouped_mm_forward_and_gradients_match_oracle(device, counts, k, n, dtype, tol):
+    from halo_amd.kernels.grouped_mm import grouped_mm
+    from oracle import grouped_mm as oracle
+
+    g = torch.Generator().manual_seed(sum(counts) + k)
+    total = sum(counts)
+    x = (torch.randn(total, k, generator=g) * 0.5).to(dtype)
+    w = (torch.randn(len(counts), k, n, generator=g) * 0.05).to(dtype)
+    dout = torch.randn(total, n, generator=g).to(dtype)
+    offs = np.cumsum(counts).astype(np.int32)
+    xd, wd = x.to(device).requires_grad_(True), w.to(device).requires_grad_(True)
+    out = grouped_mm(xd, wd, offs=_offsets(counts, device))
+    out.backward(dout.to(device))
+    assert out.dtype == dtype and out.shape == (total, n) and wd.grad.shape == w.shape
+    kw = dict(acc_dtype=torch.float64)
+    want = oracle.grouped_mm(x.double(), w.double(), offs, **kw)
+    want_dx = oracle.grouped_mm_dgrad(dout.double(), w.double(), offs, **kw)
+    want_dw = oracle.grouped_mm_wgrad(x.double(), dout.double(), offs, **kw)
+    for name, got, ref in (("out", out, want), ("dx", xd.grad, want_dx), ("dw", wd.grad, want_dw)):
+        assert torch.isfinite(got).all(), name
+        assert max_rel(got, ref) < tol, f"{name}: {max_rel(got, ref):.3e}"
+        assert cosine(got, ref) > 0.9999, f"{name}: cosine {cosine(got, ref)}"
+        if dtype == torch.bfloat16:
+            # fp32 accumulation, one rounding: the error sits at the bf16 rounding floor of the exact result
+            floor = fro_rel(ref.to(torch.bfloat16), ref)
+            assert fro_rel(got, ref) <= 1.05 * floor + 1e-12, (name, fro_rel(got, ref), floor)
+    for e, c in enumerate(counts):
+        assert (c == 0) == (not wd.grad[e].any()), f"expert {e}: an empty group's weight gradient must be exact zeros"
+
+
+def test_grouped_mm_takes_int64_offsets_transposed_weights_and_strided_rows(device):
+    from halo_amd.kernels.grouped_mm import grouped_mm
+    from oracle import grouped_mm as oracle
+
+    counts = (40, 0, 200, 16)
+    g = torch.Generator().manual_seed(0)
+    total, k, n = sum(counts), 192, 320
+    wide = (torch.randn(total, 2 * k, generator=g) * 0.5).bfloat16()
+    w_nk = (torch.randn(len(counts), n, k, generator=g) * 0.05).bfloat16()  # [G, N, K] storage, used as its transpose
+    dout = torch.randn(total, n, generator=g).bfloat16()
+    offs = np.cumsum(counts).astype(np.int32)
+    x = wide[:, :k]
+    xd = wide.to(device)[:, :k].detach().requires_grad_(True)
+    wd = w_nk.to(device).requires_grad_(True)
+    out = grouped_mm(xd, wd.transpose(1, 2), offs=torch.from_numpy(offs).long().to(device))
+    out.backward(dout.to(device))
+    w_kn = w_nk.transpose(1, 2).contiguous()
+    kw = dict(acc_dtype=torch.float64)
+    assert max_rel(out, oracle.grouped_mm(x.double(), w_kn.double(), offs, **kw)) < 2e-2
+    assert max_rel(xd.grad, oracle.grouped_mm_dgrad(dout.double(), w_kn.double(), offs, **kw)) < 2e-2
+    want_dw = oracle.grouped_mm_wgrad(x.double(), dout.double(), offs, **kw).transpose(1, 2)
+    assert wd.grad.shape == w_nk.shape and max_rel(wd.grad, want_dw) < 2e-2
+
+
+def test_grouped_mm_is_bit_reproducible_and_zero_rows(device):
+    from halo_amd.kernels.grouped_mm import grouped_mm
+
+    counts = (100, 3, 0, 500, 77)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(sum(counts), 256, generator=g).bfloat16().to(device)
+    w = (torch.randn(5, 256, 512, generator=g) * 0.05).bfloat16().to(device)
+    dout = torch.randn(sum(counts), 512, generator=g).bfloat16().to(device)
+    results = []
+    for _ in range(3):
+        xd, wd = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        out = grouped_mm(xd, wd, offs=_offsets(counts, device))
+        out.backward(dout)
+        results.append((out.detach(), xd.grad, wd.grad))
+    for other in results[1:]:
+        assert all(torch.equal(a, b) for a, b in zip(results[0], other))
+    empty = grouped_mm(torch.zeros(0, 256, device=device, dtype=torch.bfloat16, requires_grad=True), w,
+                       offs=torch.zeros(5, dtype=torch.int32, device=device))
+    assert empty.shape == (0, 512)
+    empty.sum().backward()
+
+
+# ---------------------------------------------------------------------------------------------------- block fp8
+
+@pytest.mark.parametrize("shape", [(128, 128), (256, 384), (200, 130), (5, 7), (3, 130, 129)])
+def test_block_fp8_quantiser_is_bit_exact(device, shape):
+    from halo_amd.kernels.lowp.block_fp8 import dequantize_block_fp8, quantize_block_fp8
+    from oracle import block_fp8 as oracle
+
+    torch.manual_seed(0)
+    weight = (torch.randn(shape) * torch.rand(shape).mul(4)).bfloat16()
+    q, scale = quantize_block_fp8(weight.to(device))
+    want_q, want_scale = oracle.quantize_block_fp8(weight.float().numpy())
+    assert q.dtype == torch.float8_e4m3fn and scale.dtype == torch.float32
+    assert np.array_equal(scale.cpu().numpy(), want_scale)
+    got_bits = q.view(torch.uint8).cpu().numpy()
+    nonzero = (want_q & 0x7F) != 0
+    assert np.array_equal(got_bits[nonzero], want_q[nonzero]) and not (got_bits[~nonzero] & 0x7F).any()
+    restored = dequantize_block_fp8(q, scale)
+    want_restored = torch.from_numpy(oracle.dequantize_block_fp8(want_q, want_scale)).bfloat16()
+    assert torch.equal(restored.cpu(), want_restored)
+
+
+def test_block_fp8_boundary_and_zero_block(device):
+    from halo_amd.kernels.lowp.block_fp8 import quantize_block_fp8
+
+    w = torch.zeros(128, 256)
+    w[0, 0] = 448.0 * 4
+    w[0, 128] = 448.0 * 4 * 1.0001
+    _, scale = quantize_block_fp8(w.to(device))
+    assert scale.tolist() == [[4.0, 8.0]]
+    q0, s0 = quantize_block_fp8(torch.zeros(128, 128, device=device))
+    assert torch.isfinite(s0).all() and bool((s0 > 0).all()) and not q0.float().any()
+
+
+def test_fp8_weight_grouped_gemm_equals_the_dequantised_bf16_path(device):
+    """bf16 activations times block-fp8 weights: every e4m3 value times its power-of-two scale is a bf16 value, so the
+    kernel must equal the bf16 grouped GEMM over the dequantised weights bit for bit; against the oracle's fp64
+    product it sits at the bf16 rounding floor."""
+    from halo_amd.kernels.expert_gemm import BlockFp8Weight, expert_gemm
+    from halo_amd.kernels.grouped_mm import grouped_mm
+    from halo_amd.kernels.lowp.block_fp8 import dequantize_block_fp8, quantize_block_fp8
+    from oracle import block_fp8 as fp8_oracle
+    from oracle import grouped_mm as oracle
+
+    counts = (130, 0, 257, 64)
+    g = torch.Generator().manual_seed(4)
+    k, n = 384, 640
+    x = torch.randn(sum(counts), k, generator=g).bfloat16()
+    w = (torch.randn(len(counts), k, n, generator=g) * 0.02)
+    q, scale = quantize_block_fp8(w.to(device))
+    offs = _offsets(counts, device)
+    out = expert_gemm(x.to(device), BlockFp8Weight(q, scale), offs=offs)
+    deq = dequantize_block_fp8(q, scale)
+    assert torch.equal(out, grouped_mm(x.to(device), deq, offs=offs))
+    want_q, want_scale = fp8_oracle.quantize_block_fp8(w.numpy())
+    w_ref = torch.from_numpy(fp8_oracle.dequantize_block_fp8(want_q, want_scale)).bfloat16()
+    want = oracle.grouped_mm(x.double(), w_ref.double(), np.cumsum(counts).astype(np.int32), acc_dtype=torch.float64)
+    assert max_rel(out, want) < 2e-2 and cosine(out, want) > 0.9999
