@@ -1,0 +1,148 @@
+"""Per-family glue over :class:`EPMoELayerBase`: Qwen3 (gate and up stored apart), Qwen3.5 / Qwen3.6 (fused experts and
+a sigmoid-gated shared expert) and gpt-oss (interleaved fused experts with biases, clamped SwiGLU, logit-space router
+bias).
+
+Mirrors the reference's ``halo/distributed/expert_parallel/families/qwen3.py``, ``qwen3_5.py`` and ``gpt_oss.py``.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled
+from halo_amd.kernels.moe_permute import MoEExpertBiasGather
+from halo_amd.kernels.router import SOFTMAX_TOPK, fused_topk_gate
+from halo_amd.moe_layer.config import GPT_OSS, QWEN3, QWEN3_5
+from halo_amd.moe_layer.layer import EPMoELayerBase, EPSharedExpertsMoELayerBase, dense_mm
+
+
+def split_interleaved_gate_up(interleaved: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """gpt-oss stores ``[g0, u0, g1, u1, ...]`` along the last axis (``halo/models/moe/expert_layout.py:87-88``)."""
+    return interleaved[..., ::2], interleaved[..., 1::2]
+
+
+class EPQwen3MoELayer(EPSharedExpertsMoELayerBase):
+    """``Qwen3MoeSparseMoeBlock``: fused HF experts split into matmul-convention halves, three grouped GEMMs."""
+
+    HF_MODULE_NAMES = ("Qwen3MoeSparseMoeBlock",)
+    FAMILY = QWEN3
+    # ``Qwen3MoeTopKRouter`` renormalises with no floor.
+    _TOPK_WEIGHT_NORM_EPS = 0.0
+
+    def _normalizes_topk(self) -> bool:
+        """The router's configurable ``norm_topk_prob``, read live."""
+        return bool(getattr(self.gate, "norm_topk_prob", True))
+
+
+class EPQwen3_5MoELayer(EPSharedExpertsMoELayerBase):
+    """``Qwen3_5MoeSparseMoeBlock``: fused ``gate_up_proj`` (two grouped GEMMs and the packed GLU), a router that
+    always renormalises, and a shared expert scaled by ``sigmoid(x @ w_gate^T)``."""
+
+    HF_MODULE_NAMES = ("Qwen3_5MoeSparseMoeBlock",)
+    FAMILY = QWEN3_5
+    _TOPK_WEIGHT_NORM_EPS = 0.0
+
+    def _adopt_shared_experts(self, original_layer: nn.Module) -> None:
+        super()._adopt_shared_experts(original_layer)
+        self.shared_expert_gate = original_layer.shared_expert_gate
+
+    def _shared_expert_output(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        out = super()._shared_expert_output(hidden_states)
+        gate = getattr(self, "shared_expert_gate", None)
+        if gate is None:
+            return out
+        x = hidden_states.reshape(-1, hidden_states.shape[-1])
+        # a [T, 1] projection is below the GEMM kernels' 16-byte row granularity: a matrix-vector product in torch
+        return out * torch.sigmoid(torch.nn.functional.linear(x, gate.weight.to(x.dtype))).view(
+            *hidden_states.shape[:-1], -1)
+
+    def replicated_named_params(self) -> list:
+        extra = [] if getattr(self, "shared_expert_gate", None) is None else [
+            (f"shared_expert_gate.{n}", p) for n, p in self.shared_expert_gate.named_parameters()]
+        return super().replicated_named_params() + extra
+
+
+class EPGptOssMoELayer(EPMoELayerBase):
+    """``GptOssMLP``: the interleaved ``gate_up_proj`` is stored de-interleaved for the grouped GEMMs
+    (``gate_proj_gmm`` / ``up_proj_gmm`` ``[E, H, F]``), each projection adds its expert bias through
+    :class:`MoEExpertBiasGather`, the combine is the clamped SwiGLU ``(clamp(u)+1) * g' * sigmoid(alpha g')``, and the
+    router picks on bias-inclusive logits then takes a softmax over the picks.  ``forward`` returns
+    ``(out [B, S, H], logits)``."""
+
+    HF_MODULE_NAMES = ("GptOssMLP",)
+    FAMILY = GPT_OSS
+    _ROUTER_ATTR = "router"
+
+    def _adopt_expert_compute(self, original_layer: nn.Module, experts: nn.Module) -> None:
+        self._gptoss_glu = GluCombine.gptoss(experts.alpha, experts.limit)
+        self._fused_glu_mul = self._gptoss_glu
+
+    def _adopt_expert_params(self, experts: nn.Module, weights_already_sharded: bool = False) -> None:
+        self._require_fused_experts(experts)
+        start, end = self._local_expert_range(weights_already_sharded)
+        gate, up = split_interleaved_gate_up(experts.gate_up_proj.data[start:end])  # HF keeps [E, H, 2F] here
+        self.gate_proj_gmm = nn.Parameter(gate.contiguous())
+        self.up_proj_gmm = nn.Parameter(up.contiguous())
+        if getattr(experts, "gate_up_proj_bias", None) is not None:
+            gate_bias, up_bias = split_interleaved_gate_up(experts.gate_up_proj_bias.data[start:end])
+            self.gate_proj_gmm_bias = nn.Parameter(gate_bias.contiguous())
+            self.up_proj_gmm_bias = nn.Parameter(up_bias.contiguous())
+        self.down_proj = nn.Parameter(experts.down_proj.data[start:end].clone())
+        if getattr(experts, "down_proj_bias", None) is not None:
+            self.down_proj_bias = nn.Parameter(experts.down_proj_bias.data[start:end].clone())
+
+    @classmethod
+    def from_weights(cls, *, alpha: float = 1.702, limit: float = 7.0, router_bias: torch.Tensor | None = None,
+                     **kwargs):
+        self = super().from_weights(**kwargs)
+        self._gptoss_glu = GluCombine.gptoss(alpha, limit)
+        self._fused_glu_mul = self._gptoss_glu
+        if router_bias is not None:
+            self.router.bias = nn.Parameter(router_bias)
+        return self
+
+    def _glu_combine_name(self) -> str:
+        return self._gptoss_glu.name if fused_glu_enabled() else "eager"
+
+    def forward(self, hidden_states: torch.Tensor, **kwargs) -> tuple[torch.Tensor, torch.Tensor]:
+        shape = hidden_states.shape
+        input_dtype = hidden_states.dtype
+        flat = hidden_states.reshape(-1, shape[-1])
+        logits = self._linear_router_logits(flat)
+        experts, weights = fused_topk_gate(logits, self.top_k, mode=SOFTMAX_TOPK, normalize=False)
+        result = self._dispatch_compute_combine(flat, experts, weights.float(), input_dtype)
+        return result.view(shape), logits.to(input_dtype)
+
+    def _grouped_expert_ffn(self, sorted_tokens, offs, sorted_expert_ids, output_dtype):
+        """Three grouped GEMMs (gate, up, down) on de-interleaved weights, each plus its expert bias."""
+        gate_attr, up_attr = ("gate_proj_gmm", "up_proj_gmm") if hasattr(self, "gate_proj_gmm") else (
+            "gate_proj", "up_proj")
+        gate = self._grouped_proj_with_bias(sorted_tokens, gate_attr, offs, output_dtype, sorted_expert_ids)
+        up = self._grouped_proj_with_bias(sorted_tokens, up_attr, offs, output_dtype, sorted_expert_ids)
+        gated = self._gptoss_glu(gate, up)
+        return self._grouped_proj_with_bias(gated.to(output_dtype), "down_proj", offs, output_dtype, sorted_expert_ids)
+
+    def _grouped_proj_with_bias(self, x, weight_attr, offs, out_dtype, eids):
+        out = self._expert_proj(x, weight_attr, offs, out_dtype)
+        bias = getattr(self, f"{weight_attr}_bias", None)
+        return out if bias is None else out + MoEExpertBiasGather.apply(bias.to(out_dtype), eids)
+
+
+MOE_LAYER_MAP = {name: cls for cls in (EPQwen3MoELayer, EPQwen3_5MoELayer, EPGptOssMoELayer)
+                 for name in cls.HF_MODULE_NAMES}
+
+
+def apply_ep_layers(model: nn.Module, ep_config) -> int:
+    """Swaps every HF MoE block whose class name a family claims for this package's block, in place; returns how many
+    were swapped (the module swap of the reference's ``expert_parallel/parallelize.py:22-69`` at one GPU)."""
+    import copy
+
+    swapped = 0
+    for parent in list(model.modules()):
+        for child_name, child in list(parent.named_children()):
+            cls = MOE_LAYER_MAP.get(type(child).__name__)
+            if cls is not None:
+                setattr(parent, child_name, cls(child, copy.copy(ep_config)))
+                swapped += 1
+    return swapped

@@ -1,0 +1,384 @@
+"""The MoE block on one GPU: route, sort by expert, grouped GLU FFN, weighted combine, plus the shared expert.
+
+Mirrors the parts of the reference's EP MoE layer that run at ``ep_size`` 1 or on one rank's received rows:
+``halo/distributed/expert_parallel/moe_layer/compute.py`` (``_compute_experts`` ``:207-220``,
+``_compute_experts_grouped`` ``:222-242``, ``_sort_tokens_for_grouped_mm`` ``:263-281``, ``_expert_proj`` ``:283-294``,
+``_glu_ffn`` ``:357-361``, ``_init_fused_glu_params`` ``:77-88``), ``moe_layer/layer.py`` (construction order ``:67-80``,
+``_dispatch_compute_combine{,_shared}`` ``:270-342``), ``moe_layer/routing.py`` (``_softmax_gate_weights_at``
+``:110-119``) and ``moe_layer/shared_experts_layer.py`` (``forward`` ``:20-28``).  Every tensor op on the path is a HIP
+kernel of this package; the dispatch/combine exchange, expert LoRA, balancing bias, routing replay and expert TP of the
+reference are not part of it.
+"""
+
+from __future__ import annotations
+
+import logging
+from abc import ABC, abstractmethod
+from collections.abc import Callable
+from typing import ClassVar
+
+import torch
+import torch.nn as nn
+
+from halo_amd.kernels.expert_gemm import expert_gemm
+from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled, resolve_fused_glu_mul
+from halo_amd.kernels.grouped_mm import grouped_mm
+from halo_amd.kernels.moe_permute import MoEGatherPermute, MoEWeightedUnpermute, warm_permute_kernels
+from halo_amd.kernels.moe_route_sort import sort_routing_by_expert, warm_route_sort_kernels
+from halo_amd.kernels.router import SOFTMAX_ALL, fused_topk_gate
+from halo_amd.moe_layer.config import EPConfig, MoEFamilySpec
+
+logger = logging.getLogger(__name__)
+
+ROUTER_TOPK_FIELDS = ("top_k", "num_experts_per_tok", "num_experts_per_token")
+
+
+def dense_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``x @ weight^T`` for an ``F.linear``-convention ``weight [out, in]`` on the grouped kernel with one group (the
+    router projection and the shared expert); differentiable in both operands."""
+    return grouped_mm(x, weight.unsqueeze(0).transpose(1, 2), offs=None)
+
+
+class EPMoELayerBase(nn.Module, ABC):
+    """Base class of the per-family MoE blocks.  A family fills in the declarations below, implements ``forward`` and
+    overrides the ``_adopt_*`` hooks its expert layout needs.  Built from an HF MoE block
+    (``cls(original_layer, ep_config)``, what the reference's ``apply_ep_layers`` does), or directly from tensors with
+    :meth:`from_weights`."""
+
+    FAMILY: ClassVar[MoEFamilySpec]
+    # HF class name(s) of the MoE block this layer replaces.
+    HF_MODULE_NAMES: tuple[str, ...] = ()
+    _shared_expert_attr: str = "shared_experts"
+    # Attribute the router hangs off, on the wrapped HF block and on this layer.
+    _ROUTER_ATTR: str | None = "gate"
+    # The floor the family's router adds to a top-k weight sum before renormalising by it.
+    _TOPK_WEIGHT_NORM_EPS: float = 1e-20
+
+    def __init__(self, original_layer: nn.Module, ep_config: EPConfig, weights_already_sharded: bool = False):
+        router = self._declared_router(original_layer)
+        experts = self._find_experts_container(original_layer)
+        if ep_config.num_experts is None:
+            ep_config.finalize_expert_assignment(self.detect_num_experts(original_layer))
+        self._init_ep_state(ep_config, self._detect_hidden_dim(router, experts))
+        if router is not None:
+            setattr(self, self._ROUTER_ATTR, router)
+        self._adopt_routing(original_layer)
+        self._adopt_shared_experts(original_layer)
+        self._adopt_expert_compute(original_layer, experts)
+        self._adopt_expert_params(experts, weights_already_sharded=weights_already_sharded)
+        self._finalize_expert_init()
+
+    # ---------------------------------------------------------------------------------------------- construction
+
+    @classmethod
+    def detect_num_experts(cls, layer: nn.Module) -> int:
+        experts = cls._find_experts_container(layer)
+        return len(experts) if isinstance(experts, nn.ModuleList) else experts.num_experts
+
+    @classmethod
+    def _declared_router(cls, layer: nn.Module) -> nn.Module | None:
+        if cls._ROUTER_ATTR is None:
+            return None
+        router = getattr(layer, cls._ROUTER_ATTR, None)
+        if router is None:
+            raise AttributeError(f"{cls.__name__} declares _ROUTER_ATTR='{cls._ROUTER_ATTR}', but "
+                                 f"{type(layer).__name__} has no such attribute")
+        return router
+
+    @classmethod
+    def _find_experts_container(cls, layer: nn.Module) -> nn.Module:
+        for attr in cls.FAMILY.experts_container_attrs:
+            if hasattr(layer, attr):
+                return getattr(layer, attr)
+        raise AttributeError(f"{cls.__name__}: {type(layer).__name__} carries none of "
+                             f"{cls.FAMILY.experts_container_attrs}")
+
+    @classmethod
+    def _detect_hidden_dim(cls, router: nn.Module | None, experts: nn.Module) -> int:
+        if router is not None and hasattr(router, "weight"):
+            return router.weight.shape[1]
+        return cls._require_fused_experts(experts).gate_up_proj.shape[2]
+
+    @staticmethod
+    def _require_fused_experts(experts: nn.Module) -> nn.Module:
+        missing = [name for name in ("gate_up_proj", "down_proj") if not hasattr(experts, name)]
+        if missing:
+            raise AttributeError(f"Expected fused-GLU experts carrying gate_up_proj and down_proj, but "
+                                 f"{type(experts).__name__} carries no {missing}")
+        return experts
+
+    def _init_ep_state(self, ep_config: EPConfig, hidden_dim: int) -> None:
+        super().__init__()
+        self.ep_config = ep_config
+        self.num_experts = ep_config.num_experts
+        self.experts_per_rank = ep_config.experts_per_rank
+        self.ep_rank, self.ep_size = ep_config.ep_rank, ep_config.ep_size
+        self.expert_start, self.expert_end = ep_config.expert_start_idx, ep_config.expert_end_idx
+        self.hidden_dim = hidden_dim
+        self.expert_tp_size, self.expert_tp_rank = ep_config.expert_tp_size, ep_config.expert_tp_rank
+        self.fp32_router, self.fp32_experts = ep_config.fp32_router, ep_config.fp32_experts
+        if not ep_config.grouped_gemm_enabled:
+            raise NotImplementedError("the per-expert loop is the reference's CPU path; this block runs the grouped "
+                                      "kernels only (use_grouped_gemm=True)")
+        self._use_grouped_mm = True
+        self._expert_kernels_warmed = False
+        self._lowp_quant_format = None
+        self._lowp_weight_cacheable = True
+        self._fused_glu_mul: Callable | None = None
+        # labels the dispatch / expert-compute / combine spans at no device cost (swappable, as in the reference)
+        self._perf = torch.profiler.record_function
+
+    def _adopt_routing(self, original_layer: nn.Module) -> None:
+        self.top_k = self._find_top_k(original_layer)
+
+    @classmethod
+    def _find_top_k(cls, layer: nn.Module) -> int:
+        router = getattr(layer, cls._ROUTER_ATTR, None) if cls._ROUTER_ATTR else None
+        for source in (layer, router, getattr(layer, "config", None)):
+            for attr in ROUTER_TOPK_FIELDS:
+                if source is not None and hasattr(source, attr):
+                    return int(getattr(source, attr))
+        raise AttributeError(f"Cannot determine top_k from {type(layer).__name__}: none of {ROUTER_TOPK_FIELDS}")
+
+    def _adopt_shared_experts(self, original_layer: nn.Module) -> None:
+        for attr in self.FAMILY.shared_expert_attrs:
+            if getattr(original_layer, attr, None) is not None:
+                self._shared_expert_attr = attr
+                setattr(self, attr, getattr(original_layer, attr))
+                return
+        if self.FAMILY.shared_expert_attrs:
+            raise AttributeError(f"{type(self).__name__} declares shared experts {self.FAMILY.shared_expert_attrs}, "
+                                 f"but {type(original_layer).__name__} carries none")
+
+    def _adopt_expert_compute(self, original_layer: nn.Module, experts: nn.Module) -> None:
+        act_fn = getattr(experts, "act_fn", None)
+        if act_fn is None:
+            raise AttributeError(f"{type(self).__name__}: {type(experts).__name__}.act_fn does not name the expert "
+                                 f"activation")
+        self.act_fn = act_fn
+        self._fused_glu_mul = resolve_fused_glu_mul(act_fn)
+        if self._fused_glu_mul is None:
+            raise NotImplementedError(f"expert activation {act_fn!r} has no fused combine (SiLU and tanh-GELU do)")
+
+    def _local_expert_range(self, weights_already_sharded: bool) -> tuple[int, int]:
+        return (0, self.experts_per_rank) if weights_already_sharded else (self.expert_start, self.expert_end)
+
+    def _adopt_expert_params(self, experts: nn.Module, weights_already_sharded: bool = False) -> None:
+        """HF ``gate_up_proj [E, 2F, H]`` / ``down_proj [E, H, F]`` to the matmul convention ``[E, K, N]``: fused
+        ``gate_up_proj [E, H, 2F]`` (columns ``[gate | up]``) + ``down_proj [E, F, H]``, or gate and up apart on a
+        ``separate_glu`` family."""
+        self._require_fused_experts(experts)
+        start, end = self._local_expert_range(weights_already_sharded)
+        gate_up = experts.gate_up_proj.data[start:end]
+        down = experts.down_proj.data[start:end]
+        if self.FAMILY.expert_layout == "separate_glu":
+            gate, up = gate_up.chunk(2, dim=1)
+            self.gate_proj = nn.Parameter(gate.transpose(1, 2).contiguous())
+            self.up_proj = nn.Parameter(up.transpose(1, 2).contiguous())
+        else:
+            self.gate_up_proj = nn.Parameter(gate_up.transpose(1, 2).contiguous())
+        self.down_proj = nn.Parameter(down.transpose(1, 2).contiguous())
+
+    def _finalize_expert_init(self) -> None:
+        if self.fp32_router and self._ROUTER_ATTR is not None:
+            setattr(self, self._ROUTER_ATTR, getattr(self, self._ROUTER_ATTR).float())
+        if self.fp32_experts:
+            for name, param in self.expert_named_params():
+                setattr(self, name, nn.Parameter(param.data.float(), requires_grad=param.requires_grad))
+
+    def expert_named_params(self) -> list:
+        return [(n, getattr(self, n)) for n in self.FAMILY.expert_weight_roots if hasattr(self, n)]
+
+    def replicated_named_params(self) -> list:
+        shared = getattr(self, self._shared_expert_attr, None)
+        return [] if shared is None else [(f"{self._shared_expert_attr}.{n}", p) for n, p in shared.named_parameters()]
+
+    @abstractmethod
+    def forward(self, hidden_states: torch.Tensor, **kwargs): ...
+
+    # -------------------------------------------------------------------------------------------- expert compute
+
+    def _warm_expert_kernels(self, device: torch.device, dtype: torch.dtype, hidden: int, top_k: int) -> None:
+        """Ahead-of-time binaries: nothing compiles or loads lazily on first launch.  Kept so callers of the
+        reference's hook find it; it loads the library once."""
+        if self._expert_kernels_warmed:
+            return
+        self._expert_kernels_warmed = True
+        warm_route_sort_kernels(top_k, self.experts_per_rank, device)
+        warm_permute_kernels(16, hidden, top_k, device, dtype)
+
+    def _compute_experts(self, tokens: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor,
+                         output_dtype: torch.dtype, *, recv_counts: tuple[int, ...] | None) -> torch.Tensor:
+        """``experts``/``weights`` are ``[T, top_k]`` local ids (``-1`` = not this rank's) and gate weights;
+        ``recv_counts`` counts per local expert, None at ``ep_size`` 1."""
+        if tokens.shape[0] == 0:
+            return torch.zeros((0, tokens.shape[-1]), device=tokens.device, dtype=output_dtype)
+        return self._compute_experts_grouped(tokens, experts, weights, output_dtype, recv_counts=recv_counts)
+
+    def _compute_experts_grouped(self, tokens, experts, weights, output_dtype, *, recv_counts):
+        """Sort -> grouped GLU FFN -> weighted unpermute."""
+        sorted_tokens, offs, sorted_token_idx, sorted_weights, sorted_expert_ids, inv_map = (
+            self._sort_tokens_for_grouped_mm(tokens, experts, weights, recv_counts=recv_counts)
+        )
+        expert_out = self._grouped_expert_ffn(sorted_tokens.to(output_dtype), offs, sorted_expert_ids, output_dtype)
+        return MoEWeightedUnpermute.apply(
+            expert_out.to(output_dtype).contiguous(), sorted_weights.to(output_dtype), sorted_token_idx, inv_map
+        )
+
+    def _require_recv_counts(self, recv_counts: tuple[int, ...] | None) -> tuple[int, ...]:
+        if recv_counts is None or len(recv_counts) != self.experts_per_rank:
+            raise RuntimeError(
+                f"{type(self).__name__}: the expert compute at ep_size={self.ep_size} needs the dispatch's "
+                f"per-local-expert receive counts ({self.experts_per_rank} of them), got {recv_counts!r}."
+            )
+        return recv_counts
+
+    def _sort_tokens_for_grouped_mm(self, tokens, experts, weights, *, recv_counts):
+        """``(sorted_tokens, offs, sorted_token_idx, sorted_weights, sorted_expert_ids, inv_map)`` over the valid local
+        assignments; the dispatch's -1 padding is dropped.  At ``ep_size > 1`` the host-side counts size the sort."""
+        counts = self._require_recv_counts(recv_counts) if self.ep_size > 1 else None
+        sorted_token_idx, sorted_weights, sorted_expert_ids, offs, inv_map = sort_routing_by_expert(
+            experts, weights, self.experts_per_rank, counts
+        )
+        sorted_tokens = MoEGatherPermute.apply(tokens, sorted_token_idx, inv_map)
+        return sorted_tokens, offs, sorted_token_idx, sorted_weights, sorted_expert_ids, inv_map
+
+    def _grouped_expert_ffn(self, sorted_tokens, offs, sorted_expert_ids, output_dtype):
+        return self._glu_ffn(sorted_tokens, lambda x, attr: self._expert_proj(x, attr, offs, output_dtype))
+
+    def _expert_proj(self, x: torch.Tensor, weight_attr: str, offs: torch.Tensor, out_dtype: torch.dtype):
+        weight = getattr(self, weight_attr)
+        if isinstance(weight, torch.Tensor):
+            weight = weight.to(out_dtype)
+        return self._grouped_mm(x, weight, offs=offs)
+
+    def _grouped_mm(self, mat_a, mat_b, *, offs=None, lowp: bool = True):
+        return expert_gemm(mat_a, mat_b, offs=offs, quant_format=self._lowp_quant_format if lowp else None,
+                           weight_cacheable=self._lowp_weight_cacheable)
+
+    @property
+    def _stores_fused_glu(self) -> bool:
+        return hasattr(self, "gate_up_proj")
+
+    def _glu_ffn(self, x: torch.Tensor, proj: Callable[[torch.Tensor, str], torch.Tensor]) -> torch.Tensor:
+        if self._stores_fused_glu:
+            return proj(self._glu_combine_packed(proj(x, "gate_up_proj")), "down_proj")
+        return proj(self._glu_combine(proj(x, "gate_proj"), proj(x, "up_proj")), "down_proj")
+
+    def _glu_combine(self, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+        return self._fused_glu_mul(gate, up)
+
+    def _glu_combine_packed(self, gate_up: torch.Tensor) -> torch.Tensor:
+        if isinstance(self._fused_glu_mul, GluCombine):
+            return self._fused_glu_mul.packed(gate_up)
+        gate, up = gate_up.chunk(2, dim=-1)
+        return self._glu_combine(gate, up)
+
+    def _glu_combine_name(self) -> str:
+        combine = self._fused_glu_mul
+        if combine is None or not fused_glu_enabled():
+            return "eager"
+        return combine.name if isinstance(combine, GluCombine) else getattr(combine, "__name__", "eager")
+
+    # ------------------------------------------------------------------------------------------------- routing
+
+    def _router_input(self, hidden: torch.Tensor) -> torch.Tensor:
+        router = getattr(self, self._ROUTER_ATTR) if self._ROUTER_ATTR else None
+        weight = getattr(router, "weight", None)
+        upcast = self.fp32_router and weight is not None and weight.dtype == torch.float32
+        return hidden.float() if upcast else hidden
+
+    def _linear_router_logits(self, flat: torch.Tensor) -> torch.Tensor:
+        """The router's logits at the input dtype (fp32 under ``fp32_router``), fp32 accumulation, one rounding."""
+        router = getattr(self, self._ROUTER_ATTR)
+        x = self._router_input(flat)
+        logits = dense_mm(x, router.weight.to(x.dtype))
+        bias = getattr(router, "bias", None)
+        return logits if bias is None else logits + bias.to(logits.dtype)
+
+    # ------------------------------------------------------------------------------- dispatch / compute / combine
+
+    def _dispatch_compute_combine(self, flat: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor,
+                                  input_dtype: torch.dtype) -> torch.Tensor:
+        """At ``ep_size`` 1 dispatch and combine are the identity; the spans keep the reference's names."""
+        if self.ep_size > 1:
+            raise NotImplementedError(
+                "forward() at ep_size > 1 needs the dispatch/combine exchange, which is outside this build; hand the "
+                "received rows to _compute_experts(recv_x, recv_topk_idx, recv_topk_weights, dtype, recv_counts=...)"
+            )
+        self._warm_expert_kernels(flat.device, input_dtype, flat.shape[-1], experts.shape[1])
+        with self._perf("ep.dispatch"):
+            recv_x, recv_topk_idx, recv_topk_weights, recv_counts = flat, experts, weights, None
+        with self._perf("ep.expert_compute"):
+            output = self._compute_experts(recv_x, recv_topk_idx, recv_topk_weights, input_dtype,
+                                           recv_counts=recv_counts)
+        with self._perf("ep.combine"):
+            combined = output
+        return combined
+
+    def _dispatch_compute_combine_shared(self, flat, experts, weights, input_dtype, orig_shape, shared_fn):
+        routed = self._dispatch_compute_combine(flat, experts, weights, input_dtype).view(*orig_shape)
+        return routed if shared_fn is None else routed + shared_fn()
+
+    # ---------------------------------------------------------------------------------- construction from tensors
+
+    @classmethod
+    def from_weights(cls, *, router_weight: torch.Tensor | None, top_k: int, ep_config: EPConfig | None = None,
+                     **expert_tensors: torch.Tensor):
+        """A layer built straight from tensors in the runtime layout (``gate_up_proj [E,H,2F]`` + ``down_proj [E,F,H]``,
+        or ``gate_proj``/``up_proj [E,H,F]``; optional ``*_bias``), for benches and tests that have no HF block."""
+        self = cls.__new__(cls)
+        down = expert_tensors["down_proj"]
+        local_experts = down.shape[0]
+        if ep_config is None:
+            ep_config = EPConfig(num_experts=local_experts)
+        elif ep_config.num_experts is None:
+            ep_config.finalize_expert_assignment(local_experts * ep_config.ep_size)
+        self._init_ep_state(ep_config, down.shape[2])
+        self.top_k = top_k
+        if router_weight is not None and cls._ROUTER_ATTR is not None:
+            router = nn.Module()
+            router.weight = nn.Parameter(router_weight)
+            router.top_k = top_k
+            router.norm_topk_prob = True
+            setattr(self, cls._ROUTER_ATTR, router)
+        for name, tensor in expert_tensors.items():
+            # a BlockFp8Weight (quantised serving weights) is held as it is
+            setattr(self, name, nn.Parameter(tensor) if isinstance(tensor, torch.Tensor) else tensor)
+        self._fused_glu_mul = GluCombine.silu()
+        return self
+
+
+class EPSharedExpertsMoELayerBase(EPMoELayerBase):
+    """``forward`` routes the flattened tokens, then adds the shared expert, which reads the layer input."""
+
+    _ROUTER_MODE: int = SOFTMAX_ALL
+
+    def forward(self, hidden_states: torch.Tensor, **kwargs) -> torch.Tensor:
+        orig_shape = hidden_states.shape
+        flat = hidden_states.reshape(-1, orig_shape[-1])
+        topk_indices, topk_weights = self._route_hidden_states(flat, **kwargs)
+        shared = getattr(self, self._shared_expert_attr, None)
+        shared_fn = (lambda: self._shared_expert_output(hidden_states)) if shared is not None else None
+        return self._dispatch_compute_combine_shared(
+            flat, topk_indices.long(), topk_weights.float(), hidden_states.dtype, orig_shape, shared_fn
+        )
+
+    def _normalizes_topk(self) -> bool:
+        return True
+
+    def _route_hidden_states(self, flat: torch.Tensor, **kwargs) -> tuple[torch.Tensor, torch.Tensor]:
+        """Logits projection, then the fused softmax / top-k / renormalise / cast kernel."""
+        logits = self._linear_router_logits(flat)
+        return fused_topk_gate(logits, self.top_k, mode=self._ROUTER_MODE, normalize=self._normalizes_topk(),
+                               eps=self._TOPK_WEIGHT_NORM_EPS)
+
+    def _shared_expert_output(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        """Dense GLU MLP ``down(act(gate(x)) * up(x))`` through the same GEMM and GLU kernels."""
+        shared = getattr(self, self._shared_expert_attr)
+        shape = hidden_states.shape
+        x = hidden_states.reshape(-1, shape[-1])
+        dtype = x.dtype
+        gate = dense_mm(x, shared.gate_proj.weight.to(dtype))
+        up = dense_mm(x, shared.up_proj.weight.to(dtype))
+        return dense_mm(self._fused_glu_mul(gate, up), shared.down_proj.weight.to(dtype)).view(shape)

@@ -1,0 +1,242 @@
+"""GPU parity tests of the whole MoE block: forward and every gradient against the CPU oracle's per-expert loop
+(fp32 math on the same input bits), routing bit for bit, and the blocks as drop-ins for the Hugging Face MoE modules
+they wrap.
+
+Tolerances (BASELINE.json): routing indices / offsets bit-exact; bf16 outputs and gradients max-rel <= 2e-2 and cosine
+>= 0.9999 against the fp32 result; fp32 runs max-rel <= 1e-4.
+"""
+
+import pytest
+import torch
+
+from tests.cases import CONFIG1, CONFIG2_SMALL, CONFIG4_SMALL, make_layer_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def max_rel(actual, reference):
+    a, r = actual.detach().double().cpu(), reference.detach().double().cpu()
+    return ((a - r).abs().max() / r.abs().max().clamp(min=1e-30)).item()
+
+
+def cosine(actual, reference):
+    a, r = actual.detach().double().cpu().flatten(), reference.detach().double().cpu().flatten()
+    return (torch.dot(a, r) / (a.norm() * r.norm())).item()
+
+
+def _check(name, got, want, tol):
+    assert torch.isfinite(got).all(), name
+    err, cos = max_rel(got, want), cosine(got, want)
+    assert err <= tol, f"{name}: max-rel {err:.3e} > {tol}"
+    assert cos >= 0.9999, f"{name}: cosine {cos:.6f}"
+
+
+def _build_layer(cfg, inputs, device):
+    from halo_amd.moe_layer import EPGptOssMoELayer, EPQwen3_5MoELayer, EPQwen3MoELayer
+
+    params = {k: v.to(device) for k, v in inputs["params"].items()}
+    if cfg.router == "softmax_topk":
+        renamed = {}
+        for k, v in params.items():
+            renamed[k.replace("gate_proj", "gate_proj_gmm").replace("up_proj", "up_proj_gmm")] = v
+        return EPGptOssMoELayer.from_weights(router_weight=inputs["router_weight"].to(device), top_k=cfg.top_k,
+                                             router_bias=inputs.get("router_bias", torch.zeros(cfg.experts)).to(device),
+                                             **renamed)
+    cls = EPQwen3_5MoELayer if cfg.fused else EPQwen3MoELayer
+    return cls.from_weights(router_weight=inputs["router_weight"].to(device), top_k=cfg.top_k, **params)
+
+
+def _oracle_run(cfg, inputs, indices):
+    """fp32 per-expert loop on the CPU over the same input bits, with the device's selection."""
+    from oracle import moe_layer as oracle
+    from oracle import router as router_oracle
+
+    f = lambda t: t.float().requires_grad_(True)
+    x, wr = f(inputs["x"]), f(inputs["router_weight"])
+    params = {k: f(v) for k, v in inputs["params"].items()}
+    bias = f(inputs["router_bias"]) if "router_bias" in inputs else None
+    glu = oracle.Glu("gptoss", 1.702, 7.0) if cfg.glu == "gptoss" else oracle.Glu(cfg.glu)
+    mode = router_oracle.SOFTMAX_TOPK if cfg.router == "softmax_topk" else router_oracle.SOFTMAX_ALL
+    out, logits, idx, w = oracle.moe_layer_forward(x, wr, params, glu, cfg.top_k, router_bias=bias, mode=mode,
+                                                   normalize=True, eps=0.0, indices=indices)
+    out.backward(inputs["grad_out"].float())
+    grads = {"x": x.grad, "router_weight": wr.grad, **{k: v.grad for k, v in params.items()}}
+    if bias is not None:
+        grads["router_bias"] = bias.grad
+    return out.detach(), logits.detach(), grads
+
+
+@pytest.mark.parametrize("cfg", (CONFIG1, CONFIG2_SMALL, CONFIG4_SMALL), ids=lambda c: c.name)
+def test_layer_forward_backward_matches_the_cpu_loop(device, cfg):
+    from halo_amd.kernels.router import SOFTMAX_ALL, SOFTMAX_TOPK, fused_topk_gate
+    from oracle import router as router_oracle
+
+    skew = dict(zipf_alpha=1.2, empty_experts=3) if cfg.router == "softmax_topk" else {}
+    inputs = make_layer_inputs(cfg, **skew)
+    layer = _build_layer(cfg, inputs, device)
+    x = inputs["x"].to(device).requires_grad_(True)
+    result = layer(x)
+    out = result[0] if isinstance(result, tuple) else result
+    out.backward(inputs["grad_out"].to(device))
+    assert out.dtype == cfg.dtype and out.shape == x.shape
+
+    # routing: the device's picks equal the oracle's rule on the device's own logits, bit for bit
+    with torch.no_grad():
+        logits = layer._linear_router_logits(x.detach())
+        mode = SOFTMAX_TOPK if cfg.router == "softmax_topk" else SOFTMAX_ALL
+        idx, gates = fused_topk_gate(logits, cfg.top_k, mode=mode, normalize=True, eps=0.0)
+    want_idx = router_oracle.select_topk(logits.cpu(), cfg.top_k)
+    assert torch.equal(idx.cpu(), want_idx)
+    if skew:
+        counts = torch.bincount(idx.cpu().flatten(), minlength=cfg.experts)
+        assert (counts == 0).sum() >= 3, "the skewed case should leave experts without tokens"
+        assert counts.max() > 4 * counts[counts > 0].float().median()
+
+    want_out, want_logits, want_grads = _oracle_run(cfg, inputs, idx.cpu())
+    tol = 1e-4 if cfg.dtype == torch.float32 else 2e-2
+    _check("logits", logits, want_logits, tol)
+    _check("out", out, want_out, tol)
+    _check("grad x", x.grad, want_grads["x"], tol)
+    router = getattr(layer, layer._ROUTER_ATTR)
+    _check("grad router_weight", router.weight.grad, want_grads["router_weight"], tol)
+    for name in inputs["params"]:
+        attr = name.replace("gate_proj", "gate_proj_gmm").replace("up_proj", "up_proj_gmm") \
+            if cfg.router == "softmax_topk" else name
+        got = getattr(layer, attr).grad
+        _check(f"grad {name}", got, want_grads[name], tol)
+        if got.dim() == 3 and skew:
+            empty = (torch.bincount(idx.cpu().flatten(), minlength=cfg.experts) == 0).nonzero().flatten()
+            assert not got[empty.to(device)].any(), "an expert without tokens must get an exact-zero weight gradient"
+    if "router_bias" in want_grads:
+        _check("grad router_bias", router.bias.grad, want_grads["router_bias"], tol)
+
+
+def test_layer_is_bit_reproducible(device):
+    cfg = CONFIG2_SMALL
+    inputs = make_layer_inputs(cfg)
+    runs = []
+    for _ in range(2):
+        layer = _build_layer(cfg, inputs, device)
+        x = inputs["x"].to(device).requires_grad_(True)
+        out = layer(x)
+        out.backward(inputs["grad_out"].to(device))
+        runs.append([out.detach(), x.grad, layer.gate.weight.grad, layer.gate_up_proj.grad, layer.down_proj.grad])
+    assert all(torch.equal(a, b) for a, b in zip(*runs))
+
+
+def test_one_gpus_share_of_an_ep_layer(device):
+    """Local ids with -1 for other ranks' picks plus host-side receive counts (an EP8 shard's shape, scaled down):
+    ``_compute_experts`` against the dense formula over the valid slots, and the count checks."""
+    from halo_amd.moe_layer import EPConfig, EPQwen3_5MoELayer
+    from oracle import moe_layer as oracle
+
+    g = torch.Generator().manual_seed(2)
+    local, ep, top_k, hidden, ffn, rows = 8, 8, 8, 256, 128, 700
+    picks = torch.rand(rows, local * ep, generator=g).argsort(dim=1)[:, :top_k]
+    experts = torch.where(picks < local, picks, -1)
+    experts = experts[(experts >= 0).any(dim=1)]  # a dispatch sends a token only where it has a local pick
+    n = experts.shape[0]
+    counts = tuple(torch.bincount(experts[experts >= 0], minlength=local).tolist())
+    weights = torch.rand(n, top_k, generator=g)
+    x = torch.randn(n, hidden, generator=g).bfloat16()
+    params = {"gate_up_proj": (torch.randn(local, hidden, 2 * ffn, generator=g) * 0.02).bfloat16(),
+              "down_proj": (torch.randn(local, ffn, hidden, generator=g) * 0.02).bfloat16()}
+    layer = EPQwen3_5MoELayer.from_weights(router_weight=None, top_k=top_k, ep_config=EPConfig(ep_size=ep, ep_rank=0),
+                                           **{k: v.to(device) for k, v in params.items()})
+    assert layer.experts_per_rank == local and layer.num_experts == local * ep
+    out = layer._compute_experts(x.to(device), experts.to(device), weights.to(device), torch.bfloat16,
+                                 recv_counts=counts)
+    want = oracle.compute_experts_loop(x.float(), experts, weights.bfloat16().float(),
+                                       {k: v.float() for k, v in params.items()}, oracle.Glu(), local)
+    _check("shard out", out, want, 2e-2)
+    with pytest.raises(RuntimeError, match="needs the dispatch's per-local-expert receive counts"):
+        layer._compute_experts(x.to(device), experts.to(device), weights.to(device), torch.bfloat16, recv_counts=None)
+    with pytest.raises(RuntimeError, match="needs the dispatch's per-local-expert receive counts"):
+        layer._compute_experts(x.to(device), experts.to(device), weights.to(device), torch.bfloat16,
+                               recv_counts=counts[:-1])
+    empty = layer._compute_experts(x[:0].to(device), experts[:0].to(device), weights[:0].to(device), torch.bfloat16,
+                                   recv_counts=(0,) * local)
+    assert empty.shape == (0, hidden)
+
+
+def test_quantised_weight_forward(device):
+    """Block-fp8 expert weights (BASELINE config 5, scaled down): forward only, against the dequantised-bf16 path."""
+    from halo_amd.kernels.expert_gemm import BlockFp8Weight
+    from halo_amd.kernels.lowp.block_fp8 import dequantize_block_fp8, quantize_block_fp8
+    from halo_amd.moe_layer import EPConfig, EPQwen3_5MoELayer
+
+    g = torch.Generator().manual_seed(4)
+    local, top_k, hidden, ffn, rows = 8, 8, 384, 256, 900
+    picks = torch.rand(rows, local * 8, generator=g).argsort(dim=1)[:, :top_k]
+    experts = torch.where(picks < local, picks, -1)
+    experts = experts[(experts >= 0).any(dim=1)]
+    counts = tuple(torch.bincount(experts[experts >= 0], minlength=local).tolist())
+    weights = torch.rand(experts.shape, generator=g)
+    x = torch.randn(experts.shape[0], hidden, generator=g).bfloat16().to(device)
+    w1 = (torch.randn(local, hidden, 2 * ffn, generator=g) * 0.02).to(device)
+    w2 = (torch.randn(local, ffn, hidden, generator=g) * 0.02).to(device)
+    q1, q2 = quantize_block_fp8(w1), quantize_block_fp8(w2)
+    cfg = EPConfig(ep_size=8, ep_rank=0)
+    lowp = EPQwen3_5MoELayer.from_weights(router_weight=None, top_k=top_k, ep_config=cfg,
+                                          gate_up_proj=BlockFp8Weight(*q1), down_proj=BlockFp8Weight(*q2))
+    ref = EPQwen3_5MoELayer.from_weights(router_weight=None, top_k=top_k, ep_config=EPConfig(ep_size=8, ep_rank=0),
+                                         gate_up_proj=dequantize_block_fp8(*q1), down_proj=dequantize_block_fp8(*q2))
+    with torch.no_grad():
+        got = lowp._compute_experts(x, experts.to(device), weights.to(device), torch.bfloat16, recv_counts=counts)
+        want = ref._compute_experts(x, experts.to(device), weights.to(device), torch.bfloat16, recv_counts=counts)
+    assert torch.equal(got, want)  # the dequantisation inside the kernel is exact
+
+
+# ------------------------------------------------------------------------------ drop-ins for the Hugging Face blocks
+
+def _hf_config(model_type, **kw):
+    import transformers
+
+    return getattr(transformers, model_type)(**kw)
+
+
+def test_drop_in_for_hf_qwen3_moe_block(device):
+    from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeSparseMoeBlock
+
+    from halo_amd.moe_layer import EPQwen3MoELayer, apply_ep_layers, single_process_ep_config
+
+    cfg = _hf_config("Qwen3MoeConfig", hidden_size=256, moe_intermediate_size=128, num_experts=16,
+                     num_experts_per_tok=4, norm_topk_prob=True, hidden_act="silu")
+    torch.manual_seed(0)
+    block = Qwen3MoeSparseMoeBlock(cfg)
+    for p in block.parameters():
+        torch.nn.init.normal_(p, std=0.05)
+    x = torch.randn(2, 48, 256)
+    want = block(x)
+    want.sum().backward()
+    holder = torch.nn.Sequential(torch.nn.Identity(), block.to(device))
+    assert apply_ep_layers(holder, single_process_ep_config()) == 1
+    layer = holder[1]
+    assert isinstance(layer, EPQwen3MoELayer) and hasattr(layer, "gate_proj") and not hasattr(layer, "gate_up_proj")
+    assert layer.gate_proj.shape == (16, 256, 128) and layer.down_proj.shape == (16, 128, 256)
+    xd = x.to(device).requires_grad_(True)
+    got = layer(xd)
+    got.sum().backward()
+    _check("qwen3 out", got, want, 1e-4)
+    assert max_rel(layer.gate.weight.grad, block.gate.weight.grad.cpu()) < 1e-3
+    assert {n for n, _ in layer.expert_named_params()} == {"gate_proj", "up_proj", "down_proj"}
+
+
+def test_drop_in_for_hf_gpt_oss_block(device):
+    from transformers.models.gpt_oss.modeling_gpt_oss import GptOssMLP
+
+    from halo_amd.moe_layer import EPGptOssMoELayer, single_process_ep_config
+
+    cfg = _hf_config("GptOssConfig", hidden_size=256, intermediate_size=128, num_local_experts=8,
+                     num_experts_per_tok=2)
+    torch.manual_seed(1)
+    block = GptOssMLP(cfg)
+    for p in block.parameters():
+        torch.nn.init.normal_(p, std=0.05)
+    x = torch.randn(1, 40, 256)
+    result = block(x)
+    want = result[0] if isinstance(result, tuple) else result
+    layer = EPGptOssMoELayer(block.to(device), single_process_ep_config())
+    got, logits = layer(x.to(device))
+    _check("gpt-oss out", got.view(want.shape), want, 1e-4)
+    assert logits.shape == (40, 8) and layer._glu_combine_name() == "gptoss"
