@@ -6,40 +6,60 @@
 //   wgrad  dB[g]     = A[s:e]^T @ dO[s:e]      ragged contraction, empty group -> exact zeros
 // with offs[g] the inclusive end of group g.  bf16 operands, fp32 accumulation on MFMA, one rounding.
 //
-// bf16 kernel.  One persistent launch; a workgroup (4 wavefronts) owns a 128x128 output tile and walks the
-// contraction in steps of 64.  Both operand tiles sit in LDS as [128 output index][64 contraction index] with the
-// contraction contiguous, so every MFMA fragment is one 16-byte LDS read; the 16-byte chunk index is XOR-swizzled with
-// the row so fragment reads, straight copies and transposed writes are all bank-conflict free.  An operand whose
-// contraction index is the strided one in global memory (B in fwd, both operands in wgrad) is transposed in registers
-// (8x8 blocks of bf16, v_perm_b32) on its way into LDS.  Wavefronts 0-1 load operand A, 2-3 operand B; global loads
-// for step k+1 are issued before the MFMAs of step k (register prefetch, two LDS buffers, one barrier per step).
-// MFMA v_mfma_f32_32x32x16_bf16 is issued with the operands swapped (B fragment as srcA) so that a lane owns one
-// output row and four consecutive columns per accumulator quad: stores are 8 bytes per lane.
+// bf16 kernel.  One persistent launch.  A workgroup of GM x GN wavefronts owns a (GM*WM*32) x (GN*WN*32) output
+// tile and walks the contraction in steps of 64; each wavefront owns WM x WN accumulator blocks of 32x32
+// (v_mfma_f32_32x32x16_bf16).  LDS is the scarce resource on this chip (128 B/clk/CU read, about half that written),
+// so the tile is as large as the accumulators allow: per contraction element a wavefront reads (WM+WN)*32 operand
+// values for WM*WN*1024 multiply-adds.
+// Both operand tiles sit in LDS as [output index][64 contraction], contraction contiguous, so every MFMA fragment is
+// one 16-byte LDS read; the 16-byte chunk index is XOR-swizzled with the row, which keeps fragment reads, straight
+// copies and transposed writes free of bank conflicts.  An operand whose contraction index is the strided one in
+// global memory (B in fwd, both operands in wgrad) is transposed in registers (8x8 blocks of bf16, v_perm_b32) on its
+// way into LDS.  Global loads are raw buffer loads: rows past the group's end and columns past the operand's edge
+// come back as zeros from the hardware bounds check, with no branches in the loop.  Loads for step k+1 are issued
+// before the MFMAs of step k (register staging, two LDS buffers, one barrier per step).  The MFMA is issued with the
+// operands swapped (B fragment as srcA) so that a lane owns one output row and four consecutive columns per
+// accumulator quad: stores are 8 bytes per lane.
 //
 // Tile schedule.  Every workgroup builds the per-group prefix of row tiles from offs in LDS (no host readback), so
 // ragged and empty groups cost exactly their tiles.  The logical tile order is group-major, then column tile, then
 // row tile; it is cut into 8 contiguous chunks, one per XCD (workgroup w runs on XCD w % 8), so the workgroups that
 // share an L2 work on the same expert's weights at the same time, and the tile count per XCD is balanced whatever
-// the skew of the expert loads.
+// the skew of the expert loads.  wgrad tiles are dealt round-robin so every workgroup sees every group size.
 //
 // fp32 operands take a plain LDS-tiled FMA kernel (the CPU-sized plumbing configuration and tests).
 #include "common.h"
+
+#include <cstdlib>
+#include <type_traits>
 
 namespace hmoe {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int BM = 128;  // output rows per tile (operand A's output index)
-constexpr int BN = 128;  // output cols per tile (operand B's output index)
-constexpr int BK = 64;   // contraction per step
-constexpr int kThreads = 256;
-constexpr int kTile = 128 * BK;  // elements of one operand tile
+#ifndef HMOE_ABLATE
+#define HMOE_ABLATE 0
+#endif
+
+constexpr int BK = 64;  // contraction per step
 constexpr int kXcds = 8;
 constexpr int kMaxGroups = 1024;
 
 enum Mode { kFwd = 0, kDgrad = 1, kWgrad = 2, kFwdFp8W = 3 };
+
+// Tile configuration: GM x GN wavefronts, each WM x WN blocks of 32x32.
+template <int GM_, int GN_, int WM_, int WN_>
+struct Config {
+  static constexpr int GM = GM_, GN = GN_, WM = WM_, WN = WN_;
+  static constexpr int kThreads = 64 * GM * GN;
+  static constexpr int BM = GM * WM * 32;  // output rows per tile (operand A's output index)
+  static constexpr int BN = GN * WN * 32;  // output cols per tile (operand B's output index)
+  static constexpr int kStage = (BM + BN) * BK;  // elements of one LDS stage (A tile then B tile)
+};
 
 struct GemmArgs {
   const void* a;  // fwd: A, dgrad: dO, wgrad: A
@@ -53,6 +73,7 @@ struct GemmArgs {
   int groups;
   int64_t k, n;
   const float* b_scale;  // kFwdFp8W: [G, ceil(K/128), ceil(N/128)]
+  int ablate;            // diagnostics: 1 skip global loads, 2 skip LDS stores, 4 skip MFMAs, 8 skip fragment reads
 };
 
 __device__ __forceinline__ int swizzle(int row) { return (row & 7) ^ ((row >> 3) & 7); }
@@ -73,60 +94,114 @@ __device__ __forceinline__ void group_bounds(const int32_t* offs, int g, int64_t
   end = e;
 }
 
-// One operand tile's global -> register -> LDS path for the 128 threads that serve it.  A loader describes the
-// operand (base pointer, row stride, first output index of the tile, limits) and moves one contraction step.
-// kTrans == false: element(out, con) = base[out * ld + con]  (contraction contiguous)
-// kTrans == true : element(out, con) = base[con * ld + out]  (output index contiguous), transposed on the way in
-template <bool kTrans>
-struct Bf16Loader {
-  const bf16_t* __restrict__ base;
-  int64_t ld;
-  int out0, out_lim, con_lim;
+constexpr uint32_t kOutOfRange = 0x80000000u;  // a byte offset no operand reaches: the buffer load returns zeros
 
-  __device__ __forceinline__ void load(uint4 (&reg)[8], int con0, int tt) {
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+
+// One operand tile's global -> register -> LDS path.  A loader describes the operand (a buffer resource bounded at
+// the operand's end, row stride, first output index of the tile, limits) and moves one contraction step.
+// kTrans == false: element(out, con) = base[out * ld + con]  (contraction contiguous); every thread of the
+//                  workgroup moves kRows * 8 / kThreads 16-byte chunks.
+// kTrans == true : element(out, con) = base[con * ld + out]  (output index contiguous), transposed on the way in;
+//                  the kRows 8x8 blocks of a step are dealt to threads kFirst, kFirst + 1, ...
+template <bool kTrans, int kRows, int kThreads, int kFirst>
+struct Bf16Loader {
+  static constexpr int kServing = kRows < kThreads ? kRows : kThreads;           // threads with transposing work
+  static constexpr int kBlocks = kTrans ? (kRows + kServing - 1) / kServing : 1;  // 8x8 blocks per serving thread
+  static constexpr int kChunks = kTrans ? 8 * kBlocks : kRows * 8 / kThreads;     // 16-byte loads per thread
+  static constexpr int kOffsets = kTrans ? kBlocks : kChunks;
+  static_assert(kTrans || (kRows * 8) % kThreads == 0, "tile rows must spread evenly over the workgroup");
+  static_assert(!kTrans || kRows % kServing == 0, "transposed tile must spread evenly over its threads");
+
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t voff[kOffsets];  // per chunk (direct) or per block (transposed) byte offset at contraction index 0
+  uint32_t step_bytes;      // byte distance of one contraction step
+  uint32_t row_bytes;       // transposed: byte distance of one contraction index
+  int con_lim;
+  bool serving;
+
+  // `bytes` bounds the operand (rows past the group's end fall outside it).
+  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
+                                       int con_lim_, int tid) {
+    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
+    con_lim = con_lim_;
     if constexpr (!kTrans) {
+      serving = true;
+      step_bytes = BK * 2;
+      row_bytes = 0;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int cid = tt + 128 * i;
-        const int out = out0 + (cid >> 3), con = con0 + ((cid & 7) << 3);
-        reg[i] = make_uint4(0, 0, 0, 0);
-        if (out < out_lim && con < con_lim)
-          reg[i] = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(out) * ld + con);
+      for (int i = 0; i < kChunks; ++i) {
+        const int cid = tid + kThreads * i;
+        const int out = out0 + (cid >> 3);
+        voff[i] = out < out_lim ? static_cast<uint32_t>(out) * static_cast<uint32_t>(ld) * 2u + ((cid & 7) << 4)
+                                : kOutOfRange;
       }
     } else {
-      const int out = out0 + ((tt & 15) << 3);
-      const int con_first = con0 + ((tt >> 4) << 3);
+      const int t = tid - kFirst;
+      serving = t >= 0 && t < kServing;
+      row_bytes = static_cast<uint32_t>(ld) * 2u;
+      step_bytes = BK * row_bytes;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int con = con_first + i;
-        reg[i] = make_uint4(0, 0, 0, 0);
-        if (out < out_lim && con < con_lim)
-          reg[i] = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(con) * ld + out);
+      for (int i = 0; i < kBlocks; ++i) {
+        const int blk = t + kServing * i;
+        const int ob = blk % (kRows / 8), cb = blk / (kRows / 8);
+        const int out = out0 + (ob << 3);
+        voff[i] = (serving && out < out_lim)
+                      ? static_cast<uint32_t>(cb * 8) * row_bytes + static_cast<uint32_t>(out) * 2u
+                      : kOutOfRange;
       }
     }
   }
 
-  __device__ __forceinline__ void store(const uint4 (&reg)[8], bf16_t* __restrict__ tile, int tt) const {
+  __device__ __forceinline__ void load(u32x4 (&reg)[kChunks], int step) const {
+    const uint32_t soff = static_cast<uint32_t>(step) * step_bytes;
     if constexpr (!kTrans) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int cid = tt + 128 * i;
-        *reinterpret_cast<uint4*>(tile + lds_offset(cid >> 3, cid & 7)) = reg[i];
+      for (int i = 0; i < kChunks; ++i) {
+        // only the last step can run past the contraction's end (con_lim is a multiple of 8)
+        const int con = step * BK + (((threadIdx.x + kThreads * i) & 7) << 3);
+        const uint32_t off = con < con_lim ? voff[i] : kOutOfRange;
+        reg[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, soff, 0);
       }
     } else {
-      // reg[i] holds contraction index i, output indices 0..7 (two per dword).  Row o of the 8x8 block gathers
-      // output index o from the eight registers: dword w of the result packs contraction 2w (low) and 2w+1 (high).
-      const int row0 = (tt & 15) << 3, chunk = tt >> 4;
-      const uint32_t(*r)[4] = reinterpret_cast<const uint32_t(*)[4]>(reg);
 #pragma unroll
-      for (int o = 0; o < 8; ++o) {
-        const uint32_t sel = (o & 1) ? 0x07060302u : 0x05040100u;
-        uint4 v;
-        v.x = __builtin_amdgcn_perm(r[1][o >> 1], r[0][o >> 1], sel);
-        v.y = __builtin_amdgcn_perm(r[3][o >> 1], r[2][o >> 1], sel);
-        v.z = __builtin_amdgcn_perm(r[5][o >> 1], r[4][o >> 1], sel);
-        v.w = __builtin_amdgcn_perm(r[7][o >> 1], r[6][o >> 1], sel);
-        *reinterpret_cast<uint4*>(tile + lds_offset(row0 + o, chunk)) = v;
+      for (int i = 0; i < kBlocks; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)  // rows past the contraction's end lie past the buffer's end
+          reg[i * 8 + j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff[i] + j * row_bytes, soff, 0);
+    }
+  }
+
+  // `tile` is the element offset of this operand's tile inside the workgroup's LDS array `smem` (an integer, so
+  // every access stays an LDS instruction)
+  __device__ __forceinline__ void store(const u32x4 (&reg)[kChunks], bf16_t* smem, int tile, int tid) const {
+    if constexpr (!kTrans) {
+#pragma unroll
+      for (int i = 0; i < kChunks; ++i) {
+        const int cid = tid + kThreads * i;
+        *reinterpret_cast<u32x4*>(smem + tile + lds_offset(cid >> 3, cid & 7)) = reg[i];
+      }
+    } else {
+      if (!serving) return;
+      const int t = tid - kFirst;
+#pragma unroll
+      for (int i = 0; i < kBlocks; ++i) {
+        const int blk = t + kServing * i;
+        const int row0 = (blk % (kRows / 8)) << 3, chunk = blk / (kRows / 8);
+        // reg[8i + c] holds contraction index c, output indices 0..7 (two per dword).  Row o of the 8x8 block
+        // gathers output index o: dword w of the result packs contraction 2w (low half) and 2w+1 (high half).
+#pragma unroll
+        for (int o = 0; o < 8; ++o) {
+          const uint32_t sel = (o & 1) ? 0x07060302u : 0x05040100u;
+          u32x4 v;
+          v.x = __builtin_amdgcn_perm(reg[8 * i + 1][o >> 1], reg[8 * i + 0][o >> 1], sel);
+          v.y = __builtin_amdgcn_perm(reg[8 * i + 3][o >> 1], reg[8 * i + 2][o >> 1], sel);
+          v.z = __builtin_amdgcn_perm(reg[8 * i + 5][o >> 1], reg[8 * i + 4][o >> 1], sel);
+          v.w = __builtin_amdgcn_perm(reg[8 * i + 7][o >> 1], reg[8 * i + 6][o >> 1], sel);
+          *reinterpret_cast<u32x4*>(smem + tile + lds_offset(row0 + o, chunk)) = v;
+        }
       }
     }
   }
@@ -134,149 +209,223 @@ struct Bf16Loader {
 
 // e4m3fn weights [contraction, output] (output contiguous) with one power-of-two fp32 scale per 128x128 block,
 // dequantised to bf16 (exactly: an e4m3 value times a power of two is a bf16 value) and transposed on the way into
-// LDS.  A tile spans one scale block across the outputs and at most one along the contraction step (128 % BK == 0).
+// LDS.  Each 8-column block lies inside one scale column; a step spans one scale row (128 % BK == 0).
+template <int kRows, int kThreads, int kFirst>
 struct Fp8BlockLoader {
-  const uint8_t* __restrict__ base;
-  int64_t ld;
-  int out0, out_lim, con_lim;
-  const float* __restrict__ scale;  // this group's scale grid, at column block out0 / 128
-  int scale_ld;                     // scale blocks per contraction block row
-  float step_scale;
+  static constexpr int kServing = kRows < kThreads ? kRows : kThreads;
+  static constexpr int kBlocks = (kRows + kServing - 1) / kServing;
+  static constexpr int kChunks = 4 * kBlocks;  // eight 8-byte loads per block, two per staging register
+  static_assert(kRows % kServing == 0, "transposed tile must spread evenly over its threads");
 
-  __device__ __forceinline__ void load(uint4 (&reg)[8], int con0, int tt) {
-    const int out = out0 + ((tt & 15) << 3);
-    const int con_first = con0 + ((tt >> 4) << 3);
-    step_scale = scale[static_cast<int64_t>(con0 >> 7) * scale_ld];
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t voff[kBlocks];
+  uint32_t step_bytes, row_bytes;
+  const float* scale[kBlocks];  // this block's scale column, at contraction block 0
+  int scale_ld;
+  float step_scale[kBlocks];
+  bool serving;
+
+  __device__ __forceinline__ void init(const uint8_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
+                                       const float* group_scale, int scale_ld_, int tid) {
+    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
+    const int t = tid - kFirst;
+    serving = t >= 0 && t < kServing;
+    row_bytes = static_cast<uint32_t>(ld);
+    step_bytes = BK * row_bytes;
+    scale_ld = scale_ld_;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int con = con_first + i;
-      uint2 v = make_uint2(0, 0);
-      if (out < out_lim && con < con_lim)
-        v = *reinterpret_cast<const uint2*>(base + static_cast<int64_t>(con) * ld + out);
-      reg[i].x = v.x;
-      reg[i].y = v.y;
+    for (int i = 0; i < kBlocks; ++i) {
+      const int blk = t + kServing * i;
+      const int ob = blk % (kRows / 8), cb = blk / (kRows / 8);
+      const int out = out0 + (ob << 3);
+      const bool ok = serving && out < out_lim;
+      voff[i] = ok ? static_cast<uint32_t>(cb * 8) * row_bytes + static_cast<uint32_t>(out) : kOutOfRange;
+      scale[i] = group_scale + (ok ? (out >> 7) : 0);
     }
   }
 
-  __device__ __forceinline__ void store(const uint4 (&reg)[8], bf16_t* __restrict__ tile, int tt) const {
+  __device__ __forceinline__ void load(u32x4 (&reg)[kChunks], int step) {
+    const uint32_t soff = static_cast<uint32_t>(step) * step_bytes;
+#pragma unroll
+    for (int i = 0; i < kBlocks; ++i) {
+      step_scale[i] = serving ? scale[i][static_cast<int64_t>((step * BK) >> 7) * scale_ld] : 1.0f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const u32x2 lo = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff[i] + (2 * j) * row_bytes, soff, 0);
+        const u32x2 hi = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff[i] + (2 * j + 1) * row_bytes, soff, 0);
+        reg[i * 4 + j] = u32x4{lo.x, lo.y, hi.x, hi.y};  // contraction 2j in .xy, 2j+1 in .zw
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(const u32x4 (&reg)[kChunks], bf16_t* smem, int tile, int tid) const {
     typedef float f32x2 __attribute__((ext_vector_type(2)));
-    const int row0 = (tt & 15) << 3, chunk = tt >> 4;
-    uint32_t packed[8][4];  // [output][contraction pair]
+    if (!serving) return;
+    const int t = tid - kFirst;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      float lo[8], hi[8];  // contraction 2w and 2w+1, outputs 0..7
+    for (int i = 0; i < kBlocks; ++i) {
+      const int blk = t + kServing * i;
+      const int row0 = (blk % (kRows / 8)) << 3, chunk = blk / (kRows / 8);
+      const float s = step_scale[i];
+      uint32_t packed[8][4];  // [output][contraction pair]
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const uint4 src = reg[2 * w + h];
-        float* f = h ? hi : lo;
-        const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(src.x, step_scale, false);
-        const f32x2 b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(src.x, step_scale, true);
-        const f32x2 c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(src.y, step_scale, false);
-        const f32x2 d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(src.y, step_scale, true);
-        f[0] = a.x; f[1] = a.y; f[2] = b.x; f[3] = b.y; f[4] = c.x; f[5] = c.y; f[6] = d.x; f[7] = d.y;
+      for (int w = 0; w < 4; ++w) {
+        float lo[8], hi[8];  // contraction 2w and 2w+1, outputs 0..7
+        const u32x4 src = reg[i * 4 + w];
+        const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(src.x, s, false);
+        const f32x2 b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(src.x, s, true);
+        const f32x2 c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(src.y, s, false);
+        const f32x2 d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(src.y, s, true);
+        lo[0] = a.x; lo[1] = a.y; lo[2] = b.x; lo[3] = b.y; lo[4] = c.x; lo[5] = c.y; lo[6] = d.x; lo[7] = d.y;
+        const f32x2 e = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(src.z, s, false);
+        const f32x2 f = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(src.z, s, true);
+        const f32x2 g = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(src.w, s, false);
+        const f32x2 h = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(src.w, s, true);
+        hi[0] = e.x; hi[1] = e.y; hi[2] = f.x; hi[3] = f.y; hi[4] = g.x; hi[5] = g.y; hi[6] = h.x; hi[7] = h.y;
+#pragma unroll
+        for (int o = 0; o < 8; ++o)
+          packed[o][w] =
+              static_cast<uint32_t>(f32_to_bf16(lo[o])) | (static_cast<uint32_t>(f32_to_bf16(hi[o])) << 16);
       }
 #pragma unroll
       for (int o = 0; o < 8; ++o)
-        packed[o][w] = static_cast<uint32_t>(f32_to_bf16(lo[o])) | (static_cast<uint32_t>(f32_to_bf16(hi[o])) << 16);
+        *reinterpret_cast<u32x4*>(smem + tile + lds_offset(row0 + o, chunk)) =
+            u32x4{packed[o][0], packed[o][1], packed[o][2], packed[o][3]};
     }
-#pragma unroll
-    for (int o = 0; o < 8; ++o)
-      *reinterpret_cast<uint4*>(tile + lds_offset(row0 + o, chunk)) =
-          make_uint4(packed[o][0], packed[o][1], packed[o][2], packed[o][3]);
   }
 };
 
-// C[a_out, b_out] = sum_con A(a_out, con) * B(b_out, con) over one 128x128 tile.
-template <typename LoaderA, typename LoaderB>
-__device__ __forceinline__ void compute_tile(bf16_t* __restrict__ smem, LoaderA la, LoaderB lb,
-                                             bf16_t* __restrict__ c_base, int64_t c_ld) {
+// C[a_out, b_out] = sum_con A(a_out, con) * B(b_out, con) over one BM x BN tile.
+template <typename Cfg, typename LoaderA, typename LoaderB>
+__device__ __forceinline__ void compute_tile(bf16_t* smem, LoaderA& la, LoaderB& lb, int a_out0,
+                                             int a_out_lim, int b_out0, int b_out_lim, int con_lim,
+                                             bf16_t* __restrict__ c_base, int64_t c_ld, int /*unused*/ = 0) {
+  constexpr int ablate = HMOE_ABLATE;  // compile-time diagnostics switch, 0 in the product build
+  constexpr int WM = Cfg::WM, WN = Cfg::WN;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const bool loads_a = tid < 128;
-  const int tt = tid & 127;
-  bf16_t* s_a = smem;               // [2][kTile]
-  bf16_t* s_b = smem + 2 * kTile;   // [2][kTile]
-  const int a_out0 = la.out0, a_out_lim = la.out_lim, b_out0 = lb.out0, b_out_lim = lb.out_lim;
-  const int con_lim = la.con_lim;
+  const int gm = wave / Cfg::GN, gn = wave % Cfg::GN;
+  constexpr int kTileB = Cfg::BM * BK;  // element offset of the B tile inside a stage
+  constexpr int kStoreAfter = 1;        // contraction sub-step after which the staged tile is written to LDS
 
-  uint4 reg[8];  // the thread's share of the next operand tile (A for wavefronts 0-1, B for 2-3)
-  f32x16 acc[2][2];
+  u32x4 reg_a[LoaderA::kChunks];
+  u32x4 reg_b[LoaderB::kChunks];
+  f32x16 acc[WM][WN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   const int steps = (con_lim + BK - 1) / BK;
   if (steps > 0) {
-    if (loads_a) {
-      la.load(reg, 0, tt);
-      la.store(reg, s_a, tt);
-    } else {
-      lb.load(reg, 0, tt);
-      lb.store(reg, s_b, tt);
-    }
+    la.load(reg_a, 0);
+    lb.load(reg_b, 0);
+    la.store(reg_a, smem, 0, tid);
+    lb.store(reg_b, smem, kTileB, tid);
   }
   __syncthreads();
-  for (int step = 0; step < steps; ++step) {
-    const int cur = step & 1;
-    const bool more = step + 1 < steps;
-    if (more) {
-      if (loads_a) la.load(reg, (step + 1) * BK, tt);
-      else lb.load(reg, (step + 1) * BK, tt);
-    }
-    const bf16_t* ta = s_a + cur * kTile;
-    const bf16_t* tb = s_b + cur * kTile;
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      const int chunk = kk * 2 + (lane >> 5);
-      bf16x8 fa[2], fb[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int ra = wm * 64 + i * 32 + (lane & 31);
-        const int rb = wn * 64 + i * 32 + (lane & 31);
-        fa[i] = *reinterpret_cast<const bf16x8*>(ta + lds_offset(ra, chunk));
-        fb[i] = *reinterpret_cast<const bf16x8*>(tb + lds_offset(rb, chunk));
+  const int row_a = gm * (WM * 32) + (lane & 31);
+  const int row_b = gn * (WN * 32) + (lane & 31);
+  // 32-row blocks of this wavefront that hold at least one valid output row: a group's last row tile is mostly empty,
+  // and the blocks past its end are skipped (the wavefront still moves its share of the operand tiles)
+  int live = (a_out_lim - (a_out0 + gm * (WM * 32)) + 31) >> 5;
+  live = live < 0 ? 0 : (live > WM ? WM : live);
+
+  auto run = [&](auto full_tag) {
+    constexpr bool kFull = decltype(full_tag)::value;
+    for (int step = 0; step < steps; ++step) {
+      const int cur = step & 1;
+      const bool more = step + 1 < steps;
+      if (more && !(ablate & 1)) {
+        la.load(reg_a, step + 1);
+        lb.load(reg_b, step + 1);
       }
+      const int ta = cur * Cfg::kStage;
+      const int tb = ta + kTileB;
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int kk = 0; kk < BK / 16; ++kk) {
+        const int chunk = kk * 2 + (lane >> 5);
+        bf16x8 fa[WM], fb[WN];
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < WN; ++j)
+          fb[j] = *reinterpret_cast<const bf16x8*>(smem + tb + lds_offset(row_b + j * 32, (ablate & 8) ? 0 : chunk));
+#pragma unroll
+        for (int i = 0; i < WM; ++i) {
+          if (kFull || i < live) {
+            fa[i] = *reinterpret_cast<const bf16x8*>(smem + ta + lds_offset(row_a + i * 32, (ablate & 8) ? 0 : chunk));
+            if (!(ablate & 4)) {
+#pragma unroll
+              for (int j = 0; j < WN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+            } else {
+              acc[i][0][0] += static_cast<float>(fa[i][0]) + static_cast<float>(fb[0][0]);
+            }
+          }
+        }
+        if (kk == kStoreAfter && more && !(ablate & 2)) {
+          // the next stage's LDS writes go out between the MFMAs, not after them, so they overlap matrix work
+          __builtin_amdgcn_sched_barrier(0);
+          la.store(reg_a, smem, (cur ^ 1) * Cfg::kStage, tid);
+          lb.store(reg_b, smem, (cur ^ 1) * Cfg::kStage + kTileB, tid);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      __syncthreads();
     }
-    if (more) {
-      if (loads_a) la.store(reg, s_a + (cur ^ 1) * kTile, tt);
-      else lb.store(reg, s_b + (cur ^ 1) * kTile, tt);
-    }
-    __syncthreads();
-  }
-  // lane owns output row (lane & 31) of each 32x32 block; accumulator quad q holds columns q*8 + (lane>>5)*4 .. +3
+  };
+  if (live == WM) run(std::true_type{});
+  else run(std::false_type{});
+  // Epilogue.  After the swapped MFMA a lane owns output row (lane & 31) of each 32x32 block, and accumulator quad q
+  // holds columns q*8 + (lane>>5)*4 .. +3: stored as they are, every store instruction would touch 32 different cache
+  // lines with 16 bytes each.  Instead each wavefront passes its block through a private LDS region (the operand
+  // stages are free after the last step's barrier), 64 rows at a time, and writes whole 16-byte chunks with the lanes
+  // of a row segment contiguous: full lines per instruction.
+  constexpr int kEpiPitch = WN * 32 + 8;               // elements per staged row (16 bytes of padding)
+  constexpr int kEpiRegion = 64 * kEpiPitch;           // elements per wavefront
+  constexpr int kLanesPerRow = WN * 4;                 // 16-byte chunks in a staged row
+  constexpr int kRowsPerPass = 64 / kLanesPerRow;
+  static_assert(kEpiRegion * Cfg::GM * Cfg::GN <= 2 * Cfg::kStage, "epilogue staging must fit in the operand stages");
+  bf16_t* stage = smem + wave * kEpiRegion;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int row = a_out0 + wm * 64 + i * 32 + (lane & 31);
-    if (row >= a_out_lim) continue;
-    bf16_t* c_row = c_base + static_cast<int64_t>(row) * c_ld;
+  for (int half = 0; half < (WM + 1) / 2; ++half) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int ii = 0; ii < 2; ++ii) {
+      const int i = half * 2 + ii;
+      if (i >= WM) break;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int col = b_out0 + wn * 64 + j * 32 + q * 8 + ((lane >> 5) << 2);
-        if (col < b_out_lim) {
+      for (int j = 0; j < WN; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
           uint2 packed;
           packed.x = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 0])) |
                      (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 1])) << 16);
           packed.y = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 2])) |
                      (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 3])) << 16);
-          *reinterpret_cast<uint2*>(c_row + col) = packed;
+          *reinterpret_cast<uint2*>(stage + (ii * 32 + (lane & 31)) * kEpiPitch + j * 32 + q * 8 + ((lane >> 5) << 2)) =
+              packed;
         }
       }
     }
+    __syncthreads();
+#pragma unroll
+    for (int pass = 0; pass < 64 / kRowsPerPass; ++pass) {
+      const int rr = pass * kRowsPerPass + lane / kLanesPerRow;
+      const int cc = (lane % kLanesPerRow) << 3;
+      const int row = a_out0 + gm * (WM * 32) + half * 64 + rr;
+      const int col = b_out0 + gn * (WN * 32) + cc;
+      if (half * 64 + rr < WM * 32 && row < a_out_lim && col < b_out_lim && !((ablate & 16) && c_ld != 12345)) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * kEpiPitch + cc);
+        *reinterpret_cast<u32x4*>(c_base + static_cast<int64_t>(row) * c_ld + col) = v;
+      }
+    }
+    __syncthreads();  // the region is rewritten by the next half, and by the next tile's first operand stage
   }
 }
 
 // Exclusive prefix of the per-group row-tile counts into LDS: tile_start[0..groups], by wavefront 0.
+template <int BM>
 __device__ __forceinline__ void build_tile_prefix(int32_t* tile_start, const int32_t* offs, int groups,
                                                   int64_t total_rows) {
   if (threadIdx.x < HMOE_WAVE) {
@@ -307,18 +456,23 @@ __device__ __forceinline__ void build_tile_prefix(int32_t* tile_start, const int
   __syncthreads();
 }
 
-template <int kMode>
-__global__ void __launch_bounds__(kThreads, 2) grouped_gemm_bf16_kernel(GemmArgs p) {
-  __shared__ __attribute__((aligned(16))) bf16_t smem[4 * kTile];
+template <int kMode, typename Cfg>
+__global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) bf16_t smem[];  // two stages of (A tile, B tile)
   __shared__ int32_t tile_start[kMode == kWgrad ? 1 : kMaxGroups + 1];
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, NT = Cfg::kThreads;
   const bf16_t* a = static_cast<const bf16_t*>(p.a);
   const bf16_t* b = static_cast<const bf16_t*>(p.b);
   bf16_t* c = static_cast<bf16_t*>(p.c);
+  const int tid = threadIdx.x;
 
   const int workers = gridDim.x;
   const int xcd = blockIdx.x % kXcds;
   const int local = blockIdx.x / kXcds;
   const int workers_here = (workers - xcd + kXcds - 1) / kXcds;
+  // the transposing loader of operand B takes the workgroup's last BN threads, so that in wgrad (both operands
+  // transposed) the first threads move A's blocks and the last ones B's
+  constexpr int kFirstB = BN < NT ? NT - BN : 0;
 
   if constexpr (kMode == kWgrad) {
     const int mt = static_cast<int>((p.k + BM - 1) / BM), nt = static_cast<int>((p.n + BN - 1) / BN);
@@ -331,21 +485,24 @@ __global__ void __launch_bounds__(kThreads, 2) grouped_gemm_bf16_kernel(GemmArgs
       int64_t s, e;
       group_bounds(p.offs, g, p.total_rows, s, e);
       const int rows = static_cast<int>(e - s);
-      compute_tile(smem, Bf16Loader<true>{a + s * p.lda, p.lda, m_t * BM, static_cast<int>(p.k), rows},
-                   Bf16Loader<true>{b + s * p.ldb, p.ldb, n_t * BN, static_cast<int>(p.n), rows},
-                   c + static_cast<int64_t>(g) * p.k * p.n, p.ldc);
+      Bf16Loader<true, BM, NT, 0> la;
+      Bf16Loader<true, BN, NT, kFirstB> lb;
+      la.init(a + s * p.lda, p.lda, rows * p.lda * 2, m_t * BM, static_cast<int>(p.k), rows, tid);
+      lb.init(b + s * p.ldb, p.ldb, rows * p.ldb * 2, n_t * BN, static_cast<int>(p.n), rows, tid);
+      compute_tile<Cfg>(smem, la, lb, m_t * BM, static_cast<int>(p.k), n_t * BN, static_cast<int>(p.n), rows,
+                        c + static_cast<int64_t>(g) * p.k * p.n, p.ldc, p.ablate);
     }
   } else {
-    build_tile_prefix(tile_start, p.offs, p.groups, p.total_rows);
+    build_tile_prefix<BM>(tile_start, p.offs, p.groups, p.total_rows);
     const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
-    const int64_t con = kMode == kDgrad ? p.n : p.k;
+    const int con = static_cast<int>(kMode == kDgrad ? p.n : p.k);
     const int nt = static_cast<int>((out_cols + BN - 1) / BN);
     const int64_t total = static_cast<int64_t>(tile_start[p.groups]) * nt;
     const int64_t chunk = (total + kXcds - 1) / kXcds;
     const int64_t first = xcd * chunk;
     const int64_t last = first + chunk < total ? first + chunk : total;
     for (int64_t t = first + local; t < last; t += workers_here) {
-      int lo = 0, hi = p.groups;        // largest g with tile_start[g] * nt <= t
+      int lo = 0, hi = p.groups;  // largest g with tile_start[g] * nt <= t
       while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
         if (static_cast<int64_t>(tile_start[mid]) * nt <= t) lo = mid; else hi = mid;
@@ -356,23 +513,25 @@ __global__ void __launch_bounds__(kThreads, 2) grouped_gemm_bf16_kernel(GemmArgs
       const int n_t = r / mt, m_t = r - n_t * mt;
       int64_t s, e;
       group_bounds(p.offs, g, p.total_rows, s, e);
-      const Bf16Loader<false> la{a + s * p.lda, p.lda, m_t * BM, static_cast<int>(e - s), static_cast<int>(con)};
+      const int rows = static_cast<int>(e - s);
+      Bf16Loader<false, BM, NT, 0> la;
+      la.init(a + s * p.lda, p.lda, rows * p.lda * 2, m_t * BM, rows, con, tid);
+      const int64_t w_elems = p.k * p.n;
       if constexpr (kMode == kFwd) {
-        const bf16_t* w = b + static_cast<int64_t>(g) * p.k * p.n;
-        compute_tile(smem, la, Bf16Loader<true>{w, p.ldb, n_t * BN, static_cast<int>(p.n), static_cast<int>(con)},
-                     c + s * p.ldc, p.ldc);
+        Bf16Loader<true, BN, NT, kFirstB> lb;
+        lb.init(b + g * w_elems, p.ldb, w_elems * 2, n_t * BN, static_cast<int>(p.n), con, tid);
+        compute_tile<Cfg>(smem, la, lb, m_t * BM, rows, n_t * BN, static_cast<int>(p.n), con, c + s * p.ldc, p.ldc, p.ablate);
       } else if constexpr (kMode == kDgrad) {
-        const bf16_t* w = b + static_cast<int64_t>(g) * p.k * p.n;
-        compute_tile(smem, la, Bf16Loader<false>{w, p.ldb, n_t * BN, static_cast<int>(p.k), static_cast<int>(con)},
-                     c + s * p.ldc, p.ldc);
+        Bf16Loader<false, BN, NT, 0> lb;
+        lb.init(b + g * w_elems, p.ldb, w_elems * 2, n_t * BN, static_cast<int>(p.k), con, tid);
+        compute_tile<Cfg>(smem, la, lb, m_t * BM, rows, n_t * BN, static_cast<int>(p.k), con, c + s * p.ldc, p.ldc, p.ablate);
       } else {  // kFwdFp8W
         const int scale_ld = static_cast<int>((p.n + 127) >> 7);
         const int64_t scale_blocks = ((p.k + 127) >> 7) * scale_ld;
-        const uint8_t* w = static_cast<const uint8_t*>(p.b) + static_cast<int64_t>(g) * p.k * p.n;
-        compute_tile(smem, la,
-                     Fp8BlockLoader{w, p.ldb, n_t * BN, static_cast<int>(p.n), static_cast<int>(con),
-                                    p.b_scale + g * scale_blocks + ((n_t * BN) >> 7), scale_ld, 1.0f},
-                     c + s * p.ldc, p.ldc);
+        Fp8BlockLoader<BN, NT, kFirstB> lb;
+        lb.init(static_cast<const uint8_t*>(p.b) + g * w_elems, p.ldb, w_elems, n_t * BN, static_cast<int>(p.n),
+                p.b_scale + g * scale_blocks, scale_ld, tid);
+        compute_tile<Cfg>(smem, la, lb, m_t * BM, rows, n_t * BN, static_cast<int>(p.n), con, c + s * p.ldc, p.ldc, p.ablate);
       }
     }
   }
@@ -472,20 +631,58 @@ int device_cus() {
   return cus;
 }
 
+template <int kMode, typename Cfg>
+int launch_bf16(const GemmArgs& p, int workgroups_per_cu, hipStream_t stream) {
+  // upper bound on the number of tiles, so no more workgroups start than can find work
+  const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
+  const int64_t nt = (out_cols + Cfg::BN - 1) / Cfg::BN;
+  int64_t bound;
+  if (kMode == kWgrad) bound = ((p.k + Cfg::BM - 1) / Cfg::BM) * nt * p.groups;
+  else bound = (p.total_rows / Cfg::BM + p.groups) * nt;
+  int64_t workers = static_cast<int64_t>(device_cus()) * workgroups_per_cu;
+  if (bound < workers) workers = bound;
+  workers = (workers + kXcds - 1) / kXcds * kXcds;
+  if (workers <= 0) return HMOE_OK;
+  constexpr size_t lds_bytes = 2 * Cfg::kStage * sizeof(bf16_t);
+  auto kernel = grouped_gemm_bf16_kernel<kMode, Cfg>;
+  if (lds_bytes > 48 * 1024) {
+    // raising the dynamic LDS limit is idempotent: racing threads set the same value
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(lds_bytes)) != hipSuccess)
+      return HMOE_LAUNCH_FAILED;
+  }
+  kernel<<<dim3(static_cast<unsigned>(workers)), dim3(Cfg::kThreads), lds_bytes, stream>>>(p);
+  return HMOE_OK;
+}
+
+int experiment_ablate() {
+  static int v = [] {
+    const char* e = getenv("HMOE_GEMM_ABLATE");
+    return e ? atoi(e) : 0;
+  }();
+  return v;
+}
+
+int experiment_cfg() {
+  static int cfg = [] {
+    const char* v = getenv("HMOE_GEMM_CFG");
+    return v ? atoi(v) : 0;
+  }();
+  return cfg;
+}
+
 template <int kMode>
 int launch(const GemmArgs& p, int dtype, hipStream_t stream) {
   if (dtype == HMOE_BF16) {
-    // upper bound on the number of tiles, so no more workgroups start than can find work
-    const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
-    const int64_t nt = (out_cols + BN - 1) / BN;
-    int64_t bound;
-    if (kMode == kWgrad) bound = ((p.k + BM - 1) / BM) * nt * p.groups;
-    else bound = (p.total_rows / BM + p.groups) * nt;
-    int64_t workers = static_cast<int64_t>(device_cus()) * 2;
-    if (bound < workers) workers = bound;
-    workers = (workers + kXcds - 1) / kXcds * kXcds;
-    if (workers <= 0) return HMOE_OK;
-    grouped_gemm_bf16_kernel<kMode><<<dim3(static_cast<unsigned>(workers)), dim3(kThreads), 0, stream>>>(p);
+    int rc;
+    switch (experiment_cfg()) {
+      case 1: rc = launch_bf16<kMode, Config<2, 2, 4, 4>>(p, 1, stream); break;   // 256x256, 4 waves
+      case 2: rc = launch_bf16<kMode, Config<2, 2, 4, 2>>(p, 1, stream); break;   // 256x128, 4 waves
+      case 3: rc = launch_bf16<kMode, Config<2, 2, 2, 2>>(p, 2, stream); break;   // 128x128, 4 waves, 2 WG/CU
+      case 4: rc = launch_bf16<kMode, Config<2, 2, 2, 4>>(p, 1, stream); break;   // 128x256, 4 waves
+      default: rc = launch_bf16<kMode, Config<2, 4, 4, 2>>(p, 1, stream); break;  // 256x256, 8 waves
+    }
+    if (rc) return rc;
   } else if constexpr (kMode != kFwdFp8W) {
     if (kMode == kWgrad) {
       const dim3 grid((p.k + FT - 1) / FT, (p.n + FT - 1) / FT, p.groups);
@@ -511,6 +708,11 @@ int validate(const GemmArgs& p, int dtype) {
     // 16-byte rows: the alignment torch's grouped GEMM asks for as well
     if (p.k % 8 || p.n % 8 || p.lda % 8 || p.ldb % 8 || p.ldc % 8) return HMOE_UNSUPPORTED;
     if (!aligned16(p.a) || !aligned16(p.b) || !aligned16(p.c)) return HMOE_UNSUPPORTED;
+    // buffer loads address an operand with 32-bit byte offsets: all rows of an operand and one expert's weight
+    // must each stay below 2 GiB
+    const int64_t lim = int64_t(1) << 31;
+    if (p.total_rows * p.lda * 2 >= lim || p.total_rows * p.ldb * 2 >= lim || p.k * p.n * 2 >= lim)
+      return HMOE_UNSUPPORTED;
   }
   return HMOE_OK;
 }
@@ -523,7 +725,7 @@ extern "C" {
 int hmoe_grouped_gemm_fwd(const void* a, int64_t lda, const void* b, const int32_t* offs, int64_t total_rows,
                           int num_groups, int64_t k, int64_t n, int dtype, void* out, int64_t ldo, void* stream) {
   using namespace hmoe;
-  GemmArgs p{a, lda, b, n, out, ldo, offs, total_rows, num_groups, k, n, nullptr};
+  GemmArgs p{a, lda, b, n, out, ldo, offs, total_rows, num_groups, k, n, nullptr, experiment_ablate()};
   if (int rc = validate(p, dtype)) return rc;
   if (total_rows == 0 || n == 0) return HMOE_OK;
   if (!a || !b || !out) return HMOE_INVALID_ARGUMENT;
@@ -535,7 +737,7 @@ int hmoe_grouped_gemm_fwd_fp8w(const void* a, int64_t lda, const uint8_t* bq, co
                                const int32_t* offs, int64_t total_rows, int num_groups, int64_t k, int64_t n,
                                void* out, int64_t ldo, void* stream) {
   using namespace hmoe;
-  GemmArgs p{a, lda, bq, n, out, ldo, offs, total_rows, num_groups, k, n, b_scale};
+  GemmArgs p{a, lda, bq, n, out, ldo, offs, total_rows, num_groups, k, n, b_scale, experiment_ablate()};
   if (int rc = validate(p, HMOE_BF16)) return rc;
   if (total_rows == 0 || n == 0) return HMOE_OK;
   if (!a || !bq || !b_scale || !out) return HMOE_INVALID_ARGUMENT;
@@ -547,7 +749,7 @@ int hmoe_grouped_gemm_dgrad(const void* grad_out, int64_t ldg, const void* b, co
                             int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype, void* grad_a,
                             int64_t lda, void* stream) {
   using namespace hmoe;
-  GemmArgs p{grad_out, ldg, b, n, grad_a, lda, offs, total_rows, num_groups, k, n, nullptr};
+  GemmArgs p{grad_out, ldg, b, n, grad_a, lda, offs, total_rows, num_groups, k, n, nullptr, experiment_ablate()};
   if (int rc = validate(p, dtype)) return rc;
   if (total_rows == 0 || k == 0) return HMOE_OK;
   if (!grad_out || !b || !grad_a) return HMOE_INVALID_ARGUMENT;
@@ -559,7 +761,7 @@ int hmoe_grouped_gemm_wgrad(const void* a, int64_t lda, const void* grad_out, in
                             int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype, void* grad_b,
                             void* stream) {
   using namespace hmoe;
-  GemmArgs p{a, lda, grad_out, ldg, grad_b, n, offs, total_rows, num_groups, k, n, nullptr};
+  GemmArgs p{a, lda, grad_out, ldg, grad_b, n, offs, total_rows, num_groups, k, n, nullptr, experiment_ablate()};
   if (int rc = validate(p, dtype)) return rc;
   if (k == 0 || n == 0) return HMOE_OK;
   if (!grad_b || (total_rows > 0 && (!a || !grad_out))) return HMOE_INVALID_ARGUMENT;
