@@ -537,6 +537,288 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   }
 }
 
+// ------------------------------------------------------------------------------------------- bf16 kernel, v3
+// Same tile (256 x 256 x 64, 2 x 4 wavefronts of 4 x 2 blocks) and schedule, but the operand tiles go from global
+// memory straight into LDS (buffer_load ... lds, 16 bytes per lane), so there are no staging registers, no ds_write
+// instructions and no register transposes in the loop:
+//  * a contraction-contiguous operand lands as [256 rows][64 con] with the 16-byte chunk index XOR-swizzled by row
+//    (each lane fetches the chunk that belongs in its LDS slot); fragments are one ds_read_b128;
+//  * an output-contiguous operand (B in fwd, both operands in wgrad) lands as it lies in memory, [64 con][256 out],
+//    chunks XOR-swizzled by (con & 3) << 1, and fragments are read with two ds_read_b64_tr_b16, the gfx950 LDS
+//    transpose read: within a group of 16 lanes, lane i supplies the address of row (i >> 2), columns 4 (i & 3)..+3
+//    of a 4 x 16 patch and receives the four rows of column i.
+// The loads of step k+1 are in flight during the whole of step k; the next tile's first step is issued before the
+// epilogue, which stages through the second LDS stage only.
+struct DmaDirect {   // element(out, con) = base[out * ld + con]
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t voff[4];
+  int con_first[4];  // contraction index (within a step) of the chunk each instruction's lane fetches
+  int con_lim;
+
+  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
+                                       int con_lim_, int wave, int lane) {
+    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
+    con_lim = con_lim_;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int row = (wave * 4 + t) * 8 + (lane >> 3);  // row of the tile this lane's LDS slot belongs to
+      const int logical = (lane & 7) ^ swizzle(row);
+      const int out = out0 + row;
+      con_first[t] = logical << 3;
+      voff[t] = out < out_lim ? static_cast<uint32_t>(out) * static_cast<uint32_t>(ld) * 2u + (logical << 4)
+                              : kOutOfRange;
+    }
+  }
+  // `tile` is the byte address in LDS of this operand's tile in the stage being filled
+  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave) const {
+    const uint32_t soff = static_cast<uint32_t>(step) * (BK * 2);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const uint32_t off = step * BK + con_first[t] < con_lim ? voff[t] : kOutOfRange;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * 4 + t) * 1024, 16, off, soff, 0, 0);
+    }
+  }
+  // fragment for the 32x32x16 MFMA: rows row0 + (lane & 31), contraction kk*16 + 8*(lane>>5) .. +7
+  static __device__ __forceinline__ bf16x8 fragment(const bf16_t* smem, int tile_elems, int row0, int kk, int lane) {
+    return *reinterpret_cast<const bf16x8*>(smem + tile_elems + lds_offset(row0 + (lane & 31), kk * 2 + (lane >> 5)));
+  }
+};
+
+struct DmaTransposed {   // element(out, con) = base[con * ld + out]
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t voff[4];
+  uint32_t step_bytes;
+
+  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
+                                       int /*con_lim*/, int wave, int lane) {
+    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));  // contraction rows past the end lie past the buffer
+    step_bytes = BK * static_cast<uint32_t>(ld) * 2u;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int con = (wave * 4 + t) * 2 + (lane >> 5);  // two contraction rows of 512 bytes per instruction
+      const int logical = (lane & 31) ^ ((con & 3) << 1);
+      const int out = out0 + (logical << 3);
+      voff[t] = out < out_lim ? static_cast<uint32_t>(con) * static_cast<uint32_t>(ld) * 2u + static_cast<uint32_t>(out) * 2u
+                              : kOutOfRange;
+    }
+  }
+  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave) const {
+    const uint32_t soff = static_cast<uint32_t>(step) * step_bytes;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * 4 + t) * 1024, 16, voff[t], soff, 0, 0);
+  }
+  static __device__ __forceinline__ bf16x8 fragment(const bf16_t* smem, int tile_elems, int row0, int kk, int lane) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+    const int i = lane & 15, g = lane >> 4;
+    const int out = row0 + ((g & 1) << 4) + ((i & 3) << 2);    // first of the four columns this lane points at
+    const int con = kk * 16 + ((g >> 1) << 3) + (i >> 2);        // (con & 3) == (i >> 2) for both reads
+    const int in_row = (((out >> 3) ^ ((con & 3) << 1)) << 3) + (out & 7);
+    const bf16_t* p = smem + tile_elems + con * 256 + in_row;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * 256));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(bf16x8, both);
+  }
+};
+
+using V3Cfg = Config<2, 4, 4, 2>;
+
+template <int kMode>
+__global__ void __launch_bounds__(V3Cfg::kThreads) grouped_gemm_bf16_v3_kernel(GemmArgs p) {
+  using Cfg = V3Cfg;
+  constexpr int WM = Cfg::WM, WN = Cfg::WN, BM = Cfg::BM, BN = Cfg::BN;
+  using LoaderA = typename std::conditional<kMode == kWgrad, DmaTransposed, DmaDirect>::type;
+  using LoaderB = typename std::conditional<kMode == kDgrad, DmaDirect, DmaTransposed>::type;
+  extern __shared__ __attribute__((aligned(16))) bf16_t smem[];  // two stages of (A tile, B tile), 32 KB each
+  __shared__ int32_t tile_start[kMode == kWgrad ? 1 : kMaxGroups + 1];
+  constexpr int kTileB = BM * BK;  // elements; both tiles hold 256 * 64 elements whatever their orientation
+  const bf16_t* a = static_cast<const bf16_t*>(p.a);
+  const bf16_t* b = static_cast<const bf16_t*>(p.b);
+  bf16_t* c = static_cast<bf16_t*>(p.c);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int gm = wave / Cfg::GN, gn = wave % Cfg::GN;
+  auto lds = (__attribute__((address_space(3))) char*)smem;
+
+  // ---- tile schedule (as the staged kernel)
+  const int workers = gridDim.x;
+  int64_t total, first, last, stride;
+  int nt = 1, mt_w = 1;
+  int64_t per_group = 1;
+  if constexpr (kMode == kWgrad) {
+    mt_w = static_cast<int>((p.k + BM - 1) / BM);
+    nt = static_cast<int>((p.n + BN - 1) / BN);
+    per_group = static_cast<int64_t>(mt_w) * nt;
+    total = per_group * p.groups;
+    first = blockIdx.x;
+    last = total;
+    stride = workers;
+  } else {
+    build_tile_prefix<BM>(tile_start, p.offs, p.groups, p.total_rows);
+    const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
+    nt = static_cast<int>((out_cols + BN - 1) / BN);
+    total = static_cast<int64_t>(tile_start[p.groups]) * nt;
+    const int xcd = blockIdx.x % kXcds;
+    const int64_t chunk = (total + kXcds - 1) / kXcds;
+    first = xcd * chunk + blockIdx.x / kXcds;
+    last = xcd * chunk + chunk < total ? xcd * chunk + chunk : total;
+    stride = (workers - xcd + kXcds - 1) / kXcds;
+  }
+
+  struct Tile {
+    int a_out0, a_out_lim, b_out0, b_out_lim, con_lim;
+    bf16_t* c_base;
+  };
+  LoaderA la;
+  LoaderB lb;
+  // decode tile t, describe its operands to the loaders and start its first step into stage 0
+  auto begin_tile = [&](int64_t t, Tile& tile) {
+    int g, m_t, n_t;
+    if constexpr (kMode == kWgrad) {
+      g = static_cast<int>(t / per_group);
+      const int r = static_cast<int>(t - g * per_group);
+      n_t = r / mt_w;
+      m_t = r - n_t * mt_w;
+    } else {
+      int lo = 0, hi = p.groups;  // largest g with tile_start[g] * nt <= t
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (static_cast<int64_t>(tile_start[mid]) * nt <= t) lo = mid; else hi = mid;
+      }
+      g = lo;
+      const int mt = tile_start[g + 1] - tile_start[g];
+      const int r = static_cast<int>(t - static_cast<int64_t>(tile_start[g]) * nt);
+      n_t = r / mt;
+      m_t = r - n_t * mt;
+    }
+    int64_t s, e;
+    group_bounds(p.offs, g, p.total_rows, s, e);
+    const int rows = static_cast<int>(e - s);
+    const int64_t w_elems = p.k * p.n;
+    tile.a_out0 = m_t * BM;
+    tile.b_out0 = n_t * BN;
+    if constexpr (kMode == kWgrad) {
+      tile.a_out_lim = static_cast<int>(p.k);
+      tile.b_out_lim = static_cast<int>(p.n);
+      tile.con_lim = rows;
+      tile.c_base = c + static_cast<int64_t>(g) * w_elems;
+      la.init(a + s * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, rows, wave, lane);
+      lb.init(b + s * p.ldb, p.ldb, rows * p.ldb * 2, tile.b_out0, tile.b_out_lim, rows, wave, lane);
+    } else {
+      tile.a_out_lim = rows;
+      tile.b_out_lim = static_cast<int>(kMode == kDgrad ? p.k : p.n);
+      tile.con_lim = static_cast<int>(kMode == kDgrad ? p.n : p.k);
+      tile.c_base = c + s * p.ldc;
+      la.init(a + s * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, rows, tile.con_lim, wave, lane);
+      lb.init(b + g * w_elems, p.ldb, w_elems * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, wave, lane);
+    }
+    if (tile.con_lim > 0) {
+      la.issue(lds, 0, wave);
+      lb.issue(lds + kTileB * 2, 0, wave);
+    }
+  };
+
+  Tile tile;
+  int64_t t = first;
+  if (t < last) begin_tile(t, tile);
+  while (t < last) {
+    f32x16 acc[WM][WN];
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    const int steps = (tile.con_lim + BK - 1) / BK;
+    const int row_a = gm * (WM * 32), row_b = gn * (WN * 32);
+    int live = (tile.a_out_lim - (tile.a_out0 + row_a) + 31) >> 5;
+    live = live < 0 ? 0 : (live > WM ? WM : live);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();  // step 0 of this tile has landed in stage 0
+
+    auto run = [&](auto full_tag) {
+      constexpr bool kFull = decltype(full_tag)::value;
+      for (int step = 0; step < steps; ++step) {
+        const int cur = step & 1;
+        if (step + 1 < steps) {  // the other stage is free since the barrier that ended the previous step
+          la.issue(lds + (cur ^ 1) * (Cfg::kStage * 2), step + 1, wave);
+          lb.issue(lds + (cur ^ 1) * (Cfg::kStage * 2) + kTileB * 2, step + 1, wave);
+        }
+        const int ta = cur * Cfg::kStage, tb = ta + kTileB;
+        // fragments are double-buffered: those of sub-step kk+1 are read while the MFMAs of sub-step kk run
+        bf16x8 fa[2][WM], fb[2][WN];
+        auto read_fragments = [&](int kk, int buf) {
+#pragma unroll
+          for (int j = 0; j < WN; ++j) fb[buf][j] = LoaderB::fragment(smem, tb, row_b + j * 32, kk, lane);
+#pragma unroll
+          for (int i = 0; i < WM; ++i)
+            if (kFull || i < live) fa[buf][i] = LoaderA::fragment(smem, ta, row_a + i * 32, kk, lane);
+        };
+        read_fragments(0, 0);
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+          if (kk + 1 < BK / 16) read_fragments(kk + 1, (kk + 1) & 1);
+#pragma unroll
+          for (int i = 0; i < WM; ++i) {
+            if (kFull || i < live) {
+#pragma unroll
+              for (int j = 0; j < WN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[kk & 1][j], fa[kk & 1][i], acc[i][j], 0, 0, 0);
+            }
+          }
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+      }
+    };
+    if (live == WM) run(std::true_type{});
+    else run(std::false_type{});
+
+    // both stages are free: start the next tile's first step into stage 0 before this tile's epilogue
+    const Tile done = tile;
+    t += stride;
+    if (t < last) begin_tile(t, tile);
+
+    // epilogue through the second stage: 32 rows at a time per wavefront, whole 16-byte chunks out
+    constexpr int kEpiPitch = WN * 32 + 8;
+    constexpr int kEpiRegion = 32 * kEpiPitch;
+    constexpr int kLanesPerRow = WN * 4;
+    constexpr int kRowsPerPass = 64 / kLanesPerRow;
+    static_assert(kEpiRegion * Cfg::GM * Cfg::GN <= Cfg::kStage, "epilogue staging must fit in one stage");
+    bf16_t* stage = smem + Cfg::kStage + wave * kEpiRegion;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+#pragma unroll
+      for (int j = 0; j < WN; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          uint2 packed;
+          packed.x = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 0])) |
+                     (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 1])) << 16);
+          packed.y = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 2])) |
+                     (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 3])) << 16);
+          *reinterpret_cast<uint2*>(stage + (lane & 31) * kEpiPitch + j * 32 + q * 8 + ((lane >> 5) << 2)) = packed;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();  // the region is private to the wavefront, whose LDS accesses stay in order
+#pragma unroll
+      for (int pass = 0; pass < 32 / kRowsPerPass; ++pass) {
+        const int rr = pass * kRowsPerPass + lane / kLanesPerRow;
+        const int cc = (lane % kLanesPerRow) << 3;
+        const int row = done.a_out0 + row_a + i * 32 + rr;
+        const int col = done.b_out0 + row_b + cc;
+        if (row < done.a_out_lim && col < done.b_out_lim) {
+          const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * kEpiPitch + cc);
+          *reinterpret_cast<u32x4*>(done.c_base + static_cast<int64_t>(row) * p.ldc + col) = v;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ fp32 path
 // 64x64 tile, contraction step 16, 256 threads each owning a 4x4 block.  grid.x walks row tiles of every group
 // (an upper bound of ceil(R/64)+G tiles; surplus workgroups exit), grid.y column tiles.
@@ -672,9 +954,38 @@ int experiment_cfg() {
 }
 
 template <int kMode>
+int launch_v3(const GemmArgs& p, hipStream_t stream) {
+  using Cfg = V3Cfg;
+  const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
+  const int64_t nt = (out_cols + Cfg::BN - 1) / Cfg::BN;
+  int64_t bound;
+  if (kMode == kWgrad) bound = ((p.k + Cfg::BM - 1) / Cfg::BM) * nt * p.groups;
+  else bound = (p.total_rows / Cfg::BM + p.groups) * nt;
+  int64_t workers = device_cus();
+  if (bound < workers) workers = bound;
+  workers = (workers + kXcds - 1) / kXcds * kXcds;
+  if (workers <= 0) return HMOE_OK;
+  constexpr size_t lds_bytes = 2 * Cfg::kStage * sizeof(bf16_t);
+  auto kernel = grouped_gemm_bf16_v3_kernel<kMode>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          static_cast<int>(lds_bytes)) != hipSuccess)
+    return HMOE_LAUNCH_FAILED;
+  kernel<<<dim3(static_cast<unsigned>(workers)), dim3(Cfg::kThreads), lds_bytes, stream>>>(p);
+  return HMOE_OK;
+}
+
+template <int kMode>
 int launch(const GemmArgs& p, int dtype, hipStream_t stream) {
   if (dtype == HMOE_BF16) {
     int rc;
+    if constexpr (kMode != kFwdFp8W) {
+      if (experiment_cfg() == 9) {
+        rc = launch_v3<kMode>(p, stream);
+        if (rc) return rc;
+        if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
+        return HMOE_OK;
+      }
+    }
     switch (experiment_cfg()) {
       case 1: rc = launch_bf16<kMode, Config<2, 2, 4, 4>>(p, 1, stream); break;   // 256x256, 4 waves
       case 2: rc = launch_bf16<kMode, Config<2, 2, 4, 2>>(p, 1, stream); break;   // 256x128, 4 waves
