@@ -61,7 +61,9 @@ def build(verbose: bool = True) -> str:
         jobs.append((src, obj))
     with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
         list(pool.map(lambda job: _run([hipcc, *HIPCC_FLAGS, "-c", job[0], "-o", job[1]]), jobs))
-    _run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", LIB_PATH, *[obj for _, obj in jobs]])
+    # -z defs: a kernel whose host stub went missing must fail the link, not the first dlopen
+    _run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-Wl,-z,defs", "-o", LIB_PATH,
+          *[obj for _, obj in jobs]])
     if verbose:
         print(f"built {LIB_PATH} from {len(jobs)} sources")
     return LIB_PATH

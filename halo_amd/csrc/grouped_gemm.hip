@@ -549,10 +549,11 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
 //    of a 4 x 16 patch and receives the four rows of column i.
 // The loads of step k+1 are in flight during the whole of step k; the next tile's first step is issued before the
 // epilogue, which stages through the second LDS stage only.
+template <int kI>  // 1 KB instructions per wavefront per tile: 32 / wavefronts
 struct DmaDirect {   // element(out, con) = base[out * ld + con]
   __amdgpu_buffer_rsrc_t rsrc;
-  uint32_t voff[4];
-  int con_first[4];  // contraction index (within a step) of the chunk each instruction's lane fetches
+  uint32_t voff[kI];
+  int con_first[kI];  // contraction index (within a step) of the chunk each instruction's lane fetches
   int con_lim;
 
   __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
@@ -560,8 +561,8 @@ struct DmaDirect {   // element(out, con) = base[out * ld + con]
     rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
     con_lim = con_lim_;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const int row = (wave * 4 + t) * 8 + (lane >> 3);  // row of the tile this lane's LDS slot belongs to
+    for (int t = 0; t < kI; ++t) {
+      const int row = (wave * kI + t) * 8 + (lane >> 3);  // row of the tile this lane's LDS slot belongs to
       const int logical = (lane & 7) ^ swizzle(row);
       const int out = out0 + row;
       con_first[t] = logical << 3;
@@ -573,9 +574,9 @@ struct DmaDirect {   // element(out, con) = base[out * ld + con]
   __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave) const {
     const uint32_t soff = static_cast<uint32_t>(step) * (BK * 2);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < kI; ++t) {
       const uint32_t off = step * BK + con_first[t] < con_lim ? voff[t] : kOutOfRange;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * 4 + t) * 1024, 16, off, soff, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * kI + t) * 1024, 16, off, soff, 0, 0);
     }
   }
   // fragment for the 32x32x16 MFMA: rows row0 + (lane & 31), contraction kk*16 + 8*(lane>>5) .. +7
@@ -584,9 +585,10 @@ struct DmaDirect {   // element(out, con) = base[out * ld + con]
   }
 };
 
+template <int kI>
 struct DmaTransposed {   // element(out, con) = base[con * ld + out]
   __amdgpu_buffer_rsrc_t rsrc;
-  uint32_t voff[4];
+  uint32_t voff[kI];
   uint32_t step_bytes;
 
   __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
@@ -594,8 +596,8 @@ struct DmaTransposed {   // element(out, con) = base[con * ld + out]
     rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));  // contraction rows past the end lie past the buffer
     step_bytes = BK * static_cast<uint32_t>(ld) * 2u;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const int con = (wave * 4 + t) * 2 + (lane >> 5);  // two contraction rows of 512 bytes per instruction
+    for (int t = 0; t < kI; ++t) {
+      const int con = (wave * kI + t) * 2 + (lane >> 5);  // two contraction rows of 512 bytes per instruction
       const int logical = (lane & 31) ^ ((con & 3) << 1);
       const int out = out0 + (logical << 3);
       voff[t] = out < out_lim ? static_cast<uint32_t>(con) * static_cast<uint32_t>(ld) * 2u + static_cast<uint32_t>(out) * 2u
@@ -605,8 +607,8 @@ struct DmaTransposed {   // element(out, con) = base[con * ld + out]
   __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave) const {
     const uint32_t soff = static_cast<uint32_t>(step) * step_bytes;
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * 4 + t) * 1024, 16, voff[t], soff, 0, 0);
+    for (int t = 0; t < kI; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * kI + t) * 1024, 16, voff[t], soff, 0, 0);
   }
   static __device__ __forceinline__ bf16x8 fragment(const bf16_t* smem, int tile_elems, int row0, int kk, int lane) {
     typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -624,14 +626,13 @@ struct DmaTransposed {   // element(out, con) = base[con * ld + out]
   }
 };
 
-using V3Cfg = Config<2, 4, 4, 2>;
-
-template <int kMode>
-__global__ void __launch_bounds__(V3Cfg::kThreads) grouped_gemm_bf16_v3_kernel(GemmArgs p) {
-  using Cfg = V3Cfg;
+template <int kMode, typename Cfg>
+__global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_v3_kernel(GemmArgs p) {
+  static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
   constexpr int WM = Cfg::WM, WN = Cfg::WN, BM = Cfg::BM, BN = Cfg::BN;
-  using LoaderA = typename std::conditional<kMode == kWgrad, DmaTransposed, DmaDirect>::type;
-  using LoaderB = typename std::conditional<kMode == kDgrad, DmaDirect, DmaTransposed>::type;
+  constexpr int kI = 32 / (Cfg::GM * Cfg::GN);
+  using LoaderA = typename std::conditional<kMode == kWgrad, DmaTransposed<kI>, DmaDirect<kI>>::type;
+  using LoaderB = typename std::conditional<kMode == kDgrad, DmaDirect<kI>, DmaTransposed<kI>>::type;
   extern __shared__ __attribute__((aligned(16))) bf16_t smem[];  // two stages of (A tile, B tile), 32 KB each
   __shared__ int32_t tile_start[kMode == kWgrad ? 1 : kMaxGroups + 1];
   constexpr int kTileB = BM * BK;  // elements; both tiles hold 256 * 64 elements whatever their orientation
@@ -742,7 +743,7 @@ __global__ void __launch_bounds__(V3Cfg::kThreads) grouped_gemm_bf16_v3_kernel(G
       constexpr bool kFull = decltype(full_tag)::value;
       for (int step = 0; step < steps; ++step) {
         const int cur = step & 1;
-        if (step + 1 < steps) {  // the other stage is free since the barrier that ended the previous step
+        if (step + 1 < steps && !(HMOE_ABLATE & 1)) {  // the other stage is free since the barrier that ended the previous step
           la.issue(lds + (cur ^ 1) * (Cfg::kStage * 2), step + 1, wave);
           lb.issue(lds + (cur ^ 1) * (Cfg::kStage * 2) + kTileB * 2, step + 1, wave);
         }
@@ -750,6 +751,10 @@ __global__ void __launch_bounds__(V3Cfg::kThreads) grouped_gemm_bf16_v3_kernel(G
         // fragments are double-buffered: those of sub-step kk+1 are read while the MFMAs of sub-step kk run
         bf16x8 fa[2][WM], fb[2][WN];
         auto read_fragments = [&](int kk, int buf) {
+          if (HMOE_ABLATE & 2) {
+            if (kk > 0 || step > 0) return;
+            kk = 0;
+          }
 #pragma unroll
           for (int j = 0; j < WN; ++j) fb[buf][j] = LoaderB::fragment(smem, tb, row_b + j * 32, kk, lane);
 #pragma unroll
@@ -764,8 +769,14 @@ __global__ void __launch_bounds__(V3Cfg::kThreads) grouped_gemm_bf16_v3_kernel(G
           for (int i = 0; i < WM; ++i) {
             if (kFull || i < live) {
 #pragma unroll
-              for (int j = 0; j < WN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[kk & 1][j], fa[kk & 1][i], acc[i][j], 0, 0, 0);
+              for (int j = 0; j < WN; ++j) {
+                if (HMOE_ABLATE & 4) {
+                  asm volatile("" ::"v"(fb[kk & 1][j]), "v"(fa[kk & 1][i]));
+                  continue;
+                }
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[(HMOE_ABLATE & 2) ? 0 : (kk & 1)][j],
+                                                                    fa[(HMOE_ABLATE & 2) ? 0 : (kk & 1)][i], acc[i][j], 0, 0, 0);
+              }
             }
           }
         }
@@ -809,7 +820,7 @@ __global__ void __launch_bounds__(V3Cfg::kThreads) grouped_gemm_bf16_v3_kernel(G
         const int cc = (lane % kLanesPerRow) << 3;
         const int row = done.a_out0 + row_a + i * 32 + rr;
         const int col = done.b_out0 + row_b + cc;
-        if (row < done.a_out_lim && col < done.b_out_lim) {
+        if (row < done.a_out_lim && col < done.b_out_lim && (!(HMOE_ABLATE & 16) || p.ablate == 77)) {
           const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * kEpiPitch + cc);
           *reinterpret_cast<u32x4*>(done.c_base + static_cast<int64_t>(row) * p.ldc + col) = v;
         }
@@ -953,20 +964,29 @@ int experiment_cfg() {
   return cfg;
 }
 
-template <int kMode>
+// explicit instantiations: the host pass has been seen to drop the stub of an implicitly instantiated one
+#define HMOE_V3_INSTANCE(mode) \
+  template __global__ void grouped_gemm_bf16_v3_kernel<mode, Config<2, 4, 4, 2>>(GemmArgs); \
+  template __global__ void grouped_gemm_bf16_v3_kernel<mode, Config<2, 2, 4, 4>>(GemmArgs);
+HMOE_V3_INSTANCE(kFwd)
+HMOE_V3_INSTANCE(kDgrad)
+HMOE_V3_INSTANCE(kWgrad)
+#undef HMOE_V3_INSTANCE
+
+template <int kMode, typename Cfg>
 int launch_v3(const GemmArgs& p, hipStream_t stream) {
-  using Cfg = V3Cfg;
   const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
   const int64_t nt = (out_cols + Cfg::BN - 1) / Cfg::BN;
   int64_t bound;
   if (kMode == kWgrad) bound = ((p.k + Cfg::BM - 1) / Cfg::BM) * nt * p.groups;
   else bound = (p.total_rows / Cfg::BM + p.groups) * nt;
   int64_t workers = device_cus();
+  if (const char* v = getenv("HMOE_GEMM_WGS")) workers = atoi(v);
   if (bound < workers) workers = bound;
   workers = (workers + kXcds - 1) / kXcds * kXcds;
   if (workers <= 0) return HMOE_OK;
   constexpr size_t lds_bytes = 2 * Cfg::kStage * sizeof(bf16_t);
-  auto kernel = grouped_gemm_bf16_v3_kernel<kMode>;
+  auto kernel = grouped_gemm_bf16_v3_kernel<kMode, Cfg>;
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                           static_cast<int>(lds_bytes)) != hipSuccess)
     return HMOE_LAUNCH_FAILED;
@@ -979,8 +999,9 @@ int launch(const GemmArgs& p, int dtype, hipStream_t stream) {
   if (dtype == HMOE_BF16) {
     int rc;
     if constexpr (kMode != kFwdFp8W) {
-      if (experiment_cfg() == 9) {
-        rc = launch_v3<kMode>(p, stream);
+      if (experiment_cfg() == 0 || experiment_cfg() >= 9) {
+        if (experiment_cfg() != 10) rc = launch_v3<kMode, Config<2, 4, 4, 2>>(p, stream);
+        else rc = launch_v3<kMode, Config<2, 2, 4, 4>>(p, stream);
         if (rc) return rc;
         if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
         return HMOE_OK;
@@ -991,7 +1012,7 @@ int launch(const GemmArgs& p, int dtype, hipStream_t stream) {
       case 2: rc = launch_bf16<kMode, Config<2, 2, 4, 2>>(p, 1, stream); break;   // 256x128, 4 waves
       case 3: rc = launch_bf16<kMode, Config<2, 2, 2, 2>>(p, 2, stream); break;   // 128x128, 4 waves, 2 WG/CU
       case 4: rc = launch_bf16<kMode, Config<2, 2, 2, 4>>(p, 1, stream); break;   // 128x256, 4 waves
-      default: rc = launch_bf16<kMode, Config<2, 4, 4, 2>>(p, 1, stream); break;  // 256x256, 8 waves
+      default: rc = launch_bf16<kMode, Config<2, 4, 4, 2>>(p, 1, stream); break;  // 256x256, 8 waves (5)
     }
     if (rc) return rc;
   } else if constexpr (kMode != kFwdFp8W) {

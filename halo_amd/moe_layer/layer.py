@@ -292,7 +292,8 @@ class EPMoELayerBase(nn.Module, ABC):
         """The router's logits at the input dtype (fp32 under ``fp32_router``), fp32 accumulation, one rounding."""
         router = getattr(self, self._ROUTER_ATTR)
         x = self._router_input(flat)
-        logits = dense_mm(x, router.weight.to(x.dtype))
+        # A plain dense projection with a tiny output ([T, E]): the library GEMM, as in the reference (F.linear).
+        logits = torch.nn.functional.linear(x, router.weight.to(x.dtype))
         bias = getattr(router, "bias", None)
         return logits if bias is None else logits + bias.to(logits.dtype)
 
