@@ -44,6 +44,9 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 #ifndef HMOE_ABLATE
 #define HMOE_ABLATE 0
 #endif
+#ifndef HMOE_PF
+#define HMOE_PF 0  // L2 prefetch distance of the direct-to-LDS kernel, in contraction steps; 0 = off
+#endif
 
 constexpr int BK = 64;  // contraction per step
 constexpr int kXcds = 8;
@@ -95,6 +98,18 @@ __device__ __forceinline__ void group_bounds(const int32_t* offs, int g, int64_t
 }
 
 constexpr uint32_t kOutOfRange = 0x80000000u;  // a byte offset no operand reaches: the buffer load returns zeros
+
+// s_barrier alone.  __syncthreads() also fences, and the fence drains every load in flight (vmcnt(0)), including
+// the direct-to-LDS loads a kernel wants to keep in flight across the barrier; the callers wait for exactly the
+// loads they need before they come here.
+__device__ __forceinline__ void workgroup_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// s_waitcnt vmcnt(v) only: expcnt and lgkmcnt left at their maxima
+#define HMOE_WAIT_VM(v) __builtin_amdgcn_s_waitcnt(((v) & 15) | (((v) >> 4) << 14) | (7 << 4) | (15 << 8))
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
@@ -570,6 +585,18 @@ struct DmaDirect {   // element(out, con) = base[out * ld + con]
                               : kOutOfRange;
     }
   }
+  // One 4-byte load from line `l` (0..255: output row out0 + l) of a later step, whose only purpose is to pull the
+  // 128-byte line into L2 ahead of the tile load that needs it.  It lands in a scrap area of LDS (`sink`, 256 bytes
+  // per wavefront): a load to LDS ties up no register, so nothing ever has to wait for it.
+  uint32_t pf_off;
+  __device__ __forceinline__ void init_prefetch(int64_t ld, int out0, int out_lim, int l) {
+    const int out = out0 + l;
+    pf_off = out < out_lim ? static_cast<uint32_t>(out) * static_cast<uint32_t>(ld) * 2u : kOutOfRange;
+  }
+  __device__ __forceinline__ void prefetch(__attribute__((address_space(3))) char* sink, int step) const {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, sink, 4, step * BK < con_lim ? pf_off : kOutOfRange,
+                                             static_cast<uint32_t>(step) * (BK * 2), 0, 0);
+  }
   // `tile` is the byte address in LDS of this operand's tile in the stage being filled
   __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave) const {
     const uint32_t soff = static_cast<uint32_t>(step) * (BK * 2);
@@ -592,17 +619,30 @@ struct DmaTransposed {   // element(out, con) = base[con * ld + out]
   uint32_t step_bytes;
 
   __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
-                                       int /*con_lim*/, int wave, int lane) {
+                                       int con_lim_, int wave, int lane) {
     rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));  // contraction rows past the end lie past the buffer
+    con_lim = con_lim_;
     step_bytes = BK * static_cast<uint32_t>(ld) * 2u;
 #pragma unroll
     for (int t = 0; t < kI; ++t) {
       const int con = (wave * kI + t) * 2 + (lane >> 5);  // two contraction rows of 512 bytes per instruction
-      const int logical = (lane & 31) ^ ((con & 3) << 1);
+      const int logical = (lane & 31) ^ ((con & 3) << 2);
       const int out = out0 + (logical << 3);
       voff[t] = out < out_lim ? static_cast<uint32_t>(con) * static_cast<uint32_t>(ld) * 2u + static_cast<uint32_t>(out) * 2u
                               : kOutOfRange;
     }
+  }
+  // line l (0..255): contraction row l >> 2 of the step, 128-byte piece l & 3 of its 512 bytes
+  uint32_t pf_off;
+  int con_lim;
+  __device__ __forceinline__ void init_prefetch(int64_t ld, int out0, int out_lim, int l) {
+    const int out = out0 + ((l & 3) << 6);
+    pf_off = out < out_lim ? static_cast<uint32_t>(l >> 2) * static_cast<uint32_t>(ld) * 2u + static_cast<uint32_t>(out) * 2u
+                           : kOutOfRange;
+  }
+  __device__ __forceinline__ void prefetch(__attribute__((address_space(3))) char* sink, int step) const {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, sink, 4, step * BK < con_lim ? pf_off : kOutOfRange,
+                                             static_cast<uint32_t>(step) * step_bytes, 0, 0);
   }
   __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave) const {
     const uint32_t soff = static_cast<uint32_t>(step) * step_bytes;
@@ -616,7 +656,7 @@ struct DmaTransposed {   // element(out, con) = base[con * ld + out]
     const int i = lane & 15, g = lane >> 4;
     const int out = row0 + ((g & 1) << 4) + ((i & 3) << 2);    // first of the four columns this lane points at
     const int con = kk * 16 + ((g >> 1) << 3) + (i >> 2);        // (con & 3) == (i >> 2) for both reads
-    const int in_row = (((out >> 3) ^ ((con & 3) << 1)) << 3) + (out & 7);
+    const int in_row = (((out >> 3) ^ ((con & 3) << 2)) << 3) + (out & 7);
     const bf16_t* p = smem + tile_elems + con * 256 + in_row;
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
     const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * 256));
@@ -674,6 +714,18 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_v3_kernel(Gem
   };
   LoaderA la;
   LoaderB lb;
+  // L2 prefetch: every thread touches one 128-byte line of a later step's operand tiles (wavefronts 0-3 operand A,
+  // 4-7 operand B; with four wavefronts every thread touches one of each).
+  auto pf_sink = lds + 2 * Cfg::kStage * 2 + wave * 256;
+  auto prefetch_line = [&](int step) {
+    if constexpr (Cfg::kThreads == 512) {
+      if (wave >> 2) lb.prefetch(pf_sink, step);
+      else la.prefetch(pf_sink, step);
+    } else {
+      la.prefetch(pf_sink, step);
+      lb.prefetch(pf_sink, step);
+    }
+  };
   // decode tile t, describe its operands to the loaders and start its first step into stage 0
   auto begin_tile = [&](int64_t t, Tile& tile) {
     int g, m_t, n_t;
@@ -719,6 +771,12 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_v3_kernel(Gem
       la.issue(lds, 0, wave);
       lb.issue(lds + kTileB * 2, 0, wave);
     }
+    if constexpr (HMOE_PF > 0) {
+      la.init_prefetch(p.lda, tile.a_out0, tile.a_out_lim, tid & 255);
+      lb.init_prefetch(p.ldb, tile.b_out0, tile.b_out_lim, tid & 255);
+#pragma unroll
+      for (int q = 1; q <= HMOE_PF; ++q) prefetch_line(q);
+    }
   };
 
   Tile tile;
@@ -737,7 +795,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_v3_kernel(Gem
     int live = (tile.a_out_lim - (tile.a_out0 + row_a) + 31) >> 5;
     live = live < 0 ? 0 : (live > WM ? WM : live);
     __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();  // step 0 of this tile has landed in stage 0
+    workgroup_barrier();  // step 0 of this tile has landed in stage 0
 
     auto run = [&](auto full_tag) {
       constexpr bool kFull = decltype(full_tag)::value;
@@ -746,6 +804,9 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_v3_kernel(Gem
         if (step + 1 < steps && !(HMOE_ABLATE & 1)) {  // the other stage is free since the barrier that ended the previous step
           la.issue(lds + (cur ^ 1) * (Cfg::kStage * 2), step + 1, wave);
           lb.issue(lds + (cur ^ 1) * (Cfg::kStage * 2) + kTileB * 2, step + 1, wave);
+        }
+        if constexpr (HMOE_PF > 0) {  // after the tile loads, so that the step's wait can leave it in flight
+          prefetch_line(step + 1 + HMOE_PF);
         }
         const int ta = cur * Cfg::kStage, tb = ta + kTileB;
         // fragments are double-buffered: those of sub-step kk+1 are read while the MFMAs of sub-step kk run
@@ -780,8 +841,10 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_v3_kernel(Gem
             }
           }
         }
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
+        if constexpr ((HMOE_ABLATE & 32) != 0) HMOE_WAIT_VM(24);  // timing experiment only: loads run three steps deep
+        else if constexpr (HMOE_PF > 0) HMOE_WAIT_VM(Cfg::kThreads == 512 ? 1 : 2);  // all but the prefetch, the youngest
+        else HMOE_WAIT_VM(0);
+        workgroup_barrier();
       }
     };
     if (live == WM) run(std::true_type{});
@@ -799,6 +862,9 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_v3_kernel(Gem
     constexpr int kRowsPerPass = 64 / kLanesPerRow;
     static_assert(kEpiRegion * Cfg::GM * Cfg::GN <= Cfg::kStage, "epilogue staging must fit in one stage");
     bf16_t* stage = smem + Cfg::kStage + wave * kEpiRegion;
+    const uint32_t stage_addr =
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) +
+        static_cast<uint32_t>((Cfg::kStage + wave * kEpiRegion + (lane & 31) * kEpiPitch + ((lane >> 5) << 2)) * 2);
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
 #pragma unroll
@@ -810,7 +876,13 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_v3_kernel(Gem
                      (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 1])) << 16);
           packed.y = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 2])) |
                      (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 3])) << 16);
-          *reinterpret_cast<uint2*>(stage + (lane & 31) * kEpiPitch + j * 32 + q * 8 + ((lane >> 5) << 2)) = packed;
+          // Written through inline assembly on purpose: before an LDS store it can see, the compiler drains every
+          // direct-to-LDS load in flight (it cannot tell that this region is not their target), which here would
+          // wait for the next tile's first step and for the prefetches.
+          asm volatile("ds_write_b64 %0, %1 offset:%2"
+                       :
+                       : "v"(stage_addr), "v"(packed), "n"((j * 32 + q * 8) * 2)
+                       : "memory");
         }
       }
       __builtin_amdgcn_wave_barrier();  // the region is private to the wavefront, whose LDS accesses stay in order
@@ -827,6 +899,511 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_v3_kernel(Gem
       }
       __builtin_amdgcn_wave_barrier();
     }
+  }
+}
+
+// ------------------------------------------------------------------------------------- bf16 kernel, ring pipeline
+// The same 256 x 256 tile and the same direct-to-LDS loads, but the contraction moves in steps of 32 through a ring of
+// four 32 KB stages, and the loads run three steps ahead of the MFMAs as ONE stream that does not stop at tile
+// boundaries: while a tile's last steps and its epilogue run, the first steps of the workgroup's next tile are already
+// in flight.  A step that misses L2 takes well over a microsecond to arrive; three stages in flight keep 64-96 KB
+// moving per CU, which is what the memory system needs to stream at the rate the MFMAs consume.
+//
+// One barrier per step, in the middle of it: before the barrier a wavefront waits until its own loads of the NEXT
+// stage have landed (s_waitcnt vmcnt(n), n = vector memory instructions it has issued since that stage's loads, so
+// younger loads and the epilogue's stores stay in flight); after the barrier every wavefront's part of the next stage
+// is visible and every wavefront is done with the previous stage, whose slot takes the loads of three steps ahead.
+// The MFMA fragments of the next step's first half are read right after the barrier, under the MFMAs of this step's
+// second half, so the matrix pipe has work across the barrier and across tile boundaries.
+constexpr int RK = 32;                  // contraction per ring stage
+constexpr int kRing = 4;                // stages
+constexpr int kOpTile = 256 * RK;       // elements of one operand tile in a stage (16 KB)
+constexpr int kSlot = 2 * kOpTile;      // elements per stage: A tile then B tile
+
+// element(out, con) = base[out * ld + con].  LDS tile: [256 out][32 con], 64-byte rows, the 16-byte chunk index
+// XOR-ed with (row >> 2) & 3 so that 16 lanes reading one chunk column of 16 rows cover all 64 banks.
+// One instruction moves 16 rows x 64 bytes; a wavefront issues kI of them per step.
+template <int kI>
+struct RingDirect {
+  __amdgpu_buffer_rsrc_t rsrc;  // bounded at the operand's last output row: rows past it load as zeros
+  uint32_t voff[kI];            // byte offset of this lane's chunk per instruction at step 0 (16 rows apart)
+  int con0;                     // contraction index within a step of this lane's chunk
+  int con_lim;
+
+  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
+                                       int con_lim_, int wave, int lane) {
+    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
+    con_lim = con_lim_;
+    const int logical = (lane & 3) ^ ((lane >> 4) & 3);  // (row >> 2) & 3 == (lane >> 4) & 3 for every instruction
+    con0 = logical << 3;
+#pragma unroll
+    for (int t = 0; t < kI; ++t) {
+      const int out = out0 + (wave * kI + t) * 16 + (lane >> 2);
+      voff[t] = out < out_lim ? static_cast<uint32_t>(out) * static_cast<uint32_t>(ld) * 2u + (logical << 4)
+                              : kOutOfRange;
+    }
+  }
+  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave) const {
+    const bool in_range = step * RK + con0 < con_lim;
+    const uint32_t soff = static_cast<uint32_t>(step) * (RK * 2);
+#pragma unroll
+    for (int t = 0; t < kI; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * kI + t) * 1024, 16,
+                                               in_range ? voff[t] : kOutOfRange, soff, 0, 0);
+  }
+  // byte offset within the operand tile of this lane's fragment for sub-step kk of block row `row0`
+  static __device__ __forceinline__ int fragment_offset(int row0, int kk, int lane) {
+    const int r = row0 + (lane & 31);
+    return r * (RK * 2) + ((((kk << 1) + (lane >> 5)) ^ ((r >> 2) & 3)) << 4);
+  }
+  static __device__ __forceinline__ bf16x8 fragment(const char* tile, int offset) {
+    return *reinterpret_cast<const bf16x8*>(tile + offset);
+  }
+};
+
+// element(out, con) = base[con * ld + out].  LDS tile: [32 con][256 out] as it lies in memory, 512-byte rows, chunk
+// index XOR-ed with (con & 3) << 2; fragments come out through the transposing LDS read.  A half-wavefront of that
+// read touches 4 contraction rows x 2 groups of 16 columns (32 bytes each): the XOR spreads the rows 64 bytes apart,
+// the column groups fill the gaps, and the eight pieces cover the 64 banks exactly once.
+// One instruction moves two contraction rows; a wavefront issues kI of them per step.
+template <int kI>
+struct RingTransposed {
+  __amdgpu_buffer_rsrc_t rsrc;  // bounded at the operand's last contraction row
+  uint32_t voff[kI];
+  uint32_t step_bytes;
+
+  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
+                                       int /*con_lim*/, int wave, int lane) {
+    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
+    step_bytes = RK * static_cast<uint32_t>(ld) * 2u;
+#pragma unroll
+    for (int t = 0; t < kI; ++t) {
+      const int con = (wave * kI + t) * 2 + (lane >> 5);
+      const int logical = (lane & 31) ^ ((con & 3) << 2);
+      const int out = out0 + (logical << 3);
+      voff[t] = out < out_lim
+                    ? static_cast<uint32_t>(con) * static_cast<uint32_t>(ld) * 2u + static_cast<uint32_t>(out) * 2u
+                    : kOutOfRange;
+    }
+  }
+  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave) const {
+    const uint32_t soff = static_cast<uint32_t>(step) * step_bytes;
+#pragma unroll
+    for (int t = 0; t < kI; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * kI + t) * 1024, 16, voff[t], soff, 0, 0);
+  }
+  static __device__ __forceinline__ int fragment_offset(int row0, int kk, int lane) {
+    const int i = lane & 15, g = lane >> 4;
+    const int out = row0 + ((g & 1) << 4) + ((i & 3) << 2);  // first of the four columns this lane points at
+    const int con = kk * 16 + ((g >> 1) << 3) + (i >> 2);     // (con & 3) == (i >> 2) for both reads
+    return (con * 256 + ((((out >> 3) ^ ((con & 3) << 2)) << 3) + (out & 7))) * 2;
+  }
+  static __device__ __forceinline__ bf16x8 fragment(const char* tile, int offset) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+    const char* p = tile + offset;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * 256 * 2));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(bf16x8, both);
+  }
+};
+
+// wait until at most `n` of this wavefront's vector memory instructions are outstanding (rounded down to a value
+// that has an encoding here: waiting for more than asked is always safe)
+__device__ __forceinline__ void wait_vm_at_most(int n, int steady) {
+  if (n == steady) {  // two younger stages in flight and nothing else: every step but the first three of a tile
+    if (steady == 8) HMOE_WAIT_VM(8);
+    else HMOE_WAIT_VM(16);
+  } else if (n >= 48) HMOE_WAIT_VM(48);
+  else if (n >= 40) HMOE_WAIT_VM(40);
+  else if (n >= 32) HMOE_WAIT_VM(32);
+  else if (n >= 24) HMOE_WAIT_VM(24);
+  else if (n >= 20) HMOE_WAIT_VM(20);
+  else if (n >= 16) HMOE_WAIT_VM(16);
+  else if (n >= 12) HMOE_WAIT_VM(12);
+  else if (n >= 8) HMOE_WAIT_VM(8);
+  else if (n >= 4) HMOE_WAIT_VM(4);
+  else HMOE_WAIT_VM(0);
+}
+
+template <typename Cfg>
+struct RingLayout {
+  static constexpr int kWaves = Cfg::GM * Cfg::GN;
+  static constexpr int kEpiPitch = Cfg::WN * 32 + 8;       // elements; the 16 bytes of padding stagger the banks
+  static constexpr int kEpiRegion = 16 * kEpiPitch;        // elements per wavefront: 16 rows of its tile
+  static constexpr size_t kRingBytes = size_t(kRing) * kSlot * sizeof(bf16_t);
+  static constexpr size_t kStagingBytes = size_t(kWaves) * kEpiRegion * sizeof(bf16_t);
+  static size_t bytes(int groups) { return kRingBytes + kStagingBytes + size_t(3 * groups + 1) * sizeof(int32_t); }
+};
+
+struct RingTile {
+  int g, a_out0, a_out_lim, b_out0, b_out_lim, con_lim, row_start;
+};
+
+// The tile walk of one workgroup.  Tile ids only grow along the walk, so the group of a tile is found by scanning on
+// from the previous tile's group.  Everything here is uniform across the workgroup and kept in scalar registers.
+template <int kMode, int BM, int BN>
+struct RingSchedule {
+  const int32_t* grp_s;
+  const int32_t* grp_e;
+  const int32_t* tile_start;
+  int nt, mt_w;
+  int64_t per_group, first, last, stride;
+  int k, n;
+
+  __device__ __forceinline__ void init(const GemmArgs& p, const int32_t* s, const int32_t* e, const int32_t* ts) {
+    grp_s = s;
+    grp_e = e;
+    tile_start = ts;
+    k = static_cast<int>(p.k);
+    n = static_cast<int>(p.n);
+    mt_w = 1;
+    per_group = 1;
+    const int workers = gridDim.x;
+    if constexpr (kMode == kWgrad) {
+      mt_w = static_cast<int>((p.k + BM - 1) / BM);
+      nt = static_cast<int>((p.n + BN - 1) / BN);
+      per_group = static_cast<int64_t>(mt_w) * nt;
+      first = blockIdx.x;
+      last = per_group * p.groups;
+      stride = workers;
+    } else {
+      const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
+      nt = static_cast<int>((out_cols + BN - 1) / BN);
+      const int64_t total = static_cast<int64_t>(__builtin_amdgcn_readfirstlane(tile_start[p.groups])) * nt;
+      const int xcd = blockIdx.x % kXcds;
+      const int64_t chunk = (total + kXcds - 1) / kXcds;
+      first = xcd * chunk + blockIdx.x / kXcds;
+      last = xcd * chunk + chunk < total ? xcd * chunk + chunk : total;
+      stride = (workers - xcd + kXcds - 1) / kXcds;
+    }
+  }
+
+  __device__ __forceinline__ RingTile decode(int64_t t, int& cursor) const {
+    int g, m_t, n_t;
+    if constexpr (kMode == kWgrad) {
+      g = static_cast<int>(t / per_group);
+      const int r = static_cast<int>(t - g * per_group);
+      n_t = r / mt_w;
+      m_t = r - n_t * mt_w;
+    } else {
+      g = cursor;
+      while (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(tile_start[g + 1])) * nt <= t) ++g;
+      cursor = g;
+      const int ts = __builtin_amdgcn_readfirstlane(tile_start[g]);
+      const int mt = __builtin_amdgcn_readfirstlane(tile_start[g + 1]) - ts;
+      const int r = static_cast<int>(t - static_cast<int64_t>(ts) * nt);
+      n_t = r / mt;
+      m_t = r - n_t * mt;
+    }
+    const int s = __builtin_amdgcn_readfirstlane(grp_s[g]);
+    const int rows = __builtin_amdgcn_readfirstlane(grp_e[g]) - s;
+    RingTile tile;
+    tile.g = g;
+    tile.row_start = s;
+    tile.a_out0 = m_t * BM;
+    tile.b_out0 = n_t * BN;
+    if constexpr (kMode == kWgrad) {
+      tile.a_out_lim = k;
+      tile.b_out_lim = n;
+      tile.con_lim = rows;
+    } else {
+      tile.a_out_lim = rows;
+      tile.b_out_lim = kMode == kDgrad ? k : n;
+      tile.con_lim = kMode == kDgrad ? n : k;
+    }
+    return tile;
+  }
+};
+
+// The load stream: (tile, step) after (tile, step) into the ring's slots, up to three steps ahead of the MFMAs.
+// `issued` counts the vector memory instructions of this wavefront (the epilogue adds its stores); seq0..2 hold its
+// value right after the loads of the stages in flight, oldest first, which is what the vmcnt waits are made from.
+template <int kMode, typename Sched, typename LoaderA, typename LoaderB, int kI>
+struct RingProducer {
+  LoaderA la;
+  LoaderB lb;
+  int64_t pt;
+  int cursor, step, steps, slot;
+  bool open;
+  int issued, seq0, seq1, seq2, in_flight;
+
+  __device__ __forceinline__ void init(const Sched& sched) {
+    pt = sched.first;
+    cursor = 0;
+    step = steps = slot = 0;
+    open = false;
+    issued = seq0 = seq1 = seq2 = in_flight = 0;
+  }
+  // position the stream on the next tile that has a contraction to load
+  __device__ __forceinline__ void open_next(const Sched& sched, const GemmArgs& p, int wave, int lane) {
+    const bf16_t* a = static_cast<const bf16_t*>(p.a);
+    const bf16_t* b = static_cast<const bf16_t*>(p.b);
+    open = false;
+    while (pt < sched.last) {
+      const RingTile tile = sched.decode(pt, cursor);
+      if (tile.con_lim > 0) {
+        if constexpr (kMode == kWgrad) {
+          const int64_t rows = tile.con_lim;
+          la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim, wave,
+                  lane);
+          lb.init(b + tile.row_start * p.ldb, p.ldb, rows * p.ldb * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, wave,
+                  lane);
+        } else {
+          const int64_t rows = tile.a_out_lim;
+          const int64_t w_elems = p.k * p.n;
+          la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim, wave,
+                  lane);
+          lb.init(b + tile.g * w_elems, p.ldb, w_elems * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, wave, lane);
+        }
+        step = 0;
+        steps = (tile.con_lim + RK - 1) / RK;
+        open = true;
+        return;
+      }
+      pt += sched.stride;
+    }
+  }
+  __device__ __forceinline__ void produce(const Sched& sched, const GemmArgs& p,
+                                          __attribute__((address_space(3))) char* lds, int wave, int lane) {
+    if (!open) return;
+    auto dst = lds + slot * (kSlot * 2);
+    if (!(HMOE_ABLATE & 1)) {
+      la.issue(dst, step, wave);
+      lb.issue(dst + kOpTile * 2, step, wave);
+      issued += 2 * kI;
+    }
+    if (in_flight == 0) seq0 = issued;
+    else if (in_flight == 1) seq1 = issued;
+    else seq2 = issued;
+    ++in_flight;
+    slot = (slot + 1) & (kRing - 1);
+    if (++step == steps) {
+      pt += sched.stride;
+      open_next(sched, p, wave, lane);
+    }
+  }
+  // wait for this wavefront's loads of the oldest stage in flight and retire it from the queue
+  __device__ __forceinline__ void await_oldest() {
+    wait_vm_at_most(issued - seq0, 4 * kI);
+    seq0 = seq1;
+    seq1 = seq2;
+    --in_flight;
+  }
+};
+
+template <int kMode, typename Cfg>
+__global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_ring_kernel(GemmArgs p) {
+  static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
+  using L = RingLayout<Cfg>;
+  constexpr int WM = Cfg::WM, WN = Cfg::WN, BM = Cfg::BM, BN = Cfg::BN;
+  constexpr int kI = 16 / L::kWaves;  // 1 KB load instructions per wavefront per operand per step
+  constexpr int kStoresPerBlockRow = 2 * (16 * WN * 32 * 2 / 1024);  // two halves of 16 rows, 1 KB per instruction
+  using LoaderA = typename std::conditional<kMode == kWgrad, RingTransposed<kI>, RingDirect<kI>>::type;
+  using LoaderB = typename std::conditional<kMode == kDgrad, RingDirect<kI>, RingTransposed<kI>>::type;
+  using Sched = RingSchedule<kMode, BM, BN>;
+  extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+  auto lds = (__attribute__((address_space(3))) char*)lds_raw;
+  bf16_t* staging_all = reinterpret_cast<bf16_t*>(lds_raw + L::kRingBytes);
+  int32_t* grp_s = reinterpret_cast<int32_t*>(lds_raw + L::kRingBytes + L::kStagingBytes);
+  int32_t* grp_e = grp_s + p.groups;
+  int32_t* tile_start = grp_e + p.groups;  // [groups + 1], fwd and dgrad only
+  bf16_t* c = static_cast<bf16_t*>(p.c);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int gm = wave / Cfg::GN, gn = wave % Cfg::GN;
+  const int row_a = gm * (WM * 32), row_b = gn * (WN * 32);
+
+  // ---- group bounds and the row-tile prefix, by wavefront 0
+  if (wave == 0) {
+    const int per = (p.groups + HMOE_WAVE - 1) / HMOE_WAVE;
+    const int g0 = lane * per;
+    int sum = 0;
+    for (int g = g0; g < g0 + per && g < p.groups; ++g) {
+      int64_t s, e;
+      group_bounds(p.offs, g, p.total_rows, s, e);
+      grp_s[g] = static_cast<int32_t>(s);
+      grp_e[g] = static_cast<int32_t>(e);
+      sum += static_cast<int>((e - s + BM - 1) / BM);
+    }
+    if constexpr (kMode != kWgrad) {
+      int incl = sum;
+#pragma unroll
+      for (int off = 1; off < HMOE_WAVE; off <<= 1) {
+        const int up = __shfl_up(incl, off, HMOE_WAVE);
+        if (lane >= off) incl += up;
+      }
+      int running = incl - sum;
+      for (int g = g0; g < g0 + per && g < p.groups; ++g) {
+        tile_start[g] = running;
+        running += (grp_e[g] - grp_s[g] + BM - 1) / BM;
+      }
+      if (lane == HMOE_WAVE - 1) tile_start[p.groups] = incl;
+    }
+  }
+  __syncthreads();
+
+  Sched sched;
+  sched.init(p, grp_s, grp_e, tile_start);
+  RingProducer<kMode, Sched, LoaderA, LoaderB, kI> prod;
+  prod.init(sched);
+  const int64_t w_elems = p.k * p.n;
+
+  // ---- fragment addresses (bytes within an operand tile); block rows are 32 output rows apart
+  int fa_off[2], fb_off[2][WN];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+    fa_off[kk] = LoaderA::fragment_offset(row_a, kk, lane);
+#pragma unroll
+    for (int j = 0; j < WN; ++j) fb_off[kk][j] = LoaderB::fragment_offset(row_b + j * 32, kk, lane);
+  }
+  constexpr int kBlockRowBytesA = std::is_same<LoaderA, RingDirect<kI>>::value ? 32 * RK * 2 : 0;
+  bf16x8 fa[2][WM], fb[2][WN];
+  int ablate_reads = 0;
+  auto read_fragments = [&](int slot, int kk) __attribute__((always_inline)) {
+    if ((HMOE_ABLATE & 2) && ablate_reads++ >= 2) return;
+    const char* ta = lds_raw + slot * (kSlot * 2);
+    const char* tb = ta + kOpTile * 2;
+#pragma unroll
+    for (int j = 0; j < WN; ++j) fb[kk][j] = LoaderB::fragment(tb, fb_off[kk][j]);
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+      if constexpr (kBlockRowBytesA != 0) fa[kk][i] = LoaderA::fragment(ta, fa_off[kk] + i * kBlockRowBytesA);
+      else fa[kk][i] = LoaderA::fragment(ta, LoaderA::fragment_offset(row_a + i * 32, kk, lane));
+    }
+  };
+
+  prod.open_next(sched, p, wave, lane);
+  prod.produce(sched, p, lds, wave, lane);
+  prod.produce(sched, p, lds, wave, lane);
+  prod.produce(sched, p, lds, wave, lane);
+  int c_slot = 0;
+  if (prod.in_flight > 0) {
+    prod.await_oldest();
+    workgroup_barrier();
+    read_fragments(0, 0);
+  }
+
+  bf16_t* staging = staging_all + wave * L::kEpiRegion;
+  // LDS byte address of this lane's 8-byte slot in its staging row (block column and quad added as offsets)
+  const uint32_t staging_addr =
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds_raw)) +
+      static_cast<uint32_t>(L::kRingBytes) +
+      static_cast<uint32_t>((wave * L::kEpiRegion + (lane & 15) * L::kEpiPitch + ((lane >> 5) << 2)) * 2);
+  int c_cursor = 0;
+  for (int64_t ct = sched.first; ct < sched.last; ct += sched.stride) {
+    const RingTile tile = sched.decode(ct, c_cursor);
+    f32x16 acc[WM][WN];
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    const int steps = (tile.con_lim + RK - 1) / RK;
+    int live = (tile.a_out_lim - (tile.a_out0 + row_a) + 31) >> 5;
+    live = live < 0 ? 0 : (live > WM ? WM : live);
+
+    auto run = [&](auto full_tag) __attribute__((always_inline)) {
+      constexpr bool kFull = decltype(full_tag)::value;
+      for (int step = 0; step < steps; ++step) {
+        read_fragments(c_slot, 1);
+#pragma unroll
+        for (int i = 0; i < WM; ++i) {
+          if (kFull || i < live) {
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+              if (HMOE_ABLATE & 4) {
+                asm volatile("" ::"v"(fb[0][j]), "v"(fa[0][i]));
+                continue;
+              }
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][j], fa[0][i], acc[i][j], 0, 0, 0);
+            }
+          }
+        }
+        const int next = (c_slot + 1) & (kRing - 1);
+        const bool more = prod.in_flight > 0;  // a further step (of this tile or the next) is on its way
+        if (more) prod.await_oldest();
+        if (!(HMOE_ABLATE & 8)) workgroup_barrier();  // the next stage is complete and visible; the previous stage's slot is free
+        // the matrix pipe gets work first; the loads three steps ahead and the next fragments go out under it
+#pragma unroll
+        for (int i = 0; i < WM; ++i) {
+          if (i == WM / 2) {
+            __builtin_amdgcn_sched_barrier(0);
+            prod.produce(sched, p, lds, wave, lane);
+            if (more) read_fragments(next, 0);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          if (kFull || i < live) {
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+              if (HMOE_ABLATE & 4) {
+                asm volatile("" ::"v"(fb[1][j]), "v"(fa[1][i]));
+                continue;
+              }
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
+            }
+          }
+        }
+        c_slot = next;
+      }
+    };
+    if (live == WM) run(std::true_type{});
+    else run(std::false_type{});
+
+    // ---- epilogue: 16 rows of the wavefront's tile at a time through its private staging rows, 16-byte chunks out
+    // through buffer stores whose offsets are forced out of range where the tile hangs over the output's edge, so
+    // the number of store instructions is known (the vmcnt arithmetic counts them).
+    constexpr int kLanesPerRow = WN * 4;
+    constexpr int kRowsPerPass = 64 / kLanesPerRow;
+    bf16_t* c_base = kMode == kWgrad ? c + tile.g * w_elems : c + tile.row_start * p.ldc;
+    const int64_t c_rows = kMode == kWgrad ? p.k : tile.a_out_lim;
+    const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(c_base, static_cast<uint32_t>(c_rows * p.ldc * 2));
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+      if (i < live) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          if (((lane >> 4) & 1) == half) {
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                uint2 packed;
+                packed.x = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 0])) |
+                           (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 1])) << 16);
+                packed.y = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 2])) |
+                           (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 3])) << 16);
+                // Written through inline assembly on purpose: for an LDS store the compiler sees, it first drains
+                // every direct-to-LDS load in flight (it cannot tell that the staging rows lie outside the ring),
+                // which would stop the load stream at every tile boundary.
+                asm volatile("ds_write_b64 %0, %1 offset:%2"
+                             :
+                             : "v"(staging_addr), "v"(packed), "n"((j * 32 + q * 8) * 2)
+                             : "memory");
+              }
+            }
+          }
+          __builtin_amdgcn_wave_barrier();  // the rows are private to the wavefront, whose LDS accesses stay in order
+#pragma unroll
+          for (int pass = 0; pass < 16 / kRowsPerPass; ++pass) {
+            const int rr = pass * kRowsPerPass + lane / kLanesPerRow;
+            const int cc = (lane % kLanesPerRow) << 3;
+            const int row = tile.a_out0 + row_a + i * 32 + half * 16 + rr;
+            const int col = tile.b_out0 + row_b + cc;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(staging + rr * L::kEpiPitch + cc);
+            const uint32_t off = row < tile.a_out_lim && col < tile.b_out_lim
+                                     ? static_cast<uint32_t>(row) * static_cast<uint32_t>(p.ldc) * 2u + col * 2u
+                                     : kOutOfRange;
+            __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, (HMOE_ABLATE & 16) ? kOutOfRange : off, 0, 0);
+          }
+          __builtin_amdgcn_wave_barrier();
+        }
+      }
+    }
+    prod.issued += live * kStoresPerBlockRow;
   }
 }
 
@@ -985,10 +1562,39 @@ int launch_v3(const GemmArgs& p, hipStream_t stream) {
   if (bound < workers) workers = bound;
   workers = (workers + kXcds - 1) / kXcds * kXcds;
   if (workers <= 0) return HMOE_OK;
-  constexpr size_t lds_bytes = 2 * Cfg::kStage * sizeof(bf16_t);
+  constexpr size_t lds_bytes = 2 * Cfg::kStage * sizeof(bf16_t) + Cfg::GM * Cfg::GN * 256;  // stages, prefetch scrap
   auto kernel = grouped_gemm_bf16_v3_kernel<kMode, Cfg>;
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                           static_cast<int>(lds_bytes)) != hipSuccess)
+    return HMOE_LAUNCH_FAILED;
+  kernel<<<dim3(static_cast<unsigned>(workers)), dim3(Cfg::kThreads), lds_bytes, stream>>>(p);
+  return HMOE_OK;
+}
+
+
+#define HMOE_RING_INSTANCE(mode) \
+  template __global__ void grouped_gemm_ring_kernel<mode, Config<2, 4, 4, 2>>(GemmArgs); \
+  template __global__ void grouped_gemm_ring_kernel<mode, Config<2, 2, 4, 4>>(GemmArgs);
+HMOE_RING_INSTANCE(kFwd)
+HMOE_RING_INSTANCE(kDgrad)
+HMOE_RING_INSTANCE(kWgrad)
+#undef HMOE_RING_INSTANCE
+
+template <int kMode, typename Cfg>
+int launch_ring(const GemmArgs& p, hipStream_t stream) {
+  const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
+  const int64_t nt = (out_cols + Cfg::BN - 1) / Cfg::BN;
+  int64_t bound;
+  if (kMode == kWgrad) bound = ((p.k + Cfg::BM - 1) / Cfg::BM) * nt * p.groups;
+  else bound = (p.total_rows / Cfg::BM + p.groups) * nt;
+  int64_t workers = device_cus();
+  if (bound < workers) workers = bound;
+  workers = (workers + kXcds - 1) / kXcds * kXcds;
+  if (workers <= 0) return HMOE_OK;
+  const size_t lds_bytes = RingLayout<Cfg>::bytes(p.groups);
+  auto kernel = grouped_gemm_ring_kernel<kMode, Cfg>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          static_cast<int>(RingLayout<Cfg>::bytes(kMaxGroups))) != hipSuccess)
     return HMOE_LAUNCH_FAILED;
   kernel<<<dim3(static_cast<unsigned>(workers)), dim3(Cfg::kThreads), lds_bytes, stream>>>(p);
   return HMOE_OK;
@@ -999,6 +1605,13 @@ int launch(const GemmArgs& p, int dtype, hipStream_t stream) {
   if (dtype == HMOE_BF16) {
     int rc;
     if constexpr (kMode != kFwdFp8W) {
+      if (experiment_cfg() == 11 || experiment_cfg() == 12) {
+        if (experiment_cfg() == 11) rc = launch_ring<kMode, Config<2, 4, 4, 2>>(p, stream);
+        else rc = launch_ring<kMode, Config<2, 2, 4, 4>>(p, stream);
+        if (rc) return rc;
+        if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
+        return HMOE_OK;
+      }
       if (experiment_cfg() == 0 || experiment_cfg() >= 9) {
         if (experiment_cfg() != 10) rc = launch_v3<kMode, Config<2, 4, 4, 2>>(p, stream);
         else rc = launch_v3<kMode, Config<2, 2, 4, 4>>(p, stream);
@@ -1043,7 +1656,8 @@ int validate(const GemmArgs& p, int dtype) {
     // buffer loads address an operand with 32-bit byte offsets: all rows of an operand and one expert's weight
     // must each stay below 2 GiB
     const int64_t lim = int64_t(1) << 31;
-    if (p.total_rows * p.lda * 2 >= lim || p.total_rows * p.ldb * 2 >= lim || p.k * p.n * 2 >= lim)
+    if (p.total_rows * p.lda * 2 >= lim || p.total_rows * p.ldb * 2 >= lim || p.total_rows * p.ldc * 2 >= lim ||
+        p.k * p.n * 2 >= lim)
       return HMOE_UNSUPPORTED;
   }
   return HMOE_OK;
