@@ -6,26 +6,39 @@
 //   wgrad  dB[g]     = A[s:e]^T @ dO[s:e]      ragged contraction, empty group -> exact zeros
 // with offs[g] the inclusive end of group g.  bf16 operands, fp32 accumulation on MFMA, one rounding.
 //
-// bf16 kernel.  One persistent launch.  A workgroup of GM x GN wavefronts owns a (GM*WM*32) x (GN*WN*32) output
-// tile and walks the contraction in steps of 64; each wavefront owns WM x WN accumulator blocks of 32x32
-// (v_mfma_f32_32x32x16_bf16).  LDS is the scarce resource on this chip (128 B/clk/CU read, about half that written),
-// so the tile is as large as the accumulators allow: per contraction element a wavefront reads (WM+WN)*32 operand
-// values for WM*WN*1024 multiply-adds.
-// Both operand tiles sit in LDS as [output index][64 contraction], contraction contiguous, so every MFMA fragment is
-// one 16-byte LDS read; the 16-byte chunk index is XOR-swizzled with the row, which keeps fragment reads, straight
-// copies and transposed writes free of bank conflicts.  An operand whose contraction index is the strided one in
-// global memory (B in fwd, both operands in wgrad) is transposed in registers (8x8 blocks of bf16, v_perm_b32) on its
-// way into LDS.  Global loads are raw buffer loads: rows past the group's end and columns past the operand's edge
-// come back as zeros from the hardware bounds check, with no branches in the loop.  Loads for step k+1 are issued
-// before the MFMAs of step k (register staging, two LDS buffers, one barrier per step).  The MFMA is issued with the
-// operands swapped (B fragment as srcA) so that a lane owns one output row and four consecutive columns per
-// accumulator quad: stores are 8 bytes per lane.
+// bf16 kernel (grouped_gemm_bf16_kernel).  One persistent launch; a workgroup of 8 wavefronts owns a 256 x 256 output
+// tile and walks the contraction in steps of 64; each wavefront owns 4 x 2 accumulator blocks of 32 x 32
+// (v_mfma_f32_32x32x16_bf16).  The tile is as large as the accumulators allow because LDS is the scarce resource here
+// (one ds_read per 8 cycles per CU whatever its width, measured): per contraction element a wavefront reads
+// (4 + 2) * 32 operand values for 4 * 2 * 1024 multiply-adds.
+//  * Operand tiles go from global memory straight into LDS (buffer_load ... lds, 16 bytes per lane): no staging
+//    registers, no ds_write, no register transposes.  Rows past a group's end and columns past an operand's edge come
+//    back as zeros from the buffer bounds check, with no branches in the loop.
+//  * A contraction-contiguous operand lands as [256 rows][64 con] with the 16-byte chunk index XOR-ed with row & 7
+//    (each lane fetches the chunk that belongs in its LDS slot); an MFMA fragment is one ds_read_b128, and the
+//    fragments of other row blocks and contraction sub-steps are immediate offsets or one XOR away.
+//  * An output-contiguous operand (B in fwd, both operands in wgrad) lands as it lies in memory, [64 con][256 out],
+//    chunks XOR-ed with (con & 3) << 2, and a fragment is two ds_read_b64_tr_b16, the gfx950 transposing LDS read:
+//    within 16 lanes, lane i supplies the address of row (i >> 2), columns 4 (i & 3)..+3 of a 4 x 16 patch and receives
+//    the four rows of column i.
+//  * Two LDS stages; the loads of step k+1 are in flight during step k.  The fragments of sub-step kk+1 are read under
+//    the MFMAs of sub-step kk, and the step's barrier sits in the middle of the last sub-step's MFMAs: the first
+//    fragments of the next step are read behind it, under the rest.  The barrier is a bare s_barrier after an explicit
+//    s_waitcnt: __syncthreads() would fence and drain loads that are meant to stay in flight.
+//  * The MFMA is issued with the operands swapped (B fragment as srcA) so that a lane owns one output row and four
+//    consecutive columns per accumulator quad.  The epilogue stages 32 rows per wavefront through LDS and writes whole
+//    16-byte chunks with buffer stores; the next tile's first loads are issued before it.
 //
-// Tile schedule.  Every workgroup builds the per-group prefix of row tiles from offs in LDS (no host readback), so
-// ragged and empty groups cost exactly their tiles.  The logical tile order is group-major, then column tile, then
-// row tile; it is cut into 8 contiguous chunks, one per XCD (workgroup w runs on XCD w % 8), so the workgroups that
-// share an L2 work on the same expert's weights at the same time, and the tile count per XCD is balanced whatever
-// the skew of the expert loads.  wgrad tiles are dealt round-robin so every workgroup sees every group size.
+// Tile schedule.  Every workgroup builds the group bounds and the per-group prefix of row tiles from offs in LDS (no
+// host readback), so ragged and empty groups cost exactly their tiles.  The logical tile order is group-major, then
+// column tile, then row tile; it is cut into 8 contiguous chunks, one per XCD (workgroup w runs on XCD w % 8), so the
+// workgroups that share an L2 work on the same expert's weights at the same time, and the tile count per XCD is
+// balanced whatever the skew of the expert loads.  wgrad tiles are dealt round-robin so every workgroup sees every
+// group size.
+//
+// Weights in block-scaled fp8 (grouped_gemm_staged_kernel, forward only) take the register-staged variant of the same
+// tiling: global -> registers (dequantised there) -> LDS as [output index][64 contraction], both operands read back
+// with ds_read_b128.
 //
 // fp32 operands take a plain LDS-tiled FMA kernel (the CPU-sized plumbing configuration and tests).
 #include "common.h"
@@ -41,12 +54,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-#ifndef HMOE_ABLATE
-#define HMOE_ABLATE 0
-#endif
-#ifndef HMOE_PF
-#define HMOE_PF 0  // L2 prefetch distance of the direct-to-LDS kernel, in contraction steps; 0 = off
-#endif
 
 constexpr int BK = 64;  // contraction per step
 constexpr int kXcds = 8;
@@ -76,7 +83,6 @@ struct GemmArgs {
   int groups;
   int64_t k, n;
   const float* b_scale;  // kFwdFp8W: [G, ceil(K/128), ceil(N/128)]
-  int ablate;            // diagnostics: 1 skip global loads, 2 skip LDS stores, 4 skip MFMAs, 8 skip fragment reads
 };
 
 __device__ __forceinline__ int swizzle(int row) { return (row & 7) ^ ((row >> 3) & 7); }
@@ -314,8 +320,7 @@ struct Fp8BlockLoader {
 template <typename Cfg, typename LoaderA, typename LoaderB>
 __device__ __forceinline__ void compute_tile(bf16_t* smem, LoaderA& la, LoaderB& lb, int a_out0,
                                              int a_out_lim, int b_out0, int b_out_lim, int con_lim,
-                                             bf16_t* __restrict__ c_base, int64_t c_ld, int /*unused*/ = 0) {
-  constexpr int ablate = HMOE_ABLATE;  // compile-time diagnostics switch, 0 in the product build
+                                             bf16_t* __restrict__ c_base, int64_t c_ld) {
   constexpr int WM = Cfg::WM, WN = Cfg::WN;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -353,7 +358,7 @@ __device__ __forceinline__ void compute_tile(bf16_t* smem, LoaderA& la, LoaderB&
     for (int step = 0; step < steps; ++step) {
       const int cur = step & 1;
       const bool more = step + 1 < steps;
-      if (more && !(ablate & 1)) {
+      if (more) {
         la.load(reg_a, step + 1);
         lb.load(reg_b, step + 1);
       }
@@ -365,21 +370,17 @@ __device__ __forceinline__ void compute_tile(bf16_t* smem, LoaderA& la, LoaderB&
         bf16x8 fa[WM], fb[WN];
 #pragma unroll
         for (int j = 0; j < WN; ++j)
-          fb[j] = *reinterpret_cast<const bf16x8*>(smem + tb + lds_offset(row_b + j * 32, (ablate & 8) ? 0 : chunk));
+          fb[j] = *reinterpret_cast<const bf16x8*>(smem + tb + lds_offset(row_b + j * 32, chunk));
 #pragma unroll
         for (int i = 0; i < WM; ++i) {
           if (kFull || i < live) {
-            fa[i] = *reinterpret_cast<const bf16x8*>(smem + ta + lds_offset(row_a + i * 32, (ablate & 8) ? 0 : chunk));
-            if (!(ablate & 4)) {
+            fa[i] = *reinterpret_cast<const bf16x8*>(smem + ta + lds_offset(row_a + i * 32, chunk));
 #pragma unroll
-              for (int j = 0; j < WN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
-            } else {
-              acc[i][0][0] += static_cast<float>(fa[i][0]) + static_cast<float>(fb[0][0]);
-            }
+            for (int j = 0; j < WN; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
           }
         }
-        if (kk == kStoreAfter && more && !(ablate & 2)) {
+        if (kk == kStoreAfter && more) {
           // the next stage's LDS writes go out between the MFMAs, not after them, so they overlap matrix work
           __builtin_amdgcn_sched_barrier(0);
           la.store(reg_a, smem, (cur ^ 1) * Cfg::kStage, tid);
@@ -430,7 +431,7 @@ __device__ __forceinline__ void compute_tile(bf16_t* smem, LoaderA& la, LoaderB&
       const int cc = (lane % kLanesPerRow) << 3;
       const int row = a_out0 + gm * (WM * 32) + half * 64 + rr;
       const int col = b_out0 + gn * (WN * 32) + cc;
-      if (half * 64 + rr < WM * 32 && row < a_out_lim && col < b_out_lim && !((ablate & 16) && c_ld != 12345)) {
+      if (half * 64 + rr < WM * 32 && row < a_out_lim && col < b_out_lim) {
         const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * kEpiPitch + cc);
         *reinterpret_cast<u32x4*>(c_base + static_cast<int64_t>(row) * c_ld + col) = v;
       }
@@ -472,7 +473,7 @@ __device__ __forceinline__ void build_tile_prefix(int32_t* tile_start, const int
 }
 
 template <int kMode, typename Cfg>
-__global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmArgs p) {
+__global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_staged_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(16))) bf16_t smem[];  // two stages of (A tile, B tile)
   __shared__ int32_t tile_start[kMode == kWgrad ? 1 : kMaxGroups + 1];
   constexpr int BM = Cfg::BM, BN = Cfg::BN, NT = Cfg::kThreads;
@@ -505,7 +506,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       la.init(a + s * p.lda, p.lda, rows * p.lda * 2, m_t * BM, static_cast<int>(p.k), rows, tid);
       lb.init(b + s * p.ldb, p.ldb, rows * p.ldb * 2, n_t * BN, static_cast<int>(p.n), rows, tid);
       compute_tile<Cfg>(smem, la, lb, m_t * BM, static_cast<int>(p.k), n_t * BN, static_cast<int>(p.n), rows,
-                        c + static_cast<int64_t>(g) * p.k * p.n, p.ldc, p.ablate);
+                        c + static_cast<int64_t>(g) * p.k * p.n, p.ldc);
     }
   } else {
     build_tile_prefix<BM>(tile_start, p.offs, p.groups, p.total_rows);
@@ -535,517 +536,32 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       if constexpr (kMode == kFwd) {
         Bf16Loader<true, BN, NT, kFirstB> lb;
         lb.init(b + g * w_elems, p.ldb, w_elems * 2, n_t * BN, static_cast<int>(p.n), con, tid);
-        compute_tile<Cfg>(smem, la, lb, m_t * BM, rows, n_t * BN, static_cast<int>(p.n), con, c + s * p.ldc, p.ldc, p.ablate);
+        compute_tile<Cfg>(smem, la, lb, m_t * BM, rows, n_t * BN, static_cast<int>(p.n), con, c + s * p.ldc, p.ldc);
       } else if constexpr (kMode == kDgrad) {
         Bf16Loader<false, BN, NT, 0> lb;
         lb.init(b + g * w_elems, p.ldb, w_elems * 2, n_t * BN, static_cast<int>(p.k), con, tid);
-        compute_tile<Cfg>(smem, la, lb, m_t * BM, rows, n_t * BN, static_cast<int>(p.k), con, c + s * p.ldc, p.ldc, p.ablate);
+        compute_tile<Cfg>(smem, la, lb, m_t * BM, rows, n_t * BN, static_cast<int>(p.k), con, c + s * p.ldc, p.ldc);
       } else {  // kFwdFp8W
         const int scale_ld = static_cast<int>((p.n + 127) >> 7);
         const int64_t scale_blocks = ((p.k + 127) >> 7) * scale_ld;
         Fp8BlockLoader<BN, NT, kFirstB> lb;
         lb.init(static_cast<const uint8_t*>(p.b) + g * w_elems, p.ldb, w_elems, n_t * BN, static_cast<int>(p.n),
                 p.b_scale + g * scale_blocks, scale_ld, tid);
-        compute_tile<Cfg>(smem, la, lb, m_t * BM, rows, n_t * BN, static_cast<int>(p.n), con, c + s * p.ldc, p.ldc, p.ablate);
+        compute_tile<Cfg>(smem, la, lb, m_t * BM, rows, n_t * BN, static_cast<int>(p.n), con, c + s * p.ldc, p.ldc);
       }
     }
   }
 }
 
-// ------------------------------------------------------------------------------------------- bf16 kernel, v3
-// Same tile (256 x 256 x 64, 2 x 4 wavefronts of 4 x 2 blocks) and schedule, but the operand tiles go from global
-// memory straight into LDS (buffer_load ... lds, 16 bytes per lane), so there are no staging registers, no ds_write
-// instructions and no register transposes in the loop:
-//  * a contraction-contiguous operand lands as [256 rows][64 con] with the 16-byte chunk index XOR-swizzled by row
-//    (each lane fetches the chunk that belongs in its LDS slot); fragments are one ds_read_b128;
-//  * an output-contiguous operand (B in fwd, both operands in wgrad) lands as it lies in memory, [64 con][256 out],
-//    chunks XOR-swizzled by (con & 3) << 1, and fragments are read with two ds_read_b64_tr_b16, the gfx950 LDS
-//    transpose read: within a group of 16 lanes, lane i supplies the address of row (i >> 2), columns 4 (i & 3)..+3
-//    of a 4 x 16 patch and receives the four rows of column i.
-// The loads of step k+1 are in flight during the whole of step k; the next tile's first step is issued before the
-// epilogue, which stages through the second LDS stage only.
-template <int kI>  // 1 KB instructions per wavefront per tile: 32 / wavefronts
-struct DmaDirect {   // element(out, con) = base[out * ld + con]
-  __amdgpu_buffer_rsrc_t rsrc;
-  uint32_t voff[kI];
-  int con_first[kI];  // contraction index (within a step) of the chunk each instruction's lane fetches
-  int con_lim;
-
-  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
-                                       int con_lim_, int wave, int lane) {
-    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
-    con_lim = con_lim_;
-#pragma unroll
-    for (int t = 0; t < kI; ++t) {
-      const int row = (wave * kI + t) * 8 + (lane >> 3);  // row of the tile this lane's LDS slot belongs to
-      const int logical = (lane & 7) ^ swizzle(row);
-      const int out = out0 + row;
-      con_first[t] = logical << 3;
-      voff[t] = out < out_lim ? static_cast<uint32_t>(out) * static_cast<uint32_t>(ld) * 2u + (logical << 4)
-                              : kOutOfRange;
-    }
-  }
-  // One 4-byte load from line `l` (0..255: output row out0 + l) of a later step, whose only purpose is to pull the
-  // 128-byte line into L2 ahead of the tile load that needs it.  It lands in a scrap area of LDS (`sink`, 256 bytes
-  // per wavefront): a load to LDS ties up no register, so nothing ever has to wait for it.
-  uint32_t pf_off;
-  __device__ __forceinline__ void init_prefetch(int64_t ld, int out0, int out_lim, int l) {
-    const int out = out0 + l;
-    pf_off = out < out_lim ? static_cast<uint32_t>(out) * static_cast<uint32_t>(ld) * 2u : kOutOfRange;
-  }
-  __device__ __forceinline__ void prefetch(__attribute__((address_space(3))) char* sink, int step) const {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, sink, 4, step * BK < con_lim ? pf_off : kOutOfRange,
-                                             static_cast<uint32_t>(step) * (BK * 2), 0, 0);
-  }
-  // `tile` is the byte address in LDS of this operand's tile in the stage being filled
-  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave) const {
-    const uint32_t soff = static_cast<uint32_t>(step) * (BK * 2);
-#pragma unroll
-    for (int t = 0; t < kI; ++t) {
-      const uint32_t off = step * BK + con_first[t] < con_lim ? voff[t] : kOutOfRange;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * kI + t) * 1024, 16, off, soff, 0, 0);
-    }
-  }
-  // fragment for the 32x32x16 MFMA: rows row0 + (lane & 31), contraction kk*16 + 8*(lane>>5) .. +7
-  static __device__ __forceinline__ bf16x8 fragment(const bf16_t* smem, int tile_elems, int row0, int kk, int lane) {
-    return *reinterpret_cast<const bf16x8*>(smem + tile_elems + lds_offset(row0 + (lane & 31), kk * 2 + (lane >> 5)));
-  }
-};
-
-template <int kI>
-struct DmaTransposed {   // element(out, con) = base[con * ld + out]
-  __amdgpu_buffer_rsrc_t rsrc;
-  uint32_t voff[kI];
-  uint32_t step_bytes;
-
-  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
-                                       int con_lim_, int wave, int lane) {
-    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));  // contraction rows past the end lie past the buffer
-    con_lim = con_lim_;
-    step_bytes = BK * static_cast<uint32_t>(ld) * 2u;
-#pragma unroll
-    for (int t = 0; t < kI; ++t) {
-      const int con = (wave * kI + t) * 2 + (lane >> 5);  // two contraction rows of 512 bytes per instruction
-      const int logical = (lane & 31) ^ ((con & 3) << 2);
-      const int out = out0 + (logical << 3);
-      voff[t] = out < out_lim ? static_cast<uint32_t>(con) * static_cast<uint32_t>(ld) * 2u + static_cast<uint32_t>(out) * 2u
-                              : kOutOfRange;
-    }
-  }
-  // line l (0..255): contraction row l >> 2 of the step, 128-byte piece l & 3 of its 512 bytes
-  uint32_t pf_off;
-  int con_lim;
-  __device__ __forceinline__ void init_prefetch(int64_t ld, int out0, int out_lim, int l) {
-    const int out = out0 + ((l & 3) << 6);
-    pf_off = out < out_lim ? static_cast<uint32_t>(l >> 2) * static_cast<uint32_t>(ld) * 2u + static_cast<uint32_t>(out) * 2u
-                           : kOutOfRange;
-  }
-  __device__ __forceinline__ void prefetch(__attribute__((address_space(3))) char* sink, int step) const {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, sink, 4, step * BK < con_lim ? pf_off : kOutOfRange,
-                                             static_cast<uint32_t>(step) * step_bytes, 0, 0);
-  }
-  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave) const {
-    const uint32_t soff = static_cast<uint32_t>(step) * step_bytes;
-#pragma unroll
-    for (int t = 0; t < kI; ++t)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * kI + t) * 1024, 16, voff[t], soff, 0, 0);
-  }
-  static __device__ __forceinline__ bf16x8 fragment(const bf16_t* smem, int tile_elems, int row0, int kk, int lane) {
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    typedef __attribute__((address_space(3))) s16x4* lds_ptr;
-    const int i = lane & 15, g = lane >> 4;
-    const int out = row0 + ((g & 1) << 4) + ((i & 3) << 2);    // first of the four columns this lane points at
-    const int con = kk * 16 + ((g >> 1) << 3) + (i >> 2);        // (con & 3) == (i >> 2) for both reads
-    const int in_row = (((out >> 3) ^ ((con & 3) << 2)) << 3) + (out & 7);
-    const bf16_t* p = smem + tile_elems + con * 256 + in_row;
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * 256));
-    typedef short s16x8 __attribute__((ext_vector_type(8)));
-    const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    return __builtin_bit_cast(bf16x8, both);
-  }
-};
-
-template <int kMode, typename Cfg>
-__global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_v3_kernel(GemmArgs p) {
-  static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
-  constexpr int WM = Cfg::WM, WN = Cfg::WN, BM = Cfg::BM, BN = Cfg::BN;
-  constexpr int kI = 32 / (Cfg::GM * Cfg::GN);
-  using LoaderA = typename std::conditional<kMode == kWgrad, DmaTransposed<kI>, DmaDirect<kI>>::type;
-  using LoaderB = typename std::conditional<kMode == kDgrad, DmaDirect<kI>, DmaTransposed<kI>>::type;
-  extern __shared__ __attribute__((aligned(16))) bf16_t smem[];  // two stages of (A tile, B tile), 32 KB each
-  __shared__ int32_t tile_start[kMode == kWgrad ? 1 : kMaxGroups + 1];
-  constexpr int kTileB = BM * BK;  // elements; both tiles hold 256 * 64 elements whatever their orientation
-  const bf16_t* a = static_cast<const bf16_t*>(p.a);
-  const bf16_t* b = static_cast<const bf16_t*>(p.b);
-  bf16_t* c = static_cast<bf16_t*>(p.c);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int gm = wave / Cfg::GN, gn = wave % Cfg::GN;
-  auto lds = (__attribute__((address_space(3))) char*)smem;
-
-  // ---- tile schedule (as the staged kernel)
-  const int workers = gridDim.x;
-  int64_t total, first, last, stride;
-  int nt = 1, mt_w = 1;
-  int64_t per_group = 1;
-  if constexpr (kMode == kWgrad) {
-    mt_w = static_cast<int>((p.k + BM - 1) / BM);
-    nt = static_cast<int>((p.n + BN - 1) / BN);
-    per_group = static_cast<int64_t>(mt_w) * nt;
-    total = per_group * p.groups;
-    first = blockIdx.x;
-    last = total;
-    stride = workers;
-  } else {
-    build_tile_prefix<BM>(tile_start, p.offs, p.groups, p.total_rows);
-    const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
-    nt = static_cast<int>((out_cols + BN - 1) / BN);
-    total = static_cast<int64_t>(tile_start[p.groups]) * nt;
-    const int xcd = blockIdx.x % kXcds;
-    const int64_t chunk = (total + kXcds - 1) / kXcds;
-    first = xcd * chunk + blockIdx.x / kXcds;
-    last = xcd * chunk + chunk < total ? xcd * chunk + chunk : total;
-    stride = (workers - xcd + kXcds - 1) / kXcds;
-  }
-
-  struct Tile {
-    int a_out0, a_out_lim, b_out0, b_out_lim, con_lim;
-    bf16_t* c_base;
-  };
-  LoaderA la;
-  LoaderB lb;
-  // L2 prefetch: every thread touches one 128-byte line of a later step's operand tiles (wavefronts 0-3 operand A,
-  // 4-7 operand B; with four wavefronts every thread touches one of each).
-  auto pf_sink = lds + 2 * Cfg::kStage * 2 + wave * 256;
-  auto prefetch_line = [&](int step) {
-    if constexpr (Cfg::kThreads == 512) {
-      if (wave >> 2) lb.prefetch(pf_sink, step);
-      else la.prefetch(pf_sink, step);
-    } else {
-      la.prefetch(pf_sink, step);
-      lb.prefetch(pf_sink, step);
-    }
-  };
-  // decode tile t, describe its operands to the loaders and start its first step into stage 0
-  auto begin_tile = [&](int64_t t, Tile& tile) {
-    int g, m_t, n_t;
-    if constexpr (kMode == kWgrad) {
-      g = static_cast<int>(t / per_group);
-      const int r = static_cast<int>(t - g * per_group);
-      n_t = r / mt_w;
-      m_t = r - n_t * mt_w;
-    } else {
-      int lo = 0, hi = p.groups;  // largest g with tile_start[g] * nt <= t
-      while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (static_cast<int64_t>(tile_start[mid]) * nt <= t) lo = mid; else hi = mid;
-      }
-      g = lo;
-      const int mt = tile_start[g + 1] - tile_start[g];
-      const int r = static_cast<int>(t - static_cast<int64_t>(tile_start[g]) * nt);
-      n_t = r / mt;
-      m_t = r - n_t * mt;
-    }
-    int64_t s, e;
-    group_bounds(p.offs, g, p.total_rows, s, e);
-    const int rows = static_cast<int>(e - s);
-    const int64_t w_elems = p.k * p.n;
-    tile.a_out0 = m_t * BM;
-    tile.b_out0 = n_t * BN;
-    if constexpr (kMode == kWgrad) {
-      tile.a_out_lim = static_cast<int>(p.k);
-      tile.b_out_lim = static_cast<int>(p.n);
-      tile.con_lim = rows;
-      tile.c_base = c + static_cast<int64_t>(g) * w_elems;
-      la.init(a + s * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, rows, wave, lane);
-      lb.init(b + s * p.ldb, p.ldb, rows * p.ldb * 2, tile.b_out0, tile.b_out_lim, rows, wave, lane);
-    } else {
-      tile.a_out_lim = rows;
-      tile.b_out_lim = static_cast<int>(kMode == kDgrad ? p.k : p.n);
-      tile.con_lim = static_cast<int>(kMode == kDgrad ? p.n : p.k);
-      tile.c_base = c + s * p.ldc;
-      la.init(a + s * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, rows, tile.con_lim, wave, lane);
-      lb.init(b + g * w_elems, p.ldb, w_elems * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, wave, lane);
-    }
-    if (tile.con_lim > 0) {
-      la.issue(lds, 0, wave);
-      lb.issue(lds + kTileB * 2, 0, wave);
-    }
-    if constexpr (HMOE_PF > 0) {
-      la.init_prefetch(p.lda, tile.a_out0, tile.a_out_lim, tid & 255);
-      lb.init_prefetch(p.ldb, tile.b_out0, tile.b_out_lim, tid & 255);
-#pragma unroll
-      for (int q = 1; q <= HMOE_PF; ++q) prefetch_line(q);
-    }
-  };
-
-  Tile tile;
-  int64_t t = first;
-  if (t < last) begin_tile(t, tile);
-  while (t < last) {
-    f32x16 acc[WM][WN];
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
-#pragma unroll
-      for (int j = 0; j < WN; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-    const int steps = (tile.con_lim + BK - 1) / BK;
-    const int row_a = gm * (WM * 32), row_b = gn * (WN * 32);
-    int live = (tile.a_out_lim - (tile.a_out0 + row_a) + 31) >> 5;
-    live = live < 0 ? 0 : (live > WM ? WM : live);
-    __builtin_amdgcn_s_waitcnt(0);
-    workgroup_barrier();  // step 0 of this tile has landed in stage 0
-
-    auto run = [&](auto full_tag) {
-      constexpr bool kFull = decltype(full_tag)::value;
-      for (int step = 0; step < steps; ++step) {
-        const int cur = step & 1;
-        if (step + 1 < steps && !(HMOE_ABLATE & 1)) {  // the other stage is free since the barrier that ended the previous step
-          la.issue(lds + (cur ^ 1) * (Cfg::kStage * 2), step + 1, wave);
-          lb.issue(lds + (cur ^ 1) * (Cfg::kStage * 2) + kTileB * 2, step + 1, wave);
-        }
-        if constexpr (HMOE_PF > 0) {  // after the tile loads, so that the step's wait can leave it in flight
-          prefetch_line(step + 1 + HMOE_PF);
-        }
-        const int ta = cur * Cfg::kStage, tb = ta + kTileB;
-        // fragments are double-buffered: those of sub-step kk+1 are read while the MFMAs of sub-step kk run
-        bf16x8 fa[2][WM], fb[2][WN];
-        auto read_fragments = [&](int kk, int buf) {
-          if (HMOE_ABLATE & 2) {
-            if (kk > 0 || step > 0) return;
-            kk = 0;
-          }
-#pragma unroll
-          for (int j = 0; j < WN; ++j) fb[buf][j] = LoaderB::fragment(smem, tb, row_b + j * 32, kk, lane);
-#pragma unroll
-          for (int i = 0; i < WM; ++i)
-            if (kFull || i < live) fa[buf][i] = LoaderA::fragment(smem, ta, row_a + i * 32, kk, lane);
-        };
-        read_fragments(0, 0);
-#pragma unroll
-        for (int kk = 0; kk < BK / 16; ++kk) {
-          if (kk + 1 < BK / 16) read_fragments(kk + 1, (kk + 1) & 1);
-#pragma unroll
-          for (int i = 0; i < WM; ++i) {
-            if (kFull || i < live) {
-#pragma unroll
-              for (int j = 0; j < WN; ++j) {
-                if (HMOE_ABLATE & 4) {
-                  asm volatile("" ::"v"(fb[kk & 1][j]), "v"(fa[kk & 1][i]));
-                  continue;
-                }
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[(HMOE_ABLATE & 2) ? 0 : (kk & 1)][j],
-                                                                    fa[(HMOE_ABLATE & 2) ? 0 : (kk & 1)][i], acc[i][j], 0, 0, 0);
-              }
-            }
-          }
-        }
-        if constexpr ((HMOE_ABLATE & 32) != 0) HMOE_WAIT_VM(24);  // timing experiment only: loads run three steps deep
-        else if constexpr (HMOE_PF > 0) HMOE_WAIT_VM(Cfg::kThreads == 512 ? 1 : 2);  // all but the prefetch, the youngest
-        else HMOE_WAIT_VM(0);
-        workgroup_barrier();
-      }
-    };
-    if (live == WM) run(std::true_type{});
-    else run(std::false_type{});
-
-    // both stages are free: start the next tile's first step into stage 0 before this tile's epilogue
-    const Tile done = tile;
-    t += stride;
-    if (t < last) begin_tile(t, tile);
-
-    // epilogue through the second stage: 32 rows at a time per wavefront, whole 16-byte chunks out
-    constexpr int kEpiPitch = WN * 32 + 8;
-    constexpr int kEpiRegion = 32 * kEpiPitch;
-    constexpr int kLanesPerRow = WN * 4;
-    constexpr int kRowsPerPass = 64 / kLanesPerRow;
-    static_assert(kEpiRegion * Cfg::GM * Cfg::GN <= Cfg::kStage, "epilogue staging must fit in one stage");
-    bf16_t* stage = smem + Cfg::kStage + wave * kEpiRegion;
-    const uint32_t stage_addr =
-        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) +
-        static_cast<uint32_t>((Cfg::kStage + wave * kEpiRegion + (lane & 31) * kEpiPitch + ((lane >> 5) << 2)) * 2);
-#pragma unroll
-    for (int i = 0; i < WM; ++i) {
-#pragma unroll
-      for (int j = 0; j < WN; ++j) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          uint2 packed;
-          packed.x = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 0])) |
-                     (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 1])) << 16);
-          packed.y = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 2])) |
-                     (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 3])) << 16);
-          // Written through inline assembly on purpose: before an LDS store it can see, the compiler drains every
-          // direct-to-LDS load in flight (it cannot tell that this region is not their target), which here would
-          // wait for the next tile's first step and for the prefetches.
-          asm volatile("ds_write_b64 %0, %1 offset:%2"
-                       :
-                       : "v"(stage_addr), "v"(packed), "n"((j * 32 + q * 8) * 2)
-                       : "memory");
-        }
-      }
-      __builtin_amdgcn_wave_barrier();  // the region is private to the wavefront, whose LDS accesses stay in order
-#pragma unroll
-      for (int pass = 0; pass < 32 / kRowsPerPass; ++pass) {
-        const int rr = pass * kRowsPerPass + lane / kLanesPerRow;
-        const int cc = (lane % kLanesPerRow) << 3;
-        const int row = done.a_out0 + row_a + i * 32 + rr;
-        const int col = done.b_out0 + row_b + cc;
-        if (row < done.a_out_lim && col < done.b_out_lim && (!(HMOE_ABLATE & 16) || p.ablate == 77)) {
-          const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * kEpiPitch + cc);
-          *reinterpret_cast<u32x4*>(done.c_base + static_cast<int64_t>(row) * p.ldc + col) = v;
-        }
-      }
-      __builtin_amdgcn_wave_barrier();
-    }
-  }
-}
-
-// ------------------------------------------------------------------------------------- bf16 kernel, ring pipeline
-// The same 256 x 256 tile and the same direct-to-LDS loads, but the contraction moves in steps of 32 through a ring of
-// four 32 KB stages, and the loads run three steps ahead of the MFMAs as ONE stream that does not stop at tile
-// boundaries: while a tile's last steps and its epilogue run, the first steps of the workgroup's next tile are already
-// in flight.  A step that misses L2 takes well over a microsecond to arrive; three stages in flight keep 64-96 KB
-// moving per CU, which is what the memory system needs to stream at the rate the MFMAs consume.
-//
-// One barrier per step, in the middle of it: before the barrier a wavefront waits until its own loads of the NEXT
-// stage have landed (s_waitcnt vmcnt(n), n = vector memory instructions it has issued since that stage's loads, so
-// younger loads and the epilogue's stores stay in flight); after the barrier every wavefront's part of the next stage
-// is visible and every wavefront is done with the previous stage, whose slot takes the loads of three steps ahead.
-// The MFMA fragments of the next step's first half are read right after the barrier, under the MFMAs of this step's
-// second half, so the matrix pipe has work across the barrier and across tile boundaries.
-constexpr int RK = 32;                  // contraction per ring stage
-constexpr int kRing = 4;                // stages
-constexpr int kOpTile = 256 * RK;       // elements of one operand tile in a stage (16 KB)
-constexpr int kSlot = 2 * kOpTile;      // elements per stage: A tile then B tile
-
-// element(out, con) = base[out * ld + con].  LDS tile: [256 out][32 con], 64-byte rows, the 16-byte chunk index
-// XOR-ed with (row >> 2) & 3 so that 16 lanes reading one chunk column of 16 rows cover all 64 banks.
-// One instruction moves 16 rows x 64 bytes; a wavefront issues kI of them per step.
-template <int kI>
-struct RingDirect {
-  __amdgpu_buffer_rsrc_t rsrc;  // bounded at the operand's last output row: rows past it load as zeros
-  uint32_t voff[kI];            // byte offset of this lane's chunk per instruction at step 0 (16 rows apart)
-  int con0;                     // contraction index within a step of this lane's chunk
-  int con_lim;
-
-  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
-                                       int con_lim_, int wave, int lane) {
-    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
-    con_lim = con_lim_;
-    const int logical = (lane & 3) ^ ((lane >> 4) & 3);  // (row >> 2) & 3 == (lane >> 4) & 3 for every instruction
-    con0 = logical << 3;
-#pragma unroll
-    for (int t = 0; t < kI; ++t) {
-      const int out = out0 + (wave * kI + t) * 16 + (lane >> 2);
-      voff[t] = out < out_lim ? static_cast<uint32_t>(out) * static_cast<uint32_t>(ld) * 2u + (logical << 4)
-                              : kOutOfRange;
-    }
-  }
-  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave) const {
-    const bool in_range = step * RK + con0 < con_lim;
-    const uint32_t soff = static_cast<uint32_t>(step) * (RK * 2);
-#pragma unroll
-    for (int t = 0; t < kI; ++t)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * kI + t) * 1024, 16,
-                                               in_range ? voff[t] : kOutOfRange, soff, 0, 0);
-  }
-  // byte offset within the operand tile of this lane's fragment for sub-step kk of block row `row0`
-  static __device__ __forceinline__ int fragment_offset(int row0, int kk, int lane) {
-    const int r = row0 + (lane & 31);
-    return r * (RK * 2) + ((((kk << 1) + (lane >> 5)) ^ ((r >> 2) & 3)) << 4);
-  }
-  static __device__ __forceinline__ bf16x8 fragment(const char* tile, int offset) {
-    return *reinterpret_cast<const bf16x8*>(tile + offset);
-  }
-};
-
-// element(out, con) = base[con * ld + out].  LDS tile: [32 con][256 out] as it lies in memory, 512-byte rows, chunk
-// index XOR-ed with (con & 3) << 2; fragments come out through the transposing LDS read.  A half-wavefront of that
-// read touches 4 contraction rows x 2 groups of 16 columns (32 bytes each): the XOR spreads the rows 64 bytes apart,
-// the column groups fill the gaps, and the eight pieces cover the 64 banks exactly once.
-// One instruction moves two contraction rows; a wavefront issues kI of them per step.
-template <int kI>
-struct RingTransposed {
-  __amdgpu_buffer_rsrc_t rsrc;  // bounded at the operand's last contraction row
-  uint32_t voff[kI];
-  uint32_t step_bytes;
-
-  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
-                                       int /*con_lim*/, int wave, int lane) {
-    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
-    step_bytes = RK * static_cast<uint32_t>(ld) * 2u;
-#pragma unroll
-    for (int t = 0; t < kI; ++t) {
-      const int con = (wave * kI + t) * 2 + (lane >> 5);
-      const int logical = (lane & 31) ^ ((con & 3) << 2);
-      const int out = out0 + (logical << 3);
-      voff[t] = out < out_lim
-                    ? static_cast<uint32_t>(con) * static_cast<uint32_t>(ld) * 2u + static_cast<uint32_t>(out) * 2u
-                    : kOutOfRange;
-    }
-  }
-  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave) const {
-    const uint32_t soff = static_cast<uint32_t>(step) * step_bytes;
-#pragma unroll
-    for (int t = 0; t < kI; ++t)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * kI + t) * 1024, 16, voff[t], soff, 0, 0);
-  }
-  static __device__ __forceinline__ int fragment_offset(int row0, int kk, int lane) {
-    const int i = lane & 15, g = lane >> 4;
-    const int out = row0 + ((g & 1) << 4) + ((i & 3) << 2);  // first of the four columns this lane points at
-    const int con = kk * 16 + ((g >> 1) << 3) + (i >> 2);     // (con & 3) == (i >> 2) for both reads
-    return (con * 256 + ((((out >> 3) ^ ((con & 3) << 2)) << 3) + (out & 7))) * 2;
-  }
-  static __device__ __forceinline__ bf16x8 fragment(const char* tile, int offset) {
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    typedef __attribute__((address_space(3))) s16x4* lds_ptr;
-    const char* p = tile + offset;
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * 256 * 2));
-    typedef short s16x8 __attribute__((ext_vector_type(8)));
-    const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    return __builtin_bit_cast(bf16x8, both);
-  }
-};
-
-// wait until at most `n` of this wavefront's vector memory instructions are outstanding (rounded down to a value
-// that has an encoding here: waiting for more than asked is always safe)
-__device__ __forceinline__ void wait_vm_at_most(int n, int steady) {
-  if (n == steady) {  // two younger stages in flight and nothing else: every step but the first three of a tile
-    if (steady == 8) HMOE_WAIT_VM(8);
-    else HMOE_WAIT_VM(16);
-  } else if (n >= 48) HMOE_WAIT_VM(48);
-  else if (n >= 40) HMOE_WAIT_VM(40);
-  else if (n >= 32) HMOE_WAIT_VM(32);
-  else if (n >= 24) HMOE_WAIT_VM(24);
-  else if (n >= 20) HMOE_WAIT_VM(20);
-  else if (n >= 16) HMOE_WAIT_VM(16);
-  else if (n >= 12) HMOE_WAIT_VM(12);
-  else if (n >= 8) HMOE_WAIT_VM(8);
-  else if (n >= 4) HMOE_WAIT_VM(4);
-  else HMOE_WAIT_VM(0);
-}
-
-template <typename Cfg>
-struct RingLayout {
-  static constexpr int kWaves = Cfg::GM * Cfg::GN;
-  static constexpr int kEpiPitch = Cfg::WN * 32 + 8;       // elements; the 16 bytes of padding stagger the banks
-  static constexpr int kEpiRegion = 16 * kEpiPitch;        // elements per wavefront: 16 rows of its tile
-  static constexpr size_t kRingBytes = size_t(kRing) * kSlot * sizeof(bf16_t);
-  static constexpr size_t kStagingBytes = size_t(kWaves) * kEpiRegion * sizeof(bf16_t);
-  static size_t bytes(int groups) { return kRingBytes + kStagingBytes + size_t(3 * groups + 1) * sizeof(int32_t); }
-};
-
-struct RingTile {
+// ---------------------------------------------------------------------------------------------- tile schedule
+struct TileInfo {
   int g, a_out0, a_out_lim, b_out0, b_out_lim, con_lim, row_start;
 };
 
 // The tile walk of one workgroup.  Tile ids only grow along the walk, so the group of a tile is found by scanning on
 // from the previous tile's group.  Everything here is uniform across the workgroup and kept in scalar registers.
 template <int kMode, int BM, int BN>
-struct RingSchedule {
+struct TileSchedule {
   const int32_t* grp_s;
   const int32_t* grp_e;
   const int32_t* tile_start;
@@ -1081,7 +597,7 @@ struct RingSchedule {
     }
   }
 
-  __device__ __forceinline__ RingTile decode(int64_t t, int& cursor) const {
+  __device__ __forceinline__ TileInfo decode(int64_t t, int& cursor) const {
     int g, m_t, n_t;
     if constexpr (kMode == kWgrad) {
       g = static_cast<int>(t / per_group);
@@ -1100,7 +616,7 @@ struct RingSchedule {
     }
     const int s = __builtin_amdgcn_readfirstlane(grp_s[g]);
     const int rows = __builtin_amdgcn_readfirstlane(grp_e[g]) - s;
-    RingTile tile;
+    TileInfo tile;
     tile.g = g;
     tile.row_start = s;
     tile.a_out0 = m_t * BM;
@@ -1118,98 +634,140 @@ struct RingSchedule {
   }
 };
 
-// The load stream: (tile, step) after (tile, step) into the ring's slots, up to three steps ahead of the MFMAs.
-// `issued` counts the vector memory instructions of this wavefront (the epilogue adds its stores); seq0..2 hold its
-// value right after the loads of the stages in flight, oldest first, which is what the vmcnt waits are made from.
-template <int kMode, typename Sched, typename LoaderA, typename LoaderB, int kI>
-struct RingProducer {
-  LoaderA la;
-  LoaderB lb;
-  int64_t pt;
-  int cursor, step, steps, slot;
-  bool open;
-  int issued, seq0, seq1, seq2, in_flight;
+// ------------------------------------------------------------------------------- bf16 kernel, direct to LDS
 
-  __device__ __forceinline__ void init(const Sched& sched) {
-    pt = sched.first;
-    cursor = 0;
-    step = steps = slot = 0;
-    open = false;
-    issued = seq0 = seq1 = seq2 = in_flight = 0;
+template <int kI>
+struct SlimDirect {  // element(out, con) = base[out * ld + con]; LDS [256 out][64 con], chunk ^= row & 7
+  __amdgpu_buffer_rsrc_t rsrc;  // bounded at the operand's last output row: rows past it load as zeros
+  uint32_t voff;                // this lane's chunk for the wavefront's first load of a step, at step 0
+  uint32_t t_stride;            // bytes between the rows of consecutive loads (8 rows)
+  int con0, con_lim;
+
+  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int /*out_lim*/,
+                                       int con_lim_, int wave, int lane) {
+    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
+    con_lim = con_lim_;
+    const int logical = (lane & 7) ^ (lane >> 3);  // row & 7 == lane >> 3 for every load
+    con0 = logical << 3;
+    t_stride = 8u * static_cast<uint32_t>(ld) * 2u;
+    voff = static_cast<uint32_t>(out0 + wave * kI * 8 + (lane >> 3)) * static_cast<uint32_t>(ld) * 2u + (logical << 4);
   }
-  // position the stream on the next tile that has a contraction to load
-  __device__ __forceinline__ void open_next(const Sched& sched, const GemmArgs& p, int wave, int lane) {
-    const bf16_t* a = static_cast<const bf16_t*>(p.a);
-    const bf16_t* b = static_cast<const bf16_t*>(p.b);
-    open = false;
-    while (pt < sched.last) {
-      const RingTile tile = sched.decode(pt, cursor);
-      if (tile.con_lim > 0) {
-        if constexpr (kMode == kWgrad) {
-          const int64_t rows = tile.con_lim;
-          la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim, wave,
-                  lane);
-          lb.init(b + tile.row_start * p.ldb, p.ldb, rows * p.ldb * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, wave,
-                  lane);
-        } else {
-          const int64_t rows = tile.a_out_lim;
-          const int64_t w_elems = p.k * p.n;
-          la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim, wave,
-                  lane);
-          lb.init(b + tile.g * w_elems, p.ldb, w_elems * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, wave, lane);
-        }
-        step = 0;
-        steps = (tile.con_lim + RK - 1) / RK;
-        open = true;
-        return;
-      }
-      pt += sched.stride;
-    }
+  // `live` false: the step lies past the contraction; the loads still issue (the schedule of the loop does not
+  // change) but every offset is out of range, and the step offset stays below the buffer's size
+  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave,
+                                        bool live = true) const {
+    const uint32_t soff = live ? static_cast<uint32_t>(step) * (BK * 2) : 0u;
+    const uint32_t base = live && step * BK + con0 < con_lim ? voff : kOutOfRange;
+#pragma unroll
+    for (int t = 0; t < kI; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * kI + t) * 1024, 16, base + t * t_stride, soff, 0,
+                                               0);
   }
-  __device__ __forceinline__ void produce(const Sched& sched, const GemmArgs& p,
-                                          __attribute__((address_space(3))) char* lds, int wave, int lane) {
-    if (!open) return;
-    auto dst = lds + slot * (kSlot * 2);
-    if (!(HMOE_ABLATE & 1)) {
-      la.issue(dst, step, wave);
-      lb.issue(dst + kOpTile * 2, step, wave);
-      issued += 2 * kI;
-    }
-    if (in_flight == 0) seq0 = issued;
-    else if (in_flight == 1) seq1 = issued;
-    else seq2 = issued;
-    ++in_flight;
-    slot = (slot + 1) & (kRing - 1);
-    if (++step == steps) {
-      pt += sched.stride;
-      open_next(sched, p, wave, lane);
-    }
+  // per-lane byte address (within the operand tile) of the fragment of sub-step 0, block 0 of the wavefront
+  static __device__ __forceinline__ int fragment_base(int row0, int lane) {
+    return (row0 + (lane & 31)) * (BK * 2) + (((lane >> 5) ^ (lane & 7)) << 4);
   }
-  // wait for this wavefront's loads of the oldest stage in flight and retire it from the queue
-  __device__ __forceinline__ void await_oldest() {
-    wait_vm_at_most(issued - seq0, 4 * kI);
-    seq0 = seq1;
-    seq1 = seq2;
-    --in_flight;
+  // block b (32 rows further) and sub-step kk from there
+  static __device__ __forceinline__ bf16x8 fragment(const char* tile, int base, int block, int kk) {
+    return *reinterpret_cast<const bf16x8*>(tile + (base ^ (kk << 5)) + block * (32 * BK * 2));
   }
 };
 
+template <int kI>
+struct SlimTransposed {  // element(out, con) = base[con * ld + out]; LDS [64 con][256 out], chunk ^= (con & 3) << 2
+  __amdgpu_buffer_rsrc_t rsrc;  // bounded at the operand's last contraction row
+  uint32_t voff[2];             // even and odd loads of a step differ in (con & 3); pairs are 4 contraction rows apart
+  uint32_t pair_stride, step_bytes;
+
+  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
+                                       int /*con_lim*/, int wave, int lane) {
+    static_assert(kI % 2 == 0, "loads come in even/odd pairs");
+    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
+    step_bytes = BK * static_cast<uint32_t>(ld) * 2u;
+    pair_stride = 4u * static_cast<uint32_t>(ld) * 2u;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int con = (wave * kI + t) * 2 + (lane >> 5);
+      const int logical = (lane & 31) ^ ((con & 3) << 2);
+      const int out = out0 + (logical << 3);
+      voff[t] = out < out_lim
+                    ? static_cast<uint32_t>(con) * static_cast<uint32_t>(ld) * 2u + static_cast<uint32_t>(out) * 2u
+                    : kOutOfRange;
+    }
+  }
+  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave,
+                                        bool live = true) const {
+    const uint32_t soff = live ? static_cast<uint32_t>(step) * step_bytes : 0u;
+    const uint32_t v0 = live ? voff[0] : kOutOfRange, v1 = live ? voff[1] : kOutOfRange;
+#pragma unroll
+    for (int t = 0; t < kI; ++t)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * kI + t) * 1024, 16,
+                                               ((t & 1) ? v1 : v0) + (t >> 1) * pair_stride, soff, 0, 0);
+  }
+  // per-lane byte address of the fragment of sub-step 0 for block `block` of the wavefront (blocks do not reduce to
+  // an immediate: the XOR reaches the bits the block index occupies)
+  static __device__ __forceinline__ int fragment_base(int row0, int lane) {
+    const int i = lane & 15, g = lane >> 4;
+    const int out = row0 + ((g & 1) << 4) + ((i & 3) << 2);
+    const int con = ((g >> 1) << 3) + (i >> 2);
+    return (con * 256 + ((((out >> 3) ^ ((con & 3) << 2)) << 3) + (out & 7))) * 2;
+  }
+  static __device__ __forceinline__ bf16x8 fragment(const char* tile, int base, int /*block*/, int kk) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+    const char* ptr = tile + base + kk * (16 * 256 * 2);
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(ptr));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(ptr + 4 * 256 * 2));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(bf16x8, both);
+  }
+};
+
+// Scheduling hint for a region of kReads LDS reads and kMfmas MFMAs: spread the reads evenly under the MFMAs.
+template <int kReads, int kMfmas, int kLoads = 0>
+__device__ __forceinline__ void interleave_reads_under_mfmas() {
+  if constexpr (kLoads > 0 && kLoads <= kMfmas && kReads <= kMfmas) {
+    // one global->LDS load behind each of the first MFMAs, LDS reads behind every (kMfmas / kReads)-th
+    constexpr int every = kMfmas / kReads;
+#pragma unroll
+    for (int m = 0; m < kMfmas; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (m < kLoads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      if (m % every == every - 1 && m / every < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+  } else if constexpr (kReads <= kMfmas) {
+    constexpr int per = kMfmas / kReads;
+#pragma unroll
+    for (int r = 0; r < kReads; ++r) {
+      __builtin_amdgcn_sched_group_barrier(0x008, per, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    if constexpr (kMfmas - per * kReads > 0) __builtin_amdgcn_sched_group_barrier(0x008, kMfmas - per * kReads, 0);
+  } else {
+    constexpr int per = (kReads + kMfmas - 1) / kMfmas;
+#pragma unroll
+    for (int m = 0; m < kMfmas; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, per, 0);
+    }
+  }
+}
+
 template <int kMode, typename Cfg>
-__global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_ring_kernel(GemmArgs p) {
+__global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmArgs p) {
   static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
-  using L = RingLayout<Cfg>;
   constexpr int WM = Cfg::WM, WN = Cfg::WN, BM = Cfg::BM, BN = Cfg::BN;
-  constexpr int kI = 16 / L::kWaves;  // 1 KB load instructions per wavefront per operand per step
-  constexpr int kStoresPerBlockRow = 2 * (16 * WN * 32 * 2 / 1024);  // two halves of 16 rows, 1 KB per instruction
-  using LoaderA = typename std::conditional<kMode == kWgrad, RingTransposed<kI>, RingDirect<kI>>::type;
-  using LoaderB = typename std::conditional<kMode == kDgrad, RingDirect<kI>, RingTransposed<kI>>::type;
-  using Sched = RingSchedule<kMode, BM, BN>;
-  extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+  constexpr int kWaves = Cfg::GM * Cfg::GN;
+  constexpr int kI = 32 / kWaves;
+  constexpr bool kDirectA = kMode != kWgrad, kDirectB = kMode == kDgrad;
+  using LoaderA = typename std::conditional<kDirectA, SlimDirect<kI>, SlimTransposed<kI>>::type;
+  using LoaderB = typename std::conditional<kDirectB, SlimDirect<kI>, SlimTransposed<kI>>::type;
+  using Sched = TileSchedule<kMode, BM, BN>;
+  extern __shared__ __attribute__((aligned(16))) char lds_raw[];  // two stages of (A tile, B tile), 32 KB each
+  __shared__ int32_t grp_s[kMaxGroups], grp_e[kMaxGroups], tile_start[kMode == kWgrad ? 1 : kMaxGroups + 1];
   auto lds = (__attribute__((address_space(3))) char*)lds_raw;
-  bf16_t* staging_all = reinterpret_cast<bf16_t*>(lds_raw + L::kRingBytes);
-  int32_t* grp_s = reinterpret_cast<int32_t*>(lds_raw + L::kRingBytes + L::kStagingBytes);
-  int32_t* grp_e = grp_s + p.groups;
-  int32_t* tile_start = grp_e + p.groups;  // [groups + 1], fwd and dgrad only
+  constexpr int kTileBytes = 256 * BK * 2, kStageBytes = 2 * kTileBytes;
   bf16_t* c = static_cast<bf16_t*>(p.c);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1244,57 +802,68 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_ring_kernel(GemmAr
     }
   }
   __syncthreads();
-
   Sched sched;
   sched.init(p, grp_s, grp_e, tile_start);
-  RingProducer<kMode, Sched, LoaderA, LoaderB, kI> prod;
-  prod.init(sched);
   const int64_t w_elems = p.k * p.n;
 
-  // ---- fragment addresses (bytes within an operand tile); block rows are 32 output rows apart
-  int fa_off[2], fb_off[2][WN];
-#pragma unroll
-  for (int kk = 0; kk < 2; ++kk) {
-    fa_off[kk] = LoaderA::fragment_offset(row_a, kk, lane);
-#pragma unroll
-    for (int j = 0; j < WN; ++j) fb_off[kk][j] = LoaderB::fragment_offset(row_b + j * 32, kk, lane);
-  }
-  constexpr int kBlockRowBytesA = std::is_same<LoaderA, RingDirect<kI>>::value ? 32 * RK * 2 : 0;
-  bf16x8 fa[2][WM], fb[2][WN];
-  int ablate_reads = 0;
-  auto read_fragments = [&](int slot, int kk) __attribute__((always_inline)) {
-    if ((HMOE_ABLATE & 2) && ablate_reads++ >= 2) return;
-    const char* ta = lds_raw + slot * (kSlot * 2);
-    const char* tb = ta + kOpTile * 2;
-#pragma unroll
-    for (int j = 0; j < WN; ++j) fb[kk][j] = LoaderB::fragment(tb, fb_off[kk][j]);
-#pragma unroll
-    for (int i = 0; i < WM; ++i) {
-      if constexpr (kBlockRowBytesA != 0) fa[kk][i] = LoaderA::fragment(ta, fa_off[kk] + i * kBlockRowBytesA);
-      else fa[kk][i] = LoaderA::fragment(ta, LoaderA::fragment_offset(row_a + i * 32, kk, lane));
+  LoaderA la;
+  LoaderB lb;
+  int cursor = 0;
+  // describe tile `t`'s operands to the loaders and start its first step into stage 0
+  auto begin_tile = [&](int64_t t) __attribute__((always_inline)) -> TileInfo {
+    const TileInfo tile = sched.decode(t, cursor);
+    const bf16_t* a = static_cast<const bf16_t*>(p.a);
+    const bf16_t* b = static_cast<const bf16_t*>(p.b);
+    if constexpr (kMode == kWgrad) {
+      const int64_t rows = tile.con_lim;
+      la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim, wave, lane);
+      lb.init(b + tile.row_start * p.ldb, p.ldb, rows * p.ldb * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, wave, lane);
+    } else {
+      const int64_t rows = tile.a_out_lim;
+      la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim, wave, lane);
+      lb.init(b + tile.g * w_elems, p.ldb, w_elems * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, wave, lane);
     }
+    if (tile.con_lim > 0) {
+      la.issue(lds, 0, wave);
+      lb.issue(lds + kTileBytes, 0, wave);
+    }
+    return tile;
   };
 
-  prod.open_next(sched, p, wave, lane);
-  prod.produce(sched, p, lds, wave, lane);
-  prod.produce(sched, p, lds, wave, lane);
-  prod.produce(sched, p, lds, wave, lane);
-  int c_slot = 0;
-  if (prod.in_flight > 0) {
-    prod.await_oldest();
-    workgroup_barrier();
-    read_fragments(0, 0);
-  }
+  // ---- fragment addresses
+  int fa_base[kDirectA ? 1 : WM], fb_base[kDirectB ? 1 : WN];
+  if constexpr (kDirectA) fa_base[0] = LoaderA::fragment_base(row_a, lane);
+  else
+#pragma unroll
+    for (int i = 0; i < WM; ++i) fa_base[i] = LoaderA::fragment_base(row_a + i * 32, lane);
+  if constexpr (kDirectB) fb_base[0] = LoaderB::fragment_base(row_b, lane);
+  else
+#pragma unroll
+    for (int j = 0; j < WN; ++j) fb_base[j] = LoaderB::fragment_base(row_b + j * 32, lane);
+  bf16x8 fa[2][WM], fb[2][WN];
+  auto read_fragments = [&](int stage, int kk, int buf) __attribute__((always_inline)) {
+    const char* ta = lds_raw + stage * kStageBytes;
+    const char* tb = ta + kTileBytes;
+#pragma unroll
+    for (int j = 0; j < WN; ++j) fb[buf][j] = LoaderB::fragment(tb, fb_base[kDirectB ? 0 : j], j, kk);
+#pragma unroll
+    for (int i = 0; i < WM; ++i) fa[buf][i] = LoaderA::fragment(ta, fa_base[kDirectA ? 0 : i], i, kk);
+  };
+  constexpr int kReads = WM * (kDirectA ? 1 : 2) + WN * (kDirectB ? 1 : 2);  // LDS reads of one sub-step
+  constexpr int kMfmas = WM * WN;
+  constexpr int kEpiPitch = WN * 32 + 8;
+  constexpr int kEpiRegion = 32 * kEpiPitch;
+  constexpr int kLanesPerRow = WN * 4;
+  constexpr int kRowsPerPass = 64 / kLanesPerRow;
+  static_assert(kEpiRegion * kWaves * 2 <= kStageBytes, "epilogue staging must fit in one stage");
+  const char* stage_rows = lds_raw + kStageBytes + wave * kEpiRegion * 2;
+  const uint32_t stage_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + kStageBytes +
+                              static_cast<uint32_t>((wave * kEpiRegion + (lane & 31) * kEpiPitch + ((lane >> 5) << 2)) * 2);
 
-  bf16_t* staging = staging_all + wave * L::kEpiRegion;
-  // LDS byte address of this lane's 8-byte slot in its staging row (block column and quad added as offsets)
-  const uint32_t staging_addr =
-      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds_raw)) +
-      static_cast<uint32_t>(L::kRingBytes) +
-      static_cast<uint32_t>((wave * L::kEpiRegion + (lane & 15) * L::kEpiPitch + ((lane >> 5) << 2)) * 2);
-  int c_cursor = 0;
-  for (int64_t ct = sched.first; ct < sched.last; ct += sched.stride) {
-    const RingTile tile = sched.decode(ct, c_cursor);
+  int64_t t = sched.first;
+  TileInfo tile;
+  if (t < sched.last) tile = begin_tile(t);
+  while (t < sched.last) {
     f32x16 acc[WM][WN];
 #pragma unroll
     for (int i = 0; i < WM; ++i)
@@ -1302,110 +871,108 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_ring_kernel(GemmAr
       for (int j = 0; j < WN; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-    const int steps = (tile.con_lim + RK - 1) / RK;
+    const int steps = (tile.con_lim + BK - 1) / BK;
     int live = (tile.a_out_lim - (tile.a_out0 + row_a) + 31) >> 5;
     live = live < 0 ? 0 : (live > WM ? WM : live);
+    HMOE_WAIT_VM(0);
+    workgroup_barrier();  // step 0 of this tile has landed in stage 0
+    if (steps > 0) read_fragments(0, 0, 0);
 
     auto run = [&](auto full_tag) __attribute__((always_inline)) {
       constexpr bool kFull = decltype(full_tag)::value;
+      auto mfmas = [&](int buf, int i0, int i1) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = i0; i < i1; ++i) {
+          if (kFull || i < live) {
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+          }
+        }
+      };
       for (int step = 0; step < steps; ++step) {
-        read_fragments(c_slot, 1);
+        const int cur = step & 1;
+        const bool more = step + 1 < steps;
+        // the other stage is free since the barrier inside the previous step; past the last step the loads are
+        // issued all the same, out of range, so that the loop has one shape
+        la.issue(lds + (cur ^ 1) * kStageBytes, step + 1, wave, more);
+        lb.issue(lds + (cur ^ 1) * kStageBytes + kTileBytes, step + 1, wave, more);
 #pragma unroll
-        for (int i = 0; i < WM; ++i) {
-          if (kFull || i < live) {
-#pragma unroll
-            for (int j = 0; j < WN; ++j) {
-              if (HMOE_ABLATE & 4) {
-                asm volatile("" ::"v"(fb[0][j]), "v"(fa[0][i]));
-                continue;
-              }
-              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][j], fa[0][i], acc[i][j], 0, 0, 0);
-            }
+        for (int kk = 0; kk < 3; ++kk) {
+          read_fragments(cur, kk + 1, (kk + 1) & 1);
+          mfmas(kk & 1, 0, WM);
+          if constexpr (kFull) {
+            if (kk == 0) interleave_reads_under_mfmas<kReads, kMfmas, 2 * kI>();
+            else interleave_reads_under_mfmas<kReads, kMfmas>();
           }
         }
-        const int next = (c_slot + 1) & (kRing - 1);
-        const bool more = prod.in_flight > 0;  // a further step (of this tile or the next) is on its way
-        if (more) prod.await_oldest();
-        if (!(HMOE_ABLATE & 8)) workgroup_barrier();  // the next stage is complete and visible; the previous stage's slot is free
-        // the matrix pipe gets work first; the loads three steps ahead and the next fragments go out under it
-#pragma unroll
-        for (int i = 0; i < WM; ++i) {
-          if (i == WM / 2) {
-            __builtin_amdgcn_sched_barrier(0);
-            prod.produce(sched, p, lds, wave, lane);
-            if (more) read_fragments(next, 0);
-            __builtin_amdgcn_sched_barrier(0);
-          }
-          if (kFull || i < live) {
-#pragma unroll
-            for (int j = 0; j < WN; ++j) {
-              if (HMOE_ABLATE & 4) {
-                asm volatile("" ::"v"(fb[1][j]), "v"(fa[1][i]));
-                continue;
-              }
-              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
-            }
-          }
-        }
-        c_slot = next;
+        mfmas(1, 0, WM / 2);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): the next step has landed; lgkmcnt(0): this stage is read out
+        workgroup_barrier();
+        if (more) read_fragments(cur ^ 1, 0, 0);
+        mfmas(1, WM / 2, WM);
+        if constexpr (kFull) interleave_reads_under_mfmas<kReads, kMfmas / 2>();
       }
     };
     if (live == WM) run(std::true_type{});
     else run(std::false_type{});
 
-    // ---- epilogue: 16 rows of the wavefront's tile at a time through its private staging rows, 16-byte chunks out
-    // through buffer stores whose offsets are forced out of range where the tile hangs over the output's edge, so
-    // the number of store instructions is known (the vmcnt arithmetic counts them).
-    constexpr int kLanesPerRow = WN * 4;
-    constexpr int kRowsPerPass = 64 / kLanesPerRow;
-    bf16_t* c_base = kMode == kWgrad ? c + tile.g * w_elems : c + tile.row_start * p.ldc;
-    const int64_t c_rows = kMode == kWgrad ? p.k : tile.a_out_lim;
+    // both stages are free: start the next tile's first step into stage 0 before this tile's epilogue
+    const TileInfo done = tile;
+    t += sched.stride;
+    if (t < sched.last) tile = begin_tile(t);
+
+    // epilogue through the second stage: 32 rows at a time per wavefront, whole 16-byte chunks out
+    bf16_t* c_base = kMode == kWgrad ? c + done.g * w_elems : c + done.row_start * p.ldc;
+    const int64_t c_rows = kMode == kWgrad ? p.k : done.a_out_lim;
     const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(c_base, static_cast<uint32_t>(c_rows * p.ldc * 2));
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
       if (i < live) {
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          if (((lane >> 4) & 1) == half) {
+        for (int j = 0; j < WN; ++j) {
 #pragma unroll
-            for (int j = 0; j < WN; ++j) {
-#pragma unroll
-              for (int q = 0; q < 4; ++q) {
-                uint2 packed;
-                packed.x = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 0])) |
-                           (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 1])) << 16);
-                packed.y = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 2])) |
-                           (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 3])) << 16);
-                // Written through inline assembly on purpose: for an LDS store the compiler sees, it first drains
-                // every direct-to-LDS load in flight (it cannot tell that the staging rows lie outside the ring),
-                // which would stop the load stream at every tile boundary.
-                asm volatile("ds_write_b64 %0, %1 offset:%2"
-                             :
-                             : "v"(staging_addr), "v"(packed), "n"((j * 32 + q * 8) * 2)
-                             : "memory");
-              }
-            }
+          for (int q = 0; q < 4; ++q) {
+            uint2 packed;
+            packed.x = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 0])) |
+                       (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 1])) << 16);
+            packed.y = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 2])) |
+                       (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 3])) << 16);
+            // Written through inline assembly on purpose: before an LDS store it can see, the compiler drains every
+            // direct-to-LDS load in flight (it cannot tell that these rows are not their target), which here would
+            // wait for the next tile's first step.
+            asm volatile("ds_write_b64 %0, %1 offset:%2"
+                         :
+                         : "v"(stage_addr), "v"(packed), "n"((j * 32 + q * 8) * 2)
+                         : "memory");
           }
-          __builtin_amdgcn_wave_barrier();  // the rows are private to the wavefront, whose LDS accesses stay in order
-#pragma unroll
-          for (int pass = 0; pass < 16 / kRowsPerPass; ++pass) {
-            const int rr = pass * kRowsPerPass + lane / kLanesPerRow;
-            const int cc = (lane % kLanesPerRow) << 3;
-            const int row = tile.a_out0 + row_a + i * 32 + half * 16 + rr;
-            const int col = tile.b_out0 + row_b + cc;
-            const u32x4 v = *reinterpret_cast<const u32x4*>(staging + rr * L::kEpiPitch + cc);
-            const uint32_t off = row < tile.a_out_lim && col < tile.b_out_lim
-                                     ? static_cast<uint32_t>(row) * static_cast<uint32_t>(p.ldc) * 2u + col * 2u
-                                     : kOutOfRange;
-            __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, (HMOE_ABLATE & 16) ? kOutOfRange : off, 0, 0);
-          }
-          __builtin_amdgcn_wave_barrier();
         }
+        __builtin_amdgcn_wave_barrier();  // the rows are private to the wavefront, whose LDS accesses stay in order
+#pragma unroll
+        for (int pass = 0; pass < 32 / kRowsPerPass; ++pass) {
+          const int rr = pass * kRowsPerPass + lane / kLanesPerRow;
+          const int cc = (lane % kLanesPerRow) << 3;
+          const int row = done.a_out0 + row_a + i * 32 + rr;
+          const int col = done.b_out0 + row_b + cc;
+          const u32x4 v = *reinterpret_cast<const u32x4*>(stage_rows + (rr * kEpiPitch + cc) * 2);
+          const uint32_t off = row < done.a_out_lim && col < done.b_out_lim
+                                   ? static_cast<uint32_t>(row) * static_cast<uint32_t>(p.ldc) * 2u + col * 2u
+                                   : kOutOfRange;
+          __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, off, 0, 0);
+        }
+        __builtin_amdgcn_wave_barrier();
       }
     }
-    prod.issued += live * kStoresPerBlockRow;
   }
 }
+
+#define HMOE_BF16_INSTANCE(mode) \
+  template __global__ void grouped_gemm_bf16_kernel<mode, Config<2, 4, 4, 2>>(GemmArgs);
+HMOE_BF16_INSTANCE(kFwd)
+HMOE_BF16_INSTANCE(kDgrad)
+HMOE_BF16_INSTANCE(kWgrad)
+#undef HMOE_BF16_INSTANCE
 
 // ------------------------------------------------------------------------------------------------ fp32 path
 // 64x64 tile, contraction step 16, 256 threads each owning a 4x4 block.  grid.x walks row tiles of every group
@@ -1502,7 +1069,7 @@ int device_cus() {
 }
 
 template <int kMode, typename Cfg>
-int launch_bf16(const GemmArgs& p, int workgroups_per_cu, hipStream_t stream) {
+int launch_staged(const GemmArgs& p, int workgroups_per_cu, hipStream_t stream) {
   // upper bound on the number of tiles, so no more workgroups start than can find work
   const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
   const int64_t nt = (out_cols + Cfg::BN - 1) / Cfg::BN;
@@ -1514,7 +1081,7 @@ int launch_bf16(const GemmArgs& p, int workgroups_per_cu, hipStream_t stream) {
   workers = (workers + kXcds - 1) / kXcds * kXcds;
   if (workers <= 0) return HMOE_OK;
   constexpr size_t lds_bytes = 2 * Cfg::kStage * sizeof(bf16_t);
-  auto kernel = grouped_gemm_bf16_kernel<kMode, Cfg>;
+  auto kernel = grouped_gemm_staged_kernel<kMode, Cfg>;
   if (lds_bytes > 48 * 1024) {
     // raising the dynamic LDS limit is idempotent: racing threads set the same value
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1525,76 +1092,21 @@ int launch_bf16(const GemmArgs& p, int workgroups_per_cu, hipStream_t stream) {
   return HMOE_OK;
 }
 
-int experiment_ablate() {
-  static int v = [] {
-    const char* e = getenv("HMOE_GEMM_ABLATE");
-    return e ? atoi(e) : 0;
-  }();
-  return v;
-}
-
-int experiment_cfg() {
-  static int cfg = [] {
-    const char* v = getenv("HMOE_GEMM_CFG");
-    return v ? atoi(v) : 0;
-  }();
-  return cfg;
-}
-
-// explicit instantiations: the host pass has been seen to drop the stub of an implicitly instantiated one
-#define HMOE_V3_INSTANCE(mode) \
-  template __global__ void grouped_gemm_bf16_v3_kernel<mode, Config<2, 4, 4, 2>>(GemmArgs); \
-  template __global__ void grouped_gemm_bf16_v3_kernel<mode, Config<2, 2, 4, 4>>(GemmArgs);
-HMOE_V3_INSTANCE(kFwd)
-HMOE_V3_INSTANCE(kDgrad)
-HMOE_V3_INSTANCE(kWgrad)
-#undef HMOE_V3_INSTANCE
-
 template <int kMode, typename Cfg>
-int launch_v3(const GemmArgs& p, hipStream_t stream) {
+int launch_direct(const GemmArgs& p, hipStream_t stream) {
   const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
   const int64_t nt = (out_cols + Cfg::BN - 1) / Cfg::BN;
   int64_t bound;
   if (kMode == kWgrad) bound = ((p.k + Cfg::BM - 1) / Cfg::BM) * nt * p.groups;
   else bound = (p.total_rows / Cfg::BM + p.groups) * nt;
   int64_t workers = device_cus();
-  if (const char* v = getenv("HMOE_GEMM_WGS")) workers = atoi(v);
   if (bound < workers) workers = bound;
   workers = (workers + kXcds - 1) / kXcds * kXcds;
   if (workers <= 0) return HMOE_OK;
-  constexpr size_t lds_bytes = 2 * Cfg::kStage * sizeof(bf16_t) + Cfg::GM * Cfg::GN * 256;  // stages, prefetch scrap
-  auto kernel = grouped_gemm_bf16_v3_kernel<kMode, Cfg>;
+  constexpr size_t lds_bytes = 2 * Cfg::kStage * sizeof(bf16_t);
+  auto kernel = grouped_gemm_bf16_kernel<kMode, Cfg>;
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                           static_cast<int>(lds_bytes)) != hipSuccess)
-    return HMOE_LAUNCH_FAILED;
-  kernel<<<dim3(static_cast<unsigned>(workers)), dim3(Cfg::kThreads), lds_bytes, stream>>>(p);
-  return HMOE_OK;
-}
-
-
-#define HMOE_RING_INSTANCE(mode) \
-  template __global__ void grouped_gemm_ring_kernel<mode, Config<2, 4, 4, 2>>(GemmArgs); \
-  template __global__ void grouped_gemm_ring_kernel<mode, Config<2, 2, 4, 4>>(GemmArgs);
-HMOE_RING_INSTANCE(kFwd)
-HMOE_RING_INSTANCE(kDgrad)
-HMOE_RING_INSTANCE(kWgrad)
-#undef HMOE_RING_INSTANCE
-
-template <int kMode, typename Cfg>
-int launch_ring(const GemmArgs& p, hipStream_t stream) {
-  const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
-  const int64_t nt = (out_cols + Cfg::BN - 1) / Cfg::BN;
-  int64_t bound;
-  if (kMode == kWgrad) bound = ((p.k + Cfg::BM - 1) / Cfg::BM) * nt * p.groups;
-  else bound = (p.total_rows / Cfg::BM + p.groups) * nt;
-  int64_t workers = device_cus();
-  if (bound < workers) workers = bound;
-  workers = (workers + kXcds - 1) / kXcds * kXcds;
-  if (workers <= 0) return HMOE_OK;
-  const size_t lds_bytes = RingLayout<Cfg>::bytes(p.groups);
-  auto kernel = grouped_gemm_ring_kernel<kMode, Cfg>;
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                          static_cast<int>(RingLayout<Cfg>::bytes(kMaxGroups))) != hipSuccess)
     return HMOE_LAUNCH_FAILED;
   kernel<<<dim3(static_cast<unsigned>(workers)), dim3(Cfg::kThreads), lds_bytes, stream>>>(p);
   return HMOE_OK;
@@ -1603,30 +1115,10 @@ int launch_ring(const GemmArgs& p, hipStream_t stream) {
 template <int kMode>
 int launch(const GemmArgs& p, int dtype, hipStream_t stream) {
   if (dtype == HMOE_BF16) {
+    using Tile = Config<2, 4, 4, 2>;  // 256 x 256 tile on 8 wavefronts of 4 x 2 blocks
     int rc;
-    if constexpr (kMode != kFwdFp8W) {
-      if (experiment_cfg() == 11 || experiment_cfg() == 12) {
-        if (experiment_cfg() == 11) rc = launch_ring<kMode, Config<2, 4, 4, 2>>(p, stream);
-        else rc = launch_ring<kMode, Config<2, 2, 4, 4>>(p, stream);
-        if (rc) return rc;
-        if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
-        return HMOE_OK;
-      }
-      if (experiment_cfg() == 0 || experiment_cfg() >= 9) {
-        if (experiment_cfg() != 10) rc = launch_v3<kMode, Config<2, 4, 4, 2>>(p, stream);
-        else rc = launch_v3<kMode, Config<2, 2, 4, 4>>(p, stream);
-        if (rc) return rc;
-        if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
-        return HMOE_OK;
-      }
-    }
-    switch (experiment_cfg()) {
-      case 1: rc = launch_bf16<kMode, Config<2, 2, 4, 4>>(p, 1, stream); break;   // 256x256, 4 waves
-      case 2: rc = launch_bf16<kMode, Config<2, 2, 4, 2>>(p, 1, stream); break;   // 256x128, 4 waves
-      case 3: rc = launch_bf16<kMode, Config<2, 2, 2, 2>>(p, 2, stream); break;   // 128x128, 4 waves, 2 WG/CU
-      case 4: rc = launch_bf16<kMode, Config<2, 2, 2, 4>>(p, 1, stream); break;   // 128x256, 4 waves
-      default: rc = launch_bf16<kMode, Config<2, 4, 4, 2>>(p, 1, stream); break;  // 256x256, 8 waves (5)
-    }
+    if constexpr (kMode == kFwdFp8W) rc = launch_staged<kMode, Tile>(p, 1, stream);
+    else rc = launch_direct<kMode, Tile>(p, stream);
     if (rc) return rc;
   } else if constexpr (kMode != kFwdFp8W) {
     if (kMode == kWgrad) {
@@ -1671,7 +1163,7 @@ extern "C" {
 int hmoe_grouped_gemm_fwd(const void* a, int64_t lda, const void* b, const int32_t* offs, int64_t total_rows,
                           int num_groups, int64_t k, int64_t n, int dtype, void* out, int64_t ldo, void* stream) {
   using namespace hmoe;
-  GemmArgs p{a, lda, b, n, out, ldo, offs, total_rows, num_groups, k, n, nullptr, experiment_ablate()};
+  GemmArgs p{a, lda, b, n, out, ldo, offs, total_rows, num_groups, k, n, nullptr};
   if (int rc = validate(p, dtype)) return rc;
   if (total_rows == 0 || n == 0) return HMOE_OK;
   if (!a || !b || !out) return HMOE_INVALID_ARGUMENT;
@@ -1683,7 +1175,7 @@ int hmoe_grouped_gemm_fwd_fp8w(const void* a, int64_t lda, const uint8_t* bq, co
                                const int32_t* offs, int64_t total_rows, int num_groups, int64_t k, int64_t n,
                                void* out, int64_t ldo, void* stream) {
   using namespace hmoe;
-  GemmArgs p{a, lda, bq, n, out, ldo, offs, total_rows, num_groups, k, n, b_scale, experiment_ablate()};
+  GemmArgs p{a, lda, bq, n, out, ldo, offs, total_rows, num_groups, k, n, b_scale};
   if (int rc = validate(p, HMOE_BF16)) return rc;
   if (total_rows == 0 || n == 0) return HMOE_OK;
   if (!a || !bq || !b_scale || !out) return HMOE_INVALID_ARGUMENT;
@@ -1695,7 +1187,7 @@ int hmoe_grouped_gemm_dgrad(const void* grad_out, int64_t ldg, const void* b, co
                             int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype, void* grad_a,
                             int64_t lda, void* stream) {
   using namespace hmoe;
-  GemmArgs p{grad_out, ldg, b, n, grad_a, lda, offs, total_rows, num_groups, k, n, nullptr, experiment_ablate()};
+  GemmArgs p{grad_out, ldg, b, n, grad_a, lda, offs, total_rows, num_groups, k, n, nullptr};
   if (int rc = validate(p, dtype)) return rc;
   if (total_rows == 0 || k == 0) return HMOE_OK;
   if (!grad_out || !b || !grad_a) return HMOE_INVALID_ARGUMENT;
@@ -1707,7 +1199,7 @@ int hmoe_grouped_gemm_wgrad(const void* a, int64_t lda, const void* grad_out, in
                             int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype, void* grad_b,
                             void* stream) {
   using namespace hmoe;
-  GemmArgs p{a, lda, grad_out, ldg, grad_b, n, offs, total_rows, num_groups, k, n, nullptr, experiment_ablate()};
+  GemmArgs p{a, lda, grad_out, ldg, grad_b, n, offs, total_rows, num_groups, k, n, nullptr};
   if (int rc = validate(p, dtype)) return rc;
   if (k == 0 || n == 0) return HMOE_OK;
   if (!grad_b || (total_rows > 0 && (!a || !grad_out))) return HMOE_INVALID_ARGUMENT;
