@@ -759,7 +759,10 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
   constexpr int WM = Cfg::WM, WN = Cfg::WN, BM = Cfg::BM, BN = Cfg::BN;
   constexpr int kWaves = Cfg::GM * Cfg::GN;
-  constexpr int kI = 32 / kWaves;
+  // Wavefronts 0-3 issue all the tile loads and wait for them (16 loads of 1 KB each per step, measured slightly
+  // ahead of dealing them to every wavefront); every wavefront runs the MFMAs.
+  constexpr int kLoadWaves = 4;
+  constexpr int kI = 32 / kLoadWaves;
   constexpr bool kDirectA = kMode != kWgrad, kDirectB = kMode == kDgrad;
   using LoaderA = typename std::conditional<kDirectA, SlimDirect<kI>, SlimTransposed<kI>>::type;
   using LoaderB = typename std::conditional<kDirectB, SlimDirect<kI>, SlimTransposed<kI>>::type;
@@ -773,6 +776,8 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int gm = wave / Cfg::GN, gn = wave % Cfg::GN;
   const int row_a = gm * (WM * 32), row_b = gn * (WN * 32);
+  const bool load_wave = wave < kLoadWaves;
+  const int load_slot = wave & (kLoadWaves - 1);
 
   // ---- group bounds and the row-tile prefix, by wavefront 0
   if (wave == 0) {
@@ -816,16 +821,21 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     const bf16_t* b = static_cast<const bf16_t*>(p.b);
     if constexpr (kMode == kWgrad) {
       const int64_t rows = tile.con_lim;
-      la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim, wave, lane);
-      lb.init(b + tile.row_start * p.ldb, p.ldb, rows * p.ldb * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, wave, lane);
+      la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim,
+              load_slot, lane);
+      lb.init(b + tile.row_start * p.ldb, p.ldb, rows * p.ldb * 2, tile.b_out0, tile.b_out_lim, tile.con_lim,
+              load_slot, lane);
     } else {
       const int64_t rows = tile.a_out_lim;
-      la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim, wave, lane);
-      lb.init(b + tile.g * w_elems, p.ldb, w_elems * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, wave, lane);
+      la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim,
+              load_slot, lane);
+      lb.init(b + tile.g * w_elems, p.ldb, w_elems * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, load_slot, lane);
     }
-    if (tile.con_lim > 0) {
-      la.issue(lds, 0, wave);
-      lb.issue(lds + kTileBytes, 0, wave);
+    if (load_wave) {
+      if (tile.con_lim > 0) {
+        la.issue(lds, 0, load_slot);
+        lb.issue(lds + kTileBytes, 0, load_slot);
+      }
     }
     return tile;
   };
@@ -874,7 +884,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     const int steps = (tile.con_lim + BK - 1) / BK;
     int live = (tile.a_out_lim - (tile.a_out0 + row_a) + 31) >> 5;
     live = live < 0 ? 0 : (live > WM ? WM : live);
-    HMOE_WAIT_VM(0);
+    if (load_wave) HMOE_WAIT_VM(0);
     workgroup_barrier();  // step 0 of this tile has landed in stage 0
     if (steps > 0) read_fragments(0, 0, 0);
 
@@ -895,20 +905,23 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         const bool more = step + 1 < steps;
         // the other stage is free since the barrier inside the previous step; past the last step the loads are
         // issued all the same, out of range, so that the loop has one shape
-        la.issue(lds + (cur ^ 1) * kStageBytes, step + 1, wave, more);
-        lb.issue(lds + (cur ^ 1) * kStageBytes + kTileBytes, step + 1, wave, more);
+        if (load_wave) {
+          la.issue(lds + (cur ^ 1) * kStageBytes, step + 1, load_slot, more);
+          lb.issue(lds + (cur ^ 1) * kStageBytes + kTileBytes, step + 1, load_slot, more);
+        }
 #pragma unroll
         for (int kk = 0; kk < 3; ++kk) {
           read_fragments(cur, kk + 1, (kk + 1) & 1);
           mfmas(kk & 1, 0, WM);
           if constexpr (kFull) {
-            if (kk == 0) interleave_reads_under_mfmas<kReads, kMfmas, 2 * kI>();
-            else interleave_reads_under_mfmas<kReads, kMfmas>();
+            interleave_reads_under_mfmas<kReads, kMfmas>();
           }
         }
         mfmas(1, 0, WM / 2);
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): the next step has landed; lgkmcnt(0): this stage is read out
+        // lgkmcnt(0): this stage is read out; vmcnt(0) where tile loads were issued: the next step has landed
+        if (load_wave) __builtin_amdgcn_s_waitcnt(0x0070);
+        else __builtin_amdgcn_s_waitcnt(0xC07F);
         workgroup_barrier();
         if (more) read_fragments(cur ^ 1, 0, 0);
         mfmas(1, WM / 2, WM);
@@ -965,6 +978,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       }
     }
   }
+  HMOE_WAIT_VM(0);  // no load may land in LDS after the workgroup has given it back
 }
 
 #define HMOE_BF16_INSTANCE(mode) \
