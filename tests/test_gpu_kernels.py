@@ -392,9 +392,12 @@ GEMM_CASES = (
     # counts per group, K, N
     ((7, 33, 0, 1, 64, 0), 128, 96),       # the reference's empty-group roster
     ((0, 0, 0, 0, 105, 0), 128, 96),       # one live expert
-    ((130, 1, 255, 128, 129), 256, 384),   # ragged around the 128-row tile
-    ((300, 0, 45), 2880, 360),             # widths off the tile size (2880 = 22.5 x 128)
+    ((130, 1, 255, 128, 129), 256, 384),   # ragged around half a row tile
+    ((300, 0, 45), 2880, 360),             # widths off the tile size (2880 = 11.25 x 256)
     ((64,) * 16, 512, 1536),
+    ((255, 256, 257, 0, 513, 31), 200, 264),  # ragged around the 256-row tile; K and N off the 64 / 256 steps
+    (tuple((37 * i * i + 11 * i) % 91 for i in range(150)), 320, 256),  # many small and empty groups
+    ((300,) * 36 + (7,), 256, 1024),       # more tiles than workgroups: every workgroup walks several
 )
 
 
