@@ -64,6 +64,26 @@ def _forward(mat_a: torch.Tensor, mat_b: torch.Tensor, offs: torch.Tensor | None
     return out
 
 
+def grouped_wgrad(mat_a: torch.Tensor, grad_output: torch.Tensor, offs: torch.Tensor | None,
+                  groups: int) -> torch.Tensor:
+    """``[groups, K, N]``: ``A[s:e]^T @ dO[s:e]`` per group, contiguous; an empty group's slice is exact zeros."""
+    device = _lib.require_device(mat_a, grad_output, offs)
+    if grad_output.dtype != mat_a.dtype:
+        raise TypeError("grouped_wgrad operands must share a dtype")
+    rows, k = mat_a.shape
+    n = grad_output.shape[1]
+    a = _rows(mat_a)
+    grad_output = _rows(grad_output) if grad_output.numel() else grad_output.new_empty(grad_output.shape)
+    offs32 = _offs_arg(offs, groups)
+    grad_b = torch.empty((groups, k, n), dtype=mat_a.dtype, device=device)
+    if k and n:
+        with _lib.on_device(device):
+            _lib.call("hmoe_grouped_gemm_wgrad", _lib.ptr(a), a.stride(0) if rows else k, _lib.ptr(grad_output),
+                      grad_output.stride(0) if rows else n, _lib.ptr(offs32), rows, groups, k, n,
+                      _lib.dtype_id(mat_a.dtype), _lib.ptr(grad_b), _lib.stream_ptr(device))
+    return grad_b
+
+
 def grouped_mm_grads(mat_a, mat_b, grad_output, offs, needs_a: bool, needs_b: bool):
     """``(grad_a, grad_b)``: ``dO @ B^T`` per group and ``A^T @ dO`` per group (an empty group's weight gradient is
     exact zeros).  ``grad_output`` and the operands must share a dtype.  A broadcast (zero-stride) gradient is
@@ -98,12 +118,7 @@ def grouped_mm_grads(mat_a, mat_b, grad_output, offs, needs_a: bool, needs_b: bo
                               _lib.ptr(offs32), rows, groups, k, n, dtype, _lib.ptr(grad_a), grad_a.stride(0),
                               _lib.stream_ptr(device))
         if needs_b:
-            a = _rows(mat_a)
-            grad_b = torch.empty((groups, k, n), dtype=mat_a.dtype, device=device)
-            if k and n:
-                _lib.call("hmoe_grouped_gemm_wgrad", _lib.ptr(a), a.stride(0) if rows else k, _lib.ptr(grad_output),
-                          grad_output.stride(0) if rows else n, _lib.ptr(offs32), rows, groups, k, n, dtype,
-                          _lib.ptr(grad_b), _lib.stream_ptr(device))
+            grad_b = grouped_wgrad(mat_a, grad_output, offs32, groups)
             if not mat_b.is_contiguous() and mat_b.transpose(-2, -1).is_contiguous():
                 # keep the gradient in the parameter's own layout
                 grad_b = grad_b.transpose(-2, -1).contiguous().transpose(-2, -1)

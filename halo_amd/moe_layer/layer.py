@@ -22,7 +22,7 @@ import torch.nn as nn
 
 from halo_amd.kernels.expert_gemm import expert_gemm
 from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled, resolve_fused_glu_mul
-from halo_amd.kernels.grouped_mm import grouped_mm
+from halo_amd.kernels.grouped_mm import grouped_mm, grouped_wgrad
 from halo_amd.kernels.moe_permute import MoEGatherPermute, MoEWeightedUnpermute, warm_permute_kernels
 from halo_amd.kernels.moe_route_sort import sort_routing_by_expert, warm_route_sort_kernels
 from halo_amd.kernels.router import SOFTMAX_ALL, fused_topk_gate
@@ -31,6 +31,41 @@ from halo_amd.moe_layer.config import EPConfig, MoEFamilySpec
 logger = logging.getLogger(__name__)
 
 ROUTER_TOPK_FIELDS = ("top_k", "num_experts_per_tok", "num_experts_per_token")
+
+
+class _RouterProjection(torch.autograd.Function):
+    """``F.linear(x, weight)`` for the router's logits ``[T, E]`` with the weight gradient on the grouped wgrad kernel.
+
+    Forward and the input gradient are plain dense products on the library GEMM, as in the reference.  The weight
+    gradient ``dlogits^T @ x`` is an ``[E, H]`` output contracted over all T tokens: a handful of output tiles, which
+    leaves a dense GEMM (and one grouped-GEMM group) on a few CUs.  The tokens are cut into ``_SPLITS`` slices that
+    the wgrad kernel takes as groups, one partial ``[E, H]`` each, all CUs busy; the partials are summed in fp32 in a
+    fixed order, so the result stays deterministic."""
+
+    _SPLITS = 32
+    _MIN_TOKENS = 2048
+
+    @staticmethod
+    def forward(ctx, x, weight):
+        ctx.save_for_backward(x, weight)
+        return torch.nn.functional.linear(x, weight)
+
+    @staticmethod
+    def backward(ctx, grad_logits):
+        x, weight = ctx.saved_tensors
+        grad_x = grad_weight = None
+        if ctx.needs_input_grad[0]:
+            grad_x = grad_logits @ weight
+        if ctx.needs_input_grad[1]:
+            tokens = x.shape[0]
+            splits = _RouterProjection._SPLITS
+            if x.dtype == torch.bfloat16 and tokens >= _RouterProjection._MIN_TOKENS and tokens % splits == 0:
+                offs = torch.arange(1, splits + 1, device=x.device, dtype=torch.int32) * (tokens // splits)
+                partial = grouped_wgrad(grad_logits, x, offs, splits)
+                grad_weight = partial.sum(dim=0, dtype=torch.float32).to(weight.dtype)
+            else:
+                grad_weight = grad_logits.t() @ x
+        return grad_x, grad_weight
 
 
 def dense_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
@@ -293,7 +328,7 @@ class EPMoELayerBase(nn.Module, ABC):
         router = getattr(self, self._ROUTER_ATTR)
         x = self._router_input(flat)
         # A plain dense projection with a tiny output ([T, E]): the library GEMM, as in the reference (F.linear).
-        logits = torch.nn.functional.linear(x, router.weight.to(x.dtype))
+        logits = _RouterProjection.apply(x, router.weight.to(x.dtype))
         bias = getattr(router, "bias", None)
         return logits if bias is None else logits + bias.to(logits.dtype)
 

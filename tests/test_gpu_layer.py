@@ -240,3 +240,28 @@ def test_drop_in_for_hf_gpt_oss_block(device):
     got, logits = layer(x.to(device))
     _check("gpt-oss out", got.view(want.shape), want, 1e-4)
     assert logits.shape == (40, 8) and layer._glu_combine_name() == "gptoss"
+
+
+def test_router_projection_gradients_at_a_token_count_that_splits_the_wgrad(device):
+    """The router's weight gradient goes through the grouped wgrad kernel in 32 token slices once there are enough
+    tokens; the layer configurations above are too small to take that path.  Checked against the fp64 product over
+    the same bf16 inputs (BASELINE tolerance), and for run-to-run bit equality."""
+    from halo_amd.moe_layer.layer import _RouterProjection
+
+    tokens, hidden, experts = 4096, 512, 128
+    assert tokens >= _RouterProjection._MIN_TOKENS and tokens % _RouterProjection._SPLITS == 0
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(tokens, hidden, generator=g).bfloat16()
+    w = (torch.randn(experts, hidden, generator=g) * 0.05).bfloat16()
+    dlogits = torch.randn(tokens, experts, generator=g).bfloat16()
+    results = []
+    for _ in range(2):
+        xd, wd = x.to(device).requires_grad_(True), w.to(device).requires_grad_(True)
+        logits = _RouterProjection.apply(xd, wd)
+        logits.backward(dlogits.to(device))
+        results.append((logits.detach(), xd.grad, wd.grad))
+    logits, dx, dw = results[0]
+    _check("logits", logits, x.double() @ w.double().t(), 2e-2)
+    _check("dx", dx, dlogits.double() @ w.double(), 2e-2)
+    _check("dw", dw, dlogits.double().t() @ x.double(), 2e-2)
+    assert all(torch.equal(a, b) for a, b in zip(results[0], results[1]))
