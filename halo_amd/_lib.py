@@ -38,6 +38,8 @@ SIGNATURES = {
     "hmoe_grouped_gemm_fwd": (I, [P, L, P, P, L, I, L, L, I, P, L, P]),
     "hmoe_grouped_gemm_dgrad": (I, [P, L, P, P, L, I, L, L, I, P, L, P]),
     "hmoe_grouped_gemm_wgrad": (I, [P, L, P, L, P, L, I, L, L, I, P, P]),
+    "hmoe_grouped_gemm_fwd_gather": (I, [P, L, L, P, P, P, L, I, L, L, I, P, L, P]),
+    "hmoe_grouped_gemm_wgrad_gather": (I, [P, L, L, P, P, L, P, L, I, L, L, I, P, P]),
     "hmoe_quantize_block_fp8": (I, [P, I, L, L, L, P, P, P]),
     "hmoe_dequantize_block_fp8": (I, [P, P, L, L, L, I, P, P]),
     "hmoe_grouped_gemm_fwd_fp8w": (I, [P, L, P, P, P, L, I, L, L, P, L, P]),

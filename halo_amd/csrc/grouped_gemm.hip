@@ -84,6 +84,8 @@ struct GemmArgs {
   int groups;
   int64_t k, n;
   const float* b_scale;  // kFwdFp8W: [G, ceil(K/128), ceil(N/128)]
+  const int64_t* a_index = nullptr;  // gathered A (fwd, wgrad): logical row r of A is a[a_index[r]]
+  int64_t a_rows = 0;                // rows of the array a_index points into
 };
 
 __device__ __forceinline__ int swizzle(int row) { return (row & 7) ^ ((row >> 3) & 7); }
@@ -121,6 +123,31 @@ __device__ __forceinline__ void workgroup_barrier() {
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
+
+// The same descriptor as four words, for the direct-to-LDS loads below.
+__device__ __forceinline__ u32x4 make_rsrc_words(const void* base, uint32_t bytes) {
+  const uint64_t address = reinterpret_cast<uint64_t>(base);
+  return u32x4{static_cast<uint32_t>(address), static_cast<uint32_t>(address >> 32) & 0xffffu, bytes, 0x00020000u};
+}
+
+typedef __attribute__((address_space(3))) char* lds_bytes_ptr;
+
+// Direct-to-LDS load of 16 bytes per lane: lane L's bytes land at lds_base + 16 L; an offset at or past the
+// descriptor's size loads zeros.  Written through inline assembly on purpose.  The compiler tracks the builtin form
+// as a pending LDS write and drains every load in flight (vmcnt(0)) before the next LDS store and before the next
+// transposing LDS read, which it also takes for a store; in a loop that issues the next step's loads and then reads
+// this step's fragments that serialises the two.  Issued this way the loads are invisible to it, and the kernel
+// waits for them itself (wait_loads) where it needs them.
+__device__ __forceinline__ void lds_load16(u32x4 rsrc, lds_bytes_ptr lds_base, uint32_t voffset, uint32_t soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_base))), "v"(voffset), "s"(rsrc),
+                 "s"(soffset)
+               : "memory");
+}
+
+// every direct-to-LDS load of this wavefront has landed
+__device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // One operand tile's global -> register -> LDS path.  A loader describes the operand (a buffer resource bounded at
 // the operand's end, row stride, first output index of the tile, limits) and moves one contraction step.
@@ -640,14 +667,14 @@ struct TileSchedule {
 
 template <int kI>
 struct SlimDirect {  // element(out, con) = base[out * ld + con]; LDS [256 out][64 con], chunk ^= row & 7
-  __amdgpu_buffer_rsrc_t rsrc;  // bounded at the operand's last output row: rows past it load as zeros
+  u32x4 rsrc;  // bounded at the operand's last output row: rows past it load as zeros
   uint32_t voff;                // this lane's chunk for the wavefront's first load of a step, at step 0
   uint32_t t_stride;            // bytes between the rows of consecutive loads (8 rows)
   int con0, con_lim;
 
   __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int /*out_lim*/,
                                        int con_lim_, int wave, int lane) {
-    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
+    rsrc = make_rsrc_words(base, static_cast<uint32_t>(bytes));
     con_lim = con_lim_;
     const int logical = (lane & 7) ^ (lane >> 3);  // row & 7 == lane >> 3 for every load
     con0 = logical << 3;
@@ -662,8 +689,7 @@ struct SlimDirect {  // element(out, con) = base[out * ld + con]; LDS [256 out][
     const uint32_t base = live && step * BK + con0 < con_lim ? voff : kOutOfRange;
 #pragma unroll
     for (int t = 0; t < kI; ++t)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * kI + t) * 1024, 16, base + t * t_stride, soff, 0,
-                                               0);
+      lds_load16(rsrc, tile + (wave * kI + t) * 1024, base + t * t_stride, soff);
   }
   // per-lane byte address (within the operand tile) of the fragment of sub-step 0, block 0 of the wavefront
   static __device__ __forceinline__ int fragment_base(int row0, int lane) {
@@ -677,14 +703,14 @@ struct SlimDirect {  // element(out, con) = base[out * ld + con]; LDS [256 out][
 
 template <int kI>
 struct SlimTransposed {  // element(out, con) = base[con * ld + out]; LDS [64 con][256 out], chunk ^= (con & 3) << 2
-  __amdgpu_buffer_rsrc_t rsrc;  // bounded at the operand's last contraction row
+  u32x4 rsrc;  // bounded at the operand's last contraction row
   uint32_t voff[2];             // even and odd loads of a step differ in (con & 3); pairs are 4 contraction rows apart
   uint32_t pair_stride, step_bytes;
 
   __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
                                        int /*con_lim*/, int wave, int lane) {
     static_assert(kI % 2 == 0, "loads come in even/odd pairs");
-    rsrc = make_rsrc(base, static_cast<uint32_t>(bytes));
+    rsrc = make_rsrc_words(base, static_cast<uint32_t>(bytes));
     step_bytes = BK * static_cast<uint32_t>(ld) * 2u;
     pair_stride = 4u * static_cast<uint32_t>(ld) * 2u;
 #pragma unroll
@@ -703,8 +729,7 @@ struct SlimTransposed {  // element(out, con) = base[con * ld + out]; LDS [64 co
     const uint32_t v0 = live ? voff[0] : kOutOfRange, v1 = live ? voff[1] : kOutOfRange;
 #pragma unroll
     for (int t = 0; t < kI; ++t)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, tile + (wave * kI + t) * 1024, 16,
-                                               ((t & 1) ? v1 : v0) + (t >> 1) * pair_stride, soff, 0, 0);
+      lds_load16(rsrc, tile + (wave * kI + t) * 1024, ((t & 1) ? v1 : v0) + (t >> 1) * pair_stride, soff);
   }
   // per-lane byte address of the fragment of sub-step 0 for block `block` of the wavefront (blocks do not reduce to
   // an immediate: the XOR reaches the bits the block index occupies)
@@ -723,6 +748,116 @@ struct SlimTransposed {  // element(out, con) = base[con * ld + out]; LDS [64 co
     typedef short s16x8 __attribute__((ext_vector_type(8)));
     const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     return __builtin_bit_cast(bf16x8, both);
+  }
+};
+
+// The two loaders again for an operand A whose rows are gathered: logical row r is base[index[r]] (the permute by
+// expert folded into the GEMM: the direct-to-LDS load takes a per-lane offset, so a gathered row costs what a
+// contiguous one does).  An index outside [0, a_rows) loads zeros.
+template <int kI>
+struct GatherDirect {  // LDS layout and fragments as SlimDirect
+  u32x4 rsrc;
+  uint32_t voff[kI];  // per load: this lane's chunk of its row at step 0, or out of range
+  int con0, con_lim;
+
+  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t a_rows, const int64_t* index, int out0,
+                                       int out_lim, int con_lim_, int slot, int lane) {
+    rsrc = make_rsrc_words(base, static_cast<uint32_t>(a_rows * ld * 2));
+    con_lim = con_lim_;
+    const int logical = (lane & 7) ^ (lane >> 3);
+    con0 = logical << 3;
+#pragma unroll
+    for (int t = 0; t < kI; ++t) {
+      const int out = out0 + (slot * kI + t) * 8 + (lane >> 3);
+      const int64_t row = out < out_lim ? index[out] : -1;
+      voff[t] = row >= 0 && row < a_rows ? static_cast<uint32_t>(row) * static_cast<uint32_t>(ld) * 2u + (logical << 4)
+                                         : kOutOfRange;
+    }
+  }
+  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int slot,
+                                        bool live = true) const {
+    const uint32_t soff = live ? static_cast<uint32_t>(step) * (BK * 2) : 0u;
+    const bool in_range = live && step * BK + con0 < con_lim;
+#pragma unroll
+    for (int t = 0; t < kI; ++t)
+      lds_load16(rsrc, tile + (slot * kI + t) * 1024, in_range ? voff[t] : kOutOfRange, soff);
+  }
+  static __device__ __forceinline__ int fragment_base(int row0, int lane) {
+    return SlimDirect<kI>::fragment_base(row0, lane);
+  }
+  static __device__ __forceinline__ bf16x8 fragment(const char* tile, int base, int block, int kk) {
+    return SlimDirect<kI>::fragment(tile, base, block, kk);
+  }
+};
+
+template <int kI>
+struct GatherTransposed {  // LDS layout and fragments as SlimTransposed; the gathered rows are contraction rows
+  u32x4 rsrc;
+  u32x4 index_rsrc;  // the group's row indices, bounded at its last row
+  uint32_t a_rows;
+  uint32_t col[2];       // byte offset of this lane's chunk within a row for even / odd loads, or out of range
+  uint32_t row_bytes;
+  int con_lim;
+  // A wavefront's kI loads of a step cover 2 kI contraction rows, one per half wavefront and load.  Their indices
+  // (low words) are themselves fetched straight into LDS, one step ahead, into the wavefront's own 2 x 1 KB
+  // (by step parity): a load into a register would have to be waited for, and the compiler places that wait right
+  // behind the tile loads just issued.
+  __attribute__((address_space(3))) char* rows_area;
+  int rows_valid0, rows_valid1;  // how many of the 2 kI rows exist, per parity
+
+  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t a_rows_, const int64_t* index, int out0,
+                                       int out_lim, int con_lim_, int slot, int lane) {
+    static_assert(kI % 2 == 0 && 2 * kI <= 64, "loads come in even/odd pairs");
+    rsrc = make_rsrc_words(base, static_cast<uint32_t>(a_rows_ * ld * 2));
+    index_rsrc = make_rsrc_words(index, static_cast<uint32_t>(con_lim_) * 8u);
+    a_rows = static_cast<uint32_t>(a_rows_);
+    row_bytes = static_cast<uint32_t>(ld) * 2u;
+    con_lim = con_lim_;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int con = (slot * kI + u) * 2 + (lane >> 5);
+      const int logical = (lane & 31) ^ ((con & 3) << 2);
+      const int out = out0 + (logical << 3);
+      col[u] = out < out_lim ? static_cast<uint32_t>(out) * 2u : kOutOfRange;
+    }
+  }
+  // fetch the row indices of `step`
+  __device__ __forceinline__ void load_rows(int step, int slot, int lane) {
+    load_rows_of(index_rsrc, con_lim, step, slot, lane);
+  }
+  // the same for a group given by its index buffer and its row count (the next tile's, fetched ahead)
+  __device__ __forceinline__ void load_rows_of(u32x4 group_index, int group_rows, int step, int slot,
+                                               int lane) {
+    const int first = step * BK + slot * (2 * kI);
+    if (step & 1) rows_valid1 = group_rows - first;
+    else rows_valid0 = group_rows - first;
+    // lane l < kI fetches indices first + 2l and first + 2l + 1; rows past the group's end read as 0 and are masked
+    // on use
+    lds_load16(group_index, rows_area + (step & 1) * 1024,
+               first < group_rows && lane < kI ? static_cast<uint32_t>(first + 2 * lane) * 8u : kOutOfRange, 0u);
+  }
+  // the loads of `step`, whose rows load_rows() fetched (and whose arrival the caller has waited for)
+  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int slot,
+                                        bool live = true) const {
+    const int lane = threadIdx.x & 63;
+    const int32_t rows_raw = *reinterpret_cast<const __attribute__((address_space(3))) int32_t*>(
+        rows_area + (step & 1) * 1024 + (lane & (2 * kI - 1)) * 8);  // the low word of index lane % (2 kI)
+    const int valid = (step & 1) ? rows_valid1 : rows_valid0;
+#pragma unroll
+    for (int t = 0; t < kI; ++t) {
+      const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readlane(rows_raw, 2 * t));
+      const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(rows_raw, 2 * t + 1));
+      const bool upper = (lane & 32) != 0;
+      const uint32_t row = upper ? hi : lo;
+      const bool ok = live && 2 * t + (upper ? 1 : 0) < valid && row < a_rows && (col[t & 1] & kOutOfRange) == 0;
+      lds_load16(rsrc, tile + (slot * kI + t) * 1024, ok ? row * row_bytes + col[t & 1] : kOutOfRange, 0u);
+    }
+  }
+  static __device__ __forceinline__ int fragment_base(int row0, int lane) {
+    return SlimTransposed<kI>::fragment_base(row0, lane);
+  }
+  static __device__ __forceinline__ bf16x8 fragment(const char* tile, int base, int block, int kk) {
+    return SlimTransposed<kI>::fragment(tile, base, block, kk);
   }
 };
 
@@ -756,9 +891,10 @@ __device__ __forceinline__ void interleave_reads_under_mfmas() {
   }
 }
 
-template <int kMode, typename Cfg>
+template <int kMode, typename Cfg, bool kGather = false>
 __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmArgs p) {
   static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
+  static_assert(!kGather || kMode == kFwd || kMode == kWgrad, "A is gathered in fwd and wgrad");
   constexpr int WM = Cfg::WM, WN = Cfg::WN, BM = Cfg::BM, BN = Cfg::BN;
   constexpr int kWaves = Cfg::GM * Cfg::GN;
   // Wavefronts 0-3 issue all the tile loads and wait for them (16 loads of 1 KB each per step, measured slightly
@@ -766,8 +902,11 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   constexpr int kLoadWaves = 4;
   constexpr int kI = 32 / kLoadWaves;
   constexpr bool kDirectA = kMode != kWgrad, kDirectB = kMode == kDgrad;
-  using LoaderA = typename std::conditional<kDirectA, SlimDirect<kI>, SlimTransposed<kI>>::type;
+  using PlainA = typename std::conditional<kDirectA, SlimDirect<kI>, SlimTransposed<kI>>::type;
+  using GatheredA = typename std::conditional<kDirectA, GatherDirect<kI>, GatherTransposed<kI>>::type;
+  using LoaderA = typename std::conditional<kGather, GatheredA, PlainA>::type;
   using LoaderB = typename std::conditional<kDirectB, SlimDirect<kI>, SlimTransposed<kI>>::type;
+  constexpr bool kRowsPerStep = kGather && !kDirectA;  // the gathered rows are contraction rows: new ones every step
   using Sched = TileSchedule<kMode, BM, BN>;
   extern __shared__ __attribute__((aligned(16))) char lds_raw[];  // two stages of (A tile, B tile), 32 KB each
   __shared__ int32_t grp_s[kMaxGroups], grp_e[kMaxGroups], tile_start[kMode == kWgrad ? 1 : kMaxGroups + 1];
@@ -815,31 +954,40 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
 
   LoaderA la;
   LoaderB lb;
+  if constexpr (kRowsPerStep) la.rows_area = lds + 2 * kStageBytes + load_slot * 2048;
   int cursor = 0;
   // describe tile `t`'s operands to the loaders and start its first step into stage 0
-  auto begin_tile = [&](int64_t t) __attribute__((always_inline)) -> TileInfo {
-    const TileInfo tile = sched.decode(t, cursor);
+  // `rows0_loaded`: the gathered contraction rows of its step 0 were fetched during the previous tile's last step
+  auto begin_tile = [&](const TileInfo& tile, bool rows0_loaded) __attribute__((always_inline)) {
     const bf16_t* a = static_cast<const bf16_t*>(p.a);
     const bf16_t* b = static_cast<const bf16_t*>(p.b);
-    if constexpr (kMode == kWgrad) {
-      const int64_t rows = tile.con_lim;
+    const int64_t rows = kMode == kWgrad ? tile.con_lim : tile.a_out_lim;
+    if constexpr (kGather) {
+      if (load_wave)  // the row indices are fetched by the lanes that use them
+        la.init(a, p.lda, p.a_rows, p.a_index + tile.row_start, tile.a_out0, tile.a_out_lim, tile.con_lim, load_slot,
+                lane);
+    } else {
       la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim,
               load_slot, lane);
+    }
+    if constexpr (kMode == kWgrad)
       lb.init(b + tile.row_start * p.ldb, p.ldb, rows * p.ldb * 2, tile.b_out0, tile.b_out_lim, tile.con_lim,
               load_slot, lane);
-    } else {
-      const int64_t rows = tile.a_out_lim;
-      la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim,
-              load_slot, lane);
+    else
       lb.init(b + tile.g * w_elems, p.ldb, w_elems * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, load_slot, lane);
-    }
     if (load_wave) {
+      if constexpr (kRowsPerStep) {
+        if (!rows0_loaded) {
+          la.load_rows(0, load_slot, lane);
+          wait_loads();
+        }
+      }
       if (tile.con_lim > 0) {
         la.issue(lds, 0, load_slot);
         lb.issue(lds + kTileBytes, 0, load_slot);
       }
+      if constexpr (kRowsPerStep) la.load_rows(1, load_slot, lane);
     }
-    return tile;
   };
 
   // ---- fragment addresses
@@ -873,9 +1021,15 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
                               static_cast<uint32_t>((wave * kEpiRegion + (lane & 31) * kEpiPitch + ((lane >> 5) << 2)) * 2);
 
   int64_t t = sched.first;
-  TileInfo tile;
-  if (t < sched.last) tile = begin_tile(t);
+  TileInfo tile, next;
+  if (t < sched.last) {
+    tile = sched.decode(t, cursor);
+    begin_tile(tile, false);
+  }
   while (t < sched.last) {
+    const bool has_next = t + sched.stride < sched.last;
+    if (has_next) next = sched.decode(t + sched.stride, cursor);
+    bool next_rows0_loaded = false;
     f32x16 acc[WM][WN];
 #pragma unroll
     for (int i = 0; i < WM; ++i)
@@ -886,7 +1040,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     const int steps = (tile.con_lim + BK - 1) / BK;
     int live = (tile.a_out_lim - (tile.a_out0 + row_a) + 31) >> 5;
     live = live < 0 ? 0 : (live > WM ? WM : live);
-    if (load_wave) HMOE_WAIT_VM(0);
+    if (load_wave) wait_loads();
     workgroup_barrier();  // step 0 of this tile has landed in stage 0
     if (steps > 0) read_fragments(0, 0, 0);
 
@@ -910,7 +1064,16 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         if (load_wave) {
           la.issue(lds + (cur ^ 1) * kStageBytes, step + 1, load_slot, more);
           lb.issue(lds + (cur ^ 1) * kStageBytes + kTileBytes, step + 1, load_slot, more);
+          // the rows of the step after that: their indices arrive under this step, with its tile loads; in the
+          // tile's last step that is the next tile's first
+          if constexpr (kRowsPerStep) {
+            if (more) la.load_rows(step + 2, load_slot, lane);
+            else if (has_next)
+              la.load_rows_of(make_rsrc_words(p.a_index + next.row_start, static_cast<uint32_t>(next.con_lim) * 8u),
+                              next.con_lim, 0, load_slot, lane);
+          }
         }
+        if constexpr (kRowsPerStep) next_rows0_loaded = !more && has_next;
 #pragma unroll
         for (int kk = 0; kk < 3; ++kk) {
           read_fragments(cur, kk + 1, (kk + 1) & 1);
@@ -922,8 +1085,8 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         mfmas(1, 0, WM / 2);
         __builtin_amdgcn_sched_barrier(0);
         // lgkmcnt(0): this stage is read out; vmcnt(0) where tile loads were issued: the next step has landed
-        if (load_wave) __builtin_amdgcn_s_waitcnt(0x0070);
-        else __builtin_amdgcn_s_waitcnt(0xC07F);
+        if (load_wave) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         workgroup_barrier();
         if (more) read_fragments(cur ^ 1, 0, 0);
         mfmas(1, WM / 2, WM);
@@ -936,7 +1099,10 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     // both stages are free: start the next tile's first step into stage 0 before this tile's epilogue
     const TileInfo done = tile;
     t += sched.stride;
-    if (t < sched.last) tile = begin_tile(t);
+    if (has_next) {
+      tile = next;
+      begin_tile(tile, next_rows0_loaded);
+    }
 
     // epilogue through the second stage: 32 rows at a time per wavefront, whole 16-byte chunks out
     bf16_t* c_base = kMode == kWgrad ? c + done.g * w_elems : c + done.row_start * p.ldc;
@@ -980,7 +1146,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       }
     }
   }
-  HMOE_WAIT_VM(0);  // no load may land in LDS after the workgroup has given it back
+  wait_loads();  // no load may land in LDS after the workgroup has given it back
 }
 
 #define HMOE_BF16_INSTANCE(mode) \
@@ -989,6 +1155,8 @@ HMOE_BF16_INSTANCE(kFwd)
 HMOE_BF16_INSTANCE(kDgrad)
 HMOE_BF16_INSTANCE(kWgrad)
 #undef HMOE_BF16_INSTANCE
+template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, true>(GemmArgs);
+template __global__ void grouped_gemm_bf16_kernel<kWgrad, Config<2, 4, 4, 2>, true>(GemmArgs);
 
 // ------------------------------------------------------------------------------------------------ fp32 path
 // 64x64 tile, contraction step 16, 256 threads each owning a 4x4 block.  grid.x walks row tiles of every group
@@ -1108,7 +1276,7 @@ int launch_staged(const GemmArgs& p, int workgroups_per_cu, hipStream_t stream) 
   return HMOE_OK;
 }
 
-template <int kMode, typename Cfg>
+template <int kMode, typename Cfg, bool kGather = false>
 int launch_direct(const GemmArgs& p, hipStream_t stream) {
   const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
   const int64_t nt = (out_cols + Cfg::BN - 1) / Cfg::BN;
@@ -1119,8 +1287,9 @@ int launch_direct(const GemmArgs& p, hipStream_t stream) {
   if (bound < workers) workers = bound;
   workers = (workers + kXcds - 1) / kXcds * kXcds;
   if (workers <= 0) return HMOE_OK;
-  constexpr size_t lds_bytes = 2 * Cfg::kStage * sizeof(bf16_t);
-  auto kernel = grouped_gemm_bf16_kernel<kMode, Cfg>;
+  // two stages; the gathered wgrad keeps 2 x 1 KB of row indices per loading wavefront behind them
+  constexpr size_t lds_bytes = 2 * Cfg::kStage * sizeof(bf16_t) + (kGather && kMode == kWgrad ? 4 * 2048 : 0);
+  auto kernel = grouped_gemm_bf16_kernel<kMode, Cfg, kGather>;
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                           static_cast<int>(lds_bytes)) != hipSuccess)
     return HMOE_LAUNCH_FAILED;
@@ -1133,8 +1302,13 @@ int launch(const GemmArgs& p, int dtype, hipStream_t stream) {
   if (dtype == HMOE_BF16) {
     using Tile = Config<2, 4, 4, 2>;  // 256 x 256 tile on 8 wavefronts of 4 x 2 blocks
     int rc;
-    if constexpr (kMode == kFwdFp8W) rc = launch_staged<kMode, Tile>(p, 1, stream);
-    else rc = launch_direct<kMode, Tile>(p, stream);
+    if constexpr (kMode == kFwdFp8W) {
+      rc = launch_staged<kMode, Tile>(p, 1, stream);
+    } else if constexpr (kMode == kFwd || kMode == kWgrad) {
+      rc = p.a_index ? launch_direct<kMode, Tile, true>(p, stream) : launch_direct<kMode, Tile>(p, stream);
+    } else {
+      rc = launch_direct<kMode, Tile>(p, stream);
+    }
     if (rc) return rc;
   } else if constexpr (kMode != kFwdFp8W) {
     if (kMode == kWgrad) {
@@ -1164,8 +1338,8 @@ int validate(const GemmArgs& p, int dtype) {
     // buffer loads address an operand with 32-bit byte offsets: all rows of an operand and one expert's weight
     // must each stay below 2 GiB
     const int64_t lim = int64_t(1) << 31;
-    if (p.total_rows * p.lda * 2 >= lim || p.total_rows * p.ldb * 2 >= lim || p.total_rows * p.ldc * 2 >= lim ||
-        p.k * p.n * 2 >= lim)
+    const int64_t a_extent = (p.a_index ? p.a_rows : p.total_rows) * p.lda * 2;
+    if (a_extent >= lim || p.total_rows * p.ldb * 2 >= lim || p.total_rows * p.ldc * 2 >= lim || p.k * p.n * 2 >= lim)
       return HMOE_UNSUPPORTED;
   }
   return HMOE_OK;
@@ -1185,6 +1359,34 @@ int hmoe_grouped_gemm_fwd(const void* a, int64_t lda, const void* b, const int32
   if (!a || !b || !out) return HMOE_INVALID_ARGUMENT;
   if (lda < k || ldo < n) return HMOE_INVALID_ARGUMENT;
   return launch<kFwd>(p, dtype, static_cast<hipStream_t>(stream));
+}
+
+int hmoe_grouped_gemm_fwd_gather(const void* a, int64_t lda, int64_t a_rows, const int64_t* row_index, const void* b,
+                                 const int32_t* offs, int64_t total_rows, int num_groups, int64_t k, int64_t n,
+                                 int dtype, void* out, int64_t ldo, void* stream) {
+  using namespace hmoe;
+  if (dtype != HMOE_BF16) return HMOE_UNSUPPORTED;
+  if (a_rows < 0) return HMOE_INVALID_ARGUMENT;
+  GemmArgs p{a, lda, b, n, out, ldo, offs, total_rows, num_groups, k, n, nullptr, row_index, a_rows};
+  if (int rc = validate(p, dtype)) return rc;
+  if (total_rows == 0 || n == 0) return HMOE_OK;
+  if (!a || !b || !out || !row_index) return HMOE_INVALID_ARGUMENT;
+  if (lda < k || ldo < n) return HMOE_INVALID_ARGUMENT;
+  return launch<kFwd>(p, dtype, static_cast<hipStream_t>(stream));
+}
+
+int hmoe_grouped_gemm_wgrad_gather(const void* a, int64_t lda, int64_t a_rows, const int64_t* row_index,
+                                   const void* grad_out, int64_t ldg, const int32_t* offs, int64_t total_rows,
+                                   int num_groups, int64_t k, int64_t n, int dtype, void* grad_b, void* stream) {
+  using namespace hmoe;
+  if (dtype != HMOE_BF16) return HMOE_UNSUPPORTED;
+  if (a_rows < 0) return HMOE_INVALID_ARGUMENT;
+  GemmArgs p{a, lda, grad_out, ldg, grad_b, n, offs, total_rows, num_groups, k, n, nullptr, row_index, a_rows};
+  if (int rc = validate(p, dtype)) return rc;
+  if (k == 0 || n == 0) return HMOE_OK;
+  if (!grad_b || (total_rows > 0 && (!a || !grad_out || !row_index))) return HMOE_INVALID_ARGUMENT;
+  if (lda < k || ldg < n) return HMOE_INVALID_ARGUMENT;
+  return launch<kWgrad>(p, dtype, static_cast<hipStream_t>(stream));
 }
 
 int hmoe_grouped_gemm_fwd_fp8w(const void* a, int64_t lda, const uint8_t* bq, const float* b_scale,

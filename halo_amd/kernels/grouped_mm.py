@@ -146,3 +146,107 @@ class _GroupedMMFunction(Function):
 
 def grouped_mm(mat_a, mat_b, *, offs=None):
     return _GroupedMMFunction.apply(mat_a, mat_b, offs)
+
+
+# ------------------------------------------------------------------------------------- permute folded into the GEMM
+
+def gather_fusable(tokens: torch.Tensor, mat_b) -> bool:
+    """Whether ``gather_grouped_mm`` can take these operands: bf16 rows of 16-byte multiples on the device and a plain
+    contiguous ``[G, K, N]`` weight of the same dtype."""
+    return (isinstance(mat_b, torch.Tensor) and tokens.is_cuda and tokens.dtype == torch.bfloat16
+            and mat_b.dtype == torch.bfloat16 and mat_b.dim() == 3 and mat_b.is_contiguous() and tokens.dim() == 2
+            and tokens.stride(-1) == 1 and tokens.stride(0) % 8 == 0 and tokens.shape[1] % 8 == 0
+            and mat_b.shape[2] % 8 == 0 and tokens.shape[1] == mat_b.shape[1])
+
+
+class _GatherGroupedMM(Function):
+    """``grouped_mm(tokens[row_index], mat_b, offs)`` without the permuted copy: the GEMM's loader and its weight
+    gradient's fetch the rows through ``row_index`` (``hmoe_grouped_gemm_fwd_gather`` / ``_wgrad_gather``).  This is
+    ``MoEGatherPermute`` followed by ``grouped_mm`` (reference ``moe_permute.py:130-141`` + ``grouped_mm.py:30-47``)
+    as one autograd node; the gradient for ``tokens`` is the dgrad scattered back with the atomic-free gather-reduce
+    over ``inv_map``, exactly as ``MoEGatherPermute.backward`` does."""
+
+    @staticmethod
+    def forward(ctx, tokens, row_index, inv_map, mat_b, offs):
+        device = _lib.require_device(tokens, row_index, inv_map, mat_b, offs)
+        groups, k, n = mat_b.shape
+        rows = row_index.shape[0]
+        row_index = row_index.long().contiguous()
+        offs32 = _offs_arg(offs, groups)
+        out = torch.empty((rows, n), dtype=tokens.dtype, device=device)
+        if rows and n:
+            with _lib.on_device(device):
+                _lib.call("hmoe_grouped_gemm_fwd_gather", _lib.ptr(tokens), tokens.stride(0), tokens.shape[0],
+                          _lib.ptr(row_index), _lib.ptr(mat_b), _lib.ptr(offs32), rows, groups, k, n,
+                          _lib.dtype_id(tokens.dtype), _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
+        ctx.save_for_backward(tokens, row_index, inv_map, mat_b, offs32)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from halo_amd.kernels.moe_permute import gather_reduce_rows
+
+        tokens, row_index, inv_map, mat_b, offs32 = ctx.saved_tensors
+        device = tokens.device
+        groups, k, n = mat_b.shape
+        rows = row_index.shape[0]
+        grad_output = _rows(grad_output) if grad_output.numel() else grad_output.new_empty(grad_output.shape)
+        grad_tokens = grad_b = None
+        if ctx.needs_input_grad[0]:
+            shape_only = grad_output.new_empty((1, k)).expand(rows, k)  # dgrad reads mat_a's shape and dtype only
+            grad_sorted, _ = grouped_mm_grads(shape_only, mat_b, grad_output, offs32, True, False)
+            grad_tokens = gather_reduce_rows(grad_sorted, inv_map)
+        if ctx.needs_input_grad[3]:
+            grad_b = torch.empty((groups, k, n), dtype=tokens.dtype, device=device)
+            if k and n:
+                with _lib.on_device(device):
+                    _lib.call("hmoe_grouped_gemm_wgrad_gather", _lib.ptr(tokens), tokens.stride(0), tokens.shape[0],
+                              _lib.ptr(row_index), _lib.ptr(grad_output), grad_output.stride(0) if rows else n,
+                              _lib.ptr(offs32), rows, groups, k, n, _lib.dtype_id(tokens.dtype), _lib.ptr(grad_b),
+                              _lib.stream_ptr(device))
+        return grad_tokens, None, None, grad_b, None
+
+
+def gather_grouped_mm(tokens, row_index, inv_map, mat_b, *, offs):
+    """``grouped_mm(tokens[row_index], mat_b, offs=offs)``; see :class:`_GatherGroupedMM`.  The caller checks
+    :func:`gather_fusable` first."""
+    return _GatherGroupedMM.apply(tokens, row_index, inv_map, mat_b, offs)
+
+
+class GatheredRows:
+    """``tokens[row_index]`` that nobody has copied yet: what the sort hands to the first expert projection when that
+    projection can fetch the rows itself (:func:`gather_grouped_mm`).  A consumer that cannot calls
+    :meth:`materialize`, which is ``MoEGatherPermute`` (reference ``moe_permute.py:130-141``), once."""
+
+    def __init__(self, tokens: torch.Tensor, row_index: torch.Tensor, inv_map: torch.Tensor):
+        self.tokens, self.row_index, self.inv_map = tokens, row_index, inv_map
+        self._rows = None
+
+    @property
+    def shape(self):
+        return torch.Size((self.row_index.shape[0], self.tokens.shape[1]))
+
+    @property
+    def dtype(self):
+        return self.tokens.dtype
+
+    @property
+    def device(self):
+        return self.tokens.device
+
+    def to(self, dtype: torch.dtype) -> "GatheredRows":
+        return self if dtype == self.tokens.dtype else GatheredRows(self.tokens.to(dtype), self.row_index, self.inv_map)
+
+    def materialize(self) -> torch.Tensor:
+        if self._rows is None:
+            from halo_amd.kernels.moe_permute import MoEGatherPermute
+
+            self._rows = MoEGatherPermute.apply(self.tokens, self.row_index, self.inv_map)
+        return self._rows
+
+    def grouped_mm(self, mat_b, *, offs) -> torch.Tensor | None:
+        """The projection through the gathering kernels, or None when these operands do not qualify."""
+        if not gather_fusable(self.tokens, mat_b):
+            return None
+        return gather_grouped_mm(self.tokens, self.row_index, self.inv_map, mat_b, offs=offs)
+

@@ -22,7 +22,7 @@ import torch.nn as nn
 
 from halo_amd.kernels.expert_gemm import expert_gemm
 from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled, resolve_fused_glu_mul
-from halo_amd.kernels.grouped_mm import grouped_mm, grouped_wgrad
+from halo_amd.kernels.grouped_mm import GatheredRows, grouped_mm, grouped_wgrad
 from halo_amd.kernels.moe_permute import MoEGatherPermute, MoEWeightedUnpermute, warm_permute_kernels
 from halo_amd.kernels.moe_route_sort import sort_routing_by_expert, warm_route_sort_kernels
 from halo_amd.kernels.router import SOFTMAX_ALL, fused_topk_gate
@@ -159,6 +159,8 @@ class EPMoELayerBase(nn.Module, ABC):
         self._expert_kernels_warmed = False
         self._lowp_quant_format = None
         self._lowp_weight_cacheable = True
+        # the first expert projection gathers its rows by index instead of reading a permuted copy of the tokens
+        self.fuse_permute_into_gemm = True
         self._fused_glu_mul: Callable | None = None
         # labels the dispatch / expert-compute / combine spans at no device cost (swappable, as in the reference)
         self._perf = torch.profiler.record_function
@@ -275,7 +277,12 @@ class EPMoELayerBase(nn.Module, ABC):
         sorted_token_idx, sorted_weights, sorted_expert_ids, offs, inv_map = sort_routing_by_expert(
             experts, weights, self.experts_per_rank, counts
         )
-        sorted_tokens = MoEGatherPermute.apply(tokens, sorted_token_idx, inv_map)
+        # The permuted copy is left to the first expert projection, whose loader can fetch the rows through the index
+        # (one pass over the tokens saved each way); a projection that cannot asks for the copy.  Only where one
+        # projection reads the rows (gate and up stored fused): two readers would each scatter a gradient back.
+        fuse = self.fuse_permute_into_gemm and self._stores_fused_glu
+        sorted_tokens = (GatheredRows(tokens, sorted_token_idx, inv_map) if fuse
+                         else MoEGatherPermute.apply(tokens, sorted_token_idx, inv_map))
         return sorted_tokens, offs, sorted_token_idx, sorted_weights, sorted_expert_ids, inv_map
 
     def _grouped_expert_ffn(self, sorted_tokens, offs, sorted_expert_ids, output_dtype):
@@ -285,6 +292,11 @@ class EPMoELayerBase(nn.Module, ABC):
         weight = getattr(self, weight_attr)
         if isinstance(weight, torch.Tensor):
             weight = weight.to(out_dtype)
+        if isinstance(x, GatheredRows):
+            fused = x.grouped_mm(weight, offs=offs) if self._lowp_quant_format is None else None
+            if fused is not None:
+                return fused
+            x = x.materialize()
         return self._grouped_mm(x, weight, offs=offs)
 
     def _grouped_mm(self, mat_a, mat_b, *, offs=None, lowp: bool = True):

@@ -136,6 +136,18 @@ int hmoe_grouped_gemm_wgrad(const void* a, int64_t lda, const void* grad_out, in
                             int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype, void* grad_b,
                             void* stream);
 
+/* The same two GEMMs with the rows of A gathered: logical row r of A is a[row_index[r]], a holding a_rows rows; an
+ * index outside [0, a_rows) reads as a row of zeros.  This folds MoEGatherPermute.forward
+ * (halo/kernels/moe_permute.py:133-136, tokens.index_select(0, sorted_token_idx)) into the first expert GEMM and its
+ * weight gradient (halo/kernels/grouped_mm.py:39, :26), so the permuted copy of the tokens is never written.
+ * bf16 only (HMOE_UNSUPPORTED otherwise). */
+int hmoe_grouped_gemm_fwd_gather(const void* a, int64_t lda, int64_t a_rows, const int64_t* row_index, const void* b,
+                                 const int32_t* offs, int64_t total_rows, int num_groups, int64_t k, int64_t n,
+                                 int dtype, void* out, int64_t ldo, void* stream);
+int hmoe_grouped_gemm_wgrad_gather(const void* a, int64_t lda, int64_t a_rows, const int64_t* row_index,
+                                   const void* grad_out, int64_t ldg, const int32_t* offs, int64_t total_rows,
+                                   int num_groups, int64_t k, int64_t n, int dtype, void* grad_b, void* stream);
+
 /* ------------------------------------------------------------------------------------------------- block fp8
  * Replaces quantize_block_fp8: halo/kernels/lowp/block_fp8.py:23-34.  w is [batch, rows, cols]; q (e4m3fn bytes)
  * has its shape; scale is f32 [batch, ceil(rows/128), ceil(cols/128)], a power of two per 128x128 block. */

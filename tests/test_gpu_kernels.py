@@ -536,3 +536,35 @@ def test_fp8_weight_grouped_gemm_equals_the_dequantised_bf16_path(device):
     w_ref = torch.from_numpy(fp8_oracle.dequantize_block_fp8(want_q, want_scale)).bfloat16()
     want = oracle.grouped_mm(x.double(), w_ref.double(), np.cumsum(counts).astype(np.int32), acc_dtype=torch.float64)
     assert max_rel(out, want) < 2e-2 and cosine(out, want) > 0.9999
+
+
+@pytest.mark.parametrize(("counts", "k", "n"), (((255, 256, 257, 0, 513, 31), 200, 264), ((64,) * 16, 512, 1536),
+                                                 (tuple((37 * i * i + 11 * i) % 91 for i in range(150)), 320, 256)))
+def test_gather_grouped_mm_equals_permute_then_grouped_mm(device, counts, k, n):
+    """The GEMM that gathers its A rows through the sorted token index does the same arithmetic in the same order as
+    the permute followed by the plain GEMM: outputs and all gradients are bit-equal.  Tokens are drawn so that rows
+    repeat (top-k) and some tokens are never picked."""
+    from halo_amd.kernels.grouped_mm import gather_fusable, gather_grouped_mm, grouped_mm
+    from halo_amd.kernels.moe_permute import MoEGatherPermute, build_inv_map
+
+    g = torch.Generator().manual_seed(3)
+    rows, n_tokens = sum(counts), max(8, sum(counts) // 3)
+    row_index = torch.randint(0, n_tokens, (rows,), generator=g).to(device)
+    width = int(torch.bincount(row_index.cpu(), minlength=n_tokens).max())
+    inv_map = build_inv_map(row_index, n_tokens, width)
+    tokens = torch.randn(n_tokens, k, generator=g).bfloat16().to(device)
+    w = (torch.randn(len(counts), k, n, generator=g) * 0.05).bfloat16().to(device)
+    dout = torch.randn(rows, n, generator=g).bfloat16().to(device)
+    offs = _offsets(counts, device)
+    assert gather_fusable(tokens, w)
+    results = []
+    for fused in (False, True):
+        t, wd = tokens.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        if fused:
+            out = gather_grouped_mm(t, row_index, inv_map, wd, offs=offs)
+        else:
+            out = grouped_mm(MoEGatherPermute.apply(t, row_index, inv_map), wd, offs=offs)
+        out.backward(dout)
+        results.append((out.detach(), t.grad, wd.grad))
+    for name, a, b in zip(("out", "grad_tokens", "grad_weight"), *results):
+        assert torch.equal(a, b), name

@@ -124,6 +124,27 @@ def test_layer_is_bit_reproducible(device):
     assert all(torch.equal(a, b) for a, b in zip(*runs))
 
 
+@pytest.mark.parametrize("cfg", (CONFIG1, CONFIG2_SMALL), ids=lambda c: c.name)
+def test_permute_folded_into_the_first_projection_changes_no_bit(device, cfg):
+    """By default the first expert projection fetches its rows through the sort's index instead of reading a permuted
+    copy; the output and every gradient must equal the permute-then-GEMM path's bit for bit (the products and their
+    summation order are the same, only the addressing differs).  The fp32 configuration does not qualify for the gathering
+    kernels and takes the copy either way."""
+    inputs = make_layer_inputs(cfg)
+    runs = []
+    for fuse in (True, False):
+        layer = _build_layer(cfg, inputs, device)
+        assert layer.fuse_permute_into_gemm
+        layer.fuse_permute_into_gemm = fuse
+        x = inputs["x"].to(device).requires_grad_(True)
+        out = layer(x)
+        out = out[0] if isinstance(out, tuple) else out
+        out.backward(inputs["grad_out"].to(device))
+        runs.append([out.detach(), x.grad] + [p.grad for _, p in sorted(layer.named_parameters())])
+    assert len(runs[0]) >= 4 and all(g is not None for g in runs[0])
+    assert all(torch.equal(a, b) for a, b in zip(*runs))
+
+
 def test_one_gpus_share_of_an_ep_layer(device):
     """Local ids with -1 for other ranks' picks plus host-side receive counts (an EP8 shard's shape, scaled down):
     ``_compute_experts`` against the dense formula over the valid slots, and the count checks."""
