@@ -132,6 +132,13 @@ __device__ __forceinline__ u32x4 make_rsrc_words(const void* base, uint32_t byte
 
 typedef __attribute__((address_space(3))) char* lds_bytes_ptr;
 
+// The scalar operands of the loads below, pinned to scalar registers (the compiler does not move an inline
+// assembly operand out of a vector register by itself); free where the value is already known to be uniform.
+__device__ __forceinline__ uint32_t uniform(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ u32x4 uniform(u32x4 v) {
+  return u32x4{uniform(v[0]), uniform(v[1]), uniform(v[2]), uniform(v[3])};
+}
+
 // Direct-to-LDS load of 16 bytes per lane: lane L's bytes land at lds_base + 16 L; an offset at or past the
 // descriptor's size loads zeros.  Written through inline assembly on purpose.  The compiler tracks the builtin form
 // as a pending LDS write and drains every load in flight (vmcnt(0)) before the next LDS store and before the next
@@ -141,8 +148,8 @@ typedef __attribute__((address_space(3))) char* lds_bytes_ptr;
 __device__ __forceinline__ void lds_load16(u32x4 rsrc, lds_bytes_ptr lds_base, uint32_t voffset, uint32_t soffset) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :
-               : "s"(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_base))), "v"(voffset), "s"(rsrc),
-                 "s"(soffset)
+               : "s"(uniform(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_base)))), "v"(voffset),
+                 "s"(uniform(rsrc)), "s"(uniform(soffset))
                : "memory");
 }
 
