@@ -13,7 +13,9 @@
 // (4 + 2) * 32 operand values for 4 * 2 * 1024 multiply-adds.
 //  * Operand tiles go from global memory straight into LDS (buffer_load ... lds, 16 bytes per lane): no staging
 //    registers, no ds_write, no register transposes.  Rows past a group's end and columns past an operand's edge come
-//    back as zeros from the buffer bounds check, with no branches in the loop.
+//    back as zeros from the buffer bounds check, with no branches in the loop.  The loads are issued through inline
+//    assembly and waited for explicitly (see lds_load16: the compiler would drain them before every transposing LDS
+//    read).
 //  * A contraction-contiguous operand lands as [256 rows][64 con] with the 16-byte chunk index XOR-ed with row & 7
 //    (each lane fetches the chunk that belongs in its LDS slot); an MFMA fragment is one ds_read_b128, and the
 //    fragments of other row blocks and contraction sub-steps are immediate offsets or one XOR away.
@@ -36,6 +38,11 @@
 // balanced whatever the skew of the expert loads.  wgrad walks (group, column tile, row tile) the same way: dealt
 // round-robin over all workgroups, neighbouring tiles landed on different XCDs and every operand row was fetched from
 // HBM once per tile that uses it (4x the algorithmic bytes, measured).
+//
+// Gathered operand A (template parameter kGather; fwd and wgrad).  A may be given as (array, row index): logical row
+// r is array[index[r]], which folds the reference's permute by expert (halo/kernels/moe_permute.py:130-141) into the
+// first expert projection and its weight gradient.  The direct-to-LDS load takes a per-lane offset, so a gathered row
+// costs what a contiguous one does; see GatherDirect and GatherTransposed.
 //
 // Weights in block-scaled fp8 (grouped_gemm_staged_kernel, forward only) take the register-staged variant of the same
 // tiling: global -> registers (dequantised there) -> LDS as [output index][64 contraction], both operands read back
