@@ -74,35 +74,72 @@ gather_rows_kernel(const T* __restrict__ src, int64_t src_stride, const int64_t*
   }
 }
 
-template <typename T, int W, bool kWeighted>
+// out[t] = sum over k of (weight[j] *) src[j], j = inv_map[t][k], in slot order; a slot outside [0, n_src) adds
+// nothing.  One wavefront per output row.  kTopK > 0 fixes top_k at compile time: the row's slots and weights are
+// read once, and for every 16-byte column chunk the kTopK row loads are issued together before the first is used, so
+// a lane keeps kTopK loads in flight instead of one (with one in flight the kernel reached half of the HBM rate).  An
+// invalid slot loads row 0 and contributes +0.0f, which leaves the fp32 sum exactly as skipping it does: the
+// accumulator starts at +0.0f and a sum that started there is never -0.0f.
+template <typename T, int W, bool kWeighted, int kTopK>
 __global__ void __launch_bounds__(kThreads)
 gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, const int64_t* __restrict__ inv_map,
                      T* __restrict__ out, int64_t n_out, int top_k, int64_t n_src, int64_t hidden) {
-  const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / HMOE_WAVE;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock +
+                      __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / HMOE_WAVE);
   if (row >= n_out) return;
   const int64_t* map = inv_map + row * top_k;
   T* to = out + row * hidden;
   const int64_t step = static_cast<int64_t>(HMOE_WAVE) * W;
-  for (int64_t c = static_cast<int64_t>(lane_id()) * W; c < hidden; c += step) {
-    Pack<T, W> acc;
+  if constexpr (kTopK > 0) {
+    const T* from[kTopK];
+    float w[kTopK];
+    bool valid[kTopK];
 #pragma unroll
-    for (int i = 0; i < W; ++i) acc.v[i] = 0.f;
-    for (int k = 0; k < top_k; ++k) {
+    for (int k = 0; k < kTopK; ++k) {
       const int64_t j = map[k];
-      if (j >= 0 && j < n_src) {
-        Pack<T, W> x;
-        x.load(src + j * hidden + c);
-        if constexpr (kWeighted) {
-          const float w = Elem<T>::load(weight + j);
+      valid[k] = j >= 0 && j < n_src;
+      from[k] = src + (valid[k] ? j : 0) * hidden;
+      w[k] = 1.f;
+      if constexpr (kWeighted) w[k] = Elem<T>::load(weight + (valid[k] ? j : 0));
+    }
+    for (int64_t c = static_cast<int64_t>(lane_id()) * W; c < hidden; c += step) {
+      Pack<T, W> x[kTopK], acc;
 #pragma unroll
-          for (int i = 0; i < W; ++i) acc.v[i] += x.v[i] * w;
-        } else {
+      for (int k = 0; k < kTopK; ++k) x[k].load(from[k] + c);
 #pragma unroll
-          for (int i = 0; i < W; ++i) acc.v[i] += x.v[i];
+      for (int i = 0; i < W; ++i) acc.v[i] = 0.f;
+#pragma unroll
+      for (int k = 0; k < kTopK; ++k) {
+#pragma unroll
+        for (int i = 0; i < W; ++i) {
+          const float term = kWeighted ? x[k].v[i] * w[k] : x[k].v[i];
+          acc.v[i] += valid[k] ? term : 0.f;
         }
       }
+      acc.store(to + c);
     }
-    acc.store(to + c);
+  } else {
+    for (int64_t c = static_cast<int64_t>(lane_id()) * W; c < hidden; c += step) {
+      Pack<T, W> acc;
+#pragma unroll
+      for (int i = 0; i < W; ++i) acc.v[i] = 0.f;
+      for (int k = 0; k < top_k; ++k) {
+        const int64_t j = map[k];
+        if (j >= 0 && j < n_src) {
+          Pack<T, W> x;
+          x.load(src + j * hidden + c);
+          if constexpr (kWeighted) {
+            const float w = Elem<T>::load(weight + j);
+#pragma unroll
+            for (int i = 0; i < W; ++i) acc.v[i] += x.v[i] * w;
+          } else {
+#pragma unroll
+            for (int i = 0; i < W; ++i) acc.v[i] += x.v[i];
+          }
+        }
+      }
+      acc.store(to + c);
+    }
   }
 }
 
@@ -240,17 +277,25 @@ int hmoe_gather_reduce(const void* src, const void* weight, const int64_t* inv_m
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool vec = dtype == HMOE_BF16 ? rows_vectorizable<bf16_t>(hidden, {}, {src, out})
                                       : rows_vectorizable<float>(hidden, {}, {src, out});
+  // n_src == 0: every slot is invalid and the rows come out as zeros; the generic kernel never touches src then
+  const int fixed = n_src > 0 && (top_k == 8 || top_k == 4 || top_k == 2) ? top_k : 0;
+#define HMOE_GATHER_REDUCE(WEIGHTED, TOPK)                                                                        \
+  HMOE_DISPATCH_ROWS(dtype, vec,                                                                                  \
+                     (gather_reduce_kernel<T, W, WEIGHTED, TOPK><<<row_grid(n_out), dim3(kThreads), 0, s>>>(      \
+                         static_cast<const T*>(src), static_cast<const T*>(weight), inv_map, static_cast<T*>(out), \
+                         n_out, top_k, n_src, hidden)))
   if (weight) {
-    HMOE_DISPATCH_ROWS(dtype, vec,
-                       (gather_reduce_kernel<T, W, true><<<row_grid(n_out), dim3(kThreads), 0, s>>>(
-                           static_cast<const T*>(src), static_cast<const T*>(weight), inv_map, static_cast<T*>(out),
-                           n_out, top_k, n_src, hidden)));
+    if (fixed == 8) { HMOE_GATHER_REDUCE(true, 8); }
+    else if (fixed == 4) { HMOE_GATHER_REDUCE(true, 4); }
+    else if (fixed == 2) { HMOE_GATHER_REDUCE(true, 2); }
+    else { HMOE_GATHER_REDUCE(true, 0); }
   } else {
-    HMOE_DISPATCH_ROWS(dtype, vec,
-                       (gather_reduce_kernel<T, W, false><<<row_grid(n_out), dim3(kThreads), 0, s>>>(
-                           static_cast<const T*>(src), nullptr, inv_map, static_cast<T*>(out), n_out, top_k, n_src,
-                           hidden)));
+    if (fixed == 8) { HMOE_GATHER_REDUCE(false, 8); }
+    else if (fixed == 4) { HMOE_GATHER_REDUCE(false, 4); }
+    else if (fixed == 2) { HMOE_GATHER_REDUCE(false, 2); }
+    else { HMOE_GATHER_REDUCE(false, 0); }
   }
+#undef HMOE_GATHER_REDUCE
   HMOE_CHECK_LAUNCH();
   return HMOE_OK;
 }
