@@ -130,7 +130,9 @@ def test_bincount(device):
 # -------------------------------------------------------------------------------------------- permute / combine
 
 DTYPE_TOLS = ((torch.float32, 1e-5), (torch.bfloat16, 2e-2))
-ROUTINGS = ((517, 8, 2816, 0.5), (64, 4, 100, 1.0), (33, 8, 1025, 0.1), (300, 8, 2048, 1.0))
+# top_k 2, 4 and 8 take the kernels with the slot count fixed at compile time, 3 and 6 the runtime-count loop
+ROUTINGS = ((517, 8, 2816, 0.5), (64, 4, 100, 1.0), (33, 8, 1025, 0.1), (300, 8, 2048, 1.0), (96, 2, 520, 0.7),
+            (50, 6, 512, 0.6), (40, 3, 264, 0.8), (200, 4, 768, 0.4))
 
 
 def _routing(n_tokens, top_k, n_sorted, seed):
