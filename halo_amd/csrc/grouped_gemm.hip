@@ -634,10 +634,35 @@ struct TileSchedule {
     // one contiguous chunk of the tile order per XCD (workgroup w runs on XCD w % 8): the workgroups that share an
     // L2 work on neighbouring tiles, which share operand rows
     const int xcd = blockIdx.x % kXcds;
-    const int64_t chunk = (total + kXcds - 1) / kXcds;
-    first = xcd * chunk + blockIdx.x / kXcds;
-    last = xcd * chunk + chunk < total ? xcd * chunk + chunk : total;
     stride = (workers - xcd + kXcds - 1) / kXcds;
+    if constexpr (kMode == kWgrad) {
+      // A wgrad tile walks its group's rows, so tiles cost what their group holds: the chunks are cut at equal cost,
+      // not at equal tile counts (with one expert holding a quarter of the rows, equal counts left one XCD with
+      // twice the work of the others).
+      const int64_t cost = per_group * static_cast<int64_t>(__builtin_amdgcn_readfirstlane(tile_start[p.groups]));
+      first = p.groups > 0 ? cut(cost * xcd / kXcds, p.groups) + blockIdx.x / kXcds : 0;
+      last = xcd + 1 == kXcds || p.groups == 0 ? total : cut(cost * (xcd + 1) / kXcds, p.groups);
+    } else {
+      const int64_t chunk = (total + kXcds - 1) / kXcds;
+      first = xcd * chunk + blockIdx.x / kXcds;
+      last = xcd * chunk + chunk < total ? xcd * chunk + chunk : total;
+    }
+  }
+
+  // wgrad: the first tile whose predecessors cost `target` or more (tiles in order, a tile of group g costing
+  // tile_start[g + 1] - tile_start[g])
+  __device__ __forceinline__ int64_t cut(int64_t target, int groups) const {
+    int lo = 0, hi = groups;  // the group the cut falls into: per_group * tile_start[g] <= target, largest such g
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (per_group * static_cast<int64_t>(__builtin_amdgcn_readfirstlane(tile_start[mid])) <= target) lo = mid;
+      else hi = mid;
+    }
+    const int64_t before = per_group * static_cast<int64_t>(__builtin_amdgcn_readfirstlane(tile_start[lo]));
+    const int64_t each = __builtin_amdgcn_readfirstlane(tile_start[lo + 1]) - __builtin_amdgcn_readfirstlane(tile_start[lo]);
+    int64_t within = (target - before + each - 1) / each;
+    if (within > per_group) within = per_group;
+    return lo * per_group + within;
   }
 
   __device__ __forceinline__ TileInfo decode(int64_t t, int& cursor) const {
@@ -923,7 +948,9 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   constexpr bool kRowsPerStep = kGather && !kDirectA;  // the gathered rows are contraction rows: new ones every step
   using Sched = TileSchedule<kMode, BM, BN>;
   extern __shared__ __attribute__((aligned(16))) char lds_raw[];  // two stages of (A tile, B tile), 32 KB each
-  __shared__ int32_t grp_s[kMaxGroups], grp_e[kMaxGroups], tile_start[kMode == kWgrad ? 1 : kMaxGroups + 1];
+  // tile_start: per group, the prefix of its row tiles (fwd, dgrad) or of its tiles' cost (wgrad: contraction steps
+  // + 1 per tile, the same for every tile of a group)
+  __shared__ int32_t grp_s[kMaxGroups], grp_e[kMaxGroups], tile_start[kMaxGroups + 1];
   auto lds = (__attribute__((address_space(3))) char*)lds_raw;
   constexpr int kTileBytes = 256 * BK * 2, kStageBytes = 2 * kTileBytes;
   bf16_t* c = static_cast<bf16_t*>(p.c);
@@ -944,9 +971,9 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       group_bounds(p.offs, g, p.total_rows, s, e);
       grp_s[g] = static_cast<int32_t>(s);
       grp_e[g] = static_cast<int32_t>(e);
-      sum += static_cast<int>((e - s + BM - 1) / BM);
+      sum += kMode == kWgrad ? static_cast<int>((e - s + BK - 1) / BK) + 1 : static_cast<int>((e - s + BM - 1) / BM);
     }
-    if constexpr (kMode != kWgrad) {
+    {
       int incl = sum;
 #pragma unroll
       for (int off = 1; off < HMOE_WAVE; off <<= 1) {
@@ -956,7 +983,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       int running = incl - sum;
       for (int g = g0; g < g0 + per && g < p.groups; ++g) {
         tile_start[g] = running;
-        running += (grp_e[g] - grp_s[g] + BM - 1) / BM;
+        running += kMode == kWgrad ? (grp_e[g] - grp_s[g] + BK - 1) / BK + 1 : (grp_e[g] - grp_s[g] + BM - 1) / BM;
       }
       if (lane == HMOE_WAVE - 1) tile_start[p.groups] = incl;
     }

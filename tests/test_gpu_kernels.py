@@ -250,16 +250,21 @@ def test_build_inv_map_matches_oracle(device):
     assert torch.equal(build_inv_map(token_idx.to(device), 2000, 8).cpu(), inv_map)
 
 
-def test_expert_bias_gather(device):
+@pytest.mark.parametrize(("rows", "width", "skew"), ((5000, 2880, 0), (20000, 360, 3), (700, 100, 0), (9, 64, 0)),
+                         ids=("even", "one_expert_holds_most", "unaligned_width", "tiny"))
+def test_expert_bias_gather(device, rows, width, skew):
     from halo_amd.kernels.moe_permute import MoEExpertBiasGather
     from oracle import permute as oracle
 
     g = torch.Generator().manual_seed(3)
     for dtype, tol in DTYPE_TOLS:
-        eids = torch.sort(torch.randint(0, 32, (5000,), generator=g)).values
+        ids = torch.randint(0, 32, (rows,), generator=g)
+        if skew:  # four rows in five go to one expert
+            ids = torch.where(torch.rand(rows, generator=g) < 0.8, torch.full_like(ids, skew), ids)
+        eids = torch.sort(ids).values
         eids = eids[(eids != 7) & (eids != 31)]  # two idle experts, one of them last
-        bias = torch.randn(32, 2880, generator=g).to(dtype)
-        grad = torch.randn(eids.numel(), 2880, generator=g).to(dtype)
+        bias = torch.randn(32, width, generator=g).to(dtype)
+        grad = torch.randn(eids.numel(), width, generator=g).to(dtype)
         bd = bias.to(device).requires_grad_(True)
         out = MoEExpertBiasGather.apply(bd, eids.to(device))
         assert torch.equal(out.cpu(), oracle.bias_gather(bias, eids))
