@@ -829,74 +829,85 @@ struct GatherDirect {  // LDS layout and fragments as SlimDirect
   }
 };
 
+// Gathered rows as contraction rows (wgrad): new rows every step.  The LDS tile is kept as eight panels of 32 output
+// columns, [panel][64 con][32 out] with 64-byte rows, instead of SlimTransposed's [64 con][256 out]: a lane then
+// stays on ONE contraction row for all of a step's loads (lane L: row L / 4 of the wavefront's 16, 16-byte chunk
+// L % 4 of panel t in load t), so a step costs a lane one row index, one multiply and one add per load.  (With a
+// load spanning two whole rows, as in SlimTransposed, every load needs its own pair of indices broadcast to the two
+// half-wavefronts: 16 lane reads and 8 selects per step, which made this kernel 12 % slower than the plain one.)
+// A load moves 16 rows x 64 bytes; loads t and t + 1 of a pair cover the two halves of the same 128-byte lines back
+// to back.  The transposing read of a 32-column block touches 4 rows x 64 bytes per 32 lanes: every bank once,
+// no swizzle.
 template <int kI>
-struct GatherTransposed {  // LDS layout and fragments as SlimTransposed; the gathered rows are contraction rows
+struct GatherTransposed {
+  static_assert(kI == 8, "eight panels of 32 columns, one load per panel");
   u32x4 rsrc;
   u32x4 index_rsrc;  // the group's row indices, bounded at its last row
   uint32_t a_rows;
-  uint32_t col[2];       // byte offset of this lane's chunk within a row for even / odd loads, or out of range
+  uint32_t col;       // byte offset within a row of this lane's chunk in panel 0
+  int t_lim;          // loads t < t_lim have this lane's chunk inside the operand
   uint32_t row_bytes;
   int con_lim;
-  // A wavefront's kI loads of a step cover 2 kI contraction rows, one per half wavefront and load.  Their indices
-  // (low words) are themselves fetched straight into LDS, one step ahead, into the wavefront's own 2 x 1 KB
-  // (by step parity): a load into a register would have to be waited for, and the compiler places that wait right
-  // behind the tile loads just issued.
-  __attribute__((address_space(3))) char* rows_area;
-  int rows_valid0, rows_valid1;  // how many of the 2 kI rows exist, per parity
+  // The indices of a wavefront's 16 rows of a step (low words) are themselves fetched straight into LDS, one step
+  // ahead, into the wavefront's own 2 x 1 KB (by step parity): a load into a register would have to be waited for,
+  // and the compiler places that wait right behind the tile loads just issued.
+  lds_bytes_ptr rows_area;
+  int rows_valid0, rows_valid1;  // how many of the 16 rows exist, per parity
 
   __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t a_rows_, const int64_t* index, int out0,
-                                       int out_lim, int con_lim_, int slot, int lane) {
-    static_assert(kI % 2 == 0 && 2 * kI <= 64, "loads come in even/odd pairs");
+                                       int out_lim, int con_lim_, int /*slot*/, int lane) {
     rsrc = make_rsrc_words(base, static_cast<uint32_t>(a_rows_ * ld * 2));
     index_rsrc = make_rsrc_words(index, static_cast<uint32_t>(con_lim_) * 8u);
     a_rows = static_cast<uint32_t>(a_rows_);
     row_bytes = static_cast<uint32_t>(ld) * 2u;
     con_lim = con_lim_;
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int con = (slot * kI + u) * 2 + (lane >> 5);
-      const int logical = (lane & 31) ^ ((con & 3) << 2);
-      const int out = out0 + (logical << 3);
-      col[u] = out < out_lim ? static_cast<uint32_t>(out) * 2u : kOutOfRange;
-    }
+    const int chunk = lane & 3;
+    col = static_cast<uint32_t>(out0) * 2u + chunk * 16u;
+    const int chunks = (out_lim - out0 + 7) >> 3;  // 16-byte chunks of the operand from out0 on
+    t_lim = (chunks - chunk + 3) >> 2;
   }
   // fetch the row indices of `step`
   __device__ __forceinline__ void load_rows(int step, int slot, int lane) {
     load_rows_of(index_rsrc, con_lim, step, slot, lane);
   }
   // the same for a group given by its index buffer and its row count (the next tile's, fetched ahead)
-  __device__ __forceinline__ void load_rows_of(u32x4 group_index, int group_rows, int step, int slot,
-                                               int lane) {
-    const int first = step * BK + slot * (2 * kI);
+  __device__ __forceinline__ void load_rows_of(u32x4 group_index, int group_rows, int step, int slot, int lane) {
+    const int first = step * BK + slot * 16;
     if (step & 1) rows_valid1 = group_rows - first;
     else rows_valid0 = group_rows - first;
-    // lane l < kI fetches indices first + 2l and first + 2l + 1; rows past the group's end read as 0 and are masked
+    // lane l < 8 fetches indices first + 2l and first + 2l + 1; rows past the group's end read as 0 and are masked
     // on use
     lds_load16(group_index, rows_area + (step & 1) * 1024,
-               first < group_rows && lane < kI ? static_cast<uint32_t>(first + 2 * lane) * 8u : kOutOfRange, 0u);
+               first < group_rows && lane < 8 ? static_cast<uint32_t>(first + 2 * lane) * 8u : kOutOfRange, 0u);
   }
   // the loads of `step`, whose rows load_rows() fetched (and whose arrival the caller has waited for)
-  __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int slot,
-                                        bool live = true) const {
+  __device__ __forceinline__ void issue(lds_bytes_ptr tile, int step, int slot, bool live = true) const {
     const int lane = threadIdx.x & 63;
-    const int32_t rows_raw = *reinterpret_cast<const __attribute__((address_space(3))) int32_t*>(
-        rows_area + (step & 1) * 1024 + (lane & (2 * kI - 1)) * 8);  // the low word of index lane % (2 kI)
+    const int mine = lane >> 2;  // this lane's row among the wavefront's 16
+    const uint32_t row = *reinterpret_cast<const __attribute__((address_space(3))) uint32_t*>(
+        rows_area + (step & 1) * 1024 + mine * 8);  // the index's low word
     const int valid = (step & 1) ? rows_valid1 : rows_valid0;
+    const uint32_t base = live && mine < valid && row < a_rows ? row * row_bytes + col : kOutOfRange;
 #pragma unroll
-    for (int t = 0; t < kI; ++t) {
-      const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readlane(rows_raw, 2 * t));
-      const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(rows_raw, 2 * t + 1));
-      const bool upper = (lane & 32) != 0;
-      const uint32_t row = upper ? hi : lo;
-      const bool ok = live && 2 * t + (upper ? 1 : 0) < valid && row < a_rows && (col[t & 1] & kOutOfRange) == 0;
-      lds_load16(rsrc, tile + (slot * kI + t) * 1024, ok ? row * row_bytes + col[t & 1] : kOutOfRange, 0u);
-    }
+    for (int t = 0; t < kI; ++t)  // an out-of-range base stays out of range with the panel's offset added
+      lds_load16(rsrc, tile + t * 4096 + slot * 1024, t < t_lim ? base + t * 64 : kOutOfRange, 0u);
   }
+  // per-lane byte address of the fragment of sub-step 0 for the 32-column block at row0 (a multiple of 32)
   static __device__ __forceinline__ int fragment_base(int row0, int lane) {
-    return SlimTransposed<kI>::fragment_base(row0, lane);
+    const int i = lane & 15, g = lane >> 4;
+    const int out = row0 + ((g & 1) << 4) + ((i & 3) << 2);
+    const int con = ((g >> 1) << 3) + (i >> 2);
+    return (out >> 5) * 4096 + con * 64 + (out & 31) * 2;
   }
-  static __device__ __forceinline__ bf16x8 fragment(const char* tile, int base, int block, int kk) {
-    return SlimTransposed<kI>::fragment(tile, base, block, kk);
+  static __device__ __forceinline__ bf16x8 fragment(const char* tile, int base, int /*block*/, int kk) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+    const char* ptr = tile + base + kk * (16 * 64);
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(ptr));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(ptr + 4 * 64));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(bf16x8, both);
   }
 };
 
