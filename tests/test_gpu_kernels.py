@@ -536,9 +536,16 @@ def test_fp8_weight_grouped_gemm_equals_the_dequantised_bf16_path(device):
     w = (torch.randn(len(counts), k, n, generator=g) * 0.02)
     q, scale = quantize_block_fp8(w.to(device))
     offs = _offsets(counts, device)
-    out = expert_gemm(x.to(device), BlockFp8Weight(q, scale), offs=offs)
+    weight = BlockFp8Weight(q, scale)
+    out = expert_gemm(x.to(device), weight, offs=offs, weight_cacheable=False)  # the kernel that reads the fp8 bytes
     deq = dequantize_block_fp8(q, scale)
     assert torch.equal(out, grouped_mm(x.to(device), deq, offs=offs))
+    # the route over a dequantised copy kept with the weight (taken from 64 rows per expert on) gives the same bits
+    assert weight._bf16 is None
+    assert torch.equal(expert_gemm(x.to(device), weight, offs=offs), out) and weight._bf16 is not None
+    few = x[:100].to(device)  # too few rows per expert: the fp8 kernel again
+    few_offs = _offsets((30, 0, 50, 20), device)
+    assert torch.equal(expert_gemm(few, BlockFp8Weight(q, scale), offs=few_offs), grouped_mm(few, deq, offs=few_offs))
     want_q, want_scale = fp8_oracle.quantize_block_fp8(w.numpy())
     w_ref = torch.from_numpy(fp8_oracle.dequantize_block_fp8(want_q, want_scale)).bfloat16()
     want = oracle.grouped_mm(x.double(), w_ref.double(), np.cumsum(counts).astype(np.int32), acc_dtype=torch.float64)

@@ -205,7 +205,11 @@ def test_quantised_weight_forward(device):
     with torch.no_grad():
         got = lowp._compute_experts(x, experts.to(device), weights.to(device), torch.bfloat16, recv_counts=counts)
         want = ref._compute_experts(x, experts.to(device), weights.to(device), torch.bfloat16, recv_counts=counts)
-    assert torch.equal(got, want)  # the dequantisation inside the kernel is exact
+    assert torch.equal(got, want)  # the dequantisation is exact, inside the kernel or ahead of it
+    lowp._lowp_weight_cacheable = False  # weights that may change under the layer: the fp8-reading kernel every time
+    with torch.no_grad():
+        again = lowp._compute_experts(x, experts.to(device), weights.to(device), torch.bfloat16, recv_counts=counts)
+    assert torch.equal(again, want)
 
 
 # ------------------------------------------------------------------------------ drop-ins for the Hugging Face blocks
