@@ -710,11 +710,13 @@ struct SlimDirect {  // element(out, con) = base[out * ld + con]; LDS [256 out][
   uint32_t voff;                // this lane's chunk for the wavefront's first load of a step, at step 0
   uint32_t t_stride;            // bytes between the rows of consecutive loads (8 rows)
   int con0, con_lim;
+  int t_lim;                    // loads t >= t_lim of this wavefront lie wholly past the operand's last row
 
-  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int /*out_lim*/,
+  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
                                        int con_lim_, int wave, int lane) {
     rsrc = make_rsrc_words(base, static_cast<uint32_t>(bytes));
     con_lim = con_lim_;
+    t_lim = (out_lim - out0 - wave * kI * 8 + 7) >> 3;
     const int logical = (lane & 7) ^ (lane >> 3);  // row & 7 == lane >> 3 for every load
     con0 = logical << 3;
     t_stride = 8u * static_cast<uint32_t>(ld) * 2u;
@@ -726,9 +728,17 @@ struct SlimDirect {  // element(out, con) = base[out * ld + con]; LDS [256 out][
                                         bool live = true) const {
     const uint32_t soff = live ? static_cast<uint32_t>(step) * (BK * 2) : 0u;
     const uint32_t base = live && step * BK + con0 < con_lim ? voff : kOutOfRange;
+    // A load whose eight rows all lie past the operand's end is left out: nothing reads those rows of the tile
+    // for a result that is kept (an output row takes its values from its own operand row only), and in a group's
+    // last, short row tile most loads are of that kind.
+    if (t_lim >= kI) {
 #pragma unroll
-    for (int t = 0; t < kI; ++t)
-      lds_load16(rsrc, tile + (wave * kI + t) * 1024, base + t * t_stride, soff);
+      for (int t = 0; t < kI; ++t) lds_load16(rsrc, tile + (wave * kI + t) * 1024, base + t * t_stride, soff);
+    } else {
+#pragma unroll
+      for (int t = 0; t < kI; ++t)
+        if (t < t_lim) lds_load16(rsrc, tile + (wave * kI + t) * 1024, base + t * t_stride, soff);
+    }
   }
   // per-lane byte address (within the operand tile) of the fragment of sub-step 0, block 0 of the wavefront
   static __device__ __forceinline__ int fragment_base(int row0, int lane) {
@@ -798,11 +808,13 @@ struct GatherDirect {  // LDS layout and fragments as SlimDirect
   u32x4 rsrc;
   uint32_t voff[kI];  // per load: this lane's chunk of its row at step 0, or out of range
   int con0, con_lim;
+  int t_lim;          // as in SlimDirect
 
   __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t a_rows, const int64_t* index, int out0,
                                        int out_lim, int con_lim_, int slot, int lane) {
     rsrc = make_rsrc_words(base, static_cast<uint32_t>(a_rows * ld * 2));
     con_lim = con_lim_;
+    t_lim = (out_lim - out0 - slot * kI * 8 + 7) >> 3;
     const int logical = (lane & 7) ^ (lane >> 3);
     con0 = logical << 3;
 #pragma unroll
@@ -817,9 +829,15 @@ struct GatherDirect {  // LDS layout and fragments as SlimDirect
                                         bool live = true) const {
     const uint32_t soff = live ? static_cast<uint32_t>(step) * (BK * 2) : 0u;
     const bool in_range = live && step * BK + con0 < con_lim;
+    if (t_lim >= kI) {
 #pragma unroll
-    for (int t = 0; t < kI; ++t)
-      lds_load16(rsrc, tile + (slot * kI + t) * 1024, in_range ? voff[t] : kOutOfRange, soff);
+      for (int t = 0; t < kI; ++t)
+        lds_load16(rsrc, tile + (slot * kI + t) * 1024, in_range ? voff[t] : kOutOfRange, soff);
+    } else {
+#pragma unroll
+      for (int t = 0; t < kI; ++t)
+        if (t < t_lim) lds_load16(rsrc, tile + (slot * kI + t) * 1024, in_range ? voff[t] : kOutOfRange, soff);
+    }
   }
   static __device__ __forceinline__ int fragment_base(int row0, int lane) {
     return SlimDirect<kI>::fragment_base(row0, lane);
@@ -1061,6 +1079,19 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
 #pragma unroll
     for (int i = 0; i < WM; ++i) fa[buf][i] = LoaderA::fragment(ta, fa_base[kDirectA ? 0 : i], i, kk);
   };
+  // the same for a tile whose last rows are missing: only the fragments of the `rows_live` row blocks that hold
+  // rows (a short tile's steps are otherwise bound by these reads: 64 per sub-step and CU whatever the row count)
+  auto read_live_fragments = [&](int stage, int kk, int buf, int rows_live) __attribute__((always_inline)) {
+    const char* ta = lds_raw + stage * kStageBytes;
+    const char* tb = ta + kTileBytes;
+    if (rows_live > 0) {
+#pragma unroll
+      for (int j = 0; j < WN; ++j) fb[buf][j] = LoaderB::fragment(tb, fb_base[kDirectB ? 0 : j], j, kk);
+    }
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+      if (i < rows_live) fa[buf][i] = LoaderA::fragment(ta, fa_base[kDirectA ? 0 : i], i, kk);
+  };
   constexpr int kReads = WM * (kDirectA ? 1 : 2) + WN * (kDirectB ? 1 : 2);  // LDS reads of one sub-step
   constexpr int kMfmas = WM * WN;
   constexpr int kEpiPitch = WN * 32 + 8;
@@ -1094,7 +1125,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     live = live < 0 ? 0 : (live > WM ? WM : live);
     if (load_wave) wait_loads();
     workgroup_barrier();  // step 0 of this tile has landed in stage 0
-    if (steps > 0) read_fragments(0, 0, 0);
+    if (steps > 0) read_live_fragments(0, 0, 0, live);
 
     auto run = [&](auto full_tag) __attribute__((always_inline)) {
       constexpr bool kFull = decltype(full_tag)::value;
@@ -1128,7 +1159,8 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         if constexpr (kRowsPerStep) next_rows0_loaded = !more && has_next;
 #pragma unroll
         for (int kk = 0; kk < 3; ++kk) {
-          read_fragments(cur, kk + 1, (kk + 1) & 1);
+          if constexpr (kFull) read_fragments(cur, kk + 1, (kk + 1) & 1);
+          else read_live_fragments(cur, kk + 1, (kk + 1) & 1, live);
           mfmas(kk & 1, 0, WM);
           if constexpr (kFull) {
             interleave_reads_under_mfmas<kReads, kMfmas>();
@@ -1140,7 +1172,10 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         if (load_wave) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         workgroup_barrier();
-        if (more) read_fragments(cur ^ 1, 0, 0);
+        if (more) {
+          if constexpr (kFull) read_fragments(cur ^ 1, 0, 0);
+          else read_live_fragments(cur ^ 1, 0, 0, live);
+        }
         mfmas(1, WM / 2, WM);
         if constexpr (kFull) interleave_reads_under_mfmas<kReads, kMfmas / 2>();
       }
