@@ -30,7 +30,8 @@ SIGNATURES = {
     "hmoe_gather_rows": (I, [P, L, P, L, L, I, P, P]),
     "hmoe_gather_reduce": (I, [P, P, P, L, I, L, L, I, P, P]),
     "hmoe_unpermute_bwd": (I, [P, L, P, P, P, L, L, I, P, P, P]),
-    "hmoe_expert_colsum": (I, [P, P, L, L, I, I, P, P]),
+    "hmoe_expert_colsum_workspace_bytes": (L, [L, L, I]),
+    "hmoe_expert_colsum": (I, [P, P, L, L, I, I, P, P, P]),
     "hmoe_glu_fwd": (I, [P, P, L, L, L, L, I, I, F, F, I, I, P, P]),
     "hmoe_glu_bwd": (I, [P, P, L, L, P, L, L, I, I, F, F, I, I, P, P, L, L, P]),
     "hmoe_router_topk_fwd": (I, [P, I, L, I, I, I, I, F, P, P, P]),

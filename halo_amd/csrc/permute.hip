@@ -46,6 +46,14 @@ struct Raw {
   __device__ __forceinline__ void store(T* p) const { *reinterpret_cast<V*>(p) = bits; }
 };
 
+// a chunk already in registers, as floats
+template <typename T, int W>
+__device__ __forceinline__ Pack<T, W> widen(const Raw<T, W>& raw) {
+  Pack<T, W> x;
+  x.load(reinterpret_cast<const T*>(&raw.bits));
+  return x;
+}
+
 template <typename T, int W>
 __global__ void __launch_bounds__(kThreads)
 gather_rows_kernel(const T* __restrict__ src, int64_t src_stride, const int64_t* __restrict__ index,
@@ -252,6 +260,143 @@ expert_colsum_kernel(const T* __restrict__ grad_out, const int64_t* __restrict__
   }
 }
 
+// The same sums in two launches, for 16-byte-aligned rows.  Expert loads can be very uneven (one expert holding a
+// quarter of the rows), and a workgroup per (expert, column chunk) then leaves most of the chip waiting for that
+// expert's few workgroups; here the rows are cut into blocks of 128 whatever expert they belong to.
+//   partial: grid (column chunks, row blocks).  A thread owns W columns and walks the block's rows, eight row loads in
+//            flight; the threads of a workgroup read a row side by side, so nothing is exchanged between lanes.  A
+//            row's expert id is the same for every thread (a scalar load); when it changes, the sum so far goes to
+//            row b + e of the fp32 workspace [row blocks + experts, width]: along the sorted rows the pairs
+//            (block, expert) form a staircase, so b + e names each pair once.
+//   final:   grid (experts, column chunks): expert e's row range by a 64-way search of the sorted ids, then the
+//            partial rows of the blocks it spans: four wavefronts add a quarter of them each in block order, the four
+//            sums are added in wavefront order and rounded once.
+// The order of every addition is fixed, so the result is reproducible bit for bit.
+constexpr int kColsumBlockRows = 128;
+constexpr int kPartialLoads = 8;
+static_assert(kColsumBlockRows % kPartialLoads == 0, "a block's rows come in whole batches");
+
+template <typename T, int W>
+__global__ void __launch_bounds__(1024)
+expert_colsum_partial_kernel(const T* __restrict__ grad_out, const int64_t* __restrict__ eids,
+                             float* __restrict__ partial, int64_t n_rows, int64_t width, int num_experts) {
+  const int64_t blk = blockIdx.y;
+  const int64_t row0 = blk * kColsumBlockRows;
+  const int64_t row_end = row0 + kColsumBlockRows < n_rows ? row0 + kColsumBlockRows : n_rows;
+  const int64_t c = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * W;
+  if (c >= width) return;
+  const T* col = grad_out + c;
+  float acc[W];
+#pragma unroll
+  for (int i = 0; i < W; ++i) acc[i] = 0.f;
+  int64_t current = -1;
+  auto flush = [&]() {
+    if (current >= 0 && current < num_experts) {
+      float4* to = reinterpret_cast<float4*>(partial + (blk + current) * width + c);  // W is 4 or 8: 16-byte aligned
+#pragma unroll
+      for (int i = 0; i < W / 4; ++i) to[i] = make_float4(acc[4 * i], acc[4 * i + 1], acc[4 * i + 2], acc[4 * i + 3]);
+    }
+  };
+  for (int64_t r = row0; r < row_end; r += kPartialLoads) {
+    // all the batch's loads go out before the first is used: past the block's end they repeat its last row, whose
+    // values are then left out below
+    Raw<T, W> raw[kPartialLoads];
+    int64_t id[kPartialLoads];
+#pragma unroll
+    for (int t = 0; t < kPartialLoads; ++t) {
+      const int64_t row = r + t < row_end ? r + t : row_end - 1;  // the same for every thread
+      id[t] = eids[row];
+      raw[t].load(col + row * width);
+    }
+#pragma unroll
+    for (int t = 0; t < kPartialLoads; ++t) {
+      if (r + t >= row_end) break;
+      if (id[t] != current) {
+        flush();
+        current = id[t];
+#pragma unroll
+        for (int i = 0; i < W; ++i) acc[i] = 0.f;
+      }
+      const Pack<T, W> x = widen(raw[t]);
+#pragma unroll
+      for (int i = 0; i < W; ++i) acc[i] += x.v[i];
+    }
+  }
+  flush();
+}
+
+// First index of the sorted ids that holds `key` or more, found by the wavefront together: 64 probes a round.
+__device__ __forceinline__ int64_t wave_lower_bound(const int64_t* __restrict__ ids, int64_t n, int64_t key) {
+  int64_t lo = 0, len = n;  // the answer lies in [lo, lo + len]
+  while (len > 0) {
+    const int64_t step = (len + HMOE_WAVE - 1) / HMOE_WAVE;
+    int64_t last = (static_cast<int64_t>(lane_id()) + 1) * step;  // this lane's chunk ends before lo + last
+    if (last > len) last = len;
+    const bool below = ids[lo + last - 1] < key;
+    const int chunks_below = __popcll(__ballot(below));
+    if (chunks_below * step >= len) return lo + len;
+    lo += chunks_below * step;
+    const int64_t rest = len - chunks_below * step;
+    len = (rest < step ? rest : step) - 1;  // the chunk's last id is `key` or more: the answer is it or before it
+  }
+  return lo;
+}
+
+// W is 4 or 8.  Four wavefronts share a column chunk of 64 W columns; each adds a quarter of the expert's blocks in
+// block order, and the four sums are added in wavefront order.
+template <typename T, int W>
+__global__ void __launch_bounds__(256)
+expert_colsum_final_kernel(const float* __restrict__ partial, const int64_t* __restrict__ eids,
+                           T* __restrict__ grad_bias, int64_t n_rows, int64_t width) {
+  __shared__ float quarter[4][HMOE_WAVE * W];
+  const int e = blockIdx.x;
+  const int wave = threadIdx.x / HMOE_WAVE;
+  const int64_t begin = wave_lower_bound(eids, n_rows, e);
+  const int64_t end = wave_lower_bound(eids, n_rows, static_cast<int64_t>(e) + 1);
+  const int64_t c = (static_cast<int64_t>(blockIdx.y) * HMOE_WAVE + lane_id()) * W;
+  float sum[W];
+#pragma unroll
+  for (int i = 0; i < W; ++i) sum[i] = 0.f;
+  if (begin < end && c < width) {
+    const int64_t b_first = begin / kColsumBlockRows, b_last = (end - 1) / kColsumBlockRows + 1;
+    const int64_t per_wave = (b_last - b_first + 3) / 4;
+    const int64_t b0 = b_first + wave * per_wave;
+    const int64_t b_end = b0 + per_wave < b_last ? b0 + per_wave : b_last;
+    for (int64_t b = b0; b < b_end; b += 8) {  // eight partial rows in flight
+      float4 part[8][W / 4];
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const float4* from = reinterpret_cast<const float4*>(partial + (b + t + e) * width + c);
+#pragma unroll
+        for (int i = 0; i < W / 4; ++i) part[t][i] = b + t < b_end ? from[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        if (b + t < b_end) {
+#pragma unroll
+          for (int i = 0; i < W / 4; ++i) {
+            sum[4 * i] += part[t][i].x;
+            sum[4 * i + 1] += part[t][i].y;
+            sum[4 * i + 2] += part[t][i].z;
+            sum[4 * i + 3] += part[t][i].w;
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < W; ++i) quarter[wave][lane_id() * W + i] = sum[i];
+  __syncthreads();
+  if (wave == 0 && c < width) {
+    Pack<T, W> total;
+#pragma unroll
+    for (int i = 0; i < W; ++i)
+      total.v[i] = ((quarter[0][lane_id() * W + i] + quarter[1][lane_id() * W + i]) + quarter[2][lane_id() * W + i]) +
+                   quarter[3][lane_id() * W + i];
+    total.store(grad_bias + static_cast<int64_t>(e) * width + c);
+  }
+}
+
 template <typename T>
 bool rows_vectorizable(int64_t hidden, std::initializer_list<int64_t> strides, std::initializer_list<const void*> ptrs) {
   constexpr int W = 16 / sizeof(T);
@@ -352,14 +497,52 @@ int hmoe_unpermute_bwd(const void* grad_out, int64_t grad_out_row_stride, const 
   return HMOE_OK;
 }
 
+int64_t hmoe_expert_colsum_workspace_bytes(int64_t n_rows, int64_t width, int num_experts) {
+  if (n_rows < 0 || width < 0 || num_experts < 0) return 0;
+  const int64_t blocks = (n_rows + kColsumBlockRows - 1) / kColsumBlockRows;
+  return (blocks + num_experts) * width * static_cast<int64_t>(sizeof(float));
+}
+
 int hmoe_expert_colsum(const void* grad_out, const int64_t* eids, int64_t n_rows, int64_t width, int num_experts,
-                       int dtype, void* grad_bias, void* stream) {
+                       int dtype, void* grad_bias, void* workspace, void* stream) {
   if (n_rows < 0 || width < 0 || num_experts < 0) return HMOE_INVALID_ARGUMENT;
   if (num_experts == 0 || width == 0) return HMOE_OK;
   if (!grad_bias || (n_rows > 0 && (!grad_out || !eids))) return HMOE_INVALID_ARGUMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool vec = dtype == HMOE_BF16 ? rows_vectorizable<bf16_t>(width, {}, {grad_out, grad_bias})
                                       : rows_vectorizable<float>(width, {}, {grad_out, grad_bias});
+  if (vec && workspace != nullptr && aligned16(workspace)) {
+    const unsigned blocks = static_cast<unsigned>((n_rows + kColsumBlockRows - 1) / kColsumBlockRows);
+    float* partial = static_cast<float*>(workspace);
+    if (dtype == HMOE_BF16) {
+      using T = bf16_t;
+      constexpr int W = 8;
+      const int64_t packs = width / W;
+      const unsigned threads = packs >= 1024 ? 1024u : static_cast<unsigned>((packs + HMOE_WAVE - 1) / HMOE_WAVE * HMOE_WAVE);
+      if (blocks > 0)
+        expert_colsum_partial_kernel<T, W><<<dim3(static_cast<unsigned>((packs + threads - 1) / threads), blocks),
+                                             dim3(threads), 0, s>>>(
+            static_cast<const T*>(grad_out), eids, partial, n_rows, width, num_experts);
+      expert_colsum_final_kernel<T, W><<<dim3(num_experts, (width + HMOE_WAVE * W - 1) / (HMOE_WAVE * W)), dim3(256), 0, s>>>(
+          partial, eids, static_cast<T*>(grad_bias), n_rows, width);
+    } else if (dtype == HMOE_F32) {
+      using T = float;
+      constexpr int W = 4;
+      const int64_t packs = width / W;
+      const unsigned threads = packs >= 1024 ? 1024u : static_cast<unsigned>((packs + HMOE_WAVE - 1) / HMOE_WAVE * HMOE_WAVE);
+      if (blocks > 0)
+        expert_colsum_partial_kernel<T, W><<<dim3(static_cast<unsigned>((packs + threads - 1) / threads), blocks),
+                                             dim3(threads), 0, s>>>(
+            static_cast<const T*>(grad_out), eids, partial, n_rows, width, num_experts);
+      expert_colsum_final_kernel<T, W><<<dim3(num_experts, (width + HMOE_WAVE * W - 1) / (HMOE_WAVE * W)), dim3(256), 0, s>>>(
+          partial, eids, static_cast<T*>(grad_bias), n_rows, width);
+    } else {
+      return HMOE_UNSUPPORTED;
+    }
+    HMOE_CHECK_LAUNCH();
+    return HMOE_OK;
+  }
+  // rows that are not 16-byte aligned, or no workspace: one workgroup per (expert, column chunk)
   HMOE_DISPATCH_ROWS(dtype, vec,
                      (expert_colsum_kernel<T, W><<<dim3(num_experts, (width + kColsumLanesPerRow * W - 1) /
                                                                          (kColsumLanesPerRow * W)),

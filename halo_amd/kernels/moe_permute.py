@@ -141,9 +141,13 @@ class MoEExpertBiasGather(torch.autograd.Function):
         grad_out = grad_out.contiguous()
         eids = eids.long().contiguous()
         grad_bias = torch.empty((ctx.num_experts, grad_out.shape[1]), dtype=grad_out.dtype, device=device)
+        lib = _lib.load()
+        ws_bytes = lib.hmoe_expert_colsum_workspace_bytes(grad_out.shape[0], grad_out.shape[1], ctx.num_experts)
+        workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=device)
         with _lib.on_device(device):
             _lib.call("hmoe_expert_colsum", _lib.ptr(grad_out), _lib.ptr(eids), grad_out.shape[0], grad_out.shape[1],
-                      ctx.num_experts, _lib.dtype_id(grad_out.dtype), _lib.ptr(grad_bias), _lib.stream_ptr(device))
+                      ctx.num_experts, _lib.dtype_id(grad_out.dtype), _lib.ptr(grad_bias), _lib.ptr(workspace),
+                      _lib.stream_ptr(device))
         return grad_bias, None
 
 

@@ -93,9 +93,14 @@ int hmoe_unpermute_bwd(const void* grad_out, int64_t grad_out_row_stride, const 
 
 /* Replaces MoEExpertBiasGather.backward (one-hot GEMM): halo/kernels/moe_permute.py:202-208.
  * grad_bias[e, :] = sum of grad_out rows j with eids[j] == e, fp32 accumulate in row order, one rounding.
- * eids must be non-decreasing (expert-sorted rows, the only order the expert path produces). */
+ * eids must be non-decreasing (expert-sorted rows, the only order the expert path produces).
+ * workspace: hmoe_expert_colsum_workspace_bytes(...) bytes, 16-byte aligned, or NULL.  With it (and 16-byte-aligned
+ * rows) the rows are summed in blocks of 128 whatever their expert and the block sums added per expert in block order,
+ * two launches, so that one overloaded expert does not hold the launch up; without it, one workgroup per (expert,
+ * column chunk).  Either way the order of the additions is fixed. */
+int64_t hmoe_expert_colsum_workspace_bytes(int64_t n_rows, int64_t width, int num_experts);
 int hmoe_expert_colsum(const void* grad_out, const int64_t* eids, int64_t n_rows, int64_t width, int num_experts,
-                       int dtype, void* grad_bias, void* stream);
+                       int dtype, void* grad_bias, void* workspace, void* stream);
 
 /* --------------------------------------------------------------------------------------------------- fused GLU
  * Replaces _glu_fwd_kernel / _glu_bwd_kernel: halo/kernels/fused_glu.py:118-205.  gate/up (and dgate/dup) are

@@ -272,6 +272,49 @@ def test_expert_bias_gather(device, rows, width, skew):
         want = oracle.bias_gather_backward(grad.double(), eids, 32)
         assert max_rel(bd.grad, want) < tol
         assert not bd.grad[7].any() and not bd.grad[31].any()
+        # the same sums without a workspace (one workgroup per expert and column chunk), through the C-ABI
+        plain = _colsum_without_workspace(grad.to(device), eids.to(device), 32)
+        assert max_rel(plain, want) < tol
+        assert not plain[7].any() and not plain[31].any()
+
+
+def _colsum_without_workspace(grad, eids, num_experts):
+    from halo_amd import _lib
+
+    out = torch.empty((num_experts, grad.shape[1]), dtype=grad.dtype, device=grad.device)
+    with _lib.on_device(grad.device):
+        _lib.call("hmoe_expert_colsum", _lib.ptr(grad), _lib.ptr(eids), grad.shape[0], grad.shape[1], num_experts,
+                  _lib.dtype_id(grad.dtype), _lib.ptr(out), None, _lib.stream_ptr(grad.device))
+    return out
+
+
+def test_expert_bias_gradient_in_row_blocks(device):
+    """The blocked column sums: expert boundaries on and off the 512-row block edges, an expert spanning many blocks,
+    many experts inside one block, idle experts first, in the middle and last; twice the same bits."""
+    from halo_amd.kernels.moe_permute import MoEExpertBiasGather
+    from oracle import permute as oracle
+
+    counts = [0, 512, 512, 0, 0, 1, 3000, 7, 0, 505, 1024, 1, 1, 1, 0, 2, 600, 0]
+    eids = torch.repeat_interleave(torch.arange(len(counts)), torch.tensor(counts))
+    g = torch.Generator().manual_seed(11)
+    for dtype, tol in DTYPE_TOLS:
+        for width in (64, 2880, 72):
+            grad = torch.randn(eids.numel(), width, generator=g).to(dtype)
+            bias = torch.zeros(len(counts), width, dtype=dtype, device=device, requires_grad=True)
+            results = []
+            for _ in range(2):
+                bias.grad = None
+                MoEExpertBiasGather.apply(bias, eids.to(device)).backward(grad.to(device))
+                results.append(bias.grad.clone())
+            assert torch.equal(results[0], results[1])
+            want = oracle.bias_gather_backward(grad.double(), eids, len(counts))
+            assert max_rel(results[0], want) < tol
+            for e, n in enumerate(counts):
+                if n == 0:
+                    assert not results[0][e].any()
+                elif n == 1:  # a single row comes through untouched
+                    row = int(sum(counts[:e]))
+                    assert torch.equal(results[0][e].cpu(), grad[row])
 
 
 # ---------------------------------------------------------------------------------------------------- fused GLU
