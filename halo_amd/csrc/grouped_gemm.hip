@@ -93,6 +93,7 @@ struct GemmArgs {
   const float* b_scale;  // kFwdFp8W: [G, ceil(K/128), ceil(N/128)]
   const int64_t* a_index = nullptr;  // gathered A (fwd, wgrad): logical row r of A is a[a_index[r]]
   int64_t a_rows = 0;                // rows of the array a_index points into
+  const void* bias = nullptr;        // fwd: [G, N] in the operands' dtype, added to group g's output rows
 };
 
 __device__ __forceinline__ int swizzle(int row) { return (row & 7) ^ ((row >> 3) & 7); }
@@ -158,6 +159,18 @@ __device__ __forceinline__ void lds_load16(u32x4 rsrc, lds_bytes_ptr lds_base, u
                : "s"(uniform(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_base)))), "v"(voffset),
                  "s"(uniform(rsrc)), "s"(uniform(soffset))
                : "memory");
+}
+
+// Eight bf16 values plus eight more, each sum rounded to bf16: what a bf16 tensor addition does element by element.
+__device__ __forceinline__ u32x4 add_bf16x8(u32x4 a, u32x4 b) {
+  u32x4 out;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float lo = __uint_as_float(a[w] << 16) + __uint_as_float(b[w] << 16);
+    const float hi = __uint_as_float(a[w] & 0xffff0000u) + __uint_as_float(b[w] & 0xffff0000u);
+    out[w] = static_cast<uint32_t>(f32_to_bf16(lo)) | (static_cast<uint32_t>(f32_to_bf16(hi)) << 16);
+  }
+  return out;
 }
 
 // every direct-to-LDS load of this wavefront has landed
@@ -959,9 +972,10 @@ __device__ __forceinline__ void interleave_reads_under_mfmas() {
   }
 }
 
-template <int kMode, typename Cfg, bool kGather = false>
+template <int kMode, typename Cfg, bool kGather = false, bool kBias = false>
 __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmArgs p) {
   static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
+  static_assert(!kBias || kMode == kFwd, "the expert bias belongs to the forward product");
   static_assert(!kGather || kMode == kFwd || kMode == kWgrad, "A is gathered in fwd and wgrad");
   constexpr int WM = Cfg::WM, WN = Cfg::WN, BM = Cfg::BM, BN = Cfg::BN;
   constexpr int kWaves = Cfg::GM * Cfg::GN;
@@ -1123,7 +1137,18 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     const int steps = (tile.con_lim + BK - 1) / BK;
     int live = (tile.a_out_lim - (tile.a_out0 + row_a) + 31) >> 5;
     live = live < 0 ? 0 : (live > WM ? WM : live);
+    // The expert's bias for this lane's eight output columns (the same columns in every store of the epilogue).  It
+    // is fetched here, where the tile's first loads are waited for anyway, and pinned as arrived right behind that
+    // wait: a wait placed by the compiler at its first use, in the epilogue, would be for every load in flight, the
+    // next tile's first step among them.
+    u32x4 bias_chunk = {0u, 0u, 0u, 0u};
+    if constexpr (kBias) {
+      const int col = tile.b_out0 + row_b + ((lane % kLanesPerRow) << 3);
+      if (col < tile.b_out_lim)
+        bias_chunk = *reinterpret_cast<const u32x4*>(static_cast<const bf16_t*>(p.bias) + tile.g * p.n + col);
+    }
     if (load_wave) wait_loads();
+    if constexpr (kBias) asm volatile("" : "+v"(bias_chunk));
     workgroup_barrier();  // step 0 of this tile has landed in stage 0
     if (steps > 0) read_live_fragments(0, 0, 0, live);
 
@@ -1223,7 +1248,8 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
           const int cc = (lane % kLanesPerRow) << 3;
           const int row = done.a_out0 + row_a + i * 32 + rr;
           const int col = done.b_out0 + row_b + cc;
-          const u32x4 v = *reinterpret_cast<const u32x4*>(stage_rows + (rr * kEpiPitch + cc) * 2);
+          u32x4 v = *reinterpret_cast<const u32x4*>(stage_rows + (rr * kEpiPitch + cc) * 2);
+          if constexpr (kBias) v = add_bf16x8(v, bias_chunk);
           const uint32_t off = row < done.a_out_lim && col < done.b_out_lim
                                    ? static_cast<uint32_t>(row) * static_cast<uint32_t>(p.ldc) * 2u + col * 2u
                                    : kOutOfRange;
@@ -1243,6 +1269,7 @@ HMOE_BF16_INSTANCE(kDgrad)
 HMOE_BF16_INSTANCE(kWgrad)
 #undef HMOE_BF16_INSTANCE
 template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, true>(GemmArgs);
+template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, false, true>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kWgrad, Config<2, 4, 4, 2>, true>(GemmArgs);
 
 // ------------------------------------------------------------------------------------------------ fp32 path
@@ -1326,7 +1353,11 @@ __global__ void __launch_bounds__(256) grouped_gemm_f32_kernel(GemmArgs p) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int64_t r = row0 + ty * 4 + i, cc = col0 + tx * 4 + j;
-      if (r < rows_out && cc < cols_out) out[r * p.ldc + cc] = acc[i][j];
+      if (r < rows_out && cc < cols_out) {
+        float v = acc[i][j];
+        if (kMode == kFwd && p.bias != nullptr) v += static_cast<const float*>(p.bias)[static_cast<int64_t>(g) * p.n + cc];
+        out[r * p.ldc + cc] = v;
+      }
     }
 }
 
@@ -1363,7 +1394,7 @@ int launch_staged(const GemmArgs& p, int workgroups_per_cu, hipStream_t stream) 
   return HMOE_OK;
 }
 
-template <int kMode, typename Cfg, bool kGather = false>
+template <int kMode, typename Cfg, bool kGather = false, bool kBias = false>
 int launch_direct(const GemmArgs& p, hipStream_t stream) {
   const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
   const int64_t nt = (out_cols + Cfg::BN - 1) / Cfg::BN;
@@ -1376,7 +1407,7 @@ int launch_direct(const GemmArgs& p, hipStream_t stream) {
   if (workers <= 0) return HMOE_OK;
   // two stages; the gathered wgrad keeps 2 x 1 KB of row indices per loading wavefront behind them
   constexpr size_t lds_bytes = 2 * Cfg::kStage * sizeof(bf16_t) + (kGather && kMode == kWgrad ? 4 * 2048 : 0);
-  auto kernel = grouped_gemm_bf16_kernel<kMode, Cfg, kGather>;
+  auto kernel = grouped_gemm_bf16_kernel<kMode, Cfg, kGather, kBias>;
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                           static_cast<int>(lds_bytes)) != hipSuccess)
     return HMOE_LAUNCH_FAILED;
@@ -1391,7 +1422,11 @@ int launch(const GemmArgs& p, int dtype, hipStream_t stream) {
     int rc;
     if constexpr (kMode == kFwdFp8W) {
       rc = launch_staged<kMode, Tile>(p, 1, stream);
-    } else if constexpr (kMode == kFwd || kMode == kWgrad) {
+    } else if constexpr (kMode == kFwd) {
+      rc = p.a_index ? launch_direct<kMode, Tile, true>(p, stream)
+           : p.bias  ? launch_direct<kMode, Tile, false, true>(p, stream)
+                     : launch_direct<kMode, Tile>(p, stream);
+    } else if constexpr (kMode == kWgrad) {
       rc = p.a_index ? launch_direct<kMode, Tile, true>(p, stream) : launch_direct<kMode, Tile>(p, stream);
     } else {
       rc = launch_direct<kMode, Tile>(p, stream);
@@ -1445,6 +1480,20 @@ int hmoe_grouped_gemm_fwd(const void* a, int64_t lda, const void* b, const int32
   if (total_rows == 0 || n == 0) return HMOE_OK;
   if (!a || !b || !out) return HMOE_INVALID_ARGUMENT;
   if (lda < k || ldo < n) return HMOE_INVALID_ARGUMENT;
+  return launch<kFwd>(p, dtype, static_cast<hipStream_t>(stream));
+}
+
+int hmoe_grouped_gemm_fwd_bias(const void* a, int64_t lda, const void* b, const void* bias, const int32_t* offs,
+                               int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype, void* out,
+                               int64_t ldo, void* stream) {
+  using namespace hmoe;
+  GemmArgs p{a, lda, b, n, out, ldo, offs, total_rows, num_groups, k, n, nullptr};
+  p.bias = bias;
+  if (int rc = validate(p, dtype)) return rc;
+  if (total_rows == 0 || n == 0) return HMOE_OK;
+  if (!a || !b || !out || !bias) return HMOE_INVALID_ARGUMENT;
+  if (lda < k || ldo < n) return HMOE_INVALID_ARGUMENT;
+  if (dtype == HMOE_BF16 && !aligned16(bias)) return HMOE_UNSUPPORTED;
   return launch<kFwd>(p, dtype, static_cast<hipStream_t>(stream));
 }
 

@@ -148,6 +148,59 @@ def grouped_mm(mat_a, mat_b, *, offs=None):
     return _GroupedMMFunction.apply(mat_a, mat_b, offs)
 
 
+# ------------------------------------------------------------------------------------ expert bias in the epilogue
+
+def bias_fusable(mat_a: torch.Tensor, mat_b, bias) -> bool:
+    """Whether ``grouped_mm_bias`` can take these operands: a plain contiguous ``[G, K, N]`` weight and a ``[G, N]``
+    bias on the device, all of ``mat_a``'s dtype (bf16 or fp32)."""
+    return (isinstance(mat_b, torch.Tensor) and isinstance(bias, torch.Tensor) and mat_a.is_cuda
+            and mat_a.dtype in (torch.bfloat16, torch.float32) and mat_b.dtype == mat_a.dtype
+            and bias.dtype == mat_a.dtype and mat_a.dim() == 2 and mat_b.dim() == 3 and mat_b.is_contiguous()
+            and bias.dim() == 2 and bias.shape == (mat_b.shape[0], mat_b.shape[2]) and mat_a.shape[1] == mat_b.shape[1])
+
+
+class _GroupedMMBias(Function):
+    """``grouped_mm(mat_a, mat_b, offs) + bias[eids]`` as one node: the GEMM's epilogue adds the expert's bias row
+    (``hmoe_grouped_gemm_fwd_bias``), rounding the product first and the sum again as the two tensor operations do
+    (reference ``families/gpt_oss.py:153-159``: ``_expert_proj`` then ``+ MoEExpertBiasGather.apply(bias, eids)``), so
+    neither the gathered ``[R, N]`` bias nor the sum's extra pass exists.  The bias gradient is the per-expert column
+    sum of ``grad_output``, as ``MoEExpertBiasGather.backward`` computes it."""
+
+    @staticmethod
+    def forward(ctx, mat_a, mat_b, bias, offs, eids):
+        device = _lib.require_device(mat_a, mat_b, bias, offs, eids)
+        groups, k, n = mat_b.shape
+        rows = mat_a.shape[0]
+        offs32 = _offs_arg(offs, groups)
+        ctx.save_for_backward(mat_a, mat_b, offs32, eids)
+        out = torch.empty((rows, n), dtype=mat_a.dtype, device=device)
+        if rows == 0 or n == 0:
+            return out
+        a = _rows(mat_a)
+        bias = bias.contiguous()
+        with _lib.on_device(device):
+            _lib.call("hmoe_grouped_gemm_fwd_bias", _lib.ptr(a), a.stride(0), _lib.ptr(mat_b), _lib.ptr(bias),
+                      _lib.ptr(offs32), rows, groups, k, n, _lib.dtype_id(mat_a.dtype), _lib.ptr(out), out.stride(0),
+                      _lib.stream_ptr(device))
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from halo_amd.kernels.moe_permute import expert_bias_grad
+
+        mat_a, mat_b, offs32, eids = ctx.saved_tensors
+        grad_a, grad_b = grouped_mm_grads(mat_a, mat_b, grad_output, offs32, ctx.needs_input_grad[0],
+                                          ctx.needs_input_grad[1])
+        grad_bias = expert_bias_grad(grad_output, eids, mat_b.shape[0]) if ctx.needs_input_grad[2] else None
+        return grad_a, grad_b, grad_bias, None, None
+
+
+def grouped_mm_bias(mat_a, mat_b, bias, *, offs, eids):
+    """``grouped_mm(mat_a, mat_b, offs=offs) + bias[eids]`` with ``eids`` the sorted expert id of every row (the ids
+    ``offs`` are the ends of); see ``bias_fusable`` for the operands it takes."""
+    return _GroupedMMBias.apply(mat_a, mat_b, bias, offs, eids)
+
+
 # ------------------------------------------------------------------------------------- permute folded into the GEMM
 
 def gather_fusable(tokens: torch.Tensor, mat_b) -> bool:

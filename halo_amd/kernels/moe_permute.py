@@ -124,6 +124,24 @@ class MoEWeightedUnpermute(torch.autograd.Function):
         return grad_expert, grad_weights.to(weights.dtype) if ctx.weight_grad else None, None, None
 
 
+def expert_bias_grad(grad_out: torch.Tensor, eids: torch.Tensor, num_experts: int) -> torch.Tensor:
+    """``[num_experts, width]``: per expert, the sum of the rows of ``grad_out`` that belong to it (``eids`` sorted),
+    accumulated in fp32 in a fixed order and rounded once; an expert without rows gets exact zeros.  What the
+    reference computes as ``onehot(eids)^T @ grad_out`` (``moe_permute.py:202-208``)."""
+    device = _lib.require_device(grad_out, eids)
+    grad_out = grad_out.contiguous()
+    eids = eids.long().contiguous()
+    grad_bias = torch.empty((num_experts, grad_out.shape[1]), dtype=grad_out.dtype, device=device)
+    lib = _lib.load()
+    ws_bytes = lib.hmoe_expert_colsum_workspace_bytes(grad_out.shape[0], grad_out.shape[1], num_experts)
+    workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=device)
+    with _lib.on_device(device):
+        _lib.call("hmoe_expert_colsum", _lib.ptr(grad_out), _lib.ptr(eids), grad_out.shape[0], grad_out.shape[1],
+                  num_experts, _lib.dtype_id(grad_out.dtype), _lib.ptr(grad_bias), _lib.ptr(workspace),
+                  _lib.stream_ptr(device))
+    return grad_bias
+
+
 class MoEExpertBiasGather(torch.autograd.Function):
     """``bias[eids]`` to expert-sorted tokens; ``grad_bias`` is the per-expert column sum of the incoming gradient,
     accumulated in fp32 in row order (no atomics).  ``eids`` must be non-decreasing, as the routing sort emits them."""
@@ -137,18 +155,7 @@ class MoEExpertBiasGather(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         (eids,) = ctx.saved_tensors
-        device = _lib.require_device(grad_out, eids)
-        grad_out = grad_out.contiguous()
-        eids = eids.long().contiguous()
-        grad_bias = torch.empty((ctx.num_experts, grad_out.shape[1]), dtype=grad_out.dtype, device=device)
-        lib = _lib.load()
-        ws_bytes = lib.hmoe_expert_colsum_workspace_bytes(grad_out.shape[0], grad_out.shape[1], ctx.num_experts)
-        workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=device)
-        with _lib.on_device(device):
-            _lib.call("hmoe_expert_colsum", _lib.ptr(grad_out), _lib.ptr(eids), grad_out.shape[0], grad_out.shape[1],
-                      ctx.num_experts, _lib.dtype_id(grad_out.dtype), _lib.ptr(grad_bias), _lib.ptr(workspace),
-                      _lib.stream_ptr(device))
-        return grad_bias, None
+        return expert_bias_grad(grad_out, eids, ctx.num_experts), None
 
 
 def warm_permute_kernels(num_tokens: int, hidden: int, top_k: int, device: torch.device, dtype: torch.dtype) -> None:

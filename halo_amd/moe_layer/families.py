@@ -11,6 +11,7 @@ import torch
 import torch.nn as nn
 
 from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled
+from halo_amd.kernels.grouped_mm import bias_fusable, grouped_mm_bias
 from halo_amd.kernels.moe_permute import MoEExpertBiasGather
 from halo_amd.kernels.router import SOFTMAX_TOPK, fused_topk_gate
 from halo_amd.moe_layer.config import GPT_OSS, QWEN3, QWEN3_5
@@ -124,8 +125,14 @@ class EPGptOssMoELayer(EPMoELayerBase):
         return self._grouped_proj_with_bias(gated.to(output_dtype), "down_proj", offs, output_dtype, sorted_expert_ids)
 
     def _grouped_proj_with_bias(self, x, weight_attr, offs, out_dtype, eids):
-        out = self._expert_proj(x, weight_attr, offs, out_dtype)
         bias = getattr(self, f"{weight_attr}_bias", None)
+        weight = getattr(self, weight_attr)
+        if (bias is not None and getattr(self, "fuse_bias_into_gemm", True) and self._lowp_quant_format is None
+                and isinstance(weight, torch.Tensor) and isinstance(x, torch.Tensor)):
+            weight, bias_cast = weight.to(out_dtype), bias.to(out_dtype)
+            if bias_fusable(x, weight, bias_cast):  # the projection and its bias in one kernel, the same bits
+                return grouped_mm_bias(x, weight, bias_cast, offs=offs, eids=eids)
+        out = self._expert_proj(x, weight_attr, offs, out_dtype)
         return out if bias is None else out + MoEExpertBiasGather.apply(bias.to(out_dtype), eids)
 
 

@@ -141,6 +141,14 @@ int hmoe_grouped_gemm_wgrad(const void* a, int64_t lda, const void* grad_out, in
                             int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype, void* grad_b,
                             void* stream);
 
+/* The forward GEMM plus the expert's bias row: replaces `out + MoEExpertBiasGather.apply(bias, eids)` behind a grouped
+ * projection (halo/distributed/expert_parallel/families/gpt_oss.py:153-159 with halo/kernels/moe_permute.py:192-200).
+ * bias is [num_groups, N] in dtype; rows of group g get bias[g].  The product is rounded to dtype first and the sum
+ * rounded again, as the two tensor operations it replaces do, so the result is theirs bit for bit. */
+int hmoe_grouped_gemm_fwd_bias(const void* a, int64_t lda, const void* b, const void* bias, const int32_t* offs,
+                               int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype, void* out,
+                               int64_t ldo, void* stream);
+
 /* The same two GEMMs with the rows of A gathered: logical row r of A is a[row_index[r]], a holding a_rows rows; an
  * index outside [0, a_rows) reads as a row of zeros.  This folds MoEGatherPermute.forward
  * (halo/kernels/moe_permute.py:133-136, tokens.index_select(0, sorted_token_idx)) into the first expert GEMM and its
