@@ -29,6 +29,7 @@ SIGNATURES = {
     "hmoe_bincount": (I, [P, P, L, I, I, P, P]),
     "hmoe_gather_rows": (I, [P, L, P, L, L, I, P, P]),
     "hmoe_gather_reduce": (I, [P, P, P, L, I, L, L, I, P, P]),
+    "hmoe_gather_reduce_add": (I, [P, P, P, L, I, L, L, I, P, L, P, P, P]),
     "hmoe_unpermute_bwd": (I, [P, L, P, P, P, L, L, I, P, P, P]),
     "hmoe_expert_colsum_workspace_bytes": (L, [L, L, I]),
     "hmoe_expert_colsum": (I, [P, P, L, L, I, I, P, P, P]),

@@ -32,12 +32,14 @@ struct Elem<float> {
   static constexpr int kVec = 4;  // elements per 16-byte access
   __device__ static __forceinline__ float load(const float* p) { return *p; }
   __device__ static __forceinline__ void store(float* p, float v) { *p = v; }
+  __device__ static __forceinline__ float round(float v) { return v; }  // the value a store and a load would give
 };
 template <>
 struct Elem<bf16_t> {
   static constexpr int kVec = 8;
   __device__ static __forceinline__ float load(const bf16_t* p) { return bf16_to_f32(*p); }
   __device__ static __forceinline__ void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+  __device__ static __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
 };
 
 // 16 bytes of T as floats.

@@ -91,13 +91,28 @@ gather_rows_kernel(const T* __restrict__ src, int64_t src_stride, const int64_t*
 template <typename T, int W, bool kWeighted, int kTopK>
 __global__ void __launch_bounds__(kThreads)
 gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, const int64_t* __restrict__ inv_map,
-                     T* __restrict__ out, int64_t n_out, int top_k, int64_t n_src, int64_t hidden) {
+                     T* __restrict__ out, int64_t n_out, int top_k, int64_t n_src, int64_t hidden,
+                     const T* __restrict__ addend, int64_t addend_stride, const T* __restrict__ addend_scale) {
   const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock +
                       __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / HMOE_WAVE);
   if (row >= n_out) return;
   const int64_t* map = inv_map + row * top_k;
   T* to = out + row * hidden;
   const int64_t step = static_cast<int64_t>(HMOE_WAVE) * W;
+  // Optional second term: out[r] = round(round(sum) + round(scale[r] * addend[r])), each rounding where the tensor
+  // operations `sum + scale * addend` round (the shared expert's output added to the routed one).
+  const T* extra = addend ? addend + row * addend_stride : nullptr;
+  const float extra_scale = addend_scale ? Elem<T>::load(addend_scale + row) : 1.f;
+  auto finish = [&](Pack<T, W>& acc, const Pack<T, W>& term) {
+    if (extra) {
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        float t = term.v[i];
+        if (addend_scale) t = Elem<T>::round(__fmul_rn(extra_scale, t));
+        acc.v[i] = __fadd_rn(Elem<T>::round(acc.v[i]), t);
+      }
+    }
+  };
   if constexpr (kTopK > 0) {
     const T* from[kTopK];
     float w[kTopK];
@@ -111,9 +126,10 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
       if constexpr (kWeighted) w[k] = Elem<T>::load(weight + (valid[k] ? j : 0));
     }
     for (int64_t c = static_cast<int64_t>(lane_id()) * W; c < hidden; c += step) {
-      Pack<T, W> x[kTopK], acc;
+      Pack<T, W> x[kTopK], acc, extra_chunk;
 #pragma unroll
       for (int k = 0; k < kTopK; ++k) x[k].load(from[k] + c);
+      if (extra) extra_chunk.load(extra + c);
 #pragma unroll
       for (int i = 0; i < W; ++i) acc.v[i] = 0.f;
 #pragma unroll
@@ -124,11 +140,13 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
           acc.v[i] += valid[k] ? term : 0.f;
         }
       }
+      finish(acc, extra_chunk);
       acc.store(to + c);
     }
   } else {
     for (int64_t c = static_cast<int64_t>(lane_id()) * W; c < hidden; c += step) {
-      Pack<T, W> acc;
+      Pack<T, W> acc, extra_chunk;
+      if (extra) extra_chunk.load(extra + c);
 #pragma unroll
       for (int i = 0; i < W; ++i) acc.v[i] = 0.f;
       for (int k = 0; k < top_k; ++k) {
@@ -146,6 +164,7 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
           }
         }
       }
+      finish(acc, extra_chunk);
       acc.store(to + c);
     }
   }
@@ -444,22 +463,26 @@ int hmoe_gather_rows(const void* src, int64_t src_row_stride, const int64_t* ind
   return HMOE_OK;
 }
 
-int hmoe_gather_reduce(const void* src, const void* weight, const int64_t* inv_map, int64_t n_out, int top_k,
-                       int64_t n_src, int64_t hidden, int dtype, void* out, void* stream) {
-  if (n_out < 0 || hidden < 0 || n_src < 0 || top_k < 0) return HMOE_INVALID_ARGUMENT;
+int hmoe_gather_reduce_add(const void* src, const void* weight, const int64_t* inv_map, int64_t n_out, int top_k,
+                           int64_t n_src, int64_t hidden, int dtype, const void* addend, int64_t addend_row_stride,
+                           const void* addend_scale, void* out, void* stream) {
+  if (n_out < 0 || hidden < 0 || n_src < 0 || top_k < 0 || addend_row_stride < 0) return HMOE_INVALID_ARGUMENT;
   if (n_out == 0 || hidden == 0) return HMOE_OK;
   if (!out || (top_k > 0 && !inv_map) || (n_src > 0 && !src)) return HMOE_INVALID_ARGUMENT;
+  if (addend_scale && !addend) return HMOE_INVALID_ARGUMENT;
+  if (addend && addend_row_stride < hidden) return HMOE_INVALID_ARGUMENT;
   if (n_out > (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool vec = dtype == HMOE_BF16 ? rows_vectorizable<bf16_t>(hidden, {}, {src, out})
-                                      : rows_vectorizable<float>(hidden, {}, {src, out});
+  const bool vec = dtype == HMOE_BF16 ? rows_vectorizable<bf16_t>(hidden, {addend_row_stride}, {src, out, addend})
+                                      : rows_vectorizable<float>(hidden, {addend_row_stride}, {src, out, addend});
   // n_src == 0: every slot is invalid and the rows come out as zeros; the generic kernel never touches src then
   const int fixed = n_src > 0 && (top_k == 8 || top_k == 4 || top_k == 2) ? top_k : 0;
 #define HMOE_GATHER_REDUCE(WEIGHTED, TOPK)                                                                        \
   HMOE_DISPATCH_ROWS(dtype, vec,                                                                                  \
                      (gather_reduce_kernel<T, W, WEIGHTED, TOPK><<<row_grid(n_out), dim3(kThreads), 0, s>>>(      \
                          static_cast<const T*>(src), static_cast<const T*>(weight), inv_map, static_cast<T*>(out), \
-                         n_out, top_k, n_src, hidden)))
+                         n_out, top_k, n_src, hidden, static_cast<const T*>(addend), addend_row_stride,           \
+                         static_cast<const T*>(addend_scale))))
   if (weight) {
     if (fixed == 8) { HMOE_GATHER_REDUCE(true, 8); }
     else if (fixed == 4) { HMOE_GATHER_REDUCE(true, 4); }
@@ -474,6 +497,12 @@ int hmoe_gather_reduce(const void* src, const void* weight, const int64_t* inv_m
 #undef HMOE_GATHER_REDUCE
   HMOE_CHECK_LAUNCH();
   return HMOE_OK;
+}
+
+int hmoe_gather_reduce(const void* src, const void* weight, const int64_t* inv_map, int64_t n_out, int top_k,
+                       int64_t n_src, int64_t hidden, int dtype, void* out, void* stream) {
+  return hmoe_gather_reduce_add(src, weight, inv_map, n_out, top_k, n_src, hidden, dtype, nullptr, 0, nullptr, out,
+                                stream);
 }
 
 int hmoe_unpermute_bwd(const void* grad_out, int64_t grad_out_row_stride, const void* expert_out,

@@ -30,10 +30,12 @@ def _gather_rows(src: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def gather_reduce_rows(src: torch.Tensor, inv_map: torch.Tensor, weight: torch.Tensor | None = None) -> torch.Tensor:
+def gather_reduce_rows(src: torch.Tensor, inv_map: torch.Tensor, weight: torch.Tensor | None = None, *,
+                       addend: torch.Tensor | None = None, addend_scale: torch.Tensor | None = None) -> torch.Tensor:
     """``out[r] = sum_k w[j] * src[j]`` over ``j = inv_map[r, k] < len(src)``; ``w = 1`` without a weight.  The sum is
-    taken in fp32 and rounded once to ``src``'s dtype."""
-    device = _lib.require_device(src, inv_map, weight)
+    taken in fp32 and rounded once to ``src``'s dtype.  With ``addend [len(out), hidden]`` (and ``addend_scale
+    [len(out)]``) the same pass returns ``out + addend_scale[:, None] * addend`` with that expression's roundings."""
+    device = _lib.require_device(src, inv_map, weight, addend, addend_scale)
     n_out, top_k = inv_map.shape
     hidden = src.shape[-1]
     out = torch.empty((n_out, hidden), device=device, dtype=src.dtype)
@@ -43,9 +45,22 @@ def gather_reduce_rows(src: torch.Tensor, inv_map: torch.Tensor, weight: torch.T
     if weight is not None:
         weight = weight.to(src.dtype).contiguous()
     inv_map = inv_map.long().contiguous()
+    if addend is not None:
+        if addend.shape != out.shape or addend.dtype != src.dtype:
+            raise ValueError(f"addend must be {tuple(out.shape)} {src.dtype}, got {tuple(addend.shape)} {addend.dtype}")
+        if addend.stride(-1) != 1:
+            addend = addend.contiguous()
+        if addend_scale is not None:
+            addend_scale = addend_scale.reshape(-1).to(src.dtype).contiguous()
+            if addend_scale.shape[0] != n_out:
+                raise ValueError(f"addend_scale must hold {n_out} values, got {addend_scale.shape[0]}")
+    elif addend_scale is not None:
+        raise ValueError("addend_scale without an addend")
     with _lib.on_device(device):
-        _lib.call("hmoe_gather_reduce", _lib.ptr(src), _lib.ptr(weight), _lib.ptr(inv_map), n_out, top_k,
-                  src.shape[0], hidden, _lib.dtype_id(src.dtype), _lib.ptr(out), _lib.stream_ptr(device))
+        _lib.call("hmoe_gather_reduce_add", _lib.ptr(src), _lib.ptr(weight), _lib.ptr(inv_map), n_out, top_k,
+                  src.shape[0], hidden, _lib.dtype_id(src.dtype), _lib.ptr(addend),
+                  addend.stride(0) if addend is not None else 0, _lib.ptr(addend_scale), _lib.ptr(out),
+                  _lib.stream_ptr(device))
     return out
 
 
@@ -104,24 +119,67 @@ class MoEWeightedUnpermute(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         expert_out, weights, sorted_token_idx = ctx.saved_tensors
-        device = _lib.require_device(grad_out, weights, sorted_token_idx)
-        n_sorted, hidden = sorted_token_idx.shape[0], grad_out.shape[-1]
-        # Under EP the gradient arrives as a row-strided view of the padded transport buffer, read in place.
-        if grad_out.stride(-1) != 1:
-            grad_out = grad_out.contiguous()
-        grad_expert = torch.empty((n_sorted, hidden), device=device, dtype=grad_out.dtype)
-        grad_weights = torch.empty(n_sorted if ctx.weight_grad else 0, device=device, dtype=torch.float32)
-        if n_sorted:
-            w = weights if weights.dtype == grad_out.dtype else weights.to(grad_out.dtype)
-            y = None
-            if ctx.weight_grad:
-                y = expert_out if expert_out.dtype == grad_out.dtype else expert_out.to(grad_out.dtype)
-            with _lib.on_device(device):
-                _lib.call("hmoe_unpermute_bwd", _lib.ptr(grad_out), grad_out.stride(0), _lib.ptr(y), _lib.ptr(w),
-                          _lib.ptr(sorted_token_idx), n_sorted, hidden, _lib.dtype_id(grad_out.dtype),
-                          _lib.ptr(grad_expert), _lib.ptr(grad_weights) if ctx.weight_grad else None,
-                          _lib.stream_ptr(device))
-        return grad_expert, grad_weights.to(weights.dtype) if ctx.weight_grad else None, None, None
+        grad_expert, grad_weights = _unpermute_backward(grad_out, expert_out, weights, sorted_token_idx,
+                                                        ctx.weight_grad)
+        return grad_expert, grad_weights, None, None
+
+
+def _unpermute_backward(grad_out, expert_out, weights, sorted_token_idx, weight_grad: bool):
+    """``(w[j] * grad_out[tok[j]], <grad_out[tok[j]], expert_out[j]>)``; the second only when ``weight_grad``."""
+    device = _lib.require_device(grad_out, weights, sorted_token_idx)
+    n_sorted, hidden = sorted_token_idx.shape[0], grad_out.shape[-1]
+    # Under EP the gradient arrives as a row-strided view of the padded transport buffer, read in place.
+    if grad_out.stride(-1) != 1:
+        grad_out = grad_out.contiguous()
+    grad_expert = torch.empty((n_sorted, hidden), device=device, dtype=grad_out.dtype)
+    grad_weights = torch.empty(n_sorted if weight_grad else 0, device=device, dtype=torch.float32)
+    if n_sorted:
+        w = weights if weights.dtype == grad_out.dtype else weights.to(grad_out.dtype)
+        y = None
+        if weight_grad:
+            y = expert_out if expert_out.dtype == grad_out.dtype else expert_out.to(grad_out.dtype)
+        with _lib.on_device(device):
+            _lib.call("hmoe_unpermute_bwd", _lib.ptr(grad_out), grad_out.stride(0), _lib.ptr(y), _lib.ptr(w),
+                      _lib.ptr(sorted_token_idx), n_sorted, hidden, _lib.dtype_id(grad_out.dtype),
+                      _lib.ptr(grad_expert), _lib.ptr(grad_weights) if weight_grad else None,
+                      _lib.stream_ptr(device))
+    return grad_expert, grad_weights.to(weights.dtype) if weight_grad else None
+
+
+class MoEWeightedUnpermuteAdd(torch.autograd.Function):
+    """``MoEWeightedUnpermute.apply(expert_out, weights, sorted_token_idx, inv_map) + scale[:, None] * addend`` in the
+    combine's own pass (``scale`` may be None): the routed output plus the shared expert's, which the reference adds
+    as a separate tensor operation (``expert_parallel/layer.py:270-299``; Qwen3.5's sigmoid gate on the shared expert,
+    ``families/qwen3_5.py:41-42``).  The forward rounds where those operations round, so it returns their bits; the
+    gradients are theirs as well, except that the gradient of ``scale`` is a dot product accumulated in fp32 and
+    rounded once where autograd would round every product first."""
+
+    @staticmethod
+    def forward(ctx, expert_out, weights, sorted_token_idx, inv_map, addend, scale):
+        expert_out, weights = expert_out.contiguous(), weights.contiguous()
+        ctx.weight_grad = ctx.needs_input_grad[1]
+        ctx.scaled = scale is not None
+        ctx.scale_shape = scale.shape if ctx.scaled else None
+        ctx.save_for_backward(expert_out if ctx.weight_grad else None, weights, sorted_token_idx.contiguous(),
+                              addend if ctx.scaled and ctx.needs_input_grad[5] else None, scale)
+        return gather_reduce_rows(expert_out, inv_map, weights, addend=addend, addend_scale=scale)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        expert_out, weights, sorted_token_idx, addend, scale = ctx.saved_tensors
+        grad_expert, grad_weights = _unpermute_backward(grad_out, expert_out, weights, sorted_token_idx,
+                                                        ctx.weight_grad)
+        grad_addend = grad_scale = None
+        if not ctx.scaled:
+            grad_addend = grad_out if ctx.needs_input_grad[4] else None
+        elif ctx.needs_input_grad[4] or ctx.needs_input_grad[5]:
+            # the same kernel with every row its own token: scale[r] * grad_out[r] and <grad_out[r], addend[r]>
+            rows = torch.arange(grad_out.shape[0], device=grad_out.device)
+            want_scale = ctx.needs_input_grad[5]
+            grad_addend, grad_scale = _unpermute_backward(grad_out, addend, scale.reshape(-1), rows, want_scale)
+            if want_scale:
+                grad_scale = grad_scale.to(scale.dtype).view(ctx.scale_shape)
+        return grad_expert, grad_weights, None, None, grad_addend, grad_scale
 
 
 def expert_bias_grad(grad_out: torch.Tensor, eids: torch.Tensor, num_experts: int) -> torch.Tensor:

@@ -48,15 +48,14 @@ class EPQwen3_5MoELayer(EPSharedExpertsMoELayerBase):
         super()._adopt_shared_experts(original_layer)
         self.shared_expert_gate = original_layer.shared_expert_gate
 
-    def _shared_expert_output(self, hidden_states: torch.Tensor) -> torch.Tensor:
-        out = super()._shared_expert_output(hidden_states)
+    def _shared_expert_parts(self, hidden_states: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor | None]:
+        rows, _ = super()._shared_expert_parts(hidden_states)
         gate = getattr(self, "shared_expert_gate", None)
         if gate is None:
-            return out
+            return rows, None
         x = hidden_states.reshape(-1, hidden_states.shape[-1])
         # a [T, 1] projection is below the GEMM kernels' 16-byte row granularity: a matrix-vector product in torch
-        return out * torch.sigmoid(torch.nn.functional.linear(x, gate.weight.to(x.dtype))).view(
-            *hidden_states.shape[:-1], -1)
+        return rows, torch.sigmoid(torch.nn.functional.linear(x, gate.weight.to(x.dtype))).view(-1)
 
     def replicated_named_params(self) -> list:
         extra = [] if getattr(self, "shared_expert_gate", None) is None else [

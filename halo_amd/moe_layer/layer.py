@@ -23,7 +23,8 @@ import torch.nn as nn
 from halo_amd.kernels.expert_gemm import expert_gemm
 from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled, resolve_fused_glu_mul
 from halo_amd.kernels.grouped_mm import GatheredRows, grouped_mm, grouped_wgrad
-from halo_amd.kernels.moe_permute import MoEGatherPermute, MoEWeightedUnpermute, warm_permute_kernels
+from halo_amd.kernels.moe_permute import (MoEGatherPermute, MoEWeightedUnpermute, MoEWeightedUnpermuteAdd,
+                                          warm_permute_kernels)
 from halo_amd.kernels.moe_route_sort import sort_routing_by_expert, warm_route_sort_kernels
 from halo_amd.kernels.router import SOFTMAX_ALL, fused_topk_gate
 from halo_amd.moe_layer.config import EPConfig, MoEFamilySpec
@@ -161,6 +162,8 @@ class EPMoELayerBase(nn.Module, ABC):
         self._lowp_weight_cacheable = True
         # the first expert projection gathers its rows by index instead of reading a permuted copy of the tokens
         self.fuse_permute_into_gemm = True
+        # the shared expert's output joins the routed one in the combine kernel instead of a tensor addition
+        self.fuse_shared_into_combine = True
         self._fused_glu_mul: Callable | None = None
         # labels the dispatch / expert-compute / combine spans at no device cost (swappable, as in the reference)
         self._perf = torch.profiler.record_function
@@ -245,19 +248,27 @@ class EPMoELayerBase(nn.Module, ABC):
         warm_permute_kernels(16, hidden, top_k, device, dtype)
 
     def _compute_experts(self, tokens: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor,
-                         output_dtype: torch.dtype, *, recv_counts: tuple[int, ...] | None) -> torch.Tensor:
+                         output_dtype: torch.dtype, *, recv_counts: tuple[int, ...] | None,
+                         addend: tuple[torch.Tensor, torch.Tensor | None] | None = None) -> torch.Tensor:
         """``experts``/``weights`` are ``[T, top_k]`` local ids (``-1`` = not this rank's) and gate weights;
-        ``recv_counts`` counts per local expert, None at ``ep_size`` 1."""
+        ``recv_counts`` counts per local expert, None at ``ep_size`` 1.  ``addend = (rows [T, H], scale [T] or None)``
+        (not in the reference's signature) is added to the result, ``scale[:, None] * rows``, by the combine kernel."""
         if tokens.shape[0] == 0:
             return torch.zeros((0, tokens.shape[-1]), device=tokens.device, dtype=output_dtype)
-        return self._compute_experts_grouped(tokens, experts, weights, output_dtype, recv_counts=recv_counts)
+        return self._compute_experts_grouped(tokens, experts, weights, output_dtype, recv_counts=recv_counts,
+                                             addend=addend)
 
-    def _compute_experts_grouped(self, tokens, experts, weights, output_dtype, *, recv_counts):
+    def _compute_experts_grouped(self, tokens, experts, weights, output_dtype, *, recv_counts, addend=None):
         """Sort -> grouped GLU FFN -> weighted unpermute."""
         sorted_tokens, offs, sorted_token_idx, sorted_weights, sorted_expert_ids, inv_map = (
             self._sort_tokens_for_grouped_mm(tokens, experts, weights, recv_counts=recv_counts)
         )
         expert_out = self._grouped_expert_ffn(sorted_tokens.to(output_dtype), offs, sorted_expert_ids, output_dtype)
+        if addend is not None:
+            rows, scale = addend
+            return MoEWeightedUnpermuteAdd.apply(
+                expert_out.to(output_dtype).contiguous(), sorted_weights.to(output_dtype), sorted_token_idx, inv_map,
+                rows.to(output_dtype), None if scale is None else scale.to(output_dtype))
         return MoEWeightedUnpermute.apply(
             expert_out.to(output_dtype).contiguous(), sorted_weights.to(output_dtype), sorted_token_idx, inv_map
         )
@@ -347,7 +358,7 @@ class EPMoELayerBase(nn.Module, ABC):
     # ------------------------------------------------------------------------------- dispatch / compute / combine
 
     def _dispatch_compute_combine(self, flat: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor,
-                                  input_dtype: torch.dtype) -> torch.Tensor:
+                                  input_dtype: torch.dtype, addend=None) -> torch.Tensor:
         """At ``ep_size`` 1 dispatch and combine are the identity; the spans keep the reference's names."""
         if self.ep_size > 1:
             raise NotImplementedError(
@@ -359,12 +370,18 @@ class EPMoELayerBase(nn.Module, ABC):
             recv_x, recv_topk_idx, recv_topk_weights, recv_counts = flat, experts, weights, None
         with self._perf("ep.expert_compute"):
             output = self._compute_experts(recv_x, recv_topk_idx, recv_topk_weights, input_dtype,
-                                           recv_counts=recv_counts)
+                                           recv_counts=recv_counts, addend=addend)
         with self._perf("ep.combine"):
             combined = output
         return combined
 
-    def _dispatch_compute_combine_shared(self, flat, experts, weights, input_dtype, orig_shape, shared_fn):
+    def _dispatch_compute_combine_shared(self, flat, experts, weights, input_dtype, orig_shape, shared_fn,
+                                         shared_parts_fn=None):
+        """``routed + shared``.  With ``shared_parts_fn`` (the shared expert's output as ``(rows [T, H], scale [T] or
+        None)``, ``shared = scale[:, None] * rows``) and tokens to route, the sum is taken by the combine kernel."""
+        if shared_parts_fn is not None and self.fuse_shared_into_combine and flat.shape[0] > 0:
+            return self._dispatch_compute_combine(flat, experts, weights, input_dtype,
+                                                  addend=shared_parts_fn()).view(*orig_shape)
         routed = self._dispatch_compute_combine(flat, experts, weights, input_dtype).view(*orig_shape)
         return routed if shared_fn is None else routed + shared_fn()
 
@@ -408,8 +425,9 @@ class EPSharedExpertsMoELayerBase(EPMoELayerBase):
         topk_indices, topk_weights = self._route_hidden_states(flat, **kwargs)
         shared = getattr(self, self._shared_expert_attr, None)
         shared_fn = (lambda: self._shared_expert_output(hidden_states)) if shared is not None else None
+        parts_fn = (lambda: self._shared_expert_parts(hidden_states)) if shared is not None else None
         return self._dispatch_compute_combine_shared(
-            flat, topk_indices.long(), topk_weights.float(), hidden_states.dtype, orig_shape, shared_fn
+            flat, topk_indices.long(), topk_weights.float(), hidden_states.dtype, orig_shape, shared_fn, parts_fn
         )
 
     def _normalizes_topk(self) -> bool:
@@ -423,10 +441,16 @@ class EPSharedExpertsMoELayerBase(EPMoELayerBase):
 
     def _shared_expert_output(self, hidden_states: torch.Tensor) -> torch.Tensor:
         """Dense GLU MLP ``down(act(gate(x)) * up(x))`` through the same GEMM and GLU kernels."""
+        rows, scale = self._shared_expert_parts(hidden_states)
+        out = rows.view(hidden_states.shape)
+        return out if scale is None else out * scale.view(*hidden_states.shape[:-1], 1)
+
+    def _shared_expert_parts(self, hidden_states: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor | None]:
+        """The shared expert's output as ``(rows [T, H], scale [T] or None)``: ``rows`` the MLP's output, ``scale`` a
+        per-token factor on it (none here; Qwen3.5's sigmoid gate)."""
         shared = getattr(self, self._shared_expert_attr)
-        shape = hidden_states.shape
-        x = hidden_states.reshape(-1, shape[-1])
+        x = hidden_states.reshape(-1, hidden_states.shape[-1])
         dtype = x.dtype
         gate = dense_mm(x, shared.gate_proj.weight.to(dtype))
         up = dense_mm(x, shared.up_proj.weight.to(dtype))
-        return dense_mm(self._fused_glu_mul(gate, up), shared.down_proj.weight.to(dtype)).view(shape)
+        return dense_mm(self._fused_glu_mul(gate, up), shared.down_proj.weight.to(dtype)), None

@@ -84,6 +84,15 @@ int hmoe_gather_rows(const void* src, int64_t src_row_stride, const int64_t* ind
 int hmoe_gather_reduce(const void* src, const void* weight, const int64_t* inv_map, int64_t n_out, int top_k,
                        int64_t n_src, int64_t hidden, int dtype, void* out, void* stream);
 
+/* The same with a second term added in the same pass: out[r] = round(round(sum) + round(scale[r] * addend[r])), the
+ * roundings where the tensor operations `combined + scale * addend` have them.  Replaces the `routed + shared_fn()` of
+ * _dispatch_compute_combine_shared (halo/distributed/expert_parallel/layer.py:270-299) behind the weighted unpermute,
+ * with Qwen3.5's sigmoid gate on the shared expert (families/qwen3_5.py:41-42) as `addend_scale` [n_out] (null: no
+ * scale).  addend is [n_out, hidden] with rows addend_row_stride elements apart, null for the plain reduction. */
+int hmoe_gather_reduce_add(const void* src, const void* weight, const int64_t* inv_map, int64_t n_out, int top_k,
+                           int64_t n_src, int64_t hidden, int dtype, const void* addend, int64_t addend_row_stride,
+                           const void* addend_scale, void* out, void* stream);
+
 /* Replaces _weighted_unpermute_bwd_kernel: halo/kernels/moe_permute.py:44-72, 158-189.
  * grad_expert[j] = w[j] * grad_out[tok[j]];  grad_weights[j] = <grad_out[tok[j]], expert_out[j]> in fp32 when
  * expert_out and grad_weights are non-null. */

@@ -661,3 +661,30 @@ def test_grouped_mm_with_the_bias_in_its_epilogue_equals_the_two_operations(devi
                       for i, (s, e) in enumerate(zip([0] + list(np.cumsum(counts)[:-1]), np.cumsum(counts)))])
     tol = 2e-2 if dtype == torch.bfloat16 else 1e-4
     assert max_rel(results[1][0], want) < tol
+
+
+@pytest.mark.parametrize("scaled", (False, True), ids=("plain", "scaled"))
+@pytest.mark.parametrize(("dtype", "top_k", "hidden"), ((torch.bfloat16, 8, 2048), (torch.bfloat16, 3, 264),
+                                                         (torch.float32, 4, 256), (torch.bfloat16, 2, 100)))
+def test_combine_with_an_added_term_equals_the_tensor_operations(device, dtype, top_k, hidden, scaled):
+    """``gather_reduce_rows(..., addend=a, addend_scale=s)`` returns the bits of ``gather_reduce_rows(...) + s * a``:
+    the reduction is rounded, the scaled term is rounded, the sum is rounded.  Rows without a valid slot and a
+    row-strided addend included."""
+    from halo_amd.kernels.moe_permute import gather_reduce_rows
+
+    g = torch.Generator().manual_seed(13)
+    n_tokens = 300
+    token_idx, inv_map = _routing(n_tokens, top_k, n_tokens * top_k * 2 // 3, seed=4)
+    n_sorted = token_idx.numel()
+    src = torch.randn(n_sorted, hidden, generator=g).to(dtype).to(device)
+    w = torch.rand(n_sorted, generator=g).to(dtype).to(device)
+    padded = torch.randn(n_tokens, hidden + 24, generator=g).to(dtype).to(device)
+    addend = padded[:, :hidden]  # rows 24 elements apart from dense
+    scale = torch.rand(n_tokens, generator=g).to(dtype).to(device) if scaled else None
+    inv_map[5] = inv_map[77] = n_sorted  # two tokens that no expert row belongs to: their output is the added term
+    inv = inv_map.to(device)
+    got = gather_reduce_rows(src, inv, w, addend=addend, addend_scale=scale)
+    combined = gather_reduce_rows(src, inv, w)
+    want = combined + (addend if scale is None else scale[:, None] * addend)
+    assert torch.equal(got, want)
+    assert torch.equal(got[5], want[5]) and combined[5].count_nonzero() == 0

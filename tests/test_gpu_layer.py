@@ -290,3 +290,80 @@ def test_router_projection_gradients_at_a_token_count_that_splits_the_wgrad(devi
     _check("dx", dx, dlogits.double() @ w.double(), 2e-2)
     _check("dw", dw, dlogits.double().t() @ x.double(), 2e-2)
     assert all(torch.equal(a, b) for a, b in zip(results[0], results[1]))
+
+
+class _SharedMlp(torch.nn.Module):
+    def __init__(self, hidden, width, dtype, generator):
+        super().__init__()
+        for name, shape in (("gate_proj", (width, hidden)), ("up_proj", (width, hidden)), ("down_proj", (hidden, width))):
+            linear = torch.nn.Linear(shape[1], shape[0], bias=False, dtype=dtype)
+            linear.weight.data = (torch.randn(shape, generator=generator) * shape[1] ** -0.5).to(dtype)
+            setattr(self, name, linear)
+
+
+def _layer_with_shared_expert(cfg, inputs, device, gated, fuse):
+    g = torch.Generator().manual_seed(21)
+    layer = _build_layer(cfg, inputs, device)
+    layer.shared_expert = _SharedMlp(cfg.hidden, 64, cfg.dtype, g).to(device)
+    layer._shared_expert_attr = "shared_expert"
+    if gated:
+        gate = torch.nn.Linear(cfg.hidden, 1, bias=False, dtype=cfg.dtype)
+        gate.weight.data = (torch.randn(1, cfg.hidden, generator=g) * cfg.hidden ** -0.5).to(cfg.dtype)
+        layer.shared_expert_gate = gate.to(device)
+    layer.fuse_shared_into_combine = fuse
+    return layer
+
+
+@pytest.mark.parametrize("gated", (False, True), ids=("plain", "sigmoid_gated"))
+@pytest.mark.parametrize("cfg", (CONFIG1, CONFIG2_SMALL), ids=lambda c: c.name)
+def test_shared_expert_added_in_the_combine_kernel(device, cfg, gated):
+    """A layer with a shared expert (Qwen3.5's carries a sigmoid gate): the sum ``routed + shared`` taken by the
+    combine kernel gives the output of the tensor addition bit for bit, and the gradients of everything that does not
+    pass through the gate's dot product bit for bit; the output and input gradient also match the fp32 loop with the
+    same selection."""
+    from halo_amd.moe_layer import EPQwen3_5MoELayer
+    from oracle import moe_layer as oracle
+
+    if not cfg.fused:
+        pytest.skip("the sigmoid-gated shared expert belongs to the fused-GLU family")
+    inputs = make_layer_inputs(cfg)
+    results = []
+    for fuse in (False, True):
+        layer = _layer_with_shared_expert(cfg, inputs, device, gated, fuse)
+        assert isinstance(layer, EPQwen3_5MoELayer)
+        x = inputs["x"].to(device).requires_grad_(True)
+        out = layer(x)
+        out.backward(inputs["grad_out"].to(device))
+        grads = {n: p.grad.clone() for n, p in layer.named_parameters() if p.grad is not None}
+        results.append((out.detach(), x.grad.clone(), grads))
+    (out_a, gx_a, grads_a), (out_b, gx_b, grads_b) = results
+    assert torch.equal(out_a, out_b)
+    assert set(grads_a) == set(grads_b) and any(n.startswith("shared_expert.") for n in grads_a)
+    tol = 1e-5 if cfg.dtype == torch.float32 else 2e-2
+    for name in grads_a:
+        if name.startswith("shared_expert_gate"):
+            assert max_rel(grads_b[name], grads_a[name]) < tol, name
+        else:
+            assert torch.equal(grads_a[name], grads_b[name]), name
+    if gated:
+        assert max_rel(gx_b, gx_a) < tol
+    else:
+        assert torch.equal(gx_a, gx_b)
+
+    # against the fp32 loop: selection taken from the device
+    from halo_amd.kernels.router import fused_topk_gate
+    with torch.no_grad():
+        idx, _ = fused_topk_gate(layer._linear_router_logits(x.detach()), cfg.top_k, normalize=True, eps=0.0)
+    f = lambda t: t.detach().float().cpu().requires_grad_(True)
+    xs, wr = f(inputs["x"]), f(inputs["router_weight"])
+    params = {k: f(v) for k, v in inputs["params"].items()}
+    shared = {n: f(getattr(layer.shared_expert, n).weight) for n in ("gate_proj", "up_proj", "down_proj")}
+    if gated:
+        shared["shared_expert_gate"] = f(layer.shared_expert_gate.weight)
+    want, _, _, _ = oracle.moe_layer_forward(xs, wr, params, oracle.Glu(cfg.glu), cfg.top_k, normalize=True, eps=0.0,
+                                             indices=idx.cpu(), shared=shared)
+    want.backward(inputs["grad_out"].float())
+    check_tol = 1e-4 if cfg.dtype == torch.float32 else 2e-2
+    _check("out with shared expert", out_b, want.detach(), check_tol)
+    _check("grad x with shared expert", gx_b, xs.grad, check_tol)
+    _check("grad shared down_proj", grads_b["shared_expert.down_proj.weight"], shared["down_proj"].grad, check_tol)
