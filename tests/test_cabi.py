@@ -72,3 +72,43 @@ def test_product_never_imports_the_oracle():
             if name.endswith(".py"):
                 text = open(os.path.join(dirpath, name)).read()
                 assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), f"{name} imports the oracle"
+
+
+def test_bad_arguments_come_back_as_status_codes_before_any_launch():
+    """Every entry point checks its arguments first and reports through its return value; none of these calls reaches
+    a kernel launch (there is no GPU here), and an empty problem is a success that launches nothing."""
+    lib = _lib.load()
+    invalid, unsupported = -1, -2
+    assert lib.hmoe_status_string(invalid) != lib.hmoe_status_string(unsupported)
+    bf16, f32 = _lib.dtype_id(torch.bfloat16), _lib.dtype_id(torch.float32)
+    fake = 0x10000  # a non-null, 16-byte aligned address that is never dereferenced on these paths
+
+    # grouped GEMM: negative sizes, several groups without offsets, rows not 16-byte multiples, too many groups
+    gemm = lib.hmoe_grouped_gemm_fwd
+    assert gemm(fake, 64, fake, fake, -1, 4, 64, 64, bf16, fake, 64, None) == invalid
+    assert gemm(fake, 64, fake, None, 8, 4, 64, 64, bf16, fake, 64, None) == invalid
+    assert gemm(fake, 60, fake, fake, 8, 4, 60, 64, bf16, fake, 64, None) == unsupported
+    assert gemm(fake, 64, fake, fake, 8, 5000, 64, 64, bf16, fake, 64, None) == unsupported
+    assert gemm(fake, 64, fake, fake, 8, 4, 64, 64, 77, fake, 64, None) == unsupported
+    assert gemm(None, 64, fake, fake, 8, 4, 64, 64, bf16, fake, 64, None) == invalid
+    assert gemm(fake, 32, fake, fake, 8, 4, 64, 64, bf16, fake, 64, None) == invalid  # row stride below the row length
+    assert gemm(None, 64, None, None, 0, 1, 64, 64, bf16, None, 64, None) == 0  # no rows: nothing to do
+    assert lib.hmoe_grouped_gemm_fwd_bias(fake, 64, fake, None, fake, 8, 4, 64, 64, bf16, fake, 64, None) == invalid
+    assert lib.hmoe_grouped_gemm_fwd_gather(fake, 64, 8, fake, fake, fake, 8, 4, 64, 64, f32, fake, 64, None) == unsupported
+    assert lib.hmoe_grouped_gemm_fwd_gather(fake, 64, -3, fake, fake, fake, 8, 4, 64, 64, bf16, fake, 64, None) == invalid
+
+    # row movers
+    assert lib.hmoe_gather_rows(fake, 64, fake, -1, 64, bf16, fake, None) == invalid
+    assert lib.hmoe_gather_rows(None, 64, None, 0, 64, bf16, None, None) == 0
+    assert lib.hmoe_gather_reduce(fake, None, None, 4, 2, 8, 64, bf16, fake, None) == invalid  # slots without a map
+    assert lib.hmoe_gather_reduce_add(fake, None, fake, 4, 2, 8, 64, bf16, None, 0, fake, fake, None) == invalid
+    assert lib.hmoe_gather_reduce_add(fake, None, fake, 4, 2, 8, 64, bf16, fake, 32, None, fake, None) == invalid
+    assert lib.hmoe_unpermute_bwd(fake, 64, fake, fake, fake, 4, 64, bf16, fake, None, None) == invalid
+    assert lib.hmoe_expert_colsum(None, None, 4, 64, 2, bf16, fake, None, None) == invalid
+    assert lib.hmoe_expert_colsum(None, None, 0, 64, 0, bf16, None, None, None) == 0
+    assert lib.hmoe_expert_colsum_workspace_bytes(1000, 64, 3) == (8 + 3) * 64 * 4
+    assert lib.hmoe_expert_colsum_workspace_bytes(-1, 64, 3) == 0
+
+    # routing sort
+    assert lib.hmoe_route_sort_workspace_bytes(-1, 2, 4) < 0
+    assert lib.hmoe_route_sort_workspace_bytes(16, 2, 4) > 0
