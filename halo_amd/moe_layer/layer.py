@@ -45,6 +45,7 @@ class _RouterProjection(torch.autograd.Function):
 
     _SPLITS = 32
     _MIN_TOKENS = 2048
+    _slice_ends: ClassVar[dict] = {}  # (device, tokens) -> the slices' row ends
 
     @staticmethod
     def forward(ctx, x, weight):
@@ -61,9 +62,13 @@ class _RouterProjection(torch.autograd.Function):
             tokens = x.shape[0]
             splits = _RouterProjection._SPLITS
             if x.dtype == torch.bfloat16 and tokens >= _RouterProjection._MIN_TOKENS and tokens % splits == 0:
-                offs = torch.arange(1, splits + 1, device=x.device, dtype=torch.int32) * (tokens // splits)
+                key = (x.device, tokens)
+                offs = _RouterProjection._slice_ends.get(key)
+                if offs is None:
+                    offs = torch.arange(1, splits + 1, device=x.device, dtype=torch.int32) * (tokens // splits)
+                    _RouterProjection._slice_ends[key] = offs
                 partial = grouped_wgrad(grad_logits, x, offs, splits)
-                grad_weight = partial.sum(dim=0, dtype=torch.float32).to(weight.dtype)
+                grad_weight = partial.sum(dim=0)  # the reduction accumulates in fp32 and rounds once
             else:
                 grad_weight = grad_logits.t() @ x
         return grad_x, grad_weight
