@@ -2,8 +2,9 @@
 SwiGLU family.  :meth:`GluCombine.packed` reads a fused ``[gate | up]`` projection in place and returns its gradient
 as one buffer, so the expert path copies on neither side of the activation.
 
-Mirrors the reference's ``halo/kernels/fused_glu.py`` (``GluCombine`` ``:306-361``, autograd functions ``:259-299``,
-resolvers ``:364-384``, activation probes ``:36-63``); the kernels are ``csrc/glu.hip``.
+Same public surface as the reference's ``halo/kernels/fused_glu.py`` (``GluCombine`` ``:306-361``, its resolvers
+``:364-384``, the activation probes ``:36-63``, the eager forms ``:66-87``, ``HALO_FUSED_GLU`` ``:21``); the kernels are
+``csrc/glu.hip`` and take the combine as (kind, alpha, limit, two flags).
 """
 
 from __future__ import annotations
@@ -14,161 +15,165 @@ from collections.abc import Callable
 from dataclasses import dataclass
 
 import torch
+import torch.nn.functional as F
 
 from halo_amd import _lib
 
 logger = logging.getLogger(__name__)
 
+# kernel-side activation kinds (csrc/glu.hip)
+_SILU, _GELU_TANH, _CLAMPED_SILU = 0, 1, 2
 
-def _env_flag(name: str, default: bool) -> bool:
-    value = os.environ.get(name)
-    if value is None:
-        return default
-    return value.strip().lower() not in ("0", "false", "no", "off", "")
-
-
-# ``HALO_FUSED_GLU=0`` runs every combine as eager torch ops on the device, the reference's escape hatch.
-_FUSED_GLU_ENABLED = _env_flag("HALO_FUSED_GLU", True)
-
-_SILU = 0
-_GELU_TANH = 1
-_CLAMPED_SILU = 2  # alpha-scaled SiLU with the clamps of the GptOss/DeepSeek-V4/Step-3.7 family
-
-# Both saturating tails, both signs, zero and near-zero; it separates every registered activation.
-_ACTIVATION_PROBE_INPUT = (-64.0, -8.0, -1.0, -0.5, -1e-3, 0.0, 1e-3, 0.5, 1.0, 8.0, 64.0)
-
-
-def _computes_exactly(act_fn: object, reference_fn: Callable[[torch.Tensor], torch.Tensor], name: str) -> bool:
-    """Bit for bit over the probe vector on the host; behavioural, since an activation module need not be
-    ``F.silu`` itself.  Callers latch the result at construction."""
-    if not callable(act_fn):
-        return False
-    try:
-        probe = torch.tensor(_ACTIVATION_PROBE_INPUT, dtype=torch.float32, device="cpu")
-        expected = reference_fn(probe)
-        with torch.no_grad():
-            out = act_fn(probe)
-        return (
-            isinstance(out, torch.Tensor)
-            and out.shape == expected.shape
-            and out.dtype == expected.dtype
-            and torch.equal(out, expected)
-        )
-    except Exception:
-        logger.warning(f"Activation {act_fn!r} could not be probed against {name}; treating it as non-{name}.")
-        return False
-
-
-def is_silu_activation(act_fn: object) -> bool:
-    return _computes_exactly(act_fn, torch.nn.functional.silu, "F.silu")
-
-
-def is_gelu_tanh_activation(act_fn: object) -> bool:
-    return _computes_exactly(act_fn, lambda x: torch.nn.functional.gelu(x, approximate="tanh"), "tanh-GELU")
-
-
-# Eager forms: plain torch ops on whatever device the operands live on (``HALO_FUSED_GLU=0``).
-def silu_mul_eager(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-    return torch.nn.functional.silu(gate) * up
-
-
-def gelu_tanh_mul_eager(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-    return torch.nn.functional.gelu(gate, approximate="tanh") * up
-
-
-def gptoss_glu_eager(gate: torch.Tensor, up: torch.Tensor, alpha: float, limit: float) -> torch.Tensor:
-    gate = gate.clamp(max=limit)
-    up = up.clamp(min=-limit, max=limit)
-    return (up + 1) * (gate * torch.sigmoid(gate * alpha))
-
-
-def clamped_silu_mul_eager(gate: torch.Tensor, up: torch.Tensor, limit: float) -> torch.Tensor:
-    return torch.nn.functional.silu(gate.clamp(max=limit)) * up.clamp(min=-limit, max=limit)
-
-
-def silu_then_clamp_mul_eager(gate: torch.Tensor, up: torch.Tensor, limit: float) -> torch.Tensor:
-    return torch.nn.functional.silu(gate).clamp(max=limit) * up.clamp(min=-limit, max=limit)
-
-
-def _as_rows(t: torch.Tensor) -> torch.Tensor:
-    if t.stride(-1) != 1:
-        t = t.contiguous()
-    return t.reshape(-1, t.shape[-1])
-
-
-def _glu_forward(gate: torch.Tensor, up: torch.Tensor, combine: "GluCombine") -> torch.Tensor:
-    device = _lib.require_device(gate, up)
-    n_rows, width = gate.shape
-    out = torch.empty((n_rows, width), device=device, dtype=gate.dtype)
-    if out.numel():
-        with _lib.on_device(device):
-            _lib.call("hmoe_glu_fwd", _lib.ptr(gate), _lib.ptr(up), gate.stride(0), up.stride(0), n_rows, width,
-                      _lib.dtype_id(gate.dtype), combine.activation, combine.alpha, combine.limit,
-                      int(combine.clamp_activated), int(combine.up_plus_one), _lib.ptr(out), _lib.stream_ptr(device))
-    return out
-
-
-def _glu_backward(gate, up, grad_out, dgate, dup, combine: "GluCombine") -> None:
-    device = _lib.require_device(gate, up, grad_out, dgate, dup)
-    n_rows, width = gate.shape
-    if n_rows == 0 or width == 0:
-        return
-    grad_out = grad_out.contiguous().view(n_rows, width)
-    with _lib.on_device(device):
-        _lib.call("hmoe_glu_bwd", _lib.ptr(gate), _lib.ptr(up), gate.stride(0), up.stride(0), _lib.ptr(grad_out),
-                  n_rows, width, _lib.dtype_id(gate.dtype), combine.activation, combine.alpha, combine.limit,
-                  int(combine.clamp_activated), int(combine.up_plus_one), _lib.ptr(dgate), _lib.ptr(dup),
-                  dgate.stride(0), dup.stride(0), _lib.stream_ptr(device))
-
-
-class _FusedGLU(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, gate: torch.Tensor, up: torch.Tensor, combine: "GluCombine") -> torch.Tensor:
-        shape = gate.shape
-        gate2d, up2d = _as_rows(gate), _as_rows(up)
-        ctx.save_for_backward(gate2d, up2d)
-        ctx.combine, ctx.shape = combine, shape
-        return _glu_forward(gate2d, up2d, combine).view(shape)
-
-    @staticmethod
-    def backward(ctx, grad_out: torch.Tensor):
-        gate, up = ctx.saved_tensors
-        dgate = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
-        dup = torch.empty(up.shape, dtype=up.dtype, device=up.device)
-        _glu_backward(gate, up, grad_out, dgate, dup, ctx.combine)
-        return dgate.view(ctx.shape), dup.view(ctx.shape), None
-
-
-class _FusedPackedGLU(torch.autograd.Function):
-    """Over a ``[..., 2M]`` ``[gate | up]`` output, read in place with the gradient written as one buffer."""
-
-    @staticmethod
-    def forward(ctx, gate_up: torch.Tensor, combine: "GluCombine") -> torch.Tensor:
-        shape = gate_up.shape
-        rows2d = _as_rows(gate_up)
-        width = shape[-1] // 2
-        ctx.save_for_backward(rows2d)
-        ctx.combine, ctx.shape = combine, shape
-        out = _glu_forward(rows2d[:, :width], rows2d[:, width:], combine)
-        return out.view(*shape[:-1], width)
-
-    @staticmethod
-    def backward(ctx, grad_out: torch.Tensor):
-        (rows2d,) = ctx.saved_tensors
-        width = rows2d.shape[-1] // 2
-        grad = torch.empty(rows2d.shape, device=rows2d.device, dtype=rows2d.dtype)
-        _glu_backward(rows2d[:, :width], rows2d[:, width:], grad_out, grad[:, :width], grad[:, width:], ctx.combine)
-        return grad.view(ctx.shape), None
+# ``HALO_FUSED_GLU=0`` (or false/no/off/empty) runs every combine as eager torch ops on the device.
+_FUSED_GLU_ENABLED = os.environ.get("HALO_FUSED_GLU", "1").strip().lower() not in ("0", "false", "no", "off", "")
 
 
 def fused_glu_enabled() -> bool:
     return _FUSED_GLU_ENABLED
 
 
+# ------------------------------------------------------------------------------------------------- eager forms
+
+def _clip_up(up: torch.Tensor, limit: float) -> torch.Tensor:
+    return torch.clamp(up, -limit, limit)
+
+
+def silu_mul_eager(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    return F.silu(gate) * up
+
+
+def gelu_tanh_mul_eager(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    return F.gelu(gate, approximate="tanh") * up
+
+
+def clamped_silu_mul_eager(gate: torch.Tensor, up: torch.Tensor, limit: float) -> torch.Tensor:
+    """The gate is cut off at ``limit`` before the SiLU, ``up`` is held within ``±limit``."""
+    return F.silu(torch.clamp(gate, max=limit)) * _clip_up(up, limit)
+
+
+def silu_then_clamp_mul_eager(gate: torch.Tensor, up: torch.Tensor, limit: float) -> torch.Tensor:
+    """As above with the cut-off applied to the SiLU's result instead of its argument."""
+    return torch.clamp(F.silu(gate), max=limit) * _clip_up(up, limit)
+
+
+def gptoss_glu_eager(gate: torch.Tensor, up: torch.Tensor, alpha: float, limit: float) -> torch.Tensor:
+    """gpt-oss: ``(clip(up) + 1) * g * sigmoid(alpha * g)`` with ``g = min(gate, limit)``."""
+    g = torch.clamp(gate, max=limit)
+    return (g * torch.sigmoid(alpha * g)) * (_clip_up(up, limit) + 1)
+
+
+# ------------------------------------------------------------------------------------------- activation probes
+
+# Both saturating tails, both signs, zero and values next to it: no two registered activations agree on all of them.
+_ACTIVATION_PROBE_INPUT = (-64.0, -8.0, -1.0, -0.5, -1e-3, 0.0, 1e-3, 0.5, 1.0, 8.0, 64.0)
+
+
+def _computes_exactly(act_fn: object, reference_fn: Callable[[torch.Tensor], torch.Tensor], name: str) -> bool:
+    """Whether ``act_fn`` returns ``reference_fn``'s bits on the probe vector (fp32, CPU).  Anything that is not
+    callable, raises, or returns another shape or dtype is taken not to be that activation."""
+    if not callable(act_fn):
+        return False
+    points = torch.tensor(_ACTIVATION_PROBE_INPUT, dtype=torch.float32)
+    want = reference_fn(points)
+    try:
+        with torch.no_grad():
+            got = act_fn(points)
+    except Exception:
+        logger.warning(f"Activation {act_fn!r} could not be probed against {name}; treating it as non-{name}.")
+        return False
+    if not isinstance(got, torch.Tensor) or got.dtype != want.dtype or got.shape != want.shape:
+        return False
+    return bool(torch.equal(got, want))
+
+
+def is_silu_activation(act_fn: object) -> bool:
+    return _computes_exactly(act_fn, F.silu, "F.silu")
+
+
+def is_gelu_tanh_activation(act_fn: object) -> bool:
+    return _computes_exactly(act_fn, lambda x: F.gelu(x, approximate="tanh"), "tanh-GELU")
+
+
+# -------------------------------------------------------------------------------------------------- launchers
+
+def _as_rows(t: torch.Tensor) -> torch.Tensor:
+    """``[rows, width]`` with unit stride along the width (the kernels take any row stride)."""
+    return (t if t.stride(-1) == 1 else t.contiguous()).reshape(-1, t.shape[-1])
+
+
+def _kernel_args(combine: "GluCombine") -> tuple:
+    return (combine.activation, combine.alpha, combine.limit, int(combine.clamp_activated), int(combine.up_plus_one))
+
+
+def _glu_forward(gate: torch.Tensor, up: torch.Tensor, combine: "GluCombine") -> torch.Tensor:
+    device = _lib.require_device(gate, up)
+    rows, width = gate.shape
+    out = gate.new_empty((rows, width))
+    if rows and width:
+        with _lib.on_device(device):
+            _lib.call("hmoe_glu_fwd", _lib.ptr(gate), _lib.ptr(up), gate.stride(0), up.stride(0), rows, width,
+                      _lib.dtype_id(gate.dtype), *_kernel_args(combine), _lib.ptr(out), _lib.stream_ptr(device))
+    return out
+
+
+def _glu_backward(gate, up, grad_out, dgate, dup, combine: "GluCombine") -> None:
+    """Writes the gradients into ``dgate`` / ``dup`` (any row stride: the halves of one packed buffer, or two)."""
+    device = _lib.require_device(gate, up, grad_out, dgate, dup)
+    rows, width = gate.shape
+    if rows and width:
+        grad_out = grad_out.contiguous().view(rows, width)
+        with _lib.on_device(device):
+            _lib.call("hmoe_glu_bwd", _lib.ptr(gate), _lib.ptr(up), gate.stride(0), up.stride(0), _lib.ptr(grad_out),
+                      rows, width, _lib.dtype_id(gate.dtype), *_kernel_args(combine), _lib.ptr(dgate), _lib.ptr(dup),
+                      dgate.stride(0), dup.stride(0), _lib.stream_ptr(device))
+
+
+class _FusedGLU(torch.autograd.Function):
+    """``combine(gate, up)`` over two tensors of one shape."""
+
+    @staticmethod
+    def forward(ctx, gate: torch.Tensor, up: torch.Tensor, combine: "GluCombine") -> torch.Tensor:
+        g, u = _as_rows(gate), _as_rows(up)
+        ctx.combine, ctx.shape = combine, gate.shape
+        ctx.save_for_backward(g, u)
+        return _glu_forward(g, u, combine).view(gate.shape)
+
+    @staticmethod
+    def backward(ctx, grad_out: torch.Tensor):
+        g, u = ctx.saved_tensors
+        dgate, dup = torch.empty_like(g), torch.empty_like(u)
+        _glu_backward(g, u, grad_out, dgate, dup, ctx.combine)
+        return dgate.view(ctx.shape), dup.view(ctx.shape), None
+
+
+class _FusedPackedGLU(torch.autograd.Function):
+    """``combine`` over the two halves of a ``[..., 2 M]`` ``[gate | up]`` tensor, read where they lie; the gradient
+    comes back as one ``[..., 2 M]`` buffer whose halves the kernel fills."""
+
+    @staticmethod
+    def forward(ctx, gate_up: torch.Tensor, combine: "GluCombine") -> torch.Tensor:
+        packed = _as_rows(gate_up)
+        half = packed.shape[1] // 2
+        ctx.combine, ctx.shape = combine, gate_up.shape
+        ctx.save_for_backward(packed)
+        return _glu_forward(packed[:, :half], packed[:, half:], combine).view(*gate_up.shape[:-1], half)
+
+    @staticmethod
+    def backward(ctx, grad_out: torch.Tensor):
+        (packed,) = ctx.saved_tensors
+        half = packed.shape[1] // 2
+        grad = torch.empty_like(packed, memory_format=torch.contiguous_format)
+        _glu_backward(packed[:, :half], packed[:, half:], grad_out, grad[:, :half], grad[:, half:], ctx.combine)
+        return grad.view(ctx.shape), None
+
+
+# ---------------------------------------------------------------------------------------------------- combine
+
 @dataclass(frozen=True)
 class GluCombine:
-    """``alpha`` and ``limit`` are runtime kernel arguments; the activation and the two clamp flags pick one of the
-    ahead-of-time kernel instances."""
+    """One of the fused ``activation(gate) * up`` forms; frozen, so two combines with the same numbers are equal and a
+    combine can key a cache.  Calling it (or ``packed``) runs the HIP kernel pair, or the eager form when
+    ``HALO_FUSED_GLU`` turns the kernels off."""
 
     activation: int
     alpha: float = 1.0
@@ -176,71 +181,76 @@ class GluCombine:
     clamp_activated: bool = False
     up_plus_one: bool = False
 
+    # constructors -----------------------------------------------------------------------------------------
     @classmethod
     def silu(cls) -> "GluCombine":
-        return cls(_SILU)
+        return cls(activation=_SILU)
 
     @classmethod
     def gelu_tanh(cls) -> "GluCombine":
-        return cls(_GELU_TANH)
+        return cls(activation=_GELU_TANH)
 
     @classmethod
     def clamped_silu(cls, limit: float, *, clamp_activated: bool = False) -> "GluCombine":
-        """The gate clamped before SiLU (DeepSeek-V4, GLM-5 Next) or, with ``clamp_activated``, after (Step-3.7)."""
-        return cls(_CLAMPED_SILU, limit=float(limit), clamp_activated=clamp_activated)
+        """SiLU with the gate cut off at ``limit`` before the activation, or after it with ``clamp_activated``;
+        ``up`` within ``±limit`` either way."""
+        return cls(activation=_CLAMPED_SILU, limit=float(limit), clamp_activated=bool(clamp_activated))
 
     @classmethod
     def gptoss(cls, alpha: float, limit: float) -> "GluCombine":
-        return cls(_CLAMPED_SILU, alpha=float(alpha), limit=float(limit), up_plus_one=True)
+        return cls(activation=_CLAMPED_SILU, alpha=float(alpha), limit=float(limit), up_plus_one=True)
 
+    # use --------------------------------------------------------------------------------------------------
     @property
     def name(self) -> str:
-        if self.activation != _CLAMPED_SILU:
-            return "silu" if self.activation == _SILU else "gelu_tanh"
-        if self.up_plus_one:
-            return "gptoss"
-        return "silu_then_clamp" if self.clamp_activated else "clamped_silu"
+        if self.activation == _CLAMPED_SILU:
+            if self.up_plus_one:
+                return "gptoss"
+            return ("clamped_silu", "silu_then_clamp")[self.clamp_activated]
+        return ("silu", "gelu_tanh")[self.activation == _GELU_TANH]
 
     def __call__(self, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-        if fused_glu_enabled():
-            return _FusedGLU.apply(gate, up, self)
-        return self._eager(gate, up)
+        return _FusedGLU.apply(gate, up, self) if _FUSED_GLU_ENABLED else self._eager(gate, up)
 
     def packed(self, gate_up: torch.Tensor) -> torch.Tensor:
-        if fused_glu_enabled():
+        if _FUSED_GLU_ENABLED:
             return _FusedPackedGLU.apply(gate_up, self)
-        return self._eager(*gate_up.chunk(2, dim=-1))
+        gate, up = gate_up.chunk(2, dim=-1)
+        return self._eager(gate, up)
 
     def _eager(self, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-        if self.activation == _SILU:
+        kind = self.name
+        if kind == "silu":
             return silu_mul_eager(gate, up)
-        if self.activation == _GELU_TANH:
+        if kind == "gelu_tanh":
             return gelu_tanh_mul_eager(gate, up)
-        if self.up_plus_one:
+        if kind == "gptoss":
             return gptoss_glu_eager(gate, up, self.alpha, self.limit)
-        if self.clamp_activated:
+        if kind == "silu_then_clamp":
             return silu_then_clamp_mul_eager(gate, up, self.limit)
         return clamped_silu_mul_eager(gate, up, self.limit)
 
 
 def resolve_fused_glu_mul(act_fn: object) -> GluCombine | None:
-    """The fused combine computing ``act_fn(gate) * up``, or None for the eager ``act_fn`` combine."""
-    if is_silu_activation(act_fn):
-        return GluCombine.silu()
-    if is_gelu_tanh_activation(act_fn):
-        return GluCombine.gelu_tanh()
+    """The fused combine that computes ``act_fn(gate) * up``; None when ``act_fn`` is neither SiLU nor tanh-GELU (the
+    caller then multiplies eagerly)."""
+    for probe, make in ((is_silu_activation, GluCombine.silu), (is_gelu_tanh_activation, GluCombine.gelu_tanh)):
+        if probe(act_fn):
+            return make()
     return None
 
 
-def resolve_clamped_glu_mul(
-    act_fn: object, limit: float, *, clamp_activated: bool
-) -> Callable[[torch.Tensor, torch.Tensor], torch.Tensor]:
-    """Fused for a SiLU gate; any other activation runs the same clamps eagerly."""
+def resolve_clamped_glu_mul(act_fn: object, limit: float, *,
+                            clamp_activated: bool) -> Callable[[torch.Tensor, torch.Tensor], torch.Tensor]:
+    """The clamped combine for ``act_fn``: fused when it is SiLU, else the same clamps around ``act_fn`` in torch."""
     if is_silu_activation(act_fn):
         return GluCombine.clamped_silu(limit, clamp_activated=clamp_activated)
 
     def clamped_glu_mul_eager(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-        activated = act_fn(gate).clamp(max=limit) if clamp_activated else act_fn(gate.clamp(max=limit))
-        return activated * up.clamp(min=-limit, max=limit)
+        if clamp_activated:
+            head = torch.clamp(act_fn(gate), max=limit)
+        else:
+            head = act_fn(torch.clamp(gate, max=limit))
+        return head * _clip_up(up, limit)
 
     return clamped_glu_mul_eager

@@ -137,11 +137,9 @@ class _GroupedMMFunction(Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        mat_a, mat_b, offs = ctx.saved_tensors
-        grad_mat_a, grad_mat_b = grouped_mm_grads(
-            mat_a, mat_b, grad_output, offs, ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        )
-        return grad_mat_a, grad_mat_b, None
+        a, b, offs = ctx.saved_tensors
+        want_a, want_b = ctx.needs_input_grad[:2]
+        return (*grouped_mm_grads(a, b, grad_output, offs, want_a, want_b), None)
 
 
 def grouped_mm(mat_a, mat_b, *, offs=None):

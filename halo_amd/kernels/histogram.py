@@ -30,6 +30,9 @@ def sync_free_bincount(
 def accumulate_bincount(
     counter: torch.Tensor | None, indices: torch.Tensor, size: int, *, weights: torch.Tensor | None = None
 ) -> torch.Tensor:
-    """``counter`` is ``None`` until the first forward that routes and is added into in place afterwards."""
-    counts = sync_free_bincount(indices, size, weights=weights)
-    return counts if counter is None else counter.add_(counts)
+    """Adds this call's histogram into ``counter`` in place and returns it; with no counter yet (None before the first
+    forward that routes) the histogram itself becomes the counter."""
+    fresh = sync_free_bincount(indices, size, weights=weights)
+    if counter is None:
+        return fresh
+    return counter.add_(fresh)

@@ -75,23 +75,24 @@ def build_inv_map(sorted_token_idx: torch.Tensor, recv_N: int, width: int) -> to
     never calls this; it serves callers holding only ``sorted_token_idx`` and is a handful of device-side torch ops
     with no host readback (stable argsort, counts, exclusive cumsum, one scatter)."""
     device = _lib.require_device(sorted_token_idx)
-    sorted_token_idx = sorted_token_idx.long()
-    n_sorted = sorted_token_idx.shape[0]
-    inv_map = torch.full((recv_N, width), n_sorted, dtype=torch.long, device=device)
-    if n_sorted == 0:
-        return inv_map
-    order = torch.argsort(sorted_token_idx, stable=True)
-    tokens = sorted_token_idx.index_select(0, order)
-    counts = torch.zeros(recv_N, dtype=torch.long, device=device)
-    counts.scatter_add_(0, sorted_token_idx, torch.ones_like(sorted_token_idx))
-    starts = torch.cumsum(counts, 0) - counts
-    column = torch.arange(n_sorted, device=device) - starts.index_select(0, tokens)
-    inv_map[tokens, column] = order
-    return inv_map
+    token_of = sorted_token_idx.to(torch.int64)
+    rows = token_of.numel()
+    result = token_of.new_full((recv_N, width), rows)  # every slot the sentinel until a row claims it
+    if rows:
+        # sorted positions grouped by token, ascending inside a token (stable), then each position's rank inside its
+        # token: its index in the grouped order minus the index at which its token's run begins
+        by_token = torch.argsort(token_of, stable=True)
+        owner = token_of[by_token]
+        per_token = torch.bincount(token_of, minlength=recv_N)
+        run_start = per_token.cumsum(0) - per_token
+        rank = torch.arange(rows, device=device) - run_start[owner]
+        result[owner, rank] = by_token
+    return result
 
 
 class MoEGatherPermute(torch.autograd.Function):
-    """``sorted = tokens[sorted_token_idx]`` with an atomic-free gather-reduce backward over ``inv_map``."""
+    """The permute by expert: row j of the result is ``tokens[sorted_token_idx[j]]``.  Backward sums, per token, the
+    gradient rows of its sorted positions (``inv_map``) in fp32 without atomics."""
 
     @staticmethod
     def forward(ctx, tokens: torch.Tensor, sorted_token_idx: torch.Tensor, inv_map: torch.Tensor):
@@ -111,10 +112,11 @@ class MoEWeightedUnpermute(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, expert_out, weights, sorted_token_idx, inv_map):
-        expert_out, weights = expert_out.contiguous(), weights.contiguous()
-        ctx.weight_grad = ctx.needs_input_grad[1]
-        ctx.save_for_backward(expert_out if ctx.weight_grad else None, weights, sorted_token_idx.contiguous())
-        return gather_reduce_rows(expert_out, inv_map, weights)
+        rows, gates = expert_out.contiguous(), weights.contiguous()
+        ctx.weight_grad = bool(ctx.needs_input_grad[1])
+        # the rows are read again only by the gate weights' gradient: kept only when that gradient is wanted
+        ctx.save_for_backward(rows if ctx.weight_grad else None, gates, sorted_token_idx.contiguous())
+        return gather_reduce_rows(rows, inv_map, gates)
 
     @staticmethod
     def backward(ctx, grad_out):

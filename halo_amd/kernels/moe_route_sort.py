@@ -32,28 +32,30 @@ def counting_sort_raw(experts: torch.Tensor, weights: torch.Tensor, num_local_ex
         raise TypeError(f"expert ids must be int64 or int32, got {experts.dtype}")
     if weights.element_size() not in (2, 4, 8):
         raise TypeError(f"unsupported gate-weight dtype {weights.dtype}")
-    n_rows, top_k = experts.shape
-    experts, weights = experts.contiguous(), weights.contiguous()
-    lib = _lib.load()
-    ws_bytes = lib.hmoe_route_sort_workspace_bytes(n_rows, top_k, num_local_experts)
+    rows, k = experts.shape
+    ids, gates = experts.contiguous(), weights.contiguous()
+    ws_bytes = _lib.load().hmoe_route_sort_workspace_bytes(rows, k, num_local_experts)
     if ws_bytes < 0:
-        raise ValueError(f"bad routing shape: rows={n_rows} top_k={top_k} experts={num_local_experts}")
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=device)
-    offs = torch.empty(num_local_experts, dtype=torch.int32, device=device)
-    ok = torch.empty(1, dtype=torch.int32, device=device)
-    dest = torch.empty(n_rows * top_k, dtype=torch.int32, device=device)
-    sorted_token_idx = torch.empty(n_valid, dtype=torch.long, device=device)
-    sorted_weights = torch.empty(n_valid, dtype=weights.dtype, device=device)
-    sorted_expert_ids = torch.empty(n_valid, dtype=experts.dtype, device=device)
-    inv_map = torch.empty((n_rows, top_k), dtype=torch.long, device=device)
+        raise ValueError(f"bad routing shape: rows={rows} top_k={k} experts={num_local_experts}")
+
+    def buffer(shape, dtype):
+        return torch.empty(shape, dtype=dtype, device=device)
+
+    workspace = buffer(ws_bytes, torch.uint8)
+    out = {
+        "sorted_token_idx": buffer(n_valid, torch.int64),
+        "sorted_weights": buffer(n_valid, gates.dtype),
+        "sorted_expert_ids": buffer(n_valid, ids.dtype),
+        "offs": buffer(num_local_experts, torch.int32),
+        "inv_map": buffer((rows, k), torch.int64),
+        "dest": buffer(rows * k, torch.int32),
+        "ok": buffer(1, torch.int32),
+    }
     with _lib.on_device(device):
-        _lib.call(
-            "hmoe_route_sort", _lib.ptr(experts), _ID_BYTES[experts.dtype], _lib.ptr(weights), weights.element_size(),
-            n_rows, top_k, num_local_experts, n_valid, _lib.ptr(sorted_token_idx), _lib.ptr(sorted_weights),
-            _lib.ptr(sorted_expert_ids), _lib.ptr(offs), _lib.ptr(inv_map), _lib.ptr(dest), _lib.ptr(ok),
-            _lib.ptr(workspace), _lib.stream_ptr(device),
-        )
-    return sorted_token_idx, sorted_weights, sorted_expert_ids, offs, inv_map, dest, ok
+        _lib.call("hmoe_route_sort", _lib.ptr(ids), _ID_BYTES[ids.dtype], _lib.ptr(gates), gates.element_size(), rows,
+                  k, num_local_experts, n_valid, *(_lib.ptr(t) for t in out.values()), _lib.ptr(workspace),
+                  _lib.stream_ptr(device))
+    return tuple(out.values())
 
 
 class _CountingSort(torch.autograd.Function):
@@ -62,32 +64,30 @@ class _CountingSort(torch.autograd.Function):
     @staticmethod
     def forward(ctx, weights: torch.Tensor, experts: torch.Tensor, num_local_experts: int,
                 counts: tuple[int, ...] | None):
-        n_rows, top_k = experts.shape
-        n_valid = n_rows * top_k if counts is None else sum(counts)
-        sorted_token_idx, sorted_weights, sorted_expert_ids, offs, inv_map, dest, ok = counting_sort_raw(
-            experts, weights, num_local_experts, n_valid
-        )
-        # Device-side, no readback: a wrong total would have written past the outputs the counts sized.
-        torch._assert_async(ok, NONLOCAL_EXPERT_ID_MESSAGE if counts is None else RECEIVE_COUNTS_DISAGREE)
+        n_valid = experts.numel() if counts is None else sum(counts)
+        token_idx, gates, expert_ids, offs, inv_map, dest, ok = counting_sort_raw(experts, weights,
+                                                                                   num_local_experts, n_valid)
+        # Checked on the device, nothing read back: with a wrong total the sort leaves the outputs unwritten.
+        torch._assert_async(ok, RECEIVE_COUNTS_DISAGREE if counts is not None else NONLOCAL_EXPERT_ID_MESSAGE)
+        ctx.n_valid, ctx.weights_shape = n_valid, weights.shape
         ctx.save_for_backward(dest)
-        ctx.weights_shape = weights.shape
-        ctx.n_valid = n_valid
-        ctx.mark_non_differentiable(sorted_token_idx, sorted_expert_ids, offs, inv_map)
-        # The integer outputs take no gradient; materialized, each would cost a zero-fill in every backward.
+        # Only ``gates`` is differentiable; without materialised gradients backward is not handed a zero tensor for
+        # each of the integer outputs.
+        ctx.mark_non_differentiable(token_idx, expert_ids, offs, inv_map)
         ctx.set_materialize_grads(False)
-        return sorted_token_idx, sorted_weights, sorted_expert_ids, offs, inv_map
+        return token_idx, gates, expert_ids, offs, inv_map
 
     @staticmethod
     def backward(ctx, _token_grad, sorted_weights_grad, _expert_grad, _offs_grad, _inv_map_grad):
-        if sorted_weights_grad is None:
-            return None, None, None, None
-        (dest,) = ctx.saved_tensors
-        grad_sorted = sorted_weights_grad.contiguous()
-        grad = torch.empty(ctx.weights_shape, dtype=grad_sorted.dtype, device=grad_sorted.device)
-        with _lib.on_device(grad.device):
-            _lib.call("hmoe_route_sort_bwd", _lib.ptr(grad_sorted), _lib.ptr(dest), dest.numel(), ctx.n_valid,
-                      grad_sorted.element_size(), _lib.ptr(grad), _lib.stream_ptr(grad.device))
-        return grad, None, None, None
+        if sorted_weights_grad is not None:
+            (dest,) = ctx.saved_tensors
+            grad_sorted = sorted_weights_grad.contiguous()
+            grad = grad_sorted.new_empty(ctx.weights_shape)
+            with _lib.on_device(grad.device):
+                _lib.call("hmoe_route_sort_bwd", _lib.ptr(grad_sorted), _lib.ptr(dest), dest.numel(), ctx.n_valid,
+                          grad_sorted.element_size(), _lib.ptr(grad), _lib.stream_ptr(grad.device))
+            return grad, None, None, None
+        return (None,) * 4
 
 
 def sort_routing_by_expert(

@@ -80,17 +80,24 @@ class EPGptOssMoELayer(EPMoELayerBase):
 
     def _adopt_expert_params(self, experts: nn.Module, weights_already_sharded: bool = False) -> None:
         self._require_fused_experts(experts)
-        start, end = self._local_expert_range(weights_already_sharded)
-        gate, up = split_interleaved_gate_up(experts.gate_up_proj.data[start:end])  # HF keeps [E, H, 2F] here
-        self.gate_proj_gmm = nn.Parameter(gate.contiguous())
-        self.up_proj_gmm = nn.Parameter(up.contiguous())
-        if getattr(experts, "gate_up_proj_bias", None) is not None:
-            gate_bias, up_bias = split_interleaved_gate_up(experts.gate_up_proj_bias.data[start:end])
-            self.gate_proj_gmm_bias = nn.Parameter(gate_bias.contiguous())
-            self.up_proj_gmm_bias = nn.Parameter(up_bias.contiguous())
-        self.down_proj = nn.Parameter(experts.down_proj.data[start:end].clone())
-        if getattr(experts, "down_proj_bias", None) is not None:
-            self.down_proj_bias = nn.Parameter(experts.down_proj_bias.data[start:end].clone())
+        local = slice(*self._local_expert_range(weights_already_sharded))
+
+        def own(tensor: torch.Tensor) -> nn.Parameter:  # this rank's experts, as a dense parameter of its own
+            return nn.Parameter(tensor.contiguous().clone() if tensor.is_contiguous() else tensor.contiguous())
+
+        # HF keeps gate and up interleaved column by column in one [E, H, 2F] weight (and one [E, 2F] bias); the
+        # grouped GEMMs take them apart
+        for source, suffix in (("gate_up_proj", ""), ("gate_up_proj_bias", "_bias")):
+            packed = getattr(experts, source, None)
+            if packed is None:
+                continue
+            gate_half, up_half = split_interleaved_gate_up(packed.data[local])
+            setattr(self, f"gate_proj_gmm{suffix}", own(gate_half))
+            setattr(self, f"up_proj_gmm{suffix}", own(up_half))
+        for source in ("down_proj", "down_proj_bias"):
+            tensor = getattr(experts, source, None)
+            if tensor is not None:
+                setattr(self, source, own(tensor.data[local]))
 
     @classmethod
     def from_weights(cls, *, alpha: float = 1.702, limit: float = 7.0, router_bias: torch.Tensor | None = None,
@@ -118,10 +125,11 @@ class EPGptOssMoELayer(EPMoELayerBase):
         """Three grouped GEMMs (gate, up, down) on de-interleaved weights, each plus its expert bias."""
         gate_attr, up_attr = ("gate_proj_gmm", "up_proj_gmm") if hasattr(self, "gate_proj_gmm") else (
             "gate_proj", "up_proj")
-        gate = self._grouped_proj_with_bias(sorted_tokens, gate_attr, offs, output_dtype, sorted_expert_ids)
-        up = self._grouped_proj_with_bias(sorted_tokens, up_attr, offs, output_dtype, sorted_expert_ids)
-        gated = self._gptoss_glu(gate, up)
-        return self._grouped_proj_with_bias(gated.to(output_dtype), "down_proj", offs, output_dtype, sorted_expert_ids)
+        def project(x, weight_attr):
+            return self._grouped_proj_with_bias(x, weight_attr, offs, output_dtype, sorted_expert_ids)
+
+        hidden = self._gptoss_glu(project(sorted_tokens, gate_attr), project(sorted_tokens, up_attr))
+        return project(hidden.to(output_dtype), "down_proj")
 
     def _grouped_proj_with_bias(self, x, weight_attr, offs, out_dtype, eids):
         bias = getattr(self, f"{weight_attr}_bias", None)

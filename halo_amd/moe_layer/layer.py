@@ -96,15 +96,19 @@ class EPMoELayerBase(nn.Module, ABC):
     _TOPK_WEIGHT_NORM_EPS: float = 1e-20
 
     def __init__(self, original_layer: nn.Module, ep_config: EPConfig, weights_already_sharded: bool = False):
-        router = self._declared_router(original_layer)
+        # what the HF block holds, found before nn.Module's own state exists
         experts = self._find_experts_container(original_layer)
-        if ep_config.num_experts is None:
+        router = self._declared_router(original_layer)
+        if ep_config.num_experts is None:  # the expert range of this rank follows from the block's expert count
             ep_config.finalize_expert_assignment(self.detect_num_experts(original_layer))
-        self._init_ep_state(ep_config, self._detect_hidden_dim(router, experts))
+        hidden = self._detect_hidden_dim(router, experts)
+        self._init_ep_state(ep_config, hidden)
+        # the hooks a family overrides, in the reference's order: router, routing fields, shared expert, activation,
+        # expert weights, dtype fix-ups
         if router is not None:
-            setattr(self, self._ROUTER_ATTR, router)
-        self._adopt_routing(original_layer)
-        self._adopt_shared_experts(original_layer)
+            self.add_module(self._ROUTER_ATTR, router)
+        for adopt in (self._adopt_routing, self._adopt_shared_experts):
+            adopt(original_layer)
         self._adopt_expert_compute(original_layer, experts)
         self._adopt_expert_params(experts, weights_already_sharded=weights_already_sharded)
         self._finalize_expert_init()
@@ -113,54 +117,58 @@ class EPMoELayerBase(nn.Module, ABC):
 
     @classmethod
     def detect_num_experts(cls, layer: nn.Module) -> int:
-        experts = cls._find_experts_container(layer)
-        return len(experts) if isinstance(experts, nn.ModuleList) else experts.num_experts
+        container = cls._find_experts_container(layer)
+        if isinstance(container, nn.ModuleList):  # one module per expert
+            return len(container)
+        return int(container.num_experts)
 
     @classmethod
     def _declared_router(cls, layer: nn.Module) -> nn.Module | None:
-        if cls._ROUTER_ATTR is None:
+        name = cls._ROUTER_ATTR
+        if name is None:  # a family whose router lives outside the block
             return None
-        router = getattr(layer, cls._ROUTER_ATTR, None)
-        if router is None:
-            raise AttributeError(f"{cls.__name__} declares _ROUTER_ATTR='{cls._ROUTER_ATTR}', but "
-                                 f"{type(layer).__name__} has no such attribute")
-        return router
+        found = getattr(layer, name, None)
+        if found is not None:
+            return found
+        raise AttributeError(f"{cls.__name__} declares _ROUTER_ATTR='{name}', but {type(layer).__name__} has no such "
+                             f"attribute")
 
     @classmethod
     def _find_experts_container(cls, layer: nn.Module) -> nn.Module:
-        for attr in cls.FAMILY.experts_container_attrs:
-            if hasattr(layer, attr):
-                return getattr(layer, attr)
-        raise AttributeError(f"{cls.__name__}: {type(layer).__name__} carries none of "
-                             f"{cls.FAMILY.experts_container_attrs}")
+        candidates = cls.FAMILY.experts_container_attrs
+        present = [name for name in candidates if hasattr(layer, name)]
+        if not present:
+            raise AttributeError(f"{cls.__name__}: {type(layer).__name__} carries none of {candidates}")
+        return getattr(layer, present[0])
 
     @classmethod
     def _detect_hidden_dim(cls, router: nn.Module | None, experts: nn.Module) -> int:
-        if router is not None and hasattr(router, "weight"):
-            return router.weight.shape[1]
-        return cls._require_fused_experts(experts).gate_up_proj.shape[2]
+        weight = getattr(router, "weight", None)
+        if weight is not None:  # [E, H]
+            return int(weight.shape[1])
+        return int(cls._require_fused_experts(experts).gate_up_proj.shape[2])  # HF layout [E, 2F, H]
 
     @staticmethod
     def _require_fused_experts(experts: nn.Module) -> nn.Module:
-        missing = [name for name in ("gate_up_proj", "down_proj") if not hasattr(experts, name)]
-        if missing:
-            raise AttributeError(f"Expected fused-GLU experts carrying gate_up_proj and down_proj, but "
-                                 f"{type(experts).__name__} carries no {missing}")
-        return experts
+        absent = [name for name in ("gate_up_proj", "down_proj") if getattr(experts, name, None) is None]
+        if not absent:
+            return experts
+        raise AttributeError(f"Expected fused-GLU experts carrying gate_up_proj and down_proj, but "
+                             f"{type(experts).__name__} carries no {absent}")
 
     def _init_ep_state(self, ep_config: EPConfig, hidden_dim: int) -> None:
-        super().__init__()
-        self.ep_config = ep_config
-        self.num_experts = ep_config.num_experts
-        self.experts_per_rank = ep_config.experts_per_rank
-        self.ep_rank, self.ep_size = ep_config.ep_rank, ep_config.ep_size
-        self.expert_start, self.expert_end = ep_config.expert_start_idx, ep_config.expert_end_idx
-        self.hidden_dim = hidden_dim
-        self.expert_tp_size, self.expert_tp_rank = ep_config.expert_tp_size, ep_config.expert_tp_rank
-        self.fp32_router, self.fp32_experts = ep_config.fp32_router, ep_config.fp32_experts
         if not ep_config.grouped_gemm_enabled:
             raise NotImplementedError("the per-expert loop is the reference's CPU path; this block runs the grouped "
                                       "kernels only (use_grouped_gemm=True)")
+        super().__init__()
+        self.ep_config, self.hidden_dim = ep_config, hidden_dim
+        # the fields the reference's block exposes, copied off the config
+        for field, source in (("num_experts", "num_experts"), ("experts_per_rank", "experts_per_rank"),
+                              ("ep_rank", "ep_rank"), ("ep_size", "ep_size"), ("expert_start", "expert_start_idx"),
+                              ("expert_end", "expert_end_idx"), ("expert_tp_size", "expert_tp_size"),
+                              ("expert_tp_rank", "expert_tp_rank"), ("fp32_router", "fp32_router"),
+                              ("fp32_experts", "fp32_experts")):
+            setattr(self, field, getattr(ep_config, source))
         self._use_grouped_mm = True
         self._expert_kernels_warmed = False
         self._lowp_quant_format = None
@@ -214,25 +222,31 @@ class EPMoELayerBase(nn.Module, ABC):
         ``separate_glu`` family."""
         self._require_fused_experts(experts)
         start, end = self._local_expert_range(weights_already_sharded)
-        gate_up = experts.gate_up_proj.data[start:end]
-        down = experts.down_proj.data[start:end]
-        if self.FAMILY.expert_layout == "separate_glu":
-            gate, up = gate_up.chunk(2, dim=1)
-            self.gate_proj = nn.Parameter(gate.transpose(1, 2).contiguous())
-            self.up_proj = nn.Parameter(up.transpose(1, 2).contiguous())
+        def to_matmul_layout(weight: torch.Tensor) -> nn.Parameter:  # [E, out, in] -> [E, in, out], dense
+            return nn.Parameter(weight.transpose(1, 2).contiguous())
+
+        local = slice(start, end)
+        fused = experts.gate_up_proj.data[local]
+        if self.FAMILY.expert_layout != "separate_glu":
+            self.gate_up_proj = to_matmul_layout(fused)
         else:
-            self.gate_up_proj = nn.Parameter(gate_up.transpose(1, 2).contiguous())
-        self.down_proj = nn.Parameter(down.transpose(1, 2).contiguous())
+            halves = fused.chunk(2, dim=1)  # rows [gate ; up] of the HF weight
+            self.gate_proj, self.up_proj = to_matmul_layout(halves[0]), to_matmul_layout(halves[1])
+        self.down_proj = to_matmul_layout(experts.down_proj.data[local])
 
     def _finalize_expert_init(self) -> None:
-        if self.fp32_router and self._ROUTER_ATTR is not None:
-            setattr(self, self._ROUTER_ATTR, getattr(self, self._ROUTER_ATTR).float())
-        if self.fp32_experts:
-            for name, param in self.expert_named_params():
-                setattr(self, name, nn.Parameter(param.data.float(), requires_grad=param.requires_grad))
+        router_name = self._ROUTER_ATTR
+        if router_name is not None and self.fp32_router:
+            getattr(self, router_name).float()  # nn.Module.float() converts in place
+        if not self.fp32_experts:
+            return
+        for name, weight in self.expert_named_params():
+            upcast = nn.Parameter(weight.data.to(torch.float32), requires_grad=weight.requires_grad)
+            setattr(self, name, upcast)
 
     def expert_named_params(self) -> list:
-        return [(n, getattr(self, n)) for n in self.FAMILY.expert_weight_roots if hasattr(self, n)]
+        held = (root for root in self.FAMILY.expert_weight_roots if hasattr(self, root))
+        return [(root, getattr(self, root)) for root in held]
 
     def replicated_named_params(self) -> list:
         shared = getattr(self, self._shared_expert_attr, None)
@@ -279,12 +293,10 @@ class EPMoELayerBase(nn.Module, ABC):
         )
 
     def _require_recv_counts(self, recv_counts: tuple[int, ...] | None) -> tuple[int, ...]:
-        if recv_counts is None or len(recv_counts) != self.experts_per_rank:
-            raise RuntimeError(
-                f"{type(self).__name__}: the expert compute at ep_size={self.ep_size} needs the dispatch's "
-                f"per-local-expert receive counts ({self.experts_per_rank} of them), got {recv_counts!r}."
-            )
-        return recv_counts
+        if recv_counts is not None and len(recv_counts) == self.experts_per_rank:
+            return recv_counts
+        raise RuntimeError(f"{type(self).__name__}: the expert compute at ep_size={self.ep_size} needs the dispatch's "
+                           f"per-local-expert receive counts ({self.experts_per_rank} of them), got {recv_counts!r}.")
 
     def _sort_tokens_for_grouped_mm(self, tokens, experts, weights, *, recv_counts):
         """``(sorted_tokens, offs, sorted_token_idx, sorted_weights, sorted_expert_ids, inv_map)`` over the valid local
@@ -324,24 +336,28 @@ class EPMoELayerBase(nn.Module, ABC):
         return hasattr(self, "gate_up_proj")
 
     def _glu_ffn(self, x: torch.Tensor, proj: Callable[[torch.Tensor, str], torch.Tensor]) -> torch.Tensor:
-        if self._stores_fused_glu:
-            return proj(self._glu_combine_packed(proj(x, "gate_up_proj")), "down_proj")
-        return proj(self._glu_combine(proj(x, "gate_proj"), proj(x, "up_proj")), "down_proj")
+        if self._stores_fused_glu:  # one projection to [gate | up], combined where it lies
+            hidden = self._glu_combine_packed(proj(x, "gate_up_proj"))
+        else:
+            hidden = self._glu_combine(proj(x, "gate_proj"), proj(x, "up_proj"))
+        return proj(hidden, "down_proj")
 
     def _glu_combine(self, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
         return self._fused_glu_mul(gate, up)
 
     def _glu_combine_packed(self, gate_up: torch.Tensor) -> torch.Tensor:
-        if isinstance(self._fused_glu_mul, GluCombine):
-            return self._fused_glu_mul.packed(gate_up)
-        gate, up = gate_up.chunk(2, dim=-1)
-        return self._glu_combine(gate, up)
+        combine = self._fused_glu_mul
+        if not isinstance(combine, GluCombine):  # an eager callable: it takes the halves as two tensors
+            return self._glu_combine(*gate_up.chunk(2, dim=-1))
+        return combine.packed(gate_up)
 
     def _glu_combine_name(self) -> str:
         combine = self._fused_glu_mul
-        if combine is None or not fused_glu_enabled():
-            return "eager"
-        return combine.name if isinstance(combine, GluCombine) else getattr(combine, "__name__", "eager")
+        if fused_glu_enabled() and combine is not None:
+            if isinstance(combine, GluCombine):
+                return combine.name
+            return getattr(combine, "__name__", "eager")
+        return "eager"
 
     # ------------------------------------------------------------------------------------------------- routing
 
