@@ -61,13 +61,15 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 
 constexpr int BK = 64;  // contraction per step
 constexpr int kXcds = 8;
 constexpr int kMaxGroups = 1024;
 
-enum Mode { kFwd = 0, kDgrad = 1, kWgrad = 2, kFwdFp8W = 3 };
+enum Mode { kFwd = 0, kDgrad = 1, kWgrad = 2, kFwdFp8W = 3, kFwdFp8 = 4 };
 
 // Tile configuration: GM x GN wavefronts, each WM x WN blocks of 32x32.
 template <int GM_, int GN_, int WM_, int WN_>
@@ -94,6 +96,11 @@ struct GemmArgs {
   const int64_t* a_index = nullptr;  // gathered A (fwd, wgrad): logical row r of A is a[a_index[r]]
   int64_t a_rows = 0;                // rows of the array a_index points into
   const void* bias = nullptr;        // fwd: [G, N] in the operands' dtype, added to group g's output rows
+  // kFwdFp8: both operands are e4m3 bytes with the contraction contiguous (A [R, K], B [G, N, K]); k, lda and ldb
+  // count 2-byte units, so a step of BK units is 128 values: one scale block
+  const uint8_t* a_scale = nullptr;  // [K / 128][a_scale_rows]: the e8m0 exponent of row r's block b at (b, r)
+  int64_t a_scale_rows = 0;
+  int k_blocks = 0, n_blocks = 0;     // the grid of b_scale [G, k_blocks, n_blocks]
 };
 
 __device__ __forceinline__ int swizzle(int row) { return (row & 7) ^ ((row >> 3) & 7); }
@@ -977,13 +984,15 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
   static_assert(!kBias || kMode == kFwd, "the expert bias belongs to the forward product");
   static_assert(!kGather || kMode == kFwd || kMode == kWgrad, "A is gathered in fwd and wgrad");
+  static_assert(kMode != kFwdFp8 || (!kGather && !kBias), "the fp8 product takes plain operands");
   constexpr int WM = Cfg::WM, WN = Cfg::WN, BM = Cfg::BM, BN = Cfg::BN;
   constexpr int kWaves = Cfg::GM * Cfg::GN;
   // Wavefronts 0-3 issue all the tile loads and wait for them (16 loads of 1 KB each per step, measured slightly
   // ahead of dealing them to every wavefront); every wavefront runs the MFMAs.
   constexpr int kLoadWaves = 4;
   constexpr int kI = 32 / kLoadWaves;
-  constexpr bool kDirectA = kMode != kWgrad, kDirectB = kMode == kDgrad;
+  constexpr bool kFp8 = kMode == kFwdFp8;
+  constexpr bool kDirectA = kMode != kWgrad, kDirectB = kMode == kDgrad || kFp8;
   using PlainA = typename std::conditional<kDirectA, SlimDirect<kI>, SlimTransposed<kI>>::type;
   using GatheredA = typename std::conditional<kDirectA, GatherDirect<kI>, GatherTransposed<kI>>::type;
   using LoaderA = typename std::conditional<kGather, GatheredA, PlainA>::type;
@@ -1106,6 +1115,23 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     for (int i = 0; i < WM; ++i)
       if (i < rows_live) fa[buf][i] = LoaderA::fragment(ta, fa_base[kDirectA ? 0 : i], i, kk);
   };
+  // fp8: a fragment of the 32x32x64 MFMA is two 16-byte reads, the chunks sub-steps 2 h and 2 h + 1 of the bf16
+  // geometry would take.  Which 32 of the 64 values a lane holds does not matter to the product as long as both
+  // operands agree, and here it does not matter to the scales either: a step is one scale block.
+  // One set of fragments: each is replaced by the next half's as soon as its last MFMA of this half is issued (a
+  // second set would not fit beside the accumulators), which the order of the MFMAs makes early enough.
+  i32x8 fa8[WM], fb8[WN];
+  auto fragment8 = [&](const char* tile_base, int base, int block, int half) __attribute__((always_inline)) {
+    const i32x4 lo = __builtin_bit_cast(i32x4, SlimDirect<kI>::fragment(tile_base, base, block, 2 * half));
+    const i32x4 hi = __builtin_bit_cast(i32x4, SlimDirect<kI>::fragment(tile_base, base, block, 2 * half + 1));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  auto read_a8 = [&](int stage, int half, int i) __attribute__((always_inline)) {
+    if constexpr (kFp8) fa8[i] = fragment8(lds_raw + stage * kStageBytes, fa_base[0], i, half);
+  };
+  auto read_b8 = [&](int stage, int half, int j) __attribute__((always_inline)) {
+    if constexpr (kFp8) fb8[j] = fragment8(lds_raw + stage * kStageBytes + kTileBytes, fb_base[0], j, half);
+  };
   constexpr int kReads = WM * (kDirectA ? 1 : 2) + WN * (kDirectB ? 1 : 2);  // LDS reads of one sub-step
   constexpr int kMfmas = WM * WN;
   constexpr int kEpiPitch = WN * 32 + 8;
@@ -1147,10 +1173,43 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       if (col < tile.b_out_lim)
         bias_chunk = *reinterpret_cast<const u32x4*>(static_cast<const bf16_t*>(p.bias) + tile.g * p.n + col);
     }
+    // fp8: the scales.  Activations: per row and step one e8m0 byte, the bytes of a step contiguous over the rows;
+    // lane L and lane L + 32 of an MFMA both answer for row L & 31.  Weights: one fp32 per step and 128 output
+    // columns, the same for the whole wavefront (its 64 columns lie in one block).  Both are fetched a step ahead
+    // and pinned as arrived at the top of the step that uses them, right behind the wait the loading wavefronts
+    // make there anyway.
+    uint32_t sa_next[kFp8 ? WM : 1] = {};
+    uint32_t sb_next = 0;
+    __amdgpu_buffer_rsrc_t sa_rsrc, sb_rsrc;
+    uint32_t sa_off = 0, sb_off = 0, sa_step = 0, sb_step = 0;
+    if constexpr (kFp8) {
+      sa_step = static_cast<uint32_t>(p.a_scale_rows);
+      sa_rsrc = make_rsrc(p.a_scale, static_cast<uint32_t>(p.k_blocks) * sa_step);
+      sb_rsrc = make_rsrc(p.b_scale, static_cast<uint32_t>(p.groups) * p.k_blocks * p.n_blocks * 4u);
+      sa_off = static_cast<uint32_t>(tile.row_start + tile.a_out0 + row_a + (lane & 31));
+      sb_step = static_cast<uint32_t>(p.n_blocks) * 4u;
+      sb_off = (static_cast<uint32_t>(tile.g) * p.k_blocks * p.n_blocks + ((tile.b_out0 + row_b) >> 7)) * 4u;
+#pragma unroll
+      for (int i = 0; i < WM; ++i) sa_next[i] = __builtin_amdgcn_raw_buffer_load_b8(sa_rsrc, sa_off, i * 32, 0);
+      sb_next = __builtin_amdgcn_raw_buffer_load_b32(sb_rsrc, sb_off, 0, 0);
+    }
     if (load_wave) wait_loads();
     if constexpr (kBias) asm volatile("" : "+v"(bias_chunk));
     workgroup_barrier();  // step 0 of this tile has landed in stage 0
-    if (steps > 0) read_live_fragments(0, 0, 0, live);
+    if (steps > 0) {
+      if constexpr (kFp8) {
+        if (live > 0) {
+#pragma unroll
+          for (int j = 0; j < WN; ++j) read_b8(0, 0, j);
+        }
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+          if (i < live) read_a8(0, 0, i);
+      } else {
+        read_live_fragments(0, 0, 0, live);
+      }
+    }
+    float mant_last = 1.0f;  // fp8: the weight scale's mantissa of the last step, still owed to the accumulators
 
     auto run = [&](auto full_tag) __attribute__((always_inline)) {
       constexpr bool kFull = decltype(full_tag)::value;
@@ -1205,8 +1264,109 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         if constexpr (kFull) interleave_reads_under_mfmas<kReads, kMfmas / 2>();
       }
     };
-    if (live == WM) run(std::true_type{});
-    else run(std::false_type{});
+    // fp8.  The MFMA takes each operand's scale as a power of two: the activations' scales are powers of two by
+    // construction and go in whole, a weight scale goes in as its exponent, and its mantissa m (1 for the scales
+    // the block quantiser makes) is carried by the accumulators: they hold sum / m of the steps so far, are
+    // multiplied by m_previous / m where the mantissa changes, and by the last m at the end.
+    auto run8 = [&](auto full_tag) __attribute__((always_inline)) {
+      constexpr bool kFull = decltype(full_tag)::value;
+      static_assert(WM == 4 && WN == 2, "the order below is written out for 4 x 2 blocks");
+      auto mfma = [&](auto row_block, auto col_block, int sa, int sb) __attribute__((always_inline)) {
+        constexpr int i = decltype(row_block)::value, j = decltype(col_block)::value;
+        if (kFull || i < live)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[j], fa8[i], acc[i][j], 0, 0, 0, sb, i, sa);
+      };
+      using std::integral_constant;
+      const integral_constant<int, 0> b0;
+      const integral_constant<int, 1> b1;
+      const integral_constant<int, 2> b2;
+      const integral_constant<int, 3> b3;
+      // The MFMAs of one half against weight fragment 0; then fragment 0 is free for the next half's.
+      auto column0 = [&](int sa, int sb) __attribute__((always_inline)) {
+        mfma(b0, b0, sa, sb);
+        mfma(b1, b0, sa, sb);
+        mfma(b2, b0, sa, sb);
+        mfma(b3, b0, sa, sb);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      // The MFMAs against weight fragment 1, each followed by the refill of its activation fragment from (stage,
+      // half), and fragment 1's own refill at the end.  A refill is three MFMAs or more ahead of its first use, and
+      // stays behind the MFMA that frees its registers (hoisted, it would need registers of its own).
+      auto column1_refilling = [&](int sa, int sb, int stage, int half) __attribute__((always_inline)) {
+        if (kFull || live > 0) read_b8(stage, half, 0);
+        auto one = [&](auto row_block) __attribute__((always_inline)) {
+          constexpr int i = decltype(row_block)::value;
+          mfma(row_block, b1, sa, sb);
+          if (kFull || i < live) read_a8(stage, half, i);
+          __builtin_amdgcn_sched_barrier(0);
+        };
+        one(b0);
+        one(b1);
+        one(b2);
+        one(b3);
+        if (kFull || live > 0) read_b8(stage, half, 1);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      for (int step = 0; step < steps; ++step) {
+        const int cur = step & 1;
+        const bool more = step + 1 < steps;
+        asm volatile("" : "+v"(sb_next));
+        const uint32_t sb_bits = uniform(sb_next);
+        // the step's activation scales in one register, block i's in byte i (the MFMA picks the byte)
+        static_assert(WM == 4, "four row blocks, four bytes");
+#pragma unroll
+        for (int i = 0; i < WM; ++i) asm volatile("" : "+v"(sa_next[i]));
+        const int sa = static_cast<int>((sa_next[0] & 0xffu) | ((sa_next[1] & 0xffu) << 8) |
+                                        ((sa_next[2] & 0xffu) << 16) | (sa_next[3] << 24));
+        if (load_wave) {
+          la.issue(lds + (cur ^ 1) * kStageBytes, step + 1, load_slot, more);
+          lb.issue(lds + (cur ^ 1) * kStageBytes + kTileBytes, step + 1, load_slot, more);
+        }
+        // past the last step these read out of range (zeros) or a neighbour's scale, and nothing uses them
+        sb_next = __builtin_amdgcn_raw_buffer_load_b32(sb_rsrc, sb_off, (step + 1) * sb_step, 0);
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+          sa_next[i] = __builtin_amdgcn_raw_buffer_load_b8(sa_rsrc, sa_off, (step + 1) * sa_step + i * 32, 0);
+        // a zero or subnormal weight scale goes in as 2^-127 with mantissa 1: its block contributes nothing either way
+        const uint32_t sb_exp = sb_bits >> 23;
+        const float mant = sb_exp ? __uint_as_float((sb_bits & 0x007fffffu) | 0x3f800000u) : 1.0f;
+        if (mant != mant_last) {
+          const float ratio = mant_last / mant;
+#pragma unroll
+          for (int i = 0; i < WM; ++i)
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+#pragma unroll
+              for (int v = 0; v < 16; ++v) acc[i][j][v] *= ratio;
+          mant_last = mant;
+        }
+        const int sb = static_cast<int>(sb_exp);
+        __builtin_amdgcn_sched_barrier(0);
+        column0(sa, sb);
+        column1_refilling(sa, sb, cur, 1);
+        column0(sa, sb);
+        // lgkmcnt(0): this stage is read out; vmcnt(0) where tile loads were issued: the next step has landed
+        if (load_wave) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        workgroup_barrier();
+        column1_refilling(sa, sb, cur ^ 1, 0);  // (after a tile's last step the refills read what nothing uses)
+      }
+    };
+    if constexpr (kFp8) {
+      if (live == WM) run8(std::true_type{});
+      else run8(std::false_type{});
+      if (mant_last != 1.0f) {
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+          for (int j = 0; j < WN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] *= mant_last;
+      }
+    } else {
+      if (live == WM) run(std::true_type{});
+      else run(std::false_type{});
+    }
 
     // both stages are free: start the next tile's first step into stage 0 before this tile's epilogue
     const TileInfo done = tile;
@@ -1271,6 +1431,7 @@ HMOE_BF16_INSTANCE(kWgrad)
 template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, true>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, false, true>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kWgrad, Config<2, 4, 4, 2>, true>(GemmArgs);
+template __global__ void grouped_gemm_bf16_kernel<kFwdFp8, Config<2, 4, 4, 2>>(GemmArgs);
 
 // ------------------------------------------------------------------------------------------------ fp32 path
 // 64x64 tile, contraction step 16, 256 threads each owning a 4x4 block.  grid.x walks row tiles of every group
@@ -1535,6 +1696,49 @@ int hmoe_grouped_gemm_fwd_fp8w(const void* a, int64_t lda, const uint8_t* bq, co
   if (!a || !bq || !b_scale || !out) return HMOE_INVALID_ARGUMENT;
   if (lda < k || ldo < n) return HMOE_INVALID_ARGUMENT;
   return launch<kFwdFp8W>(p, HMOE_BF16, static_cast<hipStream_t>(stream));
+}
+
+int hmoe_grouped_gemm_fwd_fp8(const uint8_t* a_q, int64_t lda, const uint8_t* a_scale, int64_t a_scale_rows,
+                              const uint8_t* bq_t, const float* b_scale, const int32_t* offs, int64_t total_rows,
+                              int num_groups, int64_t k, int64_t n, void* out, int64_t ldo, void* stream) {
+  using namespace hmoe;
+  if (total_rows < 0 || num_groups <= 0 || k < 0 || n < 0) return HMOE_INVALID_ARGUMENT;
+  if (offs == nullptr && num_groups != 1) return HMOE_INVALID_ARGUMENT;
+  if (num_groups > kMaxGroups) return HMOE_UNSUPPORTED;
+  // whole scale blocks along the contraction; 16-byte rows on both sides
+  if (k % 128 || n % 8 || lda % 16 || ldo % 8 || lda < k || ldo < n || a_scale_rows < total_rows)
+    return HMOE_UNSUPPORTED;
+  if (total_rows == 0 || n == 0) return HMOE_OK;
+  if (k == 0) return HMOE_UNSUPPORTED;  // an empty contraction has no scale block to speak of
+  if (!a_q || !a_scale || !bq_t || !b_scale || !out) return HMOE_INVALID_ARGUMENT;
+  if (!aligned16(a_q) || !aligned16(bq_t) || !aligned16(out) || reinterpret_cast<uintptr_t>(b_scale) % 4)
+    return HMOE_UNSUPPORTED;
+  const int64_t lim = int64_t(1) << 31;
+  const int64_t k_blocks = k / 128, n_blocks = (n + 127) / 128;
+  if (total_rows * lda >= lim || k * n >= lim || total_rows * ldo * 2 >= lim ||
+      k_blocks * a_scale_rows >= lim || num_groups * k_blocks * n_blocks * 4 >= lim)
+    return HMOE_UNSUPPORTED;
+  GemmArgs p{};
+  p.a = a_q;
+  p.lda = lda / 2;
+  p.b = bq_t;
+  p.ldb = k / 2;
+  p.c = out;
+  p.ldc = ldo;
+  p.offs = offs;
+  p.total_rows = total_rows;
+  p.groups = num_groups;
+  p.k = k / 2;
+  p.n = n;
+  p.b_scale = b_scale;
+  p.a_scale = a_scale;
+  p.a_scale_rows = a_scale_rows;
+  p.k_blocks = static_cast<int>(k_blocks);
+  p.n_blocks = static_cast<int>(n_blocks);
+  const int rc = launch_direct<kFwdFp8, Config<2, 4, 4, 2>>(p, static_cast<hipStream_t>(stream));
+  if (rc) return rc;
+  if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
+  return HMOE_OK;
 }
 
 int hmoe_grouped_gemm_dgrad(const void* grad_out, int64_t ldg, const void* b, const int32_t* offs,

@@ -78,10 +78,66 @@ dequantize_kernel(const uint8_t* __restrict__ q, const float* __restrict__ scale
   }
 }
 
+// Activation rows to e4m3 with one power-of-two scale per row and 128 values, for the fp8 MFMA product (which takes
+// an operand's scale as an e8m0 exponent byte).  Sixteen lanes share a block: each loads 8 values, the maximum goes
+// round the sixteen, and the exponent is read off its bits: with amax = m 2^x (1 <= m < 2) the smallest e for which
+// amax 2^-e <= 448 = 1.75 2^8 is x - 8, one more where m > 1.75.  Stored biased (e + 127), clamped at 0; an all-zero
+// block gets 0.  q = x 2^-e rounded to nearest even.
+__global__ void __launch_bounds__(256)
+quantize_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, int64_t rows, int k, uint8_t* __restrict__ q, int64_t ldq,
+                     uint8_t* __restrict__ scale, int64_t scale_rows) {
+  const int chunks = k >> 3;
+  const int64_t unit = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t row = unit / chunks;
+  const int chunk = static_cast<int>(unit - row * chunks);
+  if (row >= rows) return;  // whole groups of sixteen lanes leave together (chunks is a multiple of 16)
+  Vec16<bf16_t> in;
+  in.load(x + row * ldx + (chunk << 3));
+  const float* v = in.v;
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+#pragma unroll
+  for (int off = 1; off < 16; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 16));
+  const uint32_t bits = __float_as_uint(amax);
+  int biased = static_cast<int>(bits >> 23) - 8 + ((bits & 0x007fffffu) > 0x00600000u ? 1 : 0);
+  biased = biased < 0 ? 0 : biased;
+  const float inv = __uint_as_float(static_cast<uint32_t>(254 - biased) << 23);  // 2^-(biased - 127), exact
+  uint2 packed;
+  int word = 0;
+  word = __builtin_amdgcn_cvt_pk_fp8_f32(v[0] * inv, v[1] * inv, word, false);
+  word = __builtin_amdgcn_cvt_pk_fp8_f32(v[2] * inv, v[3] * inv, word, true);
+  packed.x = static_cast<uint32_t>(word);
+  word = 0;
+  word = __builtin_amdgcn_cvt_pk_fp8_f32(v[4] * inv, v[5] * inv, word, false);
+  word = __builtin_amdgcn_cvt_pk_fp8_f32(v[6] * inv, v[7] * inv, word, true);
+  packed.y = static_cast<uint32_t>(word);
+  *reinterpret_cast<uint2*>(q + row * ldq + (chunk << 3)) = packed;
+  if ((chunk & 15) == 0) scale[static_cast<int64_t>(chunk >> 4) * scale_rows + row] = static_cast<uint8_t>(biased);
+}
+
 }  // namespace
 }  // namespace hmoe
 
 extern "C" {
+
+int hmoe_quantize_rows_fp8(const void* x, int64_t ldx, int64_t rows, int64_t k, uint8_t* q, int64_t ldq,
+                           uint8_t* scale, int64_t scale_rows, void* stream) {
+  using namespace hmoe;
+  if (rows < 0 || k < 0) return HMOE_INVALID_ARGUMENT;
+  if (k % kBlock || ldx < k || ldq < k || ldx % 8 || ldq % 8 || scale_rows < rows) return HMOE_UNSUPPORTED;
+  if (rows == 0 || k == 0) return HMOE_OK;
+  if (!x || !q || !scale) return HMOE_INVALID_ARGUMENT;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(q) % 8) return HMOE_UNSUPPORTED;
+  const int64_t units = rows * (k / 8);
+  const int64_t blocks = (units + 255) / 256;
+  if (blocks >= (int64_t(1) << 31) || k >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  quantize_rows_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(
+      static_cast<const bf16_t*>(x), ldx, rows, static_cast<int>(k), q, ldq, scale, scale_rows);
+  HMOE_CHECK_LAUNCH();
+  return HMOE_OK;
+}
 
 int hmoe_quantize_block_fp8(const void* w, int dtype, int64_t batch, int64_t rows, int64_t cols, uint8_t* q,
                             float* scale, void* stream) {

@@ -58,6 +58,29 @@ def dequantize_block_fp8(weight: torch.Tensor, scale_inv: torch.Tensor, dtype: t
     return out
 
 
+def quantize_rows_fp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(q, scale_exponents)`` for bf16 activations ``x [R, K]`` (K a multiple of 128): ``q`` float8_e4m3fn ``[R, K]``
+    and uint8 ``[K / 128, R]``, the biased exponent ``e + 127`` of each row's power-of-two scale ``2^e`` per 128
+    values (the smallest that brings the block's largest magnitude to 448 or below; 0 for an all-zero block), laid out
+    block-major as the fp8 expert GEMM reads it.  ``q * 2^e`` reconstructs ``x`` to e4m3 precision.  This is the
+    "dynamic" activation scheme of :func:`block_fp8_quantization_config`, with scales the matrix instruction takes
+    as they are."""
+    device = _lib.require_device(x)
+    if x.dim() != 2 or x.dtype != torch.bfloat16:
+        raise TypeError(f"quantize_rows_fp8 takes bf16 [R, K], got {x.dtype} {tuple(x.shape)}")
+    rows, k = x.shape
+    if k % BLOCK:
+        raise ValueError(f"K = {k} is not a multiple of {BLOCK}")
+    if x.stride(1) != 1 or x.stride(0) % 8:
+        x = x.contiguous()
+    q = torch.empty((rows, k), dtype=torch.uint8, device=device)
+    scale = torch.empty((k // BLOCK, rows), dtype=torch.uint8, device=device)
+    with _lib.on_device(device):
+        _lib.call("hmoe_quantize_rows_fp8", _lib.ptr(x), x.stride(0), rows, k, _lib.ptr(q), k, _lib.ptr(scale), rows,
+                  _lib.stream_ptr(device))
+    return q.view(torch.float8_e4m3fn), scale
+
+
 def block_fp8_quantization_config(modules_to_not_convert: list[str]) -> dict:
     """The ``config.json`` ``quantization_config`` serving engines read for such a checkpoint."""
     return {

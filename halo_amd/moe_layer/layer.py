@@ -173,6 +173,8 @@ class EPMoELayerBase(nn.Module, ABC):
         self._expert_kernels_warmed = False
         self._lowp_quant_format = None
         self._lowp_weight_cacheable = True
+        # quantised weights only: quantise the activations too and multiply on the e4m3 MFMA
+        self._lowp_fp8_activations = False
         # the first expert projection gathers its rows by index instead of reading a permuted copy of the tokens
         self.fuse_permute_into_gemm = True
         # the shared expert's output joins the routed one in the combine kernel instead of a tensor addition
@@ -329,7 +331,8 @@ class EPMoELayerBase(nn.Module, ABC):
 
     def _grouped_mm(self, mat_a, mat_b, *, offs=None, lowp: bool = True):
         return expert_gemm(mat_a, mat_b, offs=offs, quant_format=self._lowp_quant_format if lowp else None,
-                           weight_cacheable=self._lowp_weight_cacheable)
+                           weight_cacheable=self._lowp_weight_cacheable,
+                           fp8_activations=lowp and getattr(self, "_lowp_fp8_activations", False))
 
     @property
     def _stores_fused_glu(self) -> bool:

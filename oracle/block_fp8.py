@@ -75,3 +75,52 @@ def dequantize_block_fp8(q_bits: np.ndarray, scale: np.ndarray) -> np.ndarray:
     n, k = q_bits.shape[-2:]
     s = np.repeat(np.repeat(scale, BLOCK, axis=-2)[..., :n, :], BLOCK, axis=-1)[..., :k]
     return decode_e4m3fn(q_bits) * s.astype(np.float32)
+
+
+# ------------------------------------------------------------------------------- activations, one row and 128 values
+# The "dynamic" activation scheme that block_fp8_quantization_config (``block_fp8.py:37-46``) names for the serving
+# engine, which the reference itself holds no code for; the restatement below is the published recipe (one scale per
+# token and 128 channels, amax / 448 rounded up to a power of two), pinned by its own properties in the tests: the
+# scale is the smallest power of two that keeps the block inside e4m3's range, and q * scale is x to e4m3 precision.
+
+def row_scale_exponents(x: np.ndarray) -> np.ndarray:
+    """Biased exponents ``e + 127`` (uint8 ``[R, K/128]``) of the smallest power of two ``2^e`` with
+    ``amax * 2^-e <= 448`` per row and 128 values; clamped at 0, which is also what an all-zero block gets."""
+    rows, k = x.shape
+    amax = np.abs(x.astype(np.float32)).reshape(rows, k // BLOCK, BLOCK).max(axis=2)
+    mantissa, exponent = np.frexp(amax)  # amax = mantissa * 2^exponent, mantissa in [0.5, 1)
+    # 448 = 0.875 * 2^9: e = exponent - 9, one more where the mantissa is above 0.875
+    e = exponent.astype(np.int64) - 9 + (mantissa > 0.875)
+    biased = np.where(amax == 0, 0, np.clip(e + 127, 0, 254))
+    return biased.astype(np.uint8)
+
+
+def quantize_rows_fp8(x: np.ndarray):
+    """``(q uint8 e4m3fn bits [R, K], biased exponents uint8 [K/128, R])`` for fp32 ``x`` holding bf16 values."""
+    rows, k = x.shape
+    biased = row_scale_exponents(x)
+    inv = np.ldexp(np.float64(1.0), 127 - biased.astype(np.int64))  # [R, K/128], exact
+    scaled = x.astype(np.float64).reshape(rows, k // BLOCK, BLOCK) * inv[:, :, None]
+    return encode_e4m3fn(scaled.reshape(rows, k).astype(np.float32)), np.ascontiguousarray(biased.T)
+
+
+def dequantize_rows_fp8(q_bits: np.ndarray, biased_t: np.ndarray) -> np.ndarray:
+    """float64 ``q * 2^e`` for the pair :func:`quantize_rows_fp8` returns."""
+    rows, k = q_bits.shape
+    scale = np.ldexp(np.float64(1.0), biased_t.T.astype(np.int64) - 127)  # [R, K/128]
+    return (decode_e4m3fn(q_bits).astype(np.float64).reshape(rows, k // BLOCK, BLOCK) * scale[:, :, None]).reshape(rows, k)
+
+
+def fp8_grouped_mm(q_bits: np.ndarray, biased_t: np.ndarray, w_bits: np.ndarray, w_scale: np.ndarray,
+                   offs: np.ndarray) -> np.ndarray:
+    """float64 ``[R, N]``: per group ``(q * 2^e)[s:e] @ (w * w_scale)[g]`` with ``w_bits [G, K, N]`` and
+    ``w_scale [G, ceil(K/128), ceil(N/128)]``.  Every product of two e4m3 values and two scales is exact in
+    float64, so this is the value the fp8 kernel's fp32 accumulation approximates."""
+    a = dequantize_rows_fp8(q_bits, biased_t)
+    w = dequantize_block_fp8(w_bits, w_scale).astype(np.float64)
+    out = np.zeros((a.shape[0], w.shape[2]))
+    start = 0
+    for g, end in enumerate(np.asarray(offs).tolist()):
+        out[start:end] = a[start:end] @ w[g]
+        start = end
+    return out

@@ -242,3 +242,53 @@ def test_layer_forward_routes_and_adds_the_shared_expert():
     assert torch.allclose(out - routed, mlp * torch.sigmoid(x @ shared["shared_expert_gate"].t()), atol=1e-5)
     assert torch.equal(idx, torch.topk(torch.softmax(logits, -1), K).indices)
     assert torch.allclose(w.sum(-1), torch.ones(T))
+
+
+def test_row_quantiser_picks_the_smallest_power_of_two_that_fits_and_keeps_e4m3_precision():
+    """Pins ``quantize_rows_fp8`` by what defines it rather than by its formula: the scale is a power of two under
+    which the block's largest magnitude is at most 448 and above 224 (one step smaller would overflow), the codes are
+    what torch's own float8_e4m3fn cast gives for the scaled values, and ``q * scale`` is within half an e4m3 step
+    (2^-4 relative for normal values) of ``x``."""
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn(64, 512, generator=g) * torch.exp2(torch.randint(-12, 12, (64, 4), generator=g)
+                                                        .repeat_interleave(128, dim=1).float())).bfloat16().float()
+    x[0, :128] = 0
+    x[1, :128] = 0
+    x[1, 3] = 448.0  # exactly at the top of the range: scale 1
+    x[2, :128] = 0
+    x[2, 3] = 449.0  # bf16 rounds this to 448 too
+    x[3, :128] = 0
+    x[3, 3] = 452.0  # the next bf16 value above 448: scale 2
+    q, exps_t = block_fp8.quantize_rows_fp8(x.numpy())
+    exps = exps_t.T.astype(np.int64)
+    assert exps_t.shape == (4, 64) and exps[0, 0] == 0 and exps[1, 0] == 127 and exps[3, 0] == 128
+    amax = x.abs().reshape(64, 4, 128).amax(dim=2).double().numpy()
+    scale = np.ldexp(1.0, exps - 127)
+    live = amax > 0
+    assert (amax[live] / scale[live] <= 448).all() and (amax[live] / scale[live] > 224).all()
+    scaled = (x.double().reshape(64, 4, 128) / torch.from_numpy(scale)[:, :, None]).reshape(64, 512).float()
+    torch_bits = scaled.to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    nonzero = (q & 0x7F) != 0
+    assert np.array_equal(q[nonzero], torch_bits[nonzero]) and not (torch_bits[~nonzero] & 0x7F).any()
+    restored = block_fp8.dequantize_rows_fp8(q, exps_t)
+    step = np.repeat(scale, 128, axis=1) * 2.0 ** -9  # half the subnormal spacing (2^-9) in the block's scale
+    assert (np.abs(restored - x.double().numpy()) <= np.maximum(np.abs(x.double().numpy()) * 2.0 ** -4, step)).all()
+
+
+def test_fp8_product_of_the_oracle_is_the_product_of_its_dequantised_operands():
+    """``fp8_grouped_mm`` against a per-element restatement on a tiny case (two experts, K = 256): the sum over k of
+    code value times row scale times code value times block scale, term by term in Python floats."""
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(5, 256, generator=g).bfloat16().float().numpy()
+    w = (torch.randn(2, 256, 136, generator=g) * 0.02).numpy()
+    q, exps_t = block_fp8.quantize_rows_fp8(x)
+    wq, ws = block_fp8.quantize_block_fp8(w)
+    ws = ws * np.float32(1.25)
+    got = block_fp8.fp8_grouped_mm(q, exps_t, wq, ws, np.array([2, 5], dtype=np.int32))
+    qa, qw = block_fp8.decode_e4m3fn(q).astype(float), block_fp8.decode_e4m3fn(wq).astype(float)
+    for r, c in ((0, 0), (1, 135), (2, 7), (4, 130)):
+        expert = 0 if r < 2 else 1
+        total = 0.0
+        for kk in range(256):
+            total += qa[r, kk] * 2.0 ** (int(exps_t[kk // 128, r]) - 127) * qw[expert, kk, c] * float(ws[expert, kk // 128, c // 128])
+        assert abs(got[r, c] - total) <= 1e-12 * max(1.0, abs(total))
