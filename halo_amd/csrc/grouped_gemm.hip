@@ -96,8 +96,8 @@ struct GemmArgs {
   const int64_t* a_index = nullptr;  // gathered A (fwd, wgrad): logical row r of A is a[a_index[r]]
   int64_t a_rows = 0;                // rows of the array a_index points into
   const void* bias = nullptr;        // fwd: [G, N] in the operands' dtype, added to group g's output rows
-  // kFwdFp8: both operands are e4m3 bytes with the contraction contiguous (A [R, K], B [G, N, K]); k, lda and ldb
-  // count 2-byte units, so a step of BK units is 128 values: one scale block
+  // kFwdFp8: both operands are e4m3 bytes in panels of 128 contraction values (A [K/128][a_scale_rows][128],
+  // B [G][K/128][N][128]); k counts 2-byte units, so a step of BK units is 128 values: one panel, one scale block
   const uint8_t* a_scale = nullptr;  // [K / 128][a_scale_rows]: the e8m0 exponent of row r's block b at (b, r)
   int64_t a_scale_rows = 0;
   int k_blocks = 0, n_blocks = 0;     // the grid of b_scale [G, k_blocks, n_blocks]
@@ -729,12 +729,14 @@ struct SlimDirect {  // element(out, con) = base[out * ld + con]; LDS [256 out][
   u32x4 rsrc;  // bounded at the operand's last output row: rows past it load as zeros
   uint32_t voff;                // this lane's chunk for the wavefront's first load of a step, at step 0
   uint32_t t_stride;            // bytes between the rows of consecutive loads (8 rows)
+  uint32_t step_bytes;          // bytes from one contraction step to the next: BK values along a row, or one panel
   int con0, con_lim;
   int t_lim;                    // loads t >= t_lim of this wavefront lie wholly past the operand's last row
 
   __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
-                                       int con_lim_, int wave, int lane) {
+                                       int con_lim_, int wave, int lane, uint32_t step_bytes_ = BK * 2) {
     rsrc = make_rsrc_words(base, static_cast<uint32_t>(bytes));
+    step_bytes = step_bytes_;
     con_lim = con_lim_;
     t_lim = (out_lim - out0 - wave * kI * 8 + 7) >> 3;
     const int logical = (lane & 7) ^ (lane >> 3);  // row & 7 == lane >> 3 for every load
@@ -746,7 +748,7 @@ struct SlimDirect {  // element(out, con) = base[out * ld + con]; LDS [256 out][
   // change) but every offset is out of range, and the step offset stays below the buffer's size
   __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave,
                                         bool live = true) const {
-    const uint32_t soff = live ? static_cast<uint32_t>(step) * (BK * 2) : 0u;
+    const uint32_t soff = live ? static_cast<uint32_t>(step) * step_bytes : 0u;
     const uint32_t base = live && step * BK + con0 < con_lim ? voff : kOutOfRange;
     // A load whose eight rows all lie past the operand's end is left out: nothing reads those rows of the tile
     // for a result that is kept (an output row takes its values from its own operand row only), and in a group's
@@ -1055,7 +1057,17 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     const bf16_t* a = static_cast<const bf16_t*>(p.a);
     const bf16_t* b = static_cast<const bf16_t*>(p.b);
     const int64_t rows = kMode == kWgrad ? tile.con_lim : tile.a_out_lim;
-    if constexpr (kGather) {
+    if constexpr (kFp8) {
+      // Panels: operand[block][row][128 values], so a tile's share of a step is one contiguous run per operand.
+      // A row is 64 two-byte units; a step moves on by a whole panel.  Rows past the tile's last in a load of eight
+      // are the next rows of the panel (another expert's, or nothing: the descriptor ends with the array); they
+      // reach only output rows and columns that are not stored.
+      const int64_t a_panel = p.a_scale_rows * 128, b_panel = p.n * 128;
+      la.init(a + tile.row_start * 64, 64, p.k_blocks * a_panel - tile.row_start * 128, tile.a_out0, tile.a_out_lim,
+              tile.con_lim, load_slot, lane, static_cast<uint32_t>(a_panel));
+      lb.init(b + tile.g * w_elems, 64, p.k_blocks * b_panel, tile.b_out0, tile.b_out_lim, tile.con_lim, load_slot,
+              lane, static_cast<uint32_t>(b_panel));
+    } else if constexpr (kGather) {
       if (load_wave)  // the row indices are fetched by the lanes that use them
         la.init(a, p.lda, p.a_rows, p.a_index + tile.row_start, tile.a_out0, tile.a_out_lim, tile.con_lim, load_slot,
                 lane);
@@ -1063,11 +1075,13 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim,
               load_slot, lane);
     }
-    if constexpr (kMode == kWgrad)
+    if constexpr (kFp8) {
+    } else if constexpr (kMode == kWgrad) {
       lb.init(b + tile.row_start * p.ldb, p.ldb, rows * p.ldb * 2, tile.b_out0, tile.b_out_lim, tile.con_lim,
               load_slot, lane);
-    else
+    } else {
       lb.init(b + tile.g * w_elems, p.ldb, w_elems * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, load_slot, lane);
+    }
     if (load_wave) {
       if constexpr (kRowsPerStep) {
         if (!rows0_loaded) {
@@ -1318,6 +1332,9 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         for (int i = 0; i < WM; ++i) asm volatile("" : "+v"(sa_next[i]));
         const int sa = static_cast<int>((sa_next[0] & 0xffu) | ((sa_next[1] & 0xffu) << 8) |
                                         ((sa_next[2] & 0xffu) << 16) | (sa_next[3] << 24));
+        // The other stage is free since the barrier inside the previous step.  (Issued right behind that barrier
+        // instead, a refill would have a whole step to land rather than three quarters of one; measured 8 % slower:
+        // the sixteen issues then stand between the barrier and the fragment reads the next MFMAs wait for.)
         if (load_wave) {
           la.issue(lds + (cur ^ 1) * kStageBytes, step + 1, load_slot, more);
           lb.issue(lds + (cur ^ 1) * kStageBytes + kTileBytes, step + 1, load_slot, more);
@@ -1345,11 +1362,27 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         column0(sa, sb);
         column1_refilling(sa, sb, cur, 1);
         column0(sa, sb);
+        // The barrier comes as late as the refills allow, after 14 of the step's 16 MFMAs: the step's refill has
+        // that much longer to land, and the first fragments of the next step still have two MFMAs to arrive under.
+        mfma(b0, b1, sa, sb);
+        mfma(b1, b1, sa, sb);
+        __builtin_amdgcn_sched_barrier(0);
         // lgkmcnt(0): this stage is read out; vmcnt(0) where tile loads were issued: the next step has landed
         if (load_wave) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         workgroup_barrier();
-        column1_refilling(sa, sb, cur ^ 1, 0);  // (after a tile's last step the refills read what nothing uses)
+        // (after a tile's last step the refills read what nothing uses)
+        if (kFull || live > 0) read_b8(cur ^ 1, 0, 0);
+        if (kFull || 0 < live) read_a8(cur ^ 1, 0, 0);
+        if (kFull || 1 < live) read_a8(cur ^ 1, 0, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(b2, b1, sa, sb);
+        if (kFull || 2 < live) read_a8(cur ^ 1, 0, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(b3, b1, sa, sb);
+        if (kFull || 3 < live) read_a8(cur ^ 1, 0, 3);
+        if (kFull || live > 0) read_b8(cur ^ 1, 0, 1);
+        __builtin_amdgcn_sched_barrier(0);
       }
     };
     if constexpr (kFp8) {
@@ -1698,31 +1731,29 @@ int hmoe_grouped_gemm_fwd_fp8w(const void* a, int64_t lda, const uint8_t* bq, co
   return launch<kFwdFp8W>(p, HMOE_BF16, static_cast<hipStream_t>(stream));
 }
 
-int hmoe_grouped_gemm_fwd_fp8(const uint8_t* a_q, int64_t lda, const uint8_t* a_scale, int64_t a_scale_rows,
-                              const uint8_t* bq_t, const float* b_scale, const int32_t* offs, int64_t total_rows,
-                              int num_groups, int64_t k, int64_t n, void* out, int64_t ldo, void* stream) {
+int hmoe_grouped_gemm_fwd_fp8(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
+                              const float* b_scale, const int32_t* offs, int64_t total_rows, int num_groups, int64_t k,
+                              int64_t n, void* out, int64_t ldo, void* stream) {
   using namespace hmoe;
   if (total_rows < 0 || num_groups <= 0 || k < 0 || n < 0) return HMOE_INVALID_ARGUMENT;
   if (offs == nullptr && num_groups != 1) return HMOE_INVALID_ARGUMENT;
   if (num_groups > kMaxGroups) return HMOE_UNSUPPORTED;
   // whole scale blocks along the contraction; 16-byte rows on both sides
-  if (k % 128 || n % 8 || lda % 16 || ldo % 8 || lda < k || ldo < n || a_scale_rows < total_rows)
-    return HMOE_UNSUPPORTED;
+  if (k % 128 || n % 8 || ldo % 8 || ldo < n || a_rows < total_rows) return HMOE_UNSUPPORTED;
   if (total_rows == 0 || n == 0) return HMOE_OK;
   if (k == 0) return HMOE_UNSUPPORTED;  // an empty contraction has no scale block to speak of
-  if (!a_q || !a_scale || !bq_t || !b_scale || !out) return HMOE_INVALID_ARGUMENT;
-  if (!aligned16(a_q) || !aligned16(bq_t) || !aligned16(out) || reinterpret_cast<uintptr_t>(b_scale) % 4)
+  if (!a_q || !a_scale || !bq || !b_scale || !out) return HMOE_INVALID_ARGUMENT;
+  if (!aligned16(a_q) || !aligned16(bq) || !aligned16(out) || reinterpret_cast<uintptr_t>(b_scale) % 4)
     return HMOE_UNSUPPORTED;
   const int64_t lim = int64_t(1) << 31;
   const int64_t k_blocks = k / 128, n_blocks = (n + 127) / 128;
-  if (total_rows * lda >= lim || k * n >= lim || total_rows * ldo * 2 >= lim ||
-      k_blocks * a_scale_rows >= lim || num_groups * k_blocks * n_blocks * 4 >= lim)
+  if (a_rows * k >= lim || k * n >= lim || total_rows * ldo * 2 >= lim || num_groups * k_blocks * n_blocks * 4 >= lim)
     return HMOE_UNSUPPORTED;
   GemmArgs p{};
   p.a = a_q;
-  p.lda = lda / 2;
-  p.b = bq_t;
-  p.ldb = k / 2;
+  p.lda = 64;
+  p.b = bq;
+  p.ldb = 64;
   p.c = out;
   p.ldc = ldo;
   p.offs = offs;
@@ -1732,7 +1763,7 @@ int hmoe_grouped_gemm_fwd_fp8(const uint8_t* a_q, int64_t lda, const uint8_t* a_
   p.n = n;
   p.b_scale = b_scale;
   p.a_scale = a_scale;
-  p.a_scale_rows = a_scale_rows;
+  p.a_scale_rows = a_rows;
   p.k_blocks = static_cast<int>(k_blocks);
   p.n_blocks = static_cast<int>(n_blocks);
   const int rc = launch_direct<kFwdFp8, Config<2, 4, 4, 2>>(p, static_cast<hipStream_t>(stream));

@@ -84,8 +84,8 @@ dequantize_kernel(const uint8_t* __restrict__ q, const float* __restrict__ scale
 // amax 2^-e <= 448 = 1.75 2^8 is x - 8, one more where m > 1.75.  Stored biased (e + 127), clamped at 0; an all-zero
 // block gets 0.  q = x 2^-e rounded to nearest even.
 __global__ void __launch_bounds__(256)
-quantize_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, int64_t rows, int k, uint8_t* __restrict__ q, int64_t ldq,
-                     uint8_t* __restrict__ scale, int64_t scale_rows) {
+quantize_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, int64_t rows, int k, uint8_t* __restrict__ q,
+                     uint8_t* __restrict__ scale, int64_t out_rows) {
   const int chunks = k >> 3;
   const int64_t unit = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   const int64_t row = unit / chunks;
@@ -112,8 +112,10 @@ quantize_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, int64_t rows, in
   word = __builtin_amdgcn_cvt_pk_fp8_f32(v[4] * inv, v[5] * inv, word, false);
   word = __builtin_amdgcn_cvt_pk_fp8_f32(v[6] * inv, v[7] * inv, word, true);
   packed.y = static_cast<uint32_t>(word);
-  *reinterpret_cast<uint2*>(q + row * ldq + (chunk << 3)) = packed;
-  if ((chunk & 15) == 0) scale[static_cast<int64_t>(chunk >> 4) * scale_rows + row] = static_cast<uint8_t>(biased);
+  // panels: block b of row r at q[(b * out_rows + r) * 128], its scale at scale[b * out_rows + r]
+  const int64_t slot = static_cast<int64_t>(chunk >> 4) * out_rows + row;
+  *reinterpret_cast<uint2*>(q + slot * kBlock + ((chunk & 15) << 3)) = packed;
+  if ((chunk & 15) == 0) scale[slot] = static_cast<uint8_t>(biased);
 }
 
 }  // namespace
@@ -121,11 +123,11 @@ quantize_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, int64_t rows, in
 
 extern "C" {
 
-int hmoe_quantize_rows_fp8(const void* x, int64_t ldx, int64_t rows, int64_t k, uint8_t* q, int64_t ldq,
-                           uint8_t* scale, int64_t scale_rows, void* stream) {
+int hmoe_quantize_rows_fp8(const void* x, int64_t ldx, int64_t rows, int64_t k, uint8_t* q, uint8_t* scale,
+                           int64_t out_rows, void* stream) {
   using namespace hmoe;
   if (rows < 0 || k < 0) return HMOE_INVALID_ARGUMENT;
-  if (k % kBlock || ldx < k || ldq < k || ldx % 8 || ldq % 8 || scale_rows < rows) return HMOE_UNSUPPORTED;
+  if (k % kBlock || ldx < k || ldx % 8 || out_rows < rows) return HMOE_UNSUPPORTED;
   if (rows == 0 || k == 0) return HMOE_OK;
   if (!x || !q || !scale) return HMOE_INVALID_ARGUMENT;
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(q) % 8) return HMOE_UNSUPPORTED;
@@ -134,7 +136,7 @@ int hmoe_quantize_rows_fp8(const void* x, int64_t ldx, int64_t rows, int64_t k, 
   if (blocks >= (int64_t(1) << 31) || k >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   quantize_rows_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(
-      static_cast<const bf16_t*>(x), ldx, rows, static_cast<int>(k), q, ldq, scale, scale_rows);
+      static_cast<const bf16_t*>(x), ldx, rows, static_cast<int>(k), q, scale, out_rows);
   HMOE_CHECK_LAUNCH();
   return HMOE_OK;
 }

@@ -30,7 +30,7 @@ class BlockFp8Weight:
         self.q = q.contiguous()
         self.scale_inv = scale_inv.float().contiguous()
         self._bf16 = None
-        self._transposed = None
+        self._panels = None
 
     @property
     def shape(self):
@@ -46,12 +46,14 @@ class BlockFp8Weight:
         return self._bf16
 
 
-    def transposed(self) -> torch.Tensor:
-        """The e4m3 bytes as ``[G, N, K]`` (the contraction contiguous, as the fp8 MFMA kernel loads both operands),
-        made once and kept: the fp8 bytes once more in device memory."""
-        if self._transposed is None:
-            self._transposed = self.q.view(torch.uint8).transpose(1, 2).contiguous()
-        return self._transposed
+    def panels(self) -> torch.Tensor:
+        """The e4m3 bytes as ``[G, K / 128, N, 128]``: the contraction contiguous within a panel of 128 values and a
+        tile's columns of one panel in one run, which is how the fp8 MFMA kernel loads them.  Made once and kept: the
+        fp8 bytes once more in device memory."""
+        if self._panels is None:
+            g, k, n = self.q.shape
+            self._panels = self.q.view(torch.uint8).view(g, k // 128, 128, n).permute(0, 1, 3, 2).contiguous()
+        return self._panels
 
 
 def expert_gemm(
@@ -119,7 +121,7 @@ def fp8_mfma_usable(k: int, n: int) -> bool:
 
 def _fp8_mfma_forward(mat_a: torch.Tensor, weight: BlockFp8Weight, offs: torch.Tensor | None) -> torch.Tensor:
     """Activations to e4m3 (one launch), then the grouped GEMM on the scaled e4m3 MFMA against the weight's
-    transposed bytes and its fp32 block scales."""
+    bytes in panels and its fp32 block scales."""
     from halo_amd.kernels.lowp.block_fp8 import quantize_rows_fp8
 
     device = _lib.require_device(mat_a, weight.q, weight.scale_inv, offs)
@@ -138,9 +140,9 @@ def _fp8_mfma_forward(mat_a: torch.Tensor, weight: BlockFp8Weight, offs: torch.T
         return out
     offs32 = _offs_arg(offs, groups)
     a_q, a_scale = quantize_rows_fp8(mat_a)
-    w_t = weight.transposed()
+    w_panels = weight.panels()
     with _lib.on_device(device):
-        _lib.call("hmoe_grouped_gemm_fwd_fp8", _lib.ptr(a_q), a_q.stride(0), _lib.ptr(a_scale), a_scale.stride(0),
-                  _lib.ptr(w_t), _lib.ptr(weight.scale_inv), _lib.ptr(offs32), rows, groups, k, n, _lib.ptr(out),
-                  out.stride(0), _lib.stream_ptr(device))
+        _lib.call("hmoe_grouped_gemm_fwd_fp8", _lib.ptr(a_q), _lib.ptr(a_scale), rows, _lib.ptr(w_panels),
+                  _lib.ptr(weight.scale_inv), _lib.ptr(offs32), rows, groups, k, n, _lib.ptr(out), out.stride(0),
+                  _lib.stream_ptr(device))
     return out

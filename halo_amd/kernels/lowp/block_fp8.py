@@ -59,10 +59,11 @@ def dequantize_block_fp8(weight: torch.Tensor, scale_inv: torch.Tensor, dtype: t
 
 
 def quantize_rows_fp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
-    """``(q, scale_exponents)`` for bf16 activations ``x [R, K]`` (K a multiple of 128): ``q`` float8_e4m3fn ``[R, K]``
-    and uint8 ``[K / 128, R]``, the biased exponent ``e + 127`` of each row's power-of-two scale ``2^e`` per 128
-    values (the smallest that brings the block's largest magnitude to 448 or below; 0 for an all-zero block), laid out
-    block-major as the fp8 expert GEMM reads it.  ``q * 2^e`` reconstructs ``x`` to e4m3 precision.  This is the
+    """``(q, scale_exponents)`` for bf16 activations ``x [R, K]`` (K a multiple of 128): ``q`` float8_e4m3fn
+    ``[K / 128, R, 128]`` (panels of 128 values, as the fp8 expert GEMM reads them: ``q.permute(1, 0, 2)`` is
+    ``[R, K / 128, 128]``) and uint8 ``[K / 128, R]``, the biased exponent ``e + 127`` of each row's power-of-two
+    scale ``2^e`` per 128 values (the smallest that brings the block's largest magnitude to 448 or below; 0 for an
+    all-zero block).  ``q * 2^e`` reconstructs ``x`` to e4m3 precision.  This is the
     "dynamic" activation scheme of :func:`block_fp8_quantization_config`, with scales the matrix instruction takes
     as they are."""
     device = _lib.require_device(x)
@@ -73,10 +74,10 @@ def quantize_rows_fp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         raise ValueError(f"K = {k} is not a multiple of {BLOCK}")
     if x.stride(1) != 1 or x.stride(0) % 8:
         x = x.contiguous()
-    q = torch.empty((rows, k), dtype=torch.uint8, device=device)
+    q = torch.empty((k // BLOCK, rows, BLOCK), dtype=torch.uint8, device=device)
     scale = torch.empty((k // BLOCK, rows), dtype=torch.uint8, device=device)
     with _lib.on_device(device):
-        _lib.call("hmoe_quantize_rows_fp8", _lib.ptr(x), x.stride(0), rows, k, _lib.ptr(q), k, _lib.ptr(scale), rows,
+        _lib.call("hmoe_quantize_rows_fp8", _lib.ptr(x), x.stride(0), rows, k, _lib.ptr(q), _lib.ptr(scale), rows,
                   _lib.stream_ptr(device))
     return q.view(torch.float8_e4m3fn), scale
 

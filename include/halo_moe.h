@@ -189,19 +189,23 @@ int hmoe_grouped_gemm_fwd_fp8w(const void* a, int64_t lda, const uint8_t* bq, co
  * it: block_fp8_quantization_config (halo/kernels/lowp/block_fp8.py:37-46) hands the checkpoint to the serving
  * engine with "activation_scheme": "dynamic", i.e. activations quantised per row and 128 values at run time.
  *
- * hmoe_quantize_rows_fp8: x bf16 [rows, k] (row stride ldx) to q e4m3fn [rows, k] (row stride ldq, bytes) and
- * scale u8 [k / 128, scale_rows]: the biased exponent byte (e8m0) of the power-of-two scale of row r's block b at
- * scale[b * scale_rows + r], the smallest power of two that brings the block's largest magnitude to 448 or below.
- * k must be a multiple of 128. */
-int hmoe_quantize_rows_fp8(const void* x, int64_t ldx, int64_t rows, int64_t k, uint8_t* q, int64_t ldq,
-                           uint8_t* scale, int64_t scale_rows, void* stream);
-/* out bf16 [total_rows, n] = per group, (a_q * a_scale) [rows, k] @ (bq_t * b_scale)^T: a_q and a_scale as written
- * by hmoe_quantize_rows_fp8; bq_t e4m3fn [num_groups, n, k] (each expert's weight with the contraction contiguous)
- * and b_scale f32 [num_groups, k / 128, ceil(n / 128)], positive, any mantissa.  Accumulation in fp32, one rounding
- * to bf16.  k must be a multiple of 128, n of 8. */
-int hmoe_grouped_gemm_fwd_fp8(const uint8_t* a_q, int64_t lda, const uint8_t* a_scale, int64_t a_scale_rows,
-                              const uint8_t* bq_t, const float* b_scale, const int32_t* offs, int64_t total_rows,
-                              int num_groups, int64_t k, int64_t n, void* out, int64_t ldo, void* stream);
+ * Both operands of the product lie in panels of 128 contraction values, [k / 128][rows][128], so that a tile's
+ * share of one step is a single contiguous run.
+ *
+ * hmoe_quantize_rows_fp8: x bf16 [rows, k] (row stride ldx) to q e4m3fn [k / 128][out_rows][128] and scale u8
+ * [k / 128][out_rows]: block b of row r at q[(b * out_rows + r) * 128], and at scale[b * out_rows + r] the biased
+ * exponent byte (e8m0) of its power-of-two scale, the smallest that brings the block's largest magnitude to 448
+ * or below.  k must be a multiple of 128, out_rows >= rows. */
+int hmoe_quantize_rows_fp8(const void* x, int64_t ldx, int64_t rows, int64_t k, uint8_t* q, uint8_t* scale,
+                           int64_t out_rows, void* stream);
+/* out bf16 [total_rows, n] = per group, (a_q * a_scale) [rows, k] @ (bq * b_scale) [k, n]: a_q and a_scale as
+ * written by hmoe_quantize_rows_fp8 with out_rows = a_rows; bq e4m3fn [num_groups][k / 128][n][128] (value (kk, c)
+ * of expert g at bq[((g * (k / 128) + kk / 128) * n + c) * 128 + kk % 128]) and b_scale f32
+ * [num_groups, k / 128, ceil(n / 128)], not negative, any mantissa.  Accumulation in fp32, one rounding to bf16.
+ * k must be a multiple of 128, n of 8. */
+int hmoe_grouped_gemm_fwd_fp8(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
+                              const float* b_scale, const int32_t* offs, int64_t total_rows, int num_groups, int64_t k,
+                              int64_t n, void* out, int64_t ldo, void* stream);
 
 #ifdef __cplusplus
 }

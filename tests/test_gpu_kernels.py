@@ -617,8 +617,9 @@ def test_activation_row_quantiser_is_bit_exact(device, rows, k):
     q, exps = quantize_rows_fp8(x.to(device))
     want_q, want_exps = oracle.quantize_rows_fp8(x.float().numpy())
     assert q.dtype == torch.float8_e4m3fn and exps.dtype == torch.uint8 and exps.shape == (k // 128, rows)
+    assert q.shape == (k // 128, rows, 128)  # panels of 128 values
     assert np.array_equal(exps.cpu().numpy(), want_exps)
-    got_bits = q.view(torch.uint8).cpu().numpy()
+    got_bits = q.view(torch.uint8).permute(1, 0, 2).reshape(rows, k).cpu().numpy()
     nonzero = (want_q & 0x7F) != 0
     assert np.array_equal(got_bits[nonzero], want_q[nonzero]) and not (got_bits[~nonzero] & 0x7F).any()
     assert exps[0, 0] == 0 and exps[0, 1] == 127 and exps[0, 2] == 128
@@ -646,7 +647,7 @@ def test_fp8_mfma_grouped_gemm_equals_the_exact_products(device, counts, k, n, m
     offs = _offsets(counts, device)
     out = expert_gemm(x.to(device), BlockFp8Weight(q, scale), offs=offs, fp8_activations=True)
     a_q, a_exps = quantize_rows_fp8(x.to(device))
-    want = oracle.fp8_grouped_mm(a_q.view(torch.uint8).cpu().numpy(), a_exps.cpu().numpy(),
+    want = oracle.fp8_grouped_mm(a_q.view(torch.uint8).permute(1, 0, 2).reshape(-1, k).cpu().numpy(), a_exps.cpu().numpy(),
                                  q.view(torch.uint8).cpu().numpy(), scale.cpu().numpy(),
                                  np.cumsum(counts).astype(np.int32))
     want = torch.from_numpy(want)

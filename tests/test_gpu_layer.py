@@ -210,6 +210,15 @@ def test_quantised_weight_forward(device):
     with torch.no_grad():
         again = lowp._compute_experts(x, experts.to(device), weights.to(device), torch.bfloat16, recv_counts=counts)
     assert torch.equal(again, want)
+    # activations quantised too (per row and 128 values), both products on the e4m3 MFMA: the result moves by the
+    # activations' e4m3 rounding, twice over (layer input and GLU output), and by nothing systematic
+    lowp._lowp_fp8_activations = True
+    with torch.no_grad():
+        fp8 = lowp._compute_experts(x, experts.to(device), weights.to(device), torch.bfloat16, recv_counts=counts)
+    rel = ((fp8.double() - want.double()).norm() / want.double().norm()).item()
+    assert 0.005 < rel < 0.07, rel
+    assert cosine(fp8, want) > 0.997
+    assert abs(((fp8.double() - want.double()).mean() / want.double().abs().mean()).item()) < 5e-3
 
 
 # ------------------------------------------------------------------------------ drop-ins for the Hugging Face blocks
