@@ -46,7 +46,7 @@ SIGNATURES = {
     "hmoe_quantize_block_fp8": (I, [P, I, L, L, L, P, P, P]),
     "hmoe_dequantize_block_fp8": (I, [P, P, L, L, L, I, P, P]),
     "hmoe_grouped_gemm_fwd_fp8w": (I, [P, L, P, P, P, L, I, L, L, P, L, P]),
-    "hmoe_quantize_rows_fp8": (I, [P, L, L, L, P, P, L, P]),
+    "hmoe_quantize_rows_fp8": (I, [P, L, P, L, L, L, P, P, L, P]),
     "hmoe_grouped_gemm_fwd_fp8": (I, [P, P, L, P, P, P, L, I, L, L, P, L, P]),
 }
 

@@ -82,17 +82,24 @@ dequantize_kernel(const uint8_t* __restrict__ q, const float* __restrict__ scale
 // an operand's scale as an e8m0 exponent byte).  Sixteen lanes share a block: each loads 8 values, the maximum goes
 // round the sixteen, and the exponent is read off its bits: with amax = m 2^x (1 <= m < 2) the smallest e for which
 // amax 2^-e <= 448 = 1.75 2^8 is x - 8, one more where m > 1.75.  Stored biased (e + 127), clamped at 0; an all-zero
-// block gets 0.  q = x 2^-e rounded to nearest even.
+// block gets 0.  q = x 2^-e rounded to nearest even.  With row_index, output row r is x[row_index[r]] (the permute by
+// expert taken on the way: the permuted bf16 copy is never written), zeros where the index is outside [0, x_rows).
 __global__ void __launch_bounds__(256)
-quantize_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, int64_t rows, int k, uint8_t* __restrict__ q,
-                     uint8_t* __restrict__ scale, int64_t out_rows) {
+quantize_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const int64_t* __restrict__ row_index, int64_t x_rows,
+                     int64_t rows, int k, uint8_t* __restrict__ q, uint8_t* __restrict__ scale, int64_t out_rows) {
   const int chunks = k >> 3;
   const int64_t unit = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   const int64_t row = unit / chunks;
   const int chunk = static_cast<int>(unit - row * chunks);
   if (row >= rows) return;  // whole groups of sixteen lanes leave together (chunks is a multiple of 16)
   Vec16<bf16_t> in;
-  in.load(x + row * ldx + (chunk << 3));
+  const int64_t from = row_index ? row_index[row] : row;
+  if (from >= 0 && from < x_rows) {
+    in.load(x + from * ldx + (chunk << 3));
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) in.v[i] = 0.f;
+  }
   const float* v = in.v;
   float amax = 0.f;
 #pragma unroll
@@ -123,20 +130,21 @@ quantize_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, int64_t rows, in
 
 extern "C" {
 
-int hmoe_quantize_rows_fp8(const void* x, int64_t ldx, int64_t rows, int64_t k, uint8_t* q, uint8_t* scale,
-                           int64_t out_rows, void* stream) {
+int hmoe_quantize_rows_fp8(const void* x, int64_t ldx, const int64_t* row_index, int64_t x_rows, int64_t rows, int64_t k,
+                           uint8_t* q, uint8_t* scale, int64_t out_rows, void* stream) {
   using namespace hmoe;
-  if (rows < 0 || k < 0) return HMOE_INVALID_ARGUMENT;
+  if (rows < 0 || k < 0 || x_rows < 0) return HMOE_INVALID_ARGUMENT;
+  if (!row_index && x_rows != rows) return HMOE_INVALID_ARGUMENT;
   if (k % kBlock || ldx < k || ldx % 8 || out_rows < rows) return HMOE_UNSUPPORTED;
   if (rows == 0 || k == 0) return HMOE_OK;
-  if (!x || !q || !scale) return HMOE_INVALID_ARGUMENT;
+  if (!q || !scale || (!x && x_rows > 0)) return HMOE_INVALID_ARGUMENT;
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(q) % 8) return HMOE_UNSUPPORTED;
   const int64_t units = rows * (k / 8);
   const int64_t blocks = (units + 255) / 256;
   if (blocks >= (int64_t(1) << 31) || k >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   quantize_rows_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(
-      static_cast<const bf16_t*>(x), ldx, rows, static_cast<int>(k), q, scale, out_rows);
+      static_cast<const bf16_t*>(x), ldx, row_index, x_rows, rows, static_cast<int>(k), q, scale, out_rows);
   HMOE_CHECK_LAUNCH();
   return HMOE_OK;
 }

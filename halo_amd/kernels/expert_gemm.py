@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from halo_amd import _lib
-from halo_amd.kernels.grouped_mm import _offs_arg, _rows, grouped_mm
+from halo_amd.kernels.grouped_mm import GatheredRows, _offs_arg, _rows, grouped_mm
 
 
 # rows per expert (on average) from which the dequantised-copy route is taken
@@ -120,17 +120,20 @@ def fp8_mfma_usable(k: int, n: int) -> bool:
 
 
 def _fp8_mfma_forward(mat_a: torch.Tensor, weight: BlockFp8Weight, offs: torch.Tensor | None) -> torch.Tensor:
-    """Activations to e4m3 (one launch), then the grouped GEMM on the scaled e4m3 MFMA against the weight's
-    bytes in panels and its fp32 block scales."""
+    """Activations to e4m3 (one launch, which also fetches the rows when ``mat_a`` is a :class:`GatheredRows`: the
+    permuted bf16 copy is never written), then the grouped GEMM on the scaled e4m3 MFMA against the weight's bytes in
+    panels and its fp32 block scales."""
     from halo_amd.kernels.lowp.block_fp8 import quantize_rows_fp8
 
-    device = _lib.require_device(mat_a, weight.q, weight.scale_inv, offs)
-    if mat_a.dtype != torch.bfloat16:
-        raise TypeError(f"block-fp8 expert GEMM takes bf16 activations, got {mat_a.dtype}")
-    if mat_a.requires_grad and torch.is_grad_enabled():
+    gathered = isinstance(mat_a, GatheredRows)
+    source = mat_a.tokens if gathered else mat_a
+    device = _lib.require_device(source, weight.q, weight.scale_inv, offs)
+    if source.dtype != torch.bfloat16:
+        raise TypeError(f"block-fp8 expert GEMM takes bf16 activations, got {source.dtype}")
+    if source.requires_grad and torch.is_grad_enabled():
         raise RuntimeError("the block-fp8 expert GEMM is forward only")
     groups, k, n = weight.shape
-    if mat_a.dim() != 2 or mat_a.shape[1] != k:
+    if len(mat_a.shape) != 2 or mat_a.shape[1] != k:
         raise ValueError(f"expected [R, {k}] activations, got {tuple(mat_a.shape)}")
     if not fp8_mfma_usable(k, n):
         raise ValueError(f"the fp8 MFMA product needs K % 128 == 0 and N % 8 == 0, got K = {k}, N = {n}")
@@ -139,7 +142,7 @@ def _fp8_mfma_forward(mat_a: torch.Tensor, weight: BlockFp8Weight, offs: torch.T
     if rows == 0 or n == 0:
         return out
     offs32 = _offs_arg(offs, groups)
-    a_q, a_scale = quantize_rows_fp8(mat_a)
+    a_q, a_scale = quantize_rows_fp8(source, mat_a.row_index if gathered else None)
     w_panels = weight.panels()
     with _lib.on_device(device):
         _lib.call("hmoe_grouped_gemm_fwd_fp8", _lib.ptr(a_q), _lib.ptr(a_scale), rows, _lib.ptr(w_panels),

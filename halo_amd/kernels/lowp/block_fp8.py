@@ -58,18 +58,22 @@ def dequantize_block_fp8(weight: torch.Tensor, scale_inv: torch.Tensor, dtype: t
     return out
 
 
-def quantize_rows_fp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+def quantize_rows_fp8(x: torch.Tensor, row_index: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
     """``(q, scale_exponents)`` for bf16 activations ``x [R, K]`` (K a multiple of 128): ``q`` float8_e4m3fn
     ``[K / 128, R, 128]`` (panels of 128 values, as the fp8 expert GEMM reads them: ``q.permute(1, 0, 2)`` is
     ``[R, K / 128, 128]``) and uint8 ``[K / 128, R]``, the biased exponent ``e + 127`` of each row's power-of-two
     scale ``2^e`` per 128 values (the smallest that brings the block's largest magnitude to 448 or below; 0 for an
-    all-zero block).  ``q * 2^e`` reconstructs ``x`` to e4m3 precision.  This is the
+    all-zero block).  ``q * 2^e`` reconstructs ``x`` to e4m3 precision.  With ``row_index`` (int64 ``[R]``) the rows
+    quantised are ``x[row_index]``, fetched by the kernel itself.  This is the
     "dynamic" activation scheme of :func:`block_fp8_quantization_config`, with scales the matrix instruction takes
     as they are."""
-    device = _lib.require_device(x)
+    device = _lib.require_device(x, row_index)
     if x.dim() != 2 or x.dtype != torch.bfloat16:
         raise TypeError(f"quantize_rows_fp8 takes bf16 [R, K], got {x.dtype} {tuple(x.shape)}")
-    rows, k = x.shape
+    k = x.shape[1]
+    if row_index is not None:
+        row_index = row_index.to(torch.int64).contiguous()
+    rows = x.shape[0] if row_index is None else row_index.numel()
     if k % BLOCK:
         raise ValueError(f"K = {k} is not a multiple of {BLOCK}")
     if x.stride(1) != 1 or x.stride(0) % 8:
@@ -77,8 +81,8 @@ def quantize_rows_fp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     q = torch.empty((k // BLOCK, rows, BLOCK), dtype=torch.uint8, device=device)
     scale = torch.empty((k // BLOCK, rows), dtype=torch.uint8, device=device)
     with _lib.on_device(device):
-        _lib.call("hmoe_quantize_rows_fp8", _lib.ptr(x), x.stride(0), rows, k, _lib.ptr(q), _lib.ptr(scale), rows,
-                  _lib.stream_ptr(device))
+        _lib.call("hmoe_quantize_rows_fp8", _lib.ptr(x), x.stride(0), _lib.ptr(row_index), x.shape[0], rows, k,
+                  _lib.ptr(q), _lib.ptr(scale), rows, _lib.stream_ptr(device))
     return q.view(torch.float8_e4m3fn), scale
 
 

@@ -20,7 +20,7 @@ from typing import ClassVar
 import torch
 import torch.nn as nn
 
-from halo_amd.kernels.expert_gemm import expert_gemm
+from halo_amd.kernels.expert_gemm import BlockFp8Weight, expert_gemm, fp8_mfma_usable
 from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled, resolve_fused_glu_mul
 from halo_amd.kernels.grouped_mm import GatheredRows, grouped_mm, grouped_wgrad
 from halo_amd.kernels.moe_permute import (MoEGatherPermute, MoEWeightedUnpermute, MoEWeightedUnpermuteAdd,
@@ -323,6 +323,9 @@ class EPMoELayerBase(nn.Module, ABC):
         if isinstance(weight, torch.Tensor):
             weight = weight.to(out_dtype)
         if isinstance(x, GatheredRows):
+            if (isinstance(weight, BlockFp8Weight) and self._lowp_fp8_activations and x.dtype == torch.bfloat16
+                    and fp8_mfma_usable(weight.shape[1], weight.shape[2])):
+                return self._grouped_mm(x, weight, offs=offs)  # the row quantiser fetches the rows itself
             fused = x.grouped_mm(weight, offs=offs) if self._lowp_quant_format is None else None
             if fused is not None:
                 return fused

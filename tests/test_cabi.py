@@ -106,10 +106,11 @@ def test_bad_arguments_come_back_as_status_codes_before_any_launch():
     assert fp8(fake, fake, 8, fake, fake, fake, -1, 4, 256, 128, fake, 128, None) == invalid
     assert fp8(fake, None, 8, fake, fake, fake, 8, 4, 256, 128, fake, 128, None) == invalid
     assert fp8(None, None, 0, None, None, None, 0, 1, 256, 128, None, 128, None) == 0
-    assert lib.hmoe_quantize_rows_fp8(fake, 200, 8, 200, fake, fake, 8, None) == unsupported
-    assert lib.hmoe_quantize_rows_fp8(fake, 256, 8, 256, fake, fake, 4, None) == unsupported
-    assert lib.hmoe_quantize_rows_fp8(fake, 256, 8, 256, fake, None, 8, None) == invalid
-    assert lib.hmoe_quantize_rows_fp8(None, 256, 0, 256, None, None, 0, None) == 0
+    assert lib.hmoe_quantize_rows_fp8(fake, 200, None, 8, 8, 200, fake, fake, 8, None) == unsupported
+    assert lib.hmoe_quantize_rows_fp8(fake, 256, None, 8, 8, 256, fake, fake, 4, None) == unsupported
+    assert lib.hmoe_quantize_rows_fp8(fake, 256, None, 8, 8, 256, fake, None, 8, None) == invalid
+    assert lib.hmoe_quantize_rows_fp8(fake, 256, None, 9, 8, 256, fake, fake, 8, None) == invalid  # no index, other rows
+    assert lib.hmoe_quantize_rows_fp8(None, 256, None, 0, 0, 256, None, None, 0, None) == 0
 
     # row movers
     assert lib.hmoe_gather_rows(fake, 64, fake, -1, 64, bf16, fake, None) == invalid

@@ -623,6 +623,15 @@ def test_activation_row_quantiser_is_bit_exact(device, rows, k):
     nonzero = (want_q & 0x7F) != 0
     assert np.array_equal(got_bits[nonzero], want_q[nonzero]) and not (got_bits[~nonzero] & 0x7F).any()
     assert exps[0, 0] == 0 and exps[0, 1] == 127 and exps[0, 2] == 128
+    # rows fetched through an index on the way equal the rows quantised after a gather; an index outside the source
+    # gives a row of zeros
+    index = torch.randint(0, rows, (2 * rows + 3,), generator=g)
+    index[1], index[-1] = -1, rows
+    gq, gexps = quantize_rows_fp8(x.to(device), index.to(device))
+    picked = x[index.clamp(0, rows - 1)]
+    picked[1], picked[-1] = 0, 0
+    pq, pexps = quantize_rows_fp8(picked.to(device))
+    assert torch.equal(gq.view(torch.uint8), pq.view(torch.uint8)) and torch.equal(gexps, pexps)
 
 
 @pytest.mark.parametrize("mantissas", (False, True))
