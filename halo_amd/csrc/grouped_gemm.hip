@@ -1469,6 +1469,313 @@ template __global__ void grouped_gemm_bf16_kernel<kFwdFp8, Config<2, 4, 4, 2>>(G
 // ------------------------------------------------------------------------------------------------ fp32 path
 // 64x64 tile, contraction step 16, 256 threads each owning a 4x4 block.  grid.x walks row tiles of every group
 // (an upper bound of ceil(R/64)+G tiles; surplus workgroups exit), grid.y column tiles.
+// ------------------------------------------------------------------- fp8 kernel, four stages of 64 contraction bytes
+// Both operands e4m3 in panels of 64 contraction values (A [K/64][a_rows][64], B [G][K/64][N][64]); a stage is one
+// panel's share of a 256 x 256 tile, 16 KB per operand, and four stages are resident, so that three refills are in
+// flight while one stage is computed.  (With two stages of 64 KB one refill is in flight, and the step then takes as
+// long as the slowest line of that refill: the latency of a miss under load, about 1.5 us, whatever the hit rate.)
+// The scales travel with their stage: the rows' e8m0 bytes and the two weight scales of the tile's column blocks are
+// loaded into LDS beside the tiles by the same wavefronts.
+constexpr int kF8Stages = 4;
+constexpr int kF8K = 64;                              // contraction values (bytes) per stage
+constexpr int kF8Tile = 256 * kF8K;                   // one operand's share of a stage
+constexpr int kF8Stage = 2 * kF8Tile;
+constexpr int kF8ScaleA = 256 * 4, kF8ScaleB = 64 * 4;  // a dword per tile row; 64 dwords of weight scales
+constexpr int kF8ScaleBase = kF8Stages * kF8Stage;
+constexpr int kF8Lds = kF8ScaleBase + kF8Stages * (kF8ScaleA + kF8ScaleB);
+constexpr int kF8LoadsPerStage = 10;                  // per loading wavefront: 4 + 4 tile loads, 2 scale loads
+
+__device__ __forceinline__ void lds_load4(u32x4 rsrc, lds_bytes_ptr lds_base, uint32_t voffset, uint32_t soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               :
+               : "s"(uniform(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_base)))), "v"(voffset),
+                 "s"(uniform(rsrc)), "s"(uniform(soffset))
+               : "memory");
+}
+// one byte per lane, which lands zero-extended in the lane's dword
+__device__ __forceinline__ void lds_load1(u32x4 rsrc, lds_bytes_ptr lds_base, uint32_t voffset, uint32_t soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_ubyte %1, %2, %3 offen lds"
+               :
+               : "s"(uniform(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_base)))), "v"(voffset),
+                 "s"(uniform(rsrc)), "s"(uniform(soffset))
+               : "memory");
+}
+
+__global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
+  constexpr int WM = 4, WN = 2, BM = 256, BN = 256, kLoadWaves = 4;
+  using Sched = TileSchedule<kFwd, BM, BN>;
+  extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+  __shared__ int32_t grp_s[kMaxGroups], grp_e[kMaxGroups], tile_start[kMaxGroups + 1];
+  auto lds = (lds_bytes_ptr)lds_raw;
+  bf16_t* c = static_cast<bf16_t*>(p.c);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int gm = wave >> 2, gn = wave & 3;
+  const int row_a = gm * 128, row_b = gn * 64;
+  const bool load_wave = wave < kLoadWaves;
+  const int slot = wave & (kLoadWaves - 1);
+
+  if (wave == 0) {
+    const int per = (p.groups + HMOE_WAVE - 1) / HMOE_WAVE;
+    const int g0 = lane * per;
+    int sum = 0;
+    for (int g = g0; g < g0 + per && g < p.groups; ++g) {
+      int64_t s, e;
+      group_bounds(p.offs, g, p.total_rows, s, e);
+      grp_s[g] = static_cast<int32_t>(s);
+      grp_e[g] = static_cast<int32_t>(e);
+      sum += static_cast<int>((e - s + BM - 1) / BM);
+    }
+    int incl = sum;
+#pragma unroll
+    for (int off = 1; off < HMOE_WAVE; off <<= 1) {
+      const int up = __shfl_up(incl, off, HMOE_WAVE);
+      if (lane >= off) incl += up;
+    }
+    int running = incl - sum;
+    for (int g = g0; g < g0 + per && g < p.groups; ++g) {
+      tile_start[g] = running;
+      running += (grp_e[g] - grp_s[g] + BM - 1) / BM;
+    }
+    if (lane == HMOE_WAVE - 1) tile_start[p.groups] = incl;
+  }
+  __syncthreads();
+  Sched sched;
+  sched.init(p, grp_s, grp_e, tile_start);
+  const int steps = static_cast<int>(p.k / kF8K);  // the same for every tile
+  const uint32_t a_panel = static_cast<uint32_t>(p.a_scale_rows) * kF8K, b_panel = static_cast<uint32_t>(p.n) * kF8K;
+  const int64_t w_bytes = p.k * p.n;
+
+  // ---- the loading wavefronts' view of a tile
+  // A load instruction moves 16 rows of 64 bytes: lane L takes row L >> 2, and the chunk that belongs at its place
+  // under the swizzle (physical chunk = logical ^ ((row >> 2) & 3), which spreads the fragment reads of 16
+  // consecutive rows over all the banks).  Rows past the tile's last are whatever follows in the panel (another
+  // expert's rows, or zeros past the array's end): they reach only output rows and columns that are not stored.
+  const uint32_t lane_off = static_cast<uint32_t>(lane >> 2) * kF8K + (((lane & 3) ^ ((lane >> 4) & 3)) << 4);
+  u32x4 rsrc_a, rsrc_b, rsrc_sa, rsrc_sb;
+  uint32_t voff_a = 0, voff_b = 0, voff_sa = 0, voff_sb = 0;
+  auto describe = [&](const TileInfo& tile) __attribute__((always_inline)) {
+    if (load_wave) {
+      const uint8_t* a = static_cast<const uint8_t*>(p.a) + static_cast<int64_t>(tile.row_start) * kF8K;
+      rsrc_a = make_rsrc_words(a, static_cast<uint32_t>(steps) * a_panel - static_cast<uint32_t>(tile.row_start) * kF8K);
+      rsrc_b = make_rsrc_words(static_cast<const uint8_t*>(p.b) + tile.g * w_bytes, static_cast<uint32_t>(w_bytes));
+      rsrc_sa = make_rsrc_words(p.a_scale, static_cast<uint32_t>(p.k_blocks) * static_cast<uint32_t>(p.a_scale_rows));
+      rsrc_sb = make_rsrc_words(p.b_scale, static_cast<uint32_t>(p.groups) * p.k_blocks * p.n_blocks * 4u);
+      voff_a = static_cast<uint32_t>(tile.a_out0 + slot * 64) * kF8K + lane_off;
+      voff_b = static_cast<uint32_t>(tile.b_out0 + slot * 64) * kF8K + lane_off;
+      voff_sa = static_cast<uint32_t>(tile.row_start + tile.a_out0 + slot * 64 + lane);
+      int nb = (tile.b_out0 >> 7) + (lane & 1);
+      nb = nb < p.n_blocks ? nb : p.n_blocks - 1;
+      voff_sb = (static_cast<uint32_t>(tile.g) * p.k_blocks * p.n_blocks + nb) * 4u;
+    }
+  };
+  // stage `step` of the described tile into buffer step & 3: always kF8LoadsPerStage loads, so that the waits below
+  // can count them
+  auto issue = [&](int step) __attribute__((always_inline)) {
+    const int buf = step & (kF8Stages - 1);
+    lds_bytes_ptr ta = lds + buf * kF8Stage + slot * 4096;
+    const uint32_t soff_a = static_cast<uint32_t>(step) * a_panel, soff_b = static_cast<uint32_t>(step) * b_panel;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) lds_load16(rsrc_a, ta + t * 1024, voff_a + t * 1024, soff_a);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) lds_load16(rsrc_b, ta + kF8Tile + t * 1024, voff_b + t * 1024, soff_b);
+    lds_bytes_ptr sc = lds + kF8ScaleBase + buf * (kF8ScaleA + kF8ScaleB);
+    lds_load1(rsrc_sa, sc + slot * 256, voff_sa, static_cast<uint32_t>(step >> 1) * static_cast<uint32_t>(p.a_scale_rows));
+    lds_load4(rsrc_sb, sc + kF8ScaleA, voff_sb, static_cast<uint32_t>(step >> 1) * static_cast<uint32_t>(p.n_blocks) * 4u);
+  };
+
+  // ---- the computing view
+  const int frag_chunk = ((lane >> 5) ^ (((lane & 31) >> 2) & 3)) << 4;
+  const int fa0 = (row_a + (lane & 31)) * kF8K + frag_chunk;
+  const int fb0 = kF8Tile + (row_b + (lane & 31)) * kF8K + frag_chunk;
+  const int sa_at = kF8ScaleBase + (row_a + (lane & 31)) * 4;
+  const int sb_at = kF8ScaleBase + kF8ScaleA + (gn >> 1) * 4;
+  i32x8 fa8[WM], fb8[WN];
+  auto fragment = [&](int at) __attribute__((always_inline)) {
+    const i32x4 lo = *reinterpret_cast<const i32x4*>(lds_raw + at);
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(lds_raw + (at ^ 32));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  // epilogue staging in buffer 3, one 32 x 32 block at a time per wavefront
+  constexpr int kEpiPitch = 32 + 8, kEpiRegion = 32 * kEpiPitch * 2;
+  static_assert(kEpiRegion * 8 <= kF8Stage, "epilogue staging must fit in one stage");
+  const char* stage_rows = lds_raw + 3 * kF8Stage + wave * kEpiRegion;
+  const uint32_t stage_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + 3 * kF8Stage + wave * kEpiRegion +
+                              static_cast<uint32_t>(((lane & 31) * kEpiPitch + ((lane >> 5) << 2)) * 2);
+
+  int cursor = 0;
+  int64_t t = sched.first;
+  TileInfo tile, next;
+  if (t < sched.last) {
+    tile = sched.decode(t, cursor);
+    describe(tile);
+    if (load_wave)
+      for (int st = 0; st < 3 && st < steps; ++st) issue(st);
+  }
+  while (t < sched.last) {
+    const bool has_next = t + sched.stride < sched.last;
+    if (has_next) next = sched.decode(t + sched.stride, cursor);
+    f32x16 acc[WM][WN];
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    int live = (tile.a_out_lim - (tile.a_out0 + row_a) + 31) >> 5;
+    live = live < 0 ? 0 : (live > WM ? WM : live);
+    wait_loads();          // the tile's first three stages (issued before the previous tile's epilogue) are in
+    workgroup_barrier();   // and every wavefront is through with that epilogue's use of buffer 3
+    if (load_wave && steps > 3) issue(3);
+    // stage 0 into registers
+    uint32_t sa_pack, sb_bits;
+    auto read_scales = [&](int buf) __attribute__((always_inline)) {
+      const char* sc = lds_raw + buf * (kF8ScaleA + kF8ScaleB);
+      const uint32_t s0 = *reinterpret_cast<const uint32_t*>(sc + sa_at);
+      const uint32_t s1 = *reinterpret_cast<const uint32_t*>(sc + sa_at + 128);
+      const uint32_t s2 = *reinterpret_cast<const uint32_t*>(sc + sa_at + 256);
+      const uint32_t s3 = *reinterpret_cast<const uint32_t*>(sc + sa_at + 384);
+      sa_pack = (s0 & 0xffu) | ((s1 & 0xffu) << 8) | ((s2 & 0xffu) << 16) | (s3 << 24);
+      sb_bits = *reinterpret_cast<const uint32_t*>(sc + sb_at);
+    };
+    {
+#pragma unroll
+      for (int j = 0; j < WN; ++j) fb8[j] = fragment(fb0 + j * 2048);
+#pragma unroll
+      for (int i = 0; i < WM; ++i) fa8[i] = fragment(fa0 + i * 2048);
+      read_scales(0);
+    }
+    float mant_last = 1.0f;
+
+    auto run = [&](auto full_tag) __attribute__((always_inline)) {
+      constexpr bool kFull = decltype(full_tag)::value;
+      auto mfma = [&](auto row_block, auto col_block, int sa, int sb) __attribute__((always_inline)) {
+        constexpr int i = decltype(row_block)::value, j = decltype(col_block)::value;
+        if (kFull || i < live)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[j], fa8[i], acc[i][j], 0, 0, 0, sb, i, sa);
+      };
+      using std::integral_constant;
+      const integral_constant<int, 0> b0;
+      const integral_constant<int, 1> b1;
+      const integral_constant<int, 2> b2;
+      const integral_constant<int, 3> b3;
+      for (int step = 0; step < steps; ++step) {
+        const int buf = step & (kF8Stages - 1), nbuf = (step + 1) & (kF8Stages - 1);
+        // the weight scale: exponent to the MFMA, mantissa carried by the accumulators (1 for power-of-two scales);
+        // zero or subnormal goes in as 2^-127 with mantissa 1 and contributes nothing either way
+        const uint32_t bits = uniform(sb_bits);
+        const uint32_t sb_exp = bits >> 23;
+        const float mant = sb_exp ? __uint_as_float((bits & 0x007fffffu) | 0x3f800000u) : 1.0f;
+        if (mant != mant_last) {
+          const float ratio = mant_last / mant;
+#pragma unroll
+          for (int i = 0; i < WM; ++i)
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+#pragma unroll
+              for (int v = 0; v < 16; ++v) acc[i][j][v] *= ratio;
+          mant_last = mant;
+        }
+        const int sa = static_cast<int>(sa_pack), sb = static_cast<int>(sb_exp);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(b0, b0, sa, sb);
+        mfma(b1, b0, sa, sb);
+        mfma(b2, b0, sa, sb);
+        mfma(b3, b0, sa, sb);
+        __builtin_amdgcn_sched_barrier(0);
+        // stage step + 1 must be in: the loads of at most two younger stages may still be out
+        const int younger = steps - 2 - step;
+        if (load_wave) {
+          if (younger >= 2) asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)" ::: "memory");
+          else if (younger == 1) asm volatile("s_waitcnt vmcnt(10) lgkmcnt(0)" ::: "memory");
+          else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        } else {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+        workgroup_barrier();
+        // this step's buffer is read out (its fragments were taken during the previous step): refill it
+        if (load_wave && step + 4 < steps) issue(step + 4);
+        // the second column of MFMAs, each followed by the refill of its fragment from the next stage (after a
+        // tile's last step these read what nothing uses)
+        const int na = nbuf * kF8Stage;
+        if (kFull || live > 0) fb8[0] = fragment(na + fb0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(b0, b1, sa, sb);
+        if (kFull || 0 < live) fa8[0] = fragment(na + fa0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(b1, b1, sa, sb);
+        if (kFull || 1 < live) fa8[1] = fragment(na + fa0 + 2048);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(b2, b1, sa, sb);
+        if (kFull || 2 < live) fa8[2] = fragment(na + fa0 + 2 * 2048);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(b3, b1, sa, sb);
+        if (kFull || 3 < live) fa8[3] = fragment(na + fa0 + 3 * 2048);
+        if (kFull || live > 0) fb8[1] = fragment(na + fb0 + 2048);
+        read_scales(nbuf);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    if (live == WM) run(std::true_type{});
+    else run(std::false_type{});
+    if (mant_last != 1.0f) {
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[i][j][v] *= mant_last;
+    }
+
+    // buffers 0-2 are free since the last barrier: the next tile's first stages go out before this tile's epilogue
+    const TileInfo done = tile;
+    t += sched.stride;
+    if (has_next) {
+      tile = next;
+      describe(tile);
+      if (load_wave)
+        for (int st = 0; st < 3 && st < steps; ++st) issue(st);
+    }
+
+    bf16_t* c_base = c + done.row_start * p.ldc;
+    const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(c_base, static_cast<uint32_t>(done.a_out_lim * p.ldc * 2));
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+      if (i < live) {
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            uint2 packed;
+            packed.x = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 0])) |
+                       (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 1])) << 16);
+            packed.y = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 2])) |
+                       (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 3])) << 16);
+            // inline assembly: an LDS store the compiler can see makes it drain the loads in flight first
+            asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(stage_addr), "v"(packed), "n"(q * 8 * 2) : "memory");
+          }
+          __builtin_amdgcn_wave_barrier();  // the rows are private to the wavefront, whose LDS accesses stay in order
+#pragma unroll
+          for (int pass = 0; pass < 2; ++pass) {
+            const int rr = pass * 16 + (lane >> 2);
+            const int cc = (lane & 3) << 3;
+            const int row = done.a_out0 + row_a + i * 32 + rr;
+            const int col = done.b_out0 + row_b + j * 32 + cc;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(stage_rows + (rr * kEpiPitch + cc) * 2);
+            const uint32_t off = row < done.a_out_lim && col < done.b_out_lim
+                                     ? static_cast<uint32_t>(row) * static_cast<uint32_t>(p.ldc) * 2u + col * 2u
+                                     : kOutOfRange;
+            __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, off, 0, 0);
+          }
+          __builtin_amdgcn_wave_barrier();
+        }
+      }
+    }
+  }
+  wait_loads();  // no load may land in LDS after the workgroup has given it back
+}
+
+
 constexpr int FT = 64, FK = 16;
 
 template <int kMode>
@@ -1751,23 +2058,27 @@ int hmoe_grouped_gemm_fwd_fp8(const uint8_t* a_q, const uint8_t* a_scale, int64_
     return HMOE_UNSUPPORTED;
   GemmArgs p{};
   p.a = a_q;
-  p.lda = 64;
   p.b = bq;
-  p.ldb = 64;
   p.c = out;
   p.ldc = ldo;
   p.offs = offs;
   p.total_rows = total_rows;
   p.groups = num_groups;
-  p.k = k / 2;
+  p.k = k;
   p.n = n;
   p.b_scale = b_scale;
   p.a_scale = a_scale;
   p.a_scale_rows = a_rows;
   p.k_blocks = static_cast<int>(k_blocks);
   p.n_blocks = static_cast<int>(n_blocks);
-  const int rc = launch_direct<kFwdFp8, Config<2, 4, 4, 2>>(p, static_cast<hipStream_t>(stream));
-  if (rc) return rc;
+  const int64_t bound = (total_rows / 256 + num_groups) * ((n + 255) / 256);
+  int64_t workers = device_cus();
+  if (bound < workers) workers = bound;
+  workers = (workers + kXcds - 1) / kXcds * kXcds;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_fp8_kernel),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kF8Lds) != hipSuccess)
+    return HMOE_LAUNCH_FAILED;
+  grouped_gemm_fp8_kernel<<<dim3(static_cast<unsigned>(workers)), dim3(512), kF8Lds, static_cast<hipStream_t>(stream)>>>(p);
   if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
   return HMOE_OK;
 }

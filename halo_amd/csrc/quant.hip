@@ -119,10 +119,11 @@ quantize_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const int64_t* _
   word = __builtin_amdgcn_cvt_pk_fp8_f32(v[4] * inv, v[5] * inv, word, false);
   word = __builtin_amdgcn_cvt_pk_fp8_f32(v[6] * inv, v[7] * inv, word, true);
   packed.y = static_cast<uint32_t>(word);
-  // panels: block b of row r at q[(b * out_rows + r) * 128], its scale at scale[b * out_rows + r]
-  const int64_t slot = static_cast<int64_t>(chunk >> 4) * out_rows + row;
-  *reinterpret_cast<uint2*>(q + slot * kBlock + ((chunk & 15) << 3)) = packed;
-  if ((chunk & 15) == 0) scale[slot] = static_cast<uint8_t>(biased);
+  // panels of 64 values: values [64 p, 64 p + 64) of row r at q[(p * out_rows + r) * 64]; the scale of block b
+  // (panels 2 b and 2 b + 1) at scale[b * out_rows + r]
+  const int64_t slot = static_cast<int64_t>(chunk >> 3) * out_rows + row;
+  *reinterpret_cast<uint2*>(q + slot * 64 + ((chunk & 7) << 3)) = packed;
+  if ((chunk & 15) == 0) scale[static_cast<int64_t>(chunk >> 4) * out_rows + row] = static_cast<uint8_t>(biased);
 }
 
 }  // namespace

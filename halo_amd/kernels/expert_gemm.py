@@ -47,12 +47,12 @@ class BlockFp8Weight:
 
 
     def panels(self) -> torch.Tensor:
-        """The e4m3 bytes as ``[G, K / 128, N, 128]``: the contraction contiguous within a panel of 128 values and a
+        """The e4m3 bytes as ``[G, K / 64, N, 64]``: the contraction contiguous within a panel of 64 values and a
         tile's columns of one panel in one run, which is how the fp8 MFMA kernel loads them.  Made once and kept: the
         fp8 bytes once more in device memory."""
         if self._panels is None:
             g, k, n = self.q.shape
-            self._panels = self.q.view(torch.uint8).view(g, k // 128, 128, n).permute(0, 1, 3, 2).contiguous()
+            self._panels = self.q.view(torch.uint8).view(g, k // 64, 64, n).permute(0, 1, 3, 2).contiguous()
         return self._panels
 
 

@@ -60,8 +60,8 @@ def dequantize_block_fp8(weight: torch.Tensor, scale_inv: torch.Tensor, dtype: t
 
 def quantize_rows_fp8(x: torch.Tensor, row_index: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
     """``(q, scale_exponents)`` for bf16 activations ``x [R, K]`` (K a multiple of 128): ``q`` float8_e4m3fn
-    ``[K / 128, R, 128]`` (panels of 128 values, as the fp8 expert GEMM reads them: ``q.permute(1, 0, 2)`` is
-    ``[R, K / 128, 128]``) and uint8 ``[K / 128, R]``, the biased exponent ``e + 127`` of each row's power-of-two
+    ``[K / 64, R, 64]`` (panels of 64 values, as the fp8 expert GEMM reads them: ``q.permute(1, 0, 2)`` is
+    ``[R, K / 64, 64]``) and uint8 ``[K / 128, R]``, the biased exponent ``e + 127`` of each row's power-of-two
     scale ``2^e`` per 128 values (the smallest that brings the block's largest magnitude to 448 or below; 0 for an
     all-zero block).  ``q * 2^e`` reconstructs ``x`` to e4m3 precision.  With ``row_index`` (int64 ``[R]``) the rows
     quantised are ``x[row_index]``, fetched by the kernel itself.  This is the
@@ -78,7 +78,7 @@ def quantize_rows_fp8(x: torch.Tensor, row_index: torch.Tensor | None = None) ->
         raise ValueError(f"K = {k} is not a multiple of {BLOCK}")
     if x.stride(1) != 1 or x.stride(0) % 8:
         x = x.contiguous()
-    q = torch.empty((k // BLOCK, rows, BLOCK), dtype=torch.uint8, device=device)
+    q = torch.empty((k // 64, rows, 64), dtype=torch.uint8, device=device)
     scale = torch.empty((k // BLOCK, rows), dtype=torch.uint8, device=device)
     with _lib.on_device(device):
         _lib.call("hmoe_quantize_rows_fp8", _lib.ptr(x), x.stride(0), _lib.ptr(row_index), x.shape[0], rows, k,

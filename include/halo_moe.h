@@ -189,20 +189,20 @@ int hmoe_grouped_gemm_fwd_fp8w(const void* a, int64_t lda, const uint8_t* bq, co
  * it: block_fp8_quantization_config (halo/kernels/lowp/block_fp8.py:37-46) hands the checkpoint to the serving
  * engine with "activation_scheme": "dynamic", i.e. activations quantised per row and 128 values at run time.
  *
- * Both operands of the product lie in panels of 128 contraction values, [k / 128][rows][128], so that a tile's
- * share of one step is a single contiguous run.
+ * Both operands of the product lie in panels of 64 contraction values, [k / 64][rows][64], so that a tile's share
+ * of one pipeline stage is a single contiguous run.
  *
- * hmoe_quantize_rows_fp8: x bf16 [x_rows, k] (row stride ldx) to q e4m3fn [k / 128][out_rows][128] and scale u8
- * [k / 128][out_rows]: block b of row r at q[(b * out_rows + r) * 128], and at scale[b * out_rows + r] the biased
- * exponent byte (e8m0) of its power-of-two scale, the smallest that brings the block's largest magnitude to 448
- * or below.  Row r is x[row_index[r]] (the permute by expert of MoEGatherPermute, halo/kernels/moe_permute.py:130-141,
+ * hmoe_quantize_rows_fp8: x bf16 [x_rows, k] (row stride ldx) to q e4m3fn [k / 64][out_rows][64] and scale u8
+ * [k / 128][out_rows]: values [64 p, 64 p + 64) of row r at q[(p * out_rows + r) * 64], and at
+ * scale[b * out_rows + r] the biased exponent byte (e8m0) of the power-of-two scale of the row's block b of 128
+ * values, the smallest that brings the block's largest magnitude to 448 or below.  Row r is x[row_index[r]] (the permute by expert of MoEGatherPermute, halo/kernels/moe_permute.py:130-141,
  * taken on the way; an index outside [0, x_rows) gives a row of zeros), or x[r] with row_index NULL (then x_rows ==
  * rows).  k must be a multiple of 128, out_rows >= rows. */
 int hmoe_quantize_rows_fp8(const void* x, int64_t ldx, const int64_t* row_index, int64_t x_rows, int64_t rows, int64_t k,
                            uint8_t* q, uint8_t* scale, int64_t out_rows, void* stream);
 /* out bf16 [total_rows, n] = per group, (a_q * a_scale) [rows, k] @ (bq * b_scale) [k, n]: a_q and a_scale as
- * written by hmoe_quantize_rows_fp8 with out_rows = a_rows; bq e4m3fn [num_groups][k / 128][n][128] (value (kk, c)
- * of expert g at bq[((g * (k / 128) + kk / 128) * n + c) * 128 + kk % 128]) and b_scale f32
+ * written by hmoe_quantize_rows_fp8 with out_rows = a_rows; bq e4m3fn [num_groups][k / 64][n][64] (value (kk, c)
+ * of expert g at bq[((g * (k / 64) + kk / 64) * n + c) * 64 + kk % 64]) and b_scale f32
  * [num_groups, k / 128, ceil(n / 128)], not negative, any mantissa.  Accumulation in fp32, one rounding to bf16.
  * k must be a multiple of 128, n of 8. */
 int hmoe_grouped_gemm_fwd_fp8(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,

@@ -617,7 +617,7 @@ def test_activation_row_quantiser_is_bit_exact(device, rows, k):
     q, exps = quantize_rows_fp8(x.to(device))
     want_q, want_exps = oracle.quantize_rows_fp8(x.float().numpy())
     assert q.dtype == torch.float8_e4m3fn and exps.dtype == torch.uint8 and exps.shape == (k // 128, rows)
-    assert q.shape == (k // 128, rows, 128)  # panels of 128 values
+    assert q.shape == (k // 64, rows, 64)  # panels of 64 values
     assert np.array_equal(exps.cpu().numpy(), want_exps)
     got_bits = q.view(torch.uint8).permute(1, 0, 2).reshape(rows, k).cpu().numpy()
     nonzero = (want_q & 0x7F) != 0
