@@ -96,8 +96,8 @@ struct GemmArgs {
   const int64_t* a_index = nullptr;  // gathered A (fwd, wgrad): logical row r of A is a[a_index[r]]
   int64_t a_rows = 0;                // rows of the array a_index points into
   const void* bias = nullptr;        // fwd: [G, N] in the operands' dtype, added to group g's output rows
-  // kFwdFp8: both operands are e4m3 bytes in panels of 128 contraction values (A [K/128][a_scale_rows][128],
-  // B [G][K/128][N][128]); k counts 2-byte units, so a step of BK units is 128 values: one panel, one scale block
+  // kFwdFp8: both operands are e4m3 bytes in panels of 64 contraction values (A [K/64][a_scale_rows][64],
+  // B [G][K/64][N][64]); k counts values
   const uint8_t* a_scale = nullptr;  // [K / 128][a_scale_rows]: the e8m0 exponent of row r's block b at (b, r)
   int64_t a_scale_rows = 0;
   int k_blocks = 0, n_blocks = 0;     // the grid of b_scale [G, k_blocks, n_blocks]
@@ -729,14 +729,12 @@ struct SlimDirect {  // element(out, con) = base[out * ld + con]; LDS [256 out][
   u32x4 rsrc;  // bounded at the operand's last output row: rows past it load as zeros
   uint32_t voff;                // this lane's chunk for the wavefront's first load of a step, at step 0
   uint32_t t_stride;            // bytes between the rows of consecutive loads (8 rows)
-  uint32_t step_bytes;          // bytes from one contraction step to the next: BK values along a row, or one panel
   int con0, con_lim;
   int t_lim;                    // loads t >= t_lim of this wavefront lie wholly past the operand's last row
 
   __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
-                                       int con_lim_, int wave, int lane, uint32_t step_bytes_ = BK * 2) {
+                                       int con_lim_, int wave, int lane) {
     rsrc = make_rsrc_words(base, static_cast<uint32_t>(bytes));
-    step_bytes = step_bytes_;
     con_lim = con_lim_;
     t_lim = (out_lim - out0 - wave * kI * 8 + 7) >> 3;
     const int logical = (lane & 7) ^ (lane >> 3);  // row & 7 == lane >> 3 for every load
@@ -748,7 +746,7 @@ struct SlimDirect {  // element(out, con) = base[out * ld + con]; LDS [256 out][
   // change) but every offset is out of range, and the step offset stays below the buffer's size
   __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave,
                                         bool live = true) const {
-    const uint32_t soff = live ? static_cast<uint32_t>(step) * step_bytes : 0u;
+    const uint32_t soff = live ? static_cast<uint32_t>(step) * (BK * 2) : 0u;
     const uint32_t base = live && step * BK + con0 < con_lim ? voff : kOutOfRange;
     // A load whose eight rows all lie past the operand's end is left out: nothing reads those rows of the tile
     // for a result that is kept (an output row takes its values from its own operand row only), and in a group's
@@ -986,15 +984,13 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
   static_assert(!kBias || kMode == kFwd, "the expert bias belongs to the forward product");
   static_assert(!kGather || kMode == kFwd || kMode == kWgrad, "A is gathered in fwd and wgrad");
-  static_assert(kMode != kFwdFp8 || (!kGather && !kBias), "the fp8 product takes plain operands");
   constexpr int WM = Cfg::WM, WN = Cfg::WN, BM = Cfg::BM, BN = Cfg::BN;
   constexpr int kWaves = Cfg::GM * Cfg::GN;
   // Wavefronts 0-3 issue all the tile loads and wait for them (16 loads of 1 KB each per step, measured slightly
   // ahead of dealing them to every wavefront); every wavefront runs the MFMAs.
   constexpr int kLoadWaves = 4;
   constexpr int kI = 32 / kLoadWaves;
-  constexpr bool kFp8 = kMode == kFwdFp8;
-  constexpr bool kDirectA = kMode != kWgrad, kDirectB = kMode == kDgrad || kFp8;
+  constexpr bool kDirectA = kMode != kWgrad, kDirectB = kMode == kDgrad;
   using PlainA = typename std::conditional<kDirectA, SlimDirect<kI>, SlimTransposed<kI>>::type;
   using GatheredA = typename std::conditional<kDirectA, GatherDirect<kI>, GatherTransposed<kI>>::type;
   using LoaderA = typename std::conditional<kGather, GatheredA, PlainA>::type;
@@ -1057,17 +1053,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     const bf16_t* a = static_cast<const bf16_t*>(p.a);
     const bf16_t* b = static_cast<const bf16_t*>(p.b);
     const int64_t rows = kMode == kWgrad ? tile.con_lim : tile.a_out_lim;
-    if constexpr (kFp8) {
-      // Panels: operand[block][row][128 values], so a tile's share of a step is one contiguous run per operand.
-      // A row is 64 two-byte units; a step moves on by a whole panel.  Rows past the tile's last in a load of eight
-      // are the next rows of the panel (another expert's, or nothing: the descriptor ends with the array); they
-      // reach only output rows and columns that are not stored.
-      const int64_t a_panel = p.a_scale_rows * 128, b_panel = p.n * 128;
-      la.init(a + tile.row_start * 64, 64, p.k_blocks * a_panel - tile.row_start * 128, tile.a_out0, tile.a_out_lim,
-              tile.con_lim, load_slot, lane, static_cast<uint32_t>(a_panel));
-      lb.init(b + tile.g * w_elems, 64, p.k_blocks * b_panel, tile.b_out0, tile.b_out_lim, tile.con_lim, load_slot,
-              lane, static_cast<uint32_t>(b_panel));
-    } else if constexpr (kGather) {
+    if constexpr (kGather) {
       if (load_wave)  // the row indices are fetched by the lanes that use them
         la.init(a, p.lda, p.a_rows, p.a_index + tile.row_start, tile.a_out0, tile.a_out_lim, tile.con_lim, load_slot,
                 lane);
@@ -1075,13 +1061,11 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim,
               load_slot, lane);
     }
-    if constexpr (kFp8) {
-    } else if constexpr (kMode == kWgrad) {
+    if constexpr (kMode == kWgrad)
       lb.init(b + tile.row_start * p.ldb, p.ldb, rows * p.ldb * 2, tile.b_out0, tile.b_out_lim, tile.con_lim,
               load_slot, lane);
-    } else {
+    else
       lb.init(b + tile.g * w_elems, p.ldb, w_elems * 2, tile.b_out0, tile.b_out_lim, tile.con_lim, load_slot, lane);
-    }
     if (load_wave) {
       if constexpr (kRowsPerStep) {
         if (!rows0_loaded) {
@@ -1132,20 +1116,6 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   // fp8: a fragment of the 32x32x64 MFMA is two 16-byte reads, the chunks sub-steps 2 h and 2 h + 1 of the bf16
   // geometry would take.  Which 32 of the 64 values a lane holds does not matter to the product as long as both
   // operands agree, and here it does not matter to the scales either: a step is one scale block.
-  // One set of fragments: each is replaced by the next half's as soon as its last MFMA of this half is issued (a
-  // second set would not fit beside the accumulators), which the order of the MFMAs makes early enough.
-  i32x8 fa8[WM], fb8[WN];
-  auto fragment8 = [&](const char* tile_base, int base, int block, int half) __attribute__((always_inline)) {
-    const i32x4 lo = __builtin_bit_cast(i32x4, SlimDirect<kI>::fragment(tile_base, base, block, 2 * half));
-    const i32x4 hi = __builtin_bit_cast(i32x4, SlimDirect<kI>::fragment(tile_base, base, block, 2 * half + 1));
-    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-  };
-  auto read_a8 = [&](int stage, int half, int i) __attribute__((always_inline)) {
-    if constexpr (kFp8) fa8[i] = fragment8(lds_raw + stage * kStageBytes, fa_base[0], i, half);
-  };
-  auto read_b8 = [&](int stage, int half, int j) __attribute__((always_inline)) {
-    if constexpr (kFp8) fb8[j] = fragment8(lds_raw + stage * kStageBytes + kTileBytes, fb_base[0], j, half);
-  };
   constexpr int kReads = WM * (kDirectA ? 1 : 2) + WN * (kDirectB ? 1 : 2);  // LDS reads of one sub-step
   constexpr int kMfmas = WM * WN;
   constexpr int kEpiPitch = WN * 32 + 8;
@@ -1187,43 +1157,10 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       if (col < tile.b_out_lim)
         bias_chunk = *reinterpret_cast<const u32x4*>(static_cast<const bf16_t*>(p.bias) + tile.g * p.n + col);
     }
-    // fp8: the scales.  Activations: per row and step one e8m0 byte, the bytes of a step contiguous over the rows;
-    // lane L and lane L + 32 of an MFMA both answer for row L & 31.  Weights: one fp32 per step and 128 output
-    // columns, the same for the whole wavefront (its 64 columns lie in one block).  Both are fetched a step ahead
-    // and pinned as arrived at the top of the step that uses them, right behind the wait the loading wavefronts
-    // make there anyway.
-    uint32_t sa_next[kFp8 ? WM : 1] = {};
-    uint32_t sb_next = 0;
-    __amdgpu_buffer_rsrc_t sa_rsrc, sb_rsrc;
-    uint32_t sa_off = 0, sb_off = 0, sa_step = 0, sb_step = 0;
-    if constexpr (kFp8) {
-      sa_step = static_cast<uint32_t>(p.a_scale_rows);
-      sa_rsrc = make_rsrc(p.a_scale, static_cast<uint32_t>(p.k_blocks) * sa_step);
-      sb_rsrc = make_rsrc(p.b_scale, static_cast<uint32_t>(p.groups) * p.k_blocks * p.n_blocks * 4u);
-      sa_off = static_cast<uint32_t>(tile.row_start + tile.a_out0 + row_a + (lane & 31));
-      sb_step = static_cast<uint32_t>(p.n_blocks) * 4u;
-      sb_off = (static_cast<uint32_t>(tile.g) * p.k_blocks * p.n_blocks + ((tile.b_out0 + row_b) >> 7)) * 4u;
-#pragma unroll
-      for (int i = 0; i < WM; ++i) sa_next[i] = __builtin_amdgcn_raw_buffer_load_b8(sa_rsrc, sa_off, i * 32, 0);
-      sb_next = __builtin_amdgcn_raw_buffer_load_b32(sb_rsrc, sb_off, 0, 0);
-    }
     if (load_wave) wait_loads();
     if constexpr (kBias) asm volatile("" : "+v"(bias_chunk));
     workgroup_barrier();  // step 0 of this tile has landed in stage 0
-    if (steps > 0) {
-      if constexpr (kFp8) {
-        if (live > 0) {
-#pragma unroll
-          for (int j = 0; j < WN; ++j) read_b8(0, 0, j);
-        }
-#pragma unroll
-        for (int i = 0; i < WM; ++i)
-          if (i < live) read_a8(0, 0, i);
-      } else {
-        read_live_fragments(0, 0, 0, live);
-      }
-    }
-    float mant_last = 1.0f;  // fp8: the weight scale's mantissa of the last step, still owed to the accumulators
+    if (steps > 0) read_live_fragments(0, 0, 0, live);
 
     auto run = [&](auto full_tag) __attribute__((always_inline)) {
       constexpr bool kFull = decltype(full_tag)::value;
@@ -1278,128 +1215,8 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         if constexpr (kFull) interleave_reads_under_mfmas<kReads, kMfmas / 2>();
       }
     };
-    // fp8.  The MFMA takes each operand's scale as a power of two: the activations' scales are powers of two by
-    // construction and go in whole, a weight scale goes in as its exponent, and its mantissa m (1 for the scales
-    // the block quantiser makes) is carried by the accumulators: they hold sum / m of the steps so far, are
-    // multiplied by m_previous / m where the mantissa changes, and by the last m at the end.
-    auto run8 = [&](auto full_tag) __attribute__((always_inline)) {
-      constexpr bool kFull = decltype(full_tag)::value;
-      static_assert(WM == 4 && WN == 2, "the order below is written out for 4 x 2 blocks");
-      auto mfma = [&](auto row_block, auto col_block, int sa, int sb) __attribute__((always_inline)) {
-        constexpr int i = decltype(row_block)::value, j = decltype(col_block)::value;
-        if (kFull || i < live)
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[j], fa8[i], acc[i][j], 0, 0, 0, sb, i, sa);
-      };
-      using std::integral_constant;
-      const integral_constant<int, 0> b0;
-      const integral_constant<int, 1> b1;
-      const integral_constant<int, 2> b2;
-      const integral_constant<int, 3> b3;
-      // The MFMAs of one half against weight fragment 0; then fragment 0 is free for the next half's.
-      auto column0 = [&](int sa, int sb) __attribute__((always_inline)) {
-        mfma(b0, b0, sa, sb);
-        mfma(b1, b0, sa, sb);
-        mfma(b2, b0, sa, sb);
-        mfma(b3, b0, sa, sb);
-        __builtin_amdgcn_sched_barrier(0);
-      };
-      // The MFMAs against weight fragment 1, each followed by the refill of its activation fragment from (stage,
-      // half), and fragment 1's own refill at the end.  A refill is three MFMAs or more ahead of its first use, and
-      // stays behind the MFMA that frees its registers (hoisted, it would need registers of its own).
-      auto column1_refilling = [&](int sa, int sb, int stage, int half) __attribute__((always_inline)) {
-        if (kFull || live > 0) read_b8(stage, half, 0);
-        auto one = [&](auto row_block) __attribute__((always_inline)) {
-          constexpr int i = decltype(row_block)::value;
-          mfma(row_block, b1, sa, sb);
-          if (kFull || i < live) read_a8(stage, half, i);
-          __builtin_amdgcn_sched_barrier(0);
-        };
-        one(b0);
-        one(b1);
-        one(b2);
-        one(b3);
-        if (kFull || live > 0) read_b8(stage, half, 1);
-        __builtin_amdgcn_sched_barrier(0);
-      };
-      for (int step = 0; step < steps; ++step) {
-        const int cur = step & 1;
-        const bool more = step + 1 < steps;
-        asm volatile("" : "+v"(sb_next));
-        const uint32_t sb_bits = uniform(sb_next);
-        // the step's activation scales in one register, block i's in byte i (the MFMA picks the byte)
-        static_assert(WM == 4, "four row blocks, four bytes");
-#pragma unroll
-        for (int i = 0; i < WM; ++i) asm volatile("" : "+v"(sa_next[i]));
-        const int sa = static_cast<int>((sa_next[0] & 0xffu) | ((sa_next[1] & 0xffu) << 8) |
-                                        ((sa_next[2] & 0xffu) << 16) | (sa_next[3] << 24));
-        // The other stage is free since the barrier inside the previous step.  (Issued right behind that barrier
-        // instead, a refill would have a whole step to land rather than three quarters of one; measured 8 % slower:
-        // the sixteen issues then stand between the barrier and the fragment reads the next MFMAs wait for.)
-        if (load_wave) {
-          la.issue(lds + (cur ^ 1) * kStageBytes, step + 1, load_slot, more);
-          lb.issue(lds + (cur ^ 1) * kStageBytes + kTileBytes, step + 1, load_slot, more);
-        }
-        // past the last step these read out of range (zeros) or a neighbour's scale, and nothing uses them
-        sb_next = __builtin_amdgcn_raw_buffer_load_b32(sb_rsrc, sb_off, (step + 1) * sb_step, 0);
-#pragma unroll
-        for (int i = 0; i < WM; ++i)
-          sa_next[i] = __builtin_amdgcn_raw_buffer_load_b8(sa_rsrc, sa_off, (step + 1) * sa_step + i * 32, 0);
-        // a zero or subnormal weight scale goes in as 2^-127 with mantissa 1: its block contributes nothing either way
-        const uint32_t sb_exp = sb_bits >> 23;
-        const float mant = sb_exp ? __uint_as_float((sb_bits & 0x007fffffu) | 0x3f800000u) : 1.0f;
-        if (mant != mant_last) {
-          const float ratio = mant_last / mant;
-#pragma unroll
-          for (int i = 0; i < WM; ++i)
-#pragma unroll
-            for (int j = 0; j < WN; ++j)
-#pragma unroll
-              for (int v = 0; v < 16; ++v) acc[i][j][v] *= ratio;
-          mant_last = mant;
-        }
-        const int sb = static_cast<int>(sb_exp);
-        __builtin_amdgcn_sched_barrier(0);
-        column0(sa, sb);
-        column1_refilling(sa, sb, cur, 1);
-        column0(sa, sb);
-        // The barrier comes as late as the refills allow, after 14 of the step's 16 MFMAs: the step's refill has
-        // that much longer to land, and the first fragments of the next step still have two MFMAs to arrive under.
-        mfma(b0, b1, sa, sb);
-        mfma(b1, b1, sa, sb);
-        __builtin_amdgcn_sched_barrier(0);
-        // lgkmcnt(0): this stage is read out; vmcnt(0) where tile loads were issued: the next step has landed
-        if (load_wave) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        workgroup_barrier();
-        // (after a tile's last step the refills read what nothing uses)
-        if (kFull || live > 0) read_b8(cur ^ 1, 0, 0);
-        if (kFull || 0 < live) read_a8(cur ^ 1, 0, 0);
-        if (kFull || 1 < live) read_a8(cur ^ 1, 0, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma(b2, b1, sa, sb);
-        if (kFull || 2 < live) read_a8(cur ^ 1, 0, 2);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma(b3, b1, sa, sb);
-        if (kFull || 3 < live) read_a8(cur ^ 1, 0, 3);
-        if (kFull || live > 0) read_b8(cur ^ 1, 0, 1);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    };
-    if constexpr (kFp8) {
-      if (live == WM) run8(std::true_type{});
-      else run8(std::false_type{});
-      if (mant_last != 1.0f) {
-#pragma unroll
-        for (int i = 0; i < WM; ++i)
-#pragma unroll
-          for (int j = 0; j < WN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] *= mant_last;
-      }
-    } else {
-      if (live == WM) run(std::true_type{});
-      else run(std::false_type{});
-    }
+    if (live == WM) run(std::true_type{});
+    else run(std::false_type{});
 
     // both stages are free: start the next tile's first step into stage 0 before this tile's epilogue
     const TileInfo done = tile;
@@ -1464,7 +1281,6 @@ HMOE_BF16_INSTANCE(kWgrad)
 template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, true>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, false, true>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kWgrad, Config<2, 4, 4, 2>, true>(GemmArgs);
-template __global__ void grouped_gemm_bf16_kernel<kFwdFp8, Config<2, 4, 4, 2>>(GemmArgs);
 
 // ------------------------------------------------------------------------------------------------ fp32 path
 // 64x64 tile, contraction step 16, 256 threads each owning a 4x4 block.  grid.x walks row tiles of every group
@@ -1548,10 +1364,12 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
 
   // ---- the loading wavefronts' view of a tile
   // A load instruction moves 16 rows of 64 bytes: lane L takes row L >> 2, and the chunk that belongs at its place
-  // under the swizzle (physical chunk = logical ^ ((row >> 2) & 3), which spreads the fragment reads of 16
-  // consecutive rows over all the banks).  Rows past the tile's last are whatever follows in the panel (another
+  // under the swizzle: physical chunk = logical ^ ((row >> 1) & 3) ^ ((row >> 3) & 1), under which the fragment
+  // reads (one chunk of each of 32 consecutive rows) fall on distinct 16-byte slots both within any 8 consecutive
+  // rows modulo 128 bytes and within any 16 modulo 256.  Rows past the tile's last are whatever follows in the panel (another
   // expert's rows, or zeros past the array's end): they reach only output rows and columns that are not stored.
-  const uint32_t lane_off = static_cast<uint32_t>(lane >> 2) * kF8K + (((lane & 3) ^ ((lane >> 4) & 3)) << 4);
+  const uint32_t lane_off =
+      static_cast<uint32_t>(lane >> 2) * kF8K + (((lane & 3) ^ ((lane >> 3) & 3) ^ ((lane >> 5) & 1)) << 4);
   u32x4 rsrc_a, rsrc_b, rsrc_sa, rsrc_sb;
   uint32_t voff_a = 0, voff_b = 0, voff_sa = 0, voff_sb = 0;
   auto describe = [&](const TileInfo& tile) __attribute__((always_inline)) {
@@ -1585,7 +1403,7 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
   };
 
   // ---- the computing view
-  const int frag_chunk = ((lane >> 5) ^ (((lane & 31) >> 2) & 3)) << 4;
+  const int frag_chunk = ((lane >> 5) ^ ((lane >> 1) & 3) ^ ((lane >> 3) & 1)) << 4;
   const int fa0 = (row_a + (lane & 31)) * kF8K + frag_chunk;
   const int fb0 = kF8Tile + (row_b + (lane & 31)) * kF8K + frag_chunk;
   const int sa_at = kF8ScaleBase + (row_a + (lane & 31)) * 4;
