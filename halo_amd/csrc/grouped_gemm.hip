@@ -1381,7 +1381,11 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
       rsrc_sb = make_rsrc_words(p.b_scale, static_cast<uint32_t>(p.groups) * p.k_blocks * p.n_blocks * 4u);
       voff_a = static_cast<uint32_t>(tile.a_out0 + slot * 64) * kF8K + lane_off;
       voff_b = static_cast<uint32_t>(tile.b_out0 + slot * 64) * kF8K + lane_off;
-      voff_sa = static_cast<uint32_t>(tile.row_start + tile.a_out0 + slot * 64 + lane);
+      // the dword this lane's byte lands in is d = 64 slot + lane; it takes the scale of tile row
+      // (d >> 7) * 128 + (d & 3) * 32 + ((d & 127) >> 2), so that the four row blocks of a wavefront's lane lie in
+      // one 16-byte read
+      const int d = slot * 64 + lane;
+      voff_sa = static_cast<uint32_t>(tile.row_start + tile.a_out0 + (d >> 7) * 128 + (d & 3) * 32 + ((d & 127) >> 2));
       int nb = (tile.b_out0 >> 7) + (lane & 1);
       nb = nb < p.n_blocks ? nb : p.n_blocks - 1;
       voff_sb = (static_cast<uint32_t>(tile.g) * p.k_blocks * p.n_blocks + nb) * 4u;
@@ -1406,7 +1410,7 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
   const int frag_chunk = ((lane >> 5) ^ ((lane >> 1) & 3) ^ ((lane >> 3) & 1)) << 4;
   const int fa0 = (row_a + (lane & 31)) * kF8K + frag_chunk;
   const int fb0 = kF8Tile + (row_b + (lane & 31)) * kF8K + frag_chunk;
-  const int sa_at = kF8ScaleBase + (row_a + (lane & 31)) * 4;
+  const int sa_at = kF8ScaleBase + (row_a + (lane & 31) * 4) * 4;
   const int sb_at = kF8ScaleBase + kF8ScaleA + (gn >> 1) * 4;
   i32x8 fa8[WM], fb8[WN];
   auto fragment = [&](int at) __attribute__((always_inline)) {
@@ -1422,6 +1426,7 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
                               static_cast<uint32_t>(((lane & 31) * kEpiPitch + ((lane >> 5) << 2)) * 2);
 
   int cursor = 0;
+  int stores_out = 0;  // stores this wavefront issued in the previous tile's epilogue
   int64_t t = sched.first;
   TileInfo tile, next;
   if (t < sched.last) {
@@ -1442,18 +1447,22 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
     int live = (tile.a_out_lim - (tile.a_out0 + row_a) + 31) >> 5;
     live = live < 0 ? 0 : (live > WM ? WM : live);
-    wait_loads();          // the tile's first three stages (issued before the previous tile's epilogue) are in
+    // The tile's first three stages (issued before the previous tile's epilogue) must be in; that epilogue's stores,
+    // issued after them, need not be (vector memory operations complete in issue order, so "all but the youngest n"
+    // leaves exactly the stores out): they drain under this tile's first steps.
+    if (stores_out >= 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else if (stores_out == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    else if (stores_out == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if (stores_out == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else wait_loads();
     workgroup_barrier();   // and every wavefront is through with that epilogue's use of buffer 3
     if (load_wave && steps > 3) issue(3);
     // stage 0 into registers
     uint32_t sa_pack, sb_bits;
     auto read_scales = [&](int buf) __attribute__((always_inline)) {
       const char* sc = lds_raw + buf * (kF8ScaleA + kF8ScaleB);
-      const uint32_t s0 = *reinterpret_cast<const uint32_t*>(sc + sa_at);
-      const uint32_t s1 = *reinterpret_cast<const uint32_t*>(sc + sa_at + 128);
-      const uint32_t s2 = *reinterpret_cast<const uint32_t*>(sc + sa_at + 256);
-      const uint32_t s3 = *reinterpret_cast<const uint32_t*>(sc + sa_at + 384);
-      sa_pack = (s0 & 0xffu) | ((s1 & 0xffu) << 8) | ((s2 & 0xffu) << 16) | (s3 << 24);
+      const u32x4 q = *reinterpret_cast<const u32x4*>(sc + sa_at);
+      sa_pack = (q[0] & 0xffu) | ((q[1] & 0xffu) << 8) | ((q[2] & 0xffu) << 16) | (q[3] << 24);
       sb_bits = *reinterpret_cast<const uint32_t*>(sc + sb_at);
     };
     {
@@ -1500,6 +1509,10 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
         mfma(b1, b0, sa, sb);
         mfma(b2, b0, sa, sb);
         mfma(b3, b0, sa, sb);
+        // Nothing reads these accumulators before the next stage, so the compiler would sink the four MFMAs below
+        // the barrier (they are register operations: the barrier's memory clobber does not hold them), and the
+        // matrix pipe would then stand still through the wait.  Naming them in an empty statement keeps them here.
+        asm volatile("" : "+v"(acc[0][0]), "+v"(acc[1][0]), "+v"(acc[2][0]), "+v"(acc[3][0]));
         __builtin_amdgcn_sched_barrier(0);
         // stage step + 1 must be in: the loads of at most two younger stages may still be out
         const int younger = steps - 2 - step;
@@ -1557,6 +1570,7 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
 
     bf16_t* c_base = c + done.row_start * p.ldc;
     const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(c_base, static_cast<uint32_t>(done.a_out_lim * p.ldc * 2));
+    stores_out = 4 * live;
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
       if (i < live) {
