@@ -47,6 +47,7 @@ SIGNATURES = {
     "hmoe_dequantize_block_fp8": (I, [P, P, L, L, L, I, P, P]),
     "hmoe_grouped_gemm_fwd_fp8w": (I, [P, L, P, P, P, L, I, L, L, P, L, P]),
     "hmoe_quantize_rows_fp8": (I, [P, L, P, L, L, L, P, P, L, P]),
+    "hmoe_glu_fwd_quant_fp8": (I, [P, P, L, L, L, L, I, F, F, I, I, P, P, L, P]),
     "hmoe_grouped_gemm_fwd_fp8": (I, [P, P, L, P, P, P, L, I, L, L, P, L, P]),
 }
 

@@ -4,6 +4,9 @@
 //
 // Replaces _glu_fwd_kernel / _glu_bwd_kernel (halo/kernels/fused_glu.py:118-205) of the reference.
 #include "common.h"
+#include "fp8_rows.h"
+
+#include <type_traits>
 
 namespace hmoe {
 namespace {
@@ -107,6 +110,28 @@ glu_fwd_kernel(const T* __restrict__ gate, const T* __restrict__ up, T* __restri
   o.store(out + row * width + col);
 }
 
+// The forward combine with its output written as e4m3 panels and scale exponents for the fp8 expert GEMM instead of
+// as bf16: each value is rounded to bf16 first, so the result is what the row quantiser makes of glu_fwd_kernel's
+// output, bit for bit, without the bf16 round trip through memory.  bf16, eight values per lane, width a multiple
+// of 128 (sixteen lanes to a scale block).
+template <int kAct, bool kClampAct, bool kPlusOne>
+__global__ void __launch_bounds__(kThreads)
+glu_fwd_quant_kernel(const bf16_t* __restrict__ gate, const bf16_t* __restrict__ up, uint8_t* __restrict__ q,
+                     uint8_t* __restrict__ scale, int64_t out_rows, int64_t stride_gate, int64_t stride_up,
+                     int64_t n_rows, int64_t chunks_per_row, GluParams p) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t row = i / chunks_per_row;
+  if (row >= n_rows) return;  // whole groups of sixteen lanes leave together
+  const int chunk = static_cast<int>(i - row * chunks_per_row);
+  Chunk<bf16_t, 8> g, u;
+  g.load(gate + row * stride_gate + chunk * 8);
+  u.load(up + row * stride_up + chunk * 8);
+  float v[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) v[k] = Elem<bf16_t>::round(glu_value<kAct, kClampAct, kPlusOne>(g.v[k], u.v[k], p));
+  quantize_block_of_row(v, row, chunk, q, scale, out_rows);
+}
+
 template <typename T, int W, int kAct, bool kClampAct, bool kPlusOne>
 __global__ void __launch_bounds__(kThreads)
 glu_bwd_kernel(const T* __restrict__ gate, const T* __restrict__ up, const T* __restrict__ grad_out,
@@ -134,6 +159,9 @@ struct GluArgs {
   GluParams p;
   bool backward;
   hipStream_t stream;
+  uint8_t* q = nullptr;      // forward only: e4m3 panels and scale exponents instead of `out`
+  uint8_t* scale = nullptr;
+  int64_t out_rows = 0;
 };
 
 template <typename T, int W, int kAct, bool kClampAct, bool kPlusOne>
@@ -141,7 +169,12 @@ void launch(const GluArgs& a) {
   const int64_t chunks = a.width / W;
   const int64_t total = chunks * a.n_rows;
   const dim3 grid(static_cast<unsigned>((total + kThreads - 1) / kThreads)), block(kThreads);
-  if (!a.backward)
+  if (a.q) {
+    if constexpr (std::is_same<T, bf16_t>::value && W == 8)
+      glu_fwd_quant_kernel<kAct, kClampAct, kPlusOne><<<grid, block, 0, a.stream>>>(
+          static_cast<const bf16_t*>(a.gate), static_cast<const bf16_t*>(a.up), a.q, a.scale, a.out_rows,
+          a.stride_gate, a.stride_up, a.n_rows, chunks, a.p);
+  } else if (!a.backward)
     glu_fwd_kernel<T, W, kAct, kClampAct, kPlusOne><<<grid, block, 0, a.stream>>>(
         static_cast<const T*>(a.gate), static_cast<const T*>(a.up), static_cast<T*>(a.out), a.stride_gate,
         a.stride_up, a.n_rows, chunks, a.width, a.p);
@@ -172,7 +205,7 @@ int run(const GluArgs& a, int dtype, int activation, int clamp_activated, int up
   if (a.n_rows < 0 || a.width < 0) return HMOE_INVALID_ARGUMENT;
   if (a.n_rows == 0 || a.width == 0) return HMOE_OK;
   if (!a.gate || !a.up) return HMOE_INVALID_ARGUMENT;
-  if (a.backward ? (!a.grad_out || !a.dgate || !a.dup) : !a.out) return HMOE_INVALID_ARGUMENT;
+  if (a.backward ? (!a.grad_out || !a.dgate || !a.dup) : (a.q ? !a.scale : !a.out)) return HMOE_INVALID_ARGUMENT;
   if (a.n_rows * a.width / 1 >= (int64_t(1) << 40)) return HMOE_UNSUPPORTED;
   const int64_t w = dtype == HMOE_BF16 ? 8 : 4;
   bool vec = a.width % w == 0 && a.stride_gate % w == 0 && a.stride_up % w == 0 && aligned16(a.gate) &&
@@ -180,8 +213,15 @@ int run(const GluArgs& a, int dtype, int activation, int clamp_activated, int up
   if (a.backward)
     vec = vec && a.stride_dgate % w == 0 && a.stride_dup % w == 0 && aligned16(a.grad_out) && aligned16(a.dgate) &&
           aligned16(a.dup);
-  else
+  else if (!a.q)
     vec = vec && aligned16(a.out);
+  if (a.q) {
+    // the quantising form has no scalar fallback: bf16, 16-byte operands, whole 128-value blocks
+    if (dtype != HMOE_BF16 || !vec || a.width % 128 || a.out_rows < a.n_rows ||
+        (reinterpret_cast<uintptr_t>(a.q) & 7u))
+      return HMOE_UNSUPPORTED;
+    return launch_activation<bf16_t, 8>(a, activation, clamp_activated, up_plus_one);
+  }
   if (dtype == HMOE_BF16)
     return vec ? launch_activation<bf16_t, 8>(a, activation, clamp_activated, up_plus_one)
                : launch_activation<bf16_t, 1>(a, activation, clamp_activated, up_plus_one);
@@ -206,6 +246,19 @@ int hmoe_glu_fwd(const void* gate, const void* up, int64_t stride_gate, int64_t 
   a.backward = false;
   a.stream = static_cast<hipStream_t>(stream);
   return hmoe::run(a, dtype, activation, clamp_activated, up_plus_one);
+}
+
+int hmoe_glu_fwd_quant_fp8(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up, int64_t n_rows,
+                           int64_t width, int activation, float alpha, float limit, int clamp_activated,
+                           int up_plus_one, uint8_t* q, uint8_t* scale, int64_t out_rows, void* stream) {
+  hmoe::GluArgs a{};
+  a.gate = gate; a.up = up; a.q = q; a.scale = scale; a.out_rows = out_rows;
+  a.stride_gate = stride_gate; a.stride_up = stride_up; a.n_rows = n_rows; a.width = width;
+  a.p = {alpha, limit};
+  a.backward = false;
+  a.stream = static_cast<hipStream_t>(stream);
+  if (n_rows > 0 && width > 0 && !q) return HMOE_INVALID_ARGUMENT;
+  return hmoe::run(a, HMOE_BF16, activation, clamp_activated, up_plus_one);
 }
 
 int hmoe_glu_bwd(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up, const void* grad_out,

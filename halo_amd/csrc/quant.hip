@@ -6,6 +6,7 @@
 // q = clamp(x / scale, +-448) rounded to e4m3 (nearest even).  Division by a power of two is exact, so the result
 // does not depend on the device's divider.
 #include "common.h"
+#include "fp8_rows.h"
 
 namespace hmoe {
 namespace {
@@ -79,10 +80,8 @@ dequantize_kernel(const uint8_t* __restrict__ q, const float* __restrict__ scale
 }
 
 // Activation rows to e4m3 with one power-of-two scale per row and 128 values, for the fp8 MFMA product (which takes
-// an operand's scale as an e8m0 exponent byte).  Sixteen lanes share a block: each loads 8 values, the maximum goes
-// round the sixteen, and the exponent is read off its bits: with amax = m 2^x (1 <= m < 2) the smallest e for which
-// amax 2^-e <= 448 = 1.75 2^8 is x - 8, one more where m > 1.75.  Stored biased (e + 127), clamped at 0; an all-zero
-// block gets 0.  q = x 2^-e rounded to nearest even.  With row_index, output row r is x[row_index[r]] (the permute by
+// an operand's scale as an e8m0 exponent byte).  Sixteen lanes share a block: each loads 8 values and hands them to
+// quantize_block_of_row.  With row_index, output row r is x[row_index[r]] (the permute by
 // expert taken on the way: the permuted bf16 copy is never written), zeros where the index is outside [0, x_rows).
 __global__ void __launch_bounds__(256)
 quantize_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const int64_t* __restrict__ row_index, int64_t x_rows,
@@ -100,30 +99,7 @@ quantize_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const int64_t* _
 #pragma unroll
     for (int i = 0; i < 8; ++i) in.v[i] = 0.f;
   }
-  const float* v = in.v;
-  float amax = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
-#pragma unroll
-  for (int off = 1; off < 16; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 16));
-  const uint32_t bits = __float_as_uint(amax);
-  int biased = static_cast<int>(bits >> 23) - 8 + ((bits & 0x007fffffu) > 0x00600000u ? 1 : 0);
-  biased = biased < 0 ? 0 : biased;
-  const float inv = __uint_as_float(static_cast<uint32_t>(254 - biased) << 23);  // 2^-(biased - 127), exact
-  uint2 packed;
-  int word = 0;
-  word = __builtin_amdgcn_cvt_pk_fp8_f32(v[0] * inv, v[1] * inv, word, false);
-  word = __builtin_amdgcn_cvt_pk_fp8_f32(v[2] * inv, v[3] * inv, word, true);
-  packed.x = static_cast<uint32_t>(word);
-  word = 0;
-  word = __builtin_amdgcn_cvt_pk_fp8_f32(v[4] * inv, v[5] * inv, word, false);
-  word = __builtin_amdgcn_cvt_pk_fp8_f32(v[6] * inv, v[7] * inv, word, true);
-  packed.y = static_cast<uint32_t>(word);
-  // panels of 64 values: values [64 p, 64 p + 64) of row r at q[(p * out_rows + r) * 64]; the scale of block b
-  // (panels 2 b and 2 b + 1) at scale[b * out_rows + r]
-  const int64_t slot = static_cast<int64_t>(chunk >> 3) * out_rows + row;
-  *reinterpret_cast<uint2*>(q + slot * 64 + ((chunk & 7) << 3)) = packed;
-  if ((chunk & 15) == 0) scale[static_cast<int64_t>(chunk >> 4) * out_rows + row] = static_cast<uint8_t>(biased);
+  quantize_block_of_row(in.v, row, chunk, q, scale, out_rows);
 }
 
 }  // namespace

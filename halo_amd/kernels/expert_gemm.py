@@ -121,13 +121,16 @@ def fp8_mfma_usable(k: int, n: int) -> bool:
 
 def _fp8_mfma_forward(mat_a: torch.Tensor, weight: BlockFp8Weight, offs: torch.Tensor | None) -> torch.Tensor:
     """Activations to e4m3 (one launch, which also fetches the rows when ``mat_a`` is a :class:`GatheredRows`: the
-    permuted bf16 copy is never written), then the grouped GEMM on the scaled e4m3 MFMA against the weight's bytes in
+    permuted bf16 copy is never written; none at all when ``mat_a`` already is a ``QuantizedRows``), then the grouped GEMM on the scaled e4m3 MFMA against the weight's bytes in
     panels and its fp32 block scales."""
-    from halo_amd.kernels.lowp.block_fp8 import quantize_rows_fp8
+    from halo_amd.kernels.lowp.block_fp8 import QuantizedRows, quantize_rows_fp8
 
     gathered = isinstance(mat_a, GatheredRows)
-    source = mat_a.tokens if gathered else mat_a
+    quantized = isinstance(mat_a, QuantizedRows)
+    source = mat_a.tokens if gathered else (mat_a.q if quantized else mat_a)
     device = _lib.require_device(source, weight.q, weight.scale_inv, offs)
+    if quantized:
+        source = mat_a  # its dtype and gradient flag stand for the bf16 rows it was made from
     if source.dtype != torch.bfloat16:
         raise TypeError(f"block-fp8 expert GEMM takes bf16 activations, got {source.dtype}")
     if source.requires_grad and torch.is_grad_enabled():
@@ -142,7 +145,10 @@ def _fp8_mfma_forward(mat_a: torch.Tensor, weight: BlockFp8Weight, offs: torch.T
     if rows == 0 or n == 0:
         return out
     offs32 = _offs_arg(offs, groups)
-    a_q, a_scale = quantize_rows_fp8(source, mat_a.row_index if gathered else None)
+    if quantized:
+        a_q, a_scale = mat_a.q, mat_a.scale_exponents
+    else:
+        a_q, a_scale = quantize_rows_fp8(source, mat_a.row_index if gathered else None)
     w_panels = weight.panels()
     with _lib.on_device(device):
         _lib.call("hmoe_grouped_gemm_fwd_fp8", _lib.ptr(a_q), _lib.ptr(a_scale), rows, _lib.ptr(w_panels),

@@ -218,6 +218,31 @@ class GluCombine:
         gate, up = gate_up.chunk(2, dim=-1)
         return self._eager(gate, up)
 
+    def packed_quantized(self, gate_up: torch.Tensor):
+        """``packed`` with its output as e4m3 panels and scale exponents for the fp8 expert GEMM
+        (:class:`halo_amd.kernels.lowp.block_fp8.QuantizedRows`): the bits ``quantize_rows_fp8(self.packed(gate_up))``
+        gives, without the bf16 output being written.  Forward only.  None where the kernel does not apply (kernels
+        switched off, not bf16, a half width that is not a multiple of 128, rows that are not 16-byte aligned)."""
+        from halo_amd.kernels.lowp.block_fp8 import QuantizedRows
+
+        if not _FUSED_GLU_ENABLED or gate_up.dtype != torch.bfloat16 or gate_up.dim() != 2:
+            return None
+        if gate_up.requires_grad and torch.is_grad_enabled():
+            return None
+        packed = _as_rows(gate_up)
+        rows, half = packed.shape[0], packed.shape[1] // 2
+        if half == 0 or half % 128 or packed.stride(0) % 8 or packed.data_ptr() % 16:
+            return None
+        device = _lib.require_device(packed)
+        q = torch.empty((half // 64, rows, 64), dtype=torch.uint8, device=device)
+        scale = torch.empty((half // 128, rows), dtype=torch.uint8, device=device)
+        if rows:
+            gate, up = packed[:, :half], packed[:, half:]
+            with _lib.on_device(device):
+                _lib.call("hmoe_glu_fwd_quant_fp8", _lib.ptr(gate), _lib.ptr(up), gate.stride(0), up.stride(0), rows,
+                          half, *_kernel_args(self), _lib.ptr(q), _lib.ptr(scale), rows, _lib.stream_ptr(device))
+        return QuantizedRows(q.view(torch.float8_e4m3fn), scale)
+
     def _eager(self, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
         kind = self.name
         if kind == "silu":

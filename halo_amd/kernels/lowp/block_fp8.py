@@ -58,6 +58,26 @@ def dequantize_block_fp8(weight: torch.Tensor, scale_inv: torch.Tensor, dtype: t
     return out
 
 
+class QuantizedRows:
+    """Activation rows already in the fp8 expert GEMM's operand form: ``q`` e4m3 panels ``[K / 64, R, 64]`` and
+    ``scale_exponents`` uint8 ``[K / 128, R]`` as :func:`quantize_rows_fp8` returns them.  Stands where a bf16
+    ``[R, K]`` tensor would (``shape``, ``dtype``, ``device``) for a producer that quantises as it writes."""
+
+    def __init__(self, q: torch.Tensor, scale_exponents: torch.Tensor):
+        self.q, self.scale_exponents = q, scale_exponents
+
+    @property
+    def shape(self):
+        return torch.Size((self.q.shape[1], self.q.shape[0] * self.q.shape[2]))
+
+    dtype = torch.bfloat16  # the precision the values were rounded to before they were scaled
+    requires_grad = False
+
+    @property
+    def device(self):
+        return self.q.device
+
+
 def quantize_rows_fp8(x: torch.Tensor, row_index: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
     """``(q, scale_exponents)`` for bf16 activations ``x [R, K]`` (K a multiple of 128): ``q`` float8_e4m3fn
     ``[K / 64, R, 64]`` (panels of 64 values, as the fp8 expert GEMM reads them: ``q.permute(1, 0, 2)`` is

@@ -175,6 +175,8 @@ class EPMoELayerBase(nn.Module, ABC):
         self._lowp_weight_cacheable = True
         # quantised weights only: quantise the activations too and multiply on the e4m3 MFMA
         self._lowp_fp8_activations = False
+        # with it: the SwiGLU kernel writes the down projection's e4m3 operand itself
+        self.fuse_glu_quantise = True
         # the first expert projection gathers its rows by index instead of reading a permuted copy of the tokens
         self.fuse_permute_into_gemm = True
         # the shared expert's output joins the routed one in the combine kernel instead of a tensor addition
@@ -343,13 +345,27 @@ class EPMoELayerBase(nn.Module, ABC):
 
     def _glu_ffn(self, x: torch.Tensor, proj: Callable[[torch.Tensor, str], torch.Tensor]) -> torch.Tensor:
         if self._stores_fused_glu:  # one projection to [gate | up], combined where it lies
-            hidden = self._glu_combine_packed(proj(x, "gate_up_proj"))
+            gate_up = proj(x, "gate_up_proj")
+            hidden = self._glu_combine_quantized(gate_up)
+            if hidden is None:
+                hidden = self._glu_combine_packed(gate_up)
         else:
             hidden = self._glu_combine(proj(x, "gate_proj"), proj(x, "up_proj"))
         return proj(hidden, "down_proj")
 
     def _glu_combine(self, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
         return self._fused_glu_mul(gate, up)
+
+    def _glu_combine_quantized(self, gate_up: torch.Tensor):
+        """The combine writing the down projection's e4m3 operand directly, where that projection runs on the e4m3
+        MFMA (quantised weights with ``_lowp_fp8_activations``); None otherwise."""
+        down = getattr(self, "down_proj", None)
+        combine = self._fused_glu_mul
+        if not (self._lowp_fp8_activations and self.fuse_glu_quantise and isinstance(down, BlockFp8Weight)
+                and isinstance(combine, GluCombine) and isinstance(gate_up, torch.Tensor)
+                and fp8_mfma_usable(down.shape[1], down.shape[2])):
+            return None
+        return combine.packed_quantized(gate_up)
 
     def _glu_combine_packed(self, gate_up: torch.Tensor) -> torch.Tensor:
         combine = self._fused_glu_mul

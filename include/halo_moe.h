@@ -200,6 +200,12 @@ int hmoe_grouped_gemm_fwd_fp8w(const void* a, int64_t lda, const uint8_t* bq, co
  * rows).  k must be a multiple of 128, out_rows >= rows. */
 int hmoe_quantize_rows_fp8(const void* x, int64_t ldx, const int64_t* row_index, int64_t x_rows, int64_t rows, int64_t k,
                            uint8_t* q, uint8_t* scale, int64_t out_rows, void* stream);
+/* hmoe_glu_fwd with its output quantised on the way: what hmoe_quantize_rows_fp8 makes of hmoe_glu_fwd's bf16
+ * output, bit for bit (each value is rounded to bf16 before it is scaled), without that output being written.  bf16
+ * operands with 16-byte rows, width a multiple of 128; q and scale as hmoe_quantize_rows_fp8 writes them. */
+int hmoe_glu_fwd_quant_fp8(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up, int64_t n_rows,
+                           int64_t width, int activation, float alpha, float limit, int clamp_activated,
+                           int up_plus_one, uint8_t* q, uint8_t* scale, int64_t out_rows, void* stream);
 /* out bf16 [total_rows, n] = per group, (a_q * a_scale) [rows, k] @ (bq * b_scale) [k, n]: a_q and a_scale as
  * written by hmoe_quantize_rows_fp8 with out_rows = a_rows; bq e4m3fn [num_groups][k / 64][n][64] (value (kk, c)
  * of expert g at bq[((g * (k / 64) + kk / 64) * n + c) * 64 + kk % 64]) and b_scale f32

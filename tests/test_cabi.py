@@ -111,6 +111,12 @@ def test_bad_arguments_come_back_as_status_codes_before_any_launch():
     assert lib.hmoe_quantize_rows_fp8(fake, 256, None, 8, 8, 256, fake, None, 8, None) == invalid
     assert lib.hmoe_quantize_rows_fp8(fake, 256, None, 9, 8, 256, fake, fake, 8, None) == invalid  # no index, other rows
     assert lib.hmoe_quantize_rows_fp8(None, 256, None, 0, 0, 256, None, None, 0, None) == 0
+    glu_q = lib.hmoe_glu_fwd_quant_fp8
+    assert glu_q(fake, fake, 512, 512, 8, 200, 0, 1.0, 0.0, 0, 0, fake, fake, 8, None) == unsupported  # 200 % 128
+    assert glu_q(fake, fake, 512, 512, 8, 256, 0, 1.0, 0.0, 0, 0, fake, fake, 4, None) == unsupported  # out_rows < rows
+    assert glu_q(fake, fake, 512, 512, 8, 256, 0, 1.0, 0.0, 0, 0, None, fake, 8, None) == invalid
+    assert glu_q(fake, fake, 512, 512, 8, 256, 9, 1.0, 0.0, 0, 0, fake, fake, 8, None) == invalid  # no such activation
+    assert glu_q(None, None, 512, 512, 0, 256, 0, 1.0, 0.0, 0, 0, None, None, 0, None) == 0
 
     # row movers
     assert lib.hmoe_gather_rows(fake, 64, fake, -1, 64, bf16, fake, None) == invalid

@@ -634,6 +634,26 @@ def test_activation_row_quantiser_is_bit_exact(device, rows, k):
     assert torch.equal(gq.view(torch.uint8), pq.view(torch.uint8)) and torch.equal(gexps, pexps)
 
 
+@pytest.mark.parametrize("kind", ("silu", "gelu_tanh", "gptoss", "clamped"))
+def test_glu_writing_e4m3_panels_equals_glu_then_row_quantiser(device, kind):
+    from halo_amd.kernels.fused_glu import GluCombine
+    from halo_amd.kernels.lowp.block_fp8 import quantize_rows_fp8
+
+    combine = {"silu": GluCombine.silu(), "gelu_tanh": GluCombine.gelu_tanh(), "gptoss": GluCombine.gptoss(1.702, 7.0),
+               "clamped": GluCombine.clamped_silu(5.0, clamp_activated=True)}[kind]
+    g = torch.Generator().manual_seed(9)
+    for rows, half in ((77, 128), (300, 1024)):
+        gate_up = (torch.randn(rows, 2 * half, generator=g) * 3).bfloat16().to(device)
+        gate_up[3, :half] = 0
+        fused = combine.packed_quantized(gate_up)
+        q, exps = quantize_rows_fp8(combine.packed(gate_up))
+        assert fused.shape == (rows, half)
+        assert torch.equal(fused.q.view(torch.uint8), q.view(torch.uint8))
+        assert torch.equal(fused.scale_exponents, exps)
+    assert combine.packed_quantized(gate_up[:, : 2 * 96]) is None  # a half width off the block size
+    assert combine.packed_quantized(gate_up.float()) is None
+
+
 @pytest.mark.parametrize("mantissas", (False, True))
 @pytest.mark.parametrize(("counts", "k", "n"), (((130, 0, 257, 64), 128, 256), ((300, 1, 0, 255, 256, 700), 1024, 520),
                                                  ((64,) * 16, 384, 1536), ((1000,), 3072, 128)))

@@ -219,6 +219,10 @@ def test_quantised_weight_forward(device):
     assert 0.005 < rel < 0.07, rel
     assert cosine(fp8, want) > 0.997
     assert abs(((fp8.double() - want.double()).mean() / want.double().abs().mean()).item()) < 5e-3
+    lowp.fuse_glu_quantise = False  # the SwiGLU output through bf16 and the row quantiser: the same bits
+    with torch.no_grad():
+        two_step = lowp._compute_experts(x, experts.to(device), weights.to(device), torch.bfloat16, recv_counts=counts)
+    assert torch.equal(two_step, fp8)
 
 
 # ------------------------------------------------------------------------------ drop-ins for the Hugging Face blocks
