@@ -25,6 +25,15 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
   return __builtin_bit_cast(bf16_t, h);
 }
 
+// Two floats to two bf16 in one word (lo in the low half), rounded as above: one packed conversion instead of two
+// single ones and the shifts that join them.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
 template <typename T>
 struct Elem;
 template <>
@@ -74,7 +83,7 @@ struct Vec16<bf16_t> {
     uint32_t w[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      w[i] = static_cast<uint32_t>(f32_to_bf16(v[2 * i])) | (static_cast<uint32_t>(f32_to_bf16(v[2 * i + 1])) << 16);
+      w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
     *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
   }
 };

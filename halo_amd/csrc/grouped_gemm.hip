@@ -175,7 +175,7 @@ __device__ __forceinline__ u32x4 add_bf16x8(u32x4 a, u32x4 b) {
   for (int w = 0; w < 4; ++w) {
     const float lo = __uint_as_float(a[w] << 16) + __uint_as_float(b[w] << 16);
     const float hi = __uint_as_float(a[w] & 0xffff0000u) + __uint_as_float(b[w] & 0xffff0000u);
-    out[w] = static_cast<uint32_t>(f32_to_bf16(lo)) | (static_cast<uint32_t>(f32_to_bf16(hi)) << 16);
+    out[w] = pack_bf16x2(lo, hi);
   }
   return out;
 }
@@ -477,10 +477,8 @@ __device__ __forceinline__ void compute_tile(bf16_t* smem, LoaderA& la, LoaderB&
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           uint2 packed;
-          packed.x = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 0])) |
-                     (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 1])) << 16);
-          packed.y = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 2])) |
-                     (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 3])) << 16);
+          packed.x = pack_bf16x2(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1]);
+          packed.y = pack_bf16x2(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
           *reinterpret_cast<uint2*>(stage + (ii * 32 + (lane & 31)) * kEpiPitch + j * 32 + q * 8 + ((lane >> 5) << 2)) =
               packed;
         }
@@ -1238,10 +1236,8 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             uint2 packed;
-            packed.x = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 0])) |
-                       (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 1])) << 16);
-            packed.y = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 2])) |
-                       (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 3])) << 16);
+            packed.x = pack_bf16x2(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1]);
+            packed.y = pack_bf16x2(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
             // Written through inline assembly on purpose: before an LDS store it can see, the compiler drains every
             // direct-to-LDS load in flight (it cannot tell that these rows are not their target), which here would
             // wait for the next tile's first step.
@@ -1579,10 +1575,8 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             uint2 packed;
-            packed.x = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 0])) |
-                       (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 1])) << 16);
-            packed.y = static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 2])) |
-                       (static_cast<uint32_t>(f32_to_bf16(acc[i][j][q * 4 + 3])) << 16);
+            packed.x = pack_bf16x2(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1]);
+            packed.y = pack_bf16x2(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
             // inline assembly: an LDS store the compiler can see makes it drain the loads in flight first
             asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(stage_addr), "v"(packed), "n"(q * 8 * 2) : "memory");
           }
