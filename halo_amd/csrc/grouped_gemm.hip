@@ -48,6 +48,11 @@
 // tiling: global -> registers (dequantised there) -> LDS as [output index][64 contraction], both operands read back
 // with ds_read_b128.
 //
+// Both operands in e4m3 (grouped_gemm_fp8_kernel, forward only): activations quantised per row and 128 values with
+// power-of-two scales, weights with their 128 x 128 block scales, on v_mfma_scale_f32_32x32x64_f8f6f4, which takes each
+// operand's scale as an exponent byte per lane.  Same tile and schedule; operands in panels of 64 contraction values,
+// four LDS stages of 32 KB with three refills in flight, waited for by count.  Described where it is defined.
+//
 // fp32 operands take a plain LDS-tiled FMA kernel (the CPU-sized plumbing configuration and tests).
 #include "common.h"
 
