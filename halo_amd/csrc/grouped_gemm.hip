@@ -1264,7 +1264,10 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
           const uint32_t off = row < done.a_out_lim && col < done.b_out_lim
                                    ? static_cast<uint32_t>(row) * static_cast<uint32_t>(p.ldc) * 2u + col * 2u
                                    : kOutOfRange;
-          __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, off, 0, 0);
+          // a weight gradient is not read again before the optimizer: stored non-temporally, it leaves the L2's
+          // lines to the operands (measured: the two weight-gradient launches of a step 3-4 % faster; the forward
+          // and input-gradient outputs are read by the next kernel and keep the default policy)
+          __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, off, 0, kMode == kWgrad ? 2 : 0);
         }
         __builtin_amdgcn_wave_barrier();
       }
