@@ -8,4 +8,11 @@ from halo_amd.moe_layer.families import (  # noqa: F401
     EPQwen3MoELayer,
     apply_ep_layers,
 )
+from halo_amd.moe_layer.expert_lora import (  # noqa: F401
+    ExpertLoraSpec,
+    disable_expert_adapters,
+    expert_lora_delta,
+    expert_lora_layers,
+    model_has_expert_lora,
+)
 from halo_amd.moe_layer.layer import EPMoELayerBase, EPSharedExpertsMoELayerBase  # noqa: F401

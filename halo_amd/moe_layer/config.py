@@ -27,6 +27,7 @@ class EPConfig:
     experts_per_rank: int | None = None
     expert_start_idx: int | None = None
     expert_end_idx: int | None = None
+    expert_lora: object | None = None  # an ExpertLoraSpec (moe_layer/expert_lora.py): grouped adapters on the experts
 
     def __post_init__(self):
         if self.expert_tp_size != 1:

@@ -135,6 +135,7 @@ class EPGptOssMoELayer(EPMoELayerBase):
         bias = getattr(self, f"{weight_attr}_bias", None)
         weight = getattr(self, weight_attr)
         if (bias is not None and getattr(self, "fuse_bias_into_gemm", True) and self._lowp_quant_format is None
+                and not self._adapted(weight_attr)
                 and isinstance(weight, torch.Tensor) and isinstance(x, torch.Tensor)):
             weight, bias_cast = weight.to(out_dtype), bias.to(out_dtype)
             if bias_fusable(x, weight, bias_cast):  # the projection and its bias in one kernel, the same bits

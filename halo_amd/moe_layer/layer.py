@@ -6,8 +6,8 @@ Mirrors the parts of the reference's EP MoE layer that run at ``ep_size`` 1 or o
 ``_glu_ffn`` ``:357-361``, ``_init_fused_glu_params`` ``:77-88``), ``moe_layer/layer.py`` (construction order ``:67-80``,
 ``_dispatch_compute_combine{,_shared}`` ``:270-342``), ``moe_layer/routing.py`` (``_softmax_gate_weights_at``
 ``:110-119``) and ``moe_layer/shared_experts_layer.py`` (``forward`` ``:20-28``).  Every tensor op on the path is a HIP
-kernel of this package; the dispatch/combine exchange, expert LoRA, balancing bias, routing replay and expert TP of the
-reference are not part of it.
+kernel of this package; grouped expert LoRA is in as far as it computes (``moe_layer/expert_lora.py``); the
+dispatch/combine exchange, balancing bias, routing replay and expert TP of the reference are not part of it.
 """
 
 from __future__ import annotations
@@ -28,6 +28,7 @@ from halo_amd.kernels.moe_permute import (MoEGatherPermute, MoEWeightedUnpermute
 from halo_amd.kernels.moe_route_sort import sort_routing_by_expert, warm_route_sort_kernels
 from halo_amd.kernels.router import SOFTMAX_ALL, fused_topk_gate
 from halo_amd.moe_layer.config import EPConfig, MoEFamilySpec
+from halo_amd.moe_layer.expert_lora import EXPERT_LORA_SUFFIXES, init_expert_lora
 
 logger = logging.getLogger(__name__)
 
@@ -112,6 +113,7 @@ class EPMoELayerBase(nn.Module, ABC):
         self._adopt_expert_compute(original_layer, experts)
         self._adopt_expert_params(experts, weights_already_sharded=weights_already_sharded)
         self._finalize_expert_init()
+        init_expert_lora(self, ep_config.expert_lora)
 
     # ---------------------------------------------------------------------------------------------- construction
 
@@ -320,10 +322,28 @@ class EPMoELayerBase(nn.Module, ABC):
     def _grouped_expert_ffn(self, sorted_tokens, offs, sorted_expert_ids, output_dtype):
         return self._glu_ffn(sorted_tokens, lambda x, attr: self._expert_proj(x, attr, offs, output_dtype))
 
+    @property
+    def has_expert_lora(self) -> bool:
+        return bool(getattr(self, "_expert_lora_attrs", None))
+
+    def expert_lora_named_params(self) -> list:
+        names = [attr + suffix for attr in sorted(self._expert_lora_attrs) for suffix in EXPERT_LORA_SUFFIXES]
+        return [(name, getattr(self, name)) for name in names]
+
+    def _adapted(self, weight_attr: str) -> bool:
+        return self.has_expert_lora and self._expert_adapters_enabled and weight_attr in self._expert_lora_attrs
+
     def _expert_proj(self, x: torch.Tensor, weight_attr: str, offs: torch.Tensor, out_dtype: torch.dtype):
-        weight = getattr(self, weight_attr)
-        if isinstance(weight, torch.Tensor):
-            weight = weight.to(out_dtype)
+        if self._adapted(weight_attr):
+            # x @ W + scaling * (dropout(x) @ A) @ B, the adapter products in the activation dtype whatever the
+            # base weight is stored in (a scale block along a rank of 8-64 means nothing)
+            rows = x.materialize() if isinstance(x, GatheredRows) else x
+            base = self._grouped_mm(rows, self._cast_weight(weight_attr, out_dtype), offs=offs)
+            lora_a = getattr(self, weight_attr + EXPERT_LORA_SUFFIXES[0]).to(out_dtype)
+            lora_b = getattr(self, weight_attr + EXPERT_LORA_SUFFIXES[1]).to(out_dtype)
+            low = self._grouped_mm(self.expert_lora_dropout(rows), lora_a, offs=offs, lowp=False)
+            return base + self.expert_lora_scaling * self._grouped_mm(low, lora_b, offs=offs, lowp=False)
+        weight = self._cast_weight(weight_attr, out_dtype)
         if isinstance(x, GatheredRows):
             if (isinstance(weight, BlockFp8Weight) and self._lowp_fp8_activations and x.dtype == torch.bfloat16
                     and fp8_mfma_usable(weight.shape[1], weight.shape[2])):
@@ -333,6 +353,10 @@ class EPMoELayerBase(nn.Module, ABC):
                 return fused
             x = x.materialize()
         return self._grouped_mm(x, weight, offs=offs)
+
+    def _cast_weight(self, weight_attr: str, out_dtype: torch.dtype):
+        weight = getattr(self, weight_attr)
+        return weight.to(out_dtype) if isinstance(weight, torch.Tensor) else weight
 
     def _grouped_mm(self, mat_a, mat_b, *, offs=None, lowp: bool = True):
         return expert_gemm(mat_a, mat_b, offs=offs, quant_format=self._lowp_quant_format if lowp else None,
@@ -361,6 +385,8 @@ class EPMoELayerBase(nn.Module, ABC):
         MFMA (quantised weights with ``_lowp_fp8_activations``); None otherwise."""
         down = getattr(self, "down_proj", None)
         combine = self._fused_glu_mul
+        if self._adapted("down_proj"):  # the adapter products take the bf16 rows
+            return None
         if not (self._lowp_fp8_activations and self.fuse_glu_quantise and isinstance(down, BlockFp8Weight)
                 and isinstance(combine, GluCombine) and isinstance(gate_up, torch.Tensor)
                 and fp8_mfma_usable(down.shape[1], down.shape[2])):
@@ -454,6 +480,7 @@ class EPMoELayerBase(nn.Module, ABC):
             # a BlockFp8Weight (quantised serving weights) is held as it is
             setattr(self, name, nn.Parameter(tensor) if isinstance(tensor, torch.Tensor) else tensor)
         self._fused_glu_mul = GluCombine.silu()
+        init_expert_lora(self, ep_config.expert_lora)
         return self
 
 

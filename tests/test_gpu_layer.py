@@ -380,3 +380,104 @@ def test_shared_expert_added_in_the_combine_kernel(device, cfg, gated):
     _check("out with shared expert", out_b, want.detach(), check_tol)
     _check("grad x with shared expert", gx_b, xs.grad, check_tol)
     _check("grad shared down_proj", grads_b["shared_expert.down_proj.weight"], shared["down_proj"].grad, check_tol)
+
+
+# ------------------------------------------------------------------------------------------------- expert LoRA
+
+@pytest.mark.parametrize("cfg", (CONFIG2_SMALL, CONFIG4_SMALL), ids=lambda c: c.name)
+def test_expert_lora_equals_the_layer_with_merged_weights(device, cfg):
+    """``x @ W + s (x @ A) @ B`` is ``x @ (W + s A B)``: the oracle runs the fp32 loop over the merged weights (the
+    adapters as its leaves, so their gradients come out of the same graph), the layer runs the three grouped products.
+    The base weights are frozen, the adapters' initial delta is zero, and ``disable_expert_adapters`` gives the base
+    layer back."""
+    from halo_amd.kernels.router import SOFTMAX_ALL, SOFTMAX_TOPK, fused_topk_gate
+    from halo_amd.moe_layer import ExpertLoraSpec, disable_expert_adapters, expert_lora_delta
+    from halo_amd.moe_layer.config import EPConfig
+    from oracle import moe_layer as oracle
+    from oracle import router as router_oracle
+
+    inputs = make_layer_inputs(cfg)
+    base = _build_layer(cfg, inputs, device)
+    spec = ExpertLoraSpec(r=16, alpha=32.0)
+    # the same construction with adapters asked for
+    from halo_amd.moe_layer import EPGptOssMoELayer, EPQwen3_5MoELayer, EPQwen3MoELayer
+    params = {k: v.to(device) for k, v in inputs["params"].items()}
+    ep = EPConfig(expert_lora=spec)
+    if cfg.router == "softmax_topk":
+        params = {k.replace("gate_proj", "gate_proj_gmm").replace("up_proj", "up_proj_gmm"): v for k, v in params.items()}
+        layer = EPGptOssMoELayer.from_weights(router_weight=inputs["router_weight"].to(device), top_k=cfg.top_k,
+                                              router_bias=inputs.get("router_bias", torch.zeros(cfg.experts)).to(device),
+                                              ep_config=ep, **params)
+    else:
+        cls = EPQwen3_5MoELayer if cfg.fused else EPQwen3MoELayer
+        layer = cls.from_weights(router_weight=inputs["router_weight"].to(device), top_k=cfg.top_k, ep_config=ep, **params)
+    assert layer.has_expert_lora and len(layer.expert_lora_named_params()) == 2 * len(layer._expert_lora_attrs)
+    for attr in layer._expert_lora_attrs:
+        assert not getattr(layer, attr).requires_grad and getattr(layer, attr + "_lora_A").requires_grad
+        assert not getattr(layer, attr + "_lora_B").any()
+    x = inputs["x"].to(device)
+
+    def run(module, inp):
+        result = module(inp)
+        return result[0] if isinstance(result, tuple) else result
+
+    with torch.no_grad():
+        start = run(layer, x)
+        assert torch.equal(start, run(base, x))  # B = 0: the delta is an exact zero
+        g = torch.Generator().manual_seed(5)
+        for attr in layer._expert_lora_attrs:  # a delta comparable to the weights themselves
+            b = getattr(layer, attr + "_lora_B")
+            b.copy_((torch.randn(b.shape, generator=g) * 0.05).to(b.dtype))
+        assert not torch.equal(run(layer, x), start)
+        holder = torch.nn.Sequential(layer)
+        with disable_expert_adapters(holder):
+            assert torch.equal(run(layer, x), start)
+
+    xd = x.clone().requires_grad_(True)
+    out = run(layer, xd)
+    out.backward(inputs["grad_out"].to(device))
+
+    with torch.no_grad():
+        logits = layer._linear_router_logits(x)
+        mode = SOFTMAX_TOPK if cfg.router == "softmax_topk" else SOFTMAX_ALL
+        idx, _ = fused_topk_gate(logits, cfg.top_k, mode=mode, normalize=True, eps=0.0)
+    f = lambda t: t.detach().float().cpu().requires_grad_(True)
+    xr, wr = f(inputs["x"]), f(inputs["router_weight"])
+    leaves, merged = {}, {}
+    for name, value in inputs["params"].items():
+        attr = name.replace("gate_proj", "gate_proj_gmm").replace("up_proj", "up_proj_gmm") \
+            if cfg.router == "softmax_topk" else name
+        if attr in layer._expert_lora_attrs:
+            a, b = f(getattr(layer, attr + "_lora_A")), f(getattr(layer, attr + "_lora_B"))
+            leaves[attr + "_lora_A"], leaves[attr + "_lora_B"] = a, b
+            merged[name] = value.float() + expert_lora_delta(a, b, spec.scaling)
+        else:
+            merged[name] = value.float()
+    bias = inputs["router_bias"].float() if "router_bias" in inputs else None
+    glu = oracle.Glu("gptoss", 1.702, 7.0) if cfg.glu == "gptoss" else oracle.Glu(cfg.glu)
+    ref_mode = router_oracle.SOFTMAX_TOPK if cfg.router == "softmax_topk" else router_oracle.SOFTMAX_ALL
+    want, _, _, _ = oracle.moe_layer_forward(xr, wr, merged, glu, cfg.top_k, router_bias=bias, mode=ref_mode,
+                                             normalize=True, eps=0.0, indices=idx.cpu())
+    want.backward(inputs["grad_out"].float())
+    _check("out", out, want.detach(), 2e-2)
+    _check("grad x", xd.grad, xr.grad, 2e-2)
+    for name, leaf in leaves.items():
+        _check(f"grad {name}", getattr(layer, name).grad, leaf.grad, 2e-2)
+    for attr in layer._expert_lora_attrs:
+        assert getattr(layer, attr).grad is None
+
+
+def test_expert_lora_rank_must_span_whole_rows(device):
+    from halo_amd.moe_layer import EPQwen3_5MoELayer, ExpertLoraSpec
+    from halo_amd.moe_layer.config import EPConfig
+
+    w1 = torch.zeros(4, 64, 128, dtype=torch.bfloat16, device=device)
+    w2 = torch.zeros(4, 64, 64, dtype=torch.bfloat16, device=device)
+    with pytest.raises(ValueError, match="use a multiple of 8"):
+        EPQwen3_5MoELayer.from_weights(router_weight=None, top_k=2, ep_config=EPConfig(expert_lora=ExpertLoraSpec(12, 24.0)),
+                                       gate_up_proj=w1, down_proj=w2)
+    only_down = EPQwen3_5MoELayer.from_weights(
+        router_weight=None, top_k=2, gate_up_proj=w1, down_proj=w2,
+        ep_config=EPConfig(expert_lora=ExpertLoraSpec(8, 16.0, projections=frozenset({"down"}), use_rslora=True)))
+    assert only_down._expert_lora_attrs == frozenset({"down_proj"}) and only_down.gate_up_proj.requires_grad
+    assert abs(only_down.expert_lora_scaling - 16.0 / 8 ** 0.5) < 1e-12
