@@ -5,6 +5,8 @@
 // (:17-41), _weighted_unpermute_bwd_kernel (:44-72) and MoEExpertBiasGather.backward's one-hot GEMM (:202-208).
 #include "common.h"
 
+#include <type_traits>
+
 namespace hmoe {
 namespace {
 
@@ -86,8 +88,8 @@ gather_rows_kernel(const T* __restrict__ src, int64_t src_stride, const int64_t*
 // nothing.  One wavefront per output row.  kTopK > 0 fixes top_k at compile time: the row's slots and weights are
 // read once, and for every 16-byte column chunk the kTopK row loads are issued together before the first is used, so
 // a lane keeps kTopK loads in flight instead of one (with one in flight the kernel reached half of the HBM rate).  An
-// invalid slot loads row 0 and contributes +0.0f, which leaves the fp32 sum exactly as skipping it does: the
-// accumulator starts at +0.0f and a sum that started there is never -0.0f.
+// invalid slot contributes +0.0f, which leaves the fp32 sum exactly as skipping it does: the accumulator starts at
+// +0.0f and a sum that started there is never -0.0f.
 template <typename T, int W, bool kWeighted, int kTopK>
 __global__ void __launch_bounds__(kThreads)
 gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, const int64_t* __restrict__ inv_map,
@@ -125,24 +127,44 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
       w[k] = 1.f;
       if constexpr (kWeighted) w[k] = Elem<T>::load(weight + (valid[k] ? j : 0));
     }
-    for (int64_t c = static_cast<int64_t>(lane_id()) * W; c < hidden; c += step) {
-      Pack<T, W> x[kTopK], acc, extra_chunk;
+    // Two forms of the loop, chosen once per row (the slots are the same for the whole wavefront).  All slots valid:
+    // the kTopK fetches go out back to back with nothing between them.  Otherwise an invalid slot is not fetched:
+    // on one GPU's share of an expert-parallel layer most of a token's slots belong to other ranks, and eight
+    // fetches of which seven are row 0 again cost seven times the useful traffic between the L2 and the CU.  (The
+    // branches of the second form keep the compiler from batching the fetches, which costs the first 20 %.)
+    bool all_valid = true;
 #pragma unroll
-      for (int k = 0; k < kTopK; ++k) x[k].load(from[k] + c);
-      if (extra) extra_chunk.load(extra + c);
+    for (int k = 0; k < kTopK; ++k) all_valid = all_valid && valid[k];
+    auto reduce_row = [&](auto dense_tag) __attribute__((always_inline)) {
+      constexpr bool kDense = decltype(dense_tag)::value;
+      for (int64_t c = static_cast<int64_t>(lane_id()) * W; c < hidden; c += step) {
+        Pack<T, W> x[kTopK], acc, extra_chunk;
 #pragma unroll
-      for (int i = 0; i < W; ++i) acc.v[i] = 0.f;
+        for (int k = 0; k < kTopK; ++k) {
+          if (kDense || valid[k]) {
+            x[k].load(from[k] + c);
+          } else {
 #pragma unroll
-      for (int k = 0; k < kTopK; ++k) {
-#pragma unroll
-        for (int i = 0; i < W; ++i) {
-          const float term = kWeighted ? x[k].v[i] * w[k] : x[k].v[i];
-          acc.v[i] += valid[k] ? term : 0.f;
+            for (int i = 0; i < W; ++i) x[k].v[i] = 0.f;
+          }
         }
+        if (extra) extra_chunk.load(extra + c);
+#pragma unroll
+        for (int i = 0; i < W; ++i) acc.v[i] = 0.f;
+#pragma unroll
+        for (int k = 0; k < kTopK; ++k) {
+#pragma unroll
+          for (int i = 0; i < W; ++i) {
+            const float term = kWeighted ? x[k].v[i] * w[k] : x[k].v[i];
+            acc.v[i] += (kDense || valid[k]) ? term : 0.f;
+          }
+        }
+        finish(acc, extra_chunk);
+        acc.store(to + c);
       }
-      finish(acc, extra_chunk);
-      acc.store(to + c);
-    }
+    };
+    if (all_valid) reduce_row(std::true_type{});
+    else reduce_row(std::false_type{});
   } else {
     for (int64_t c = static_cast<int64_t>(lane_id()) * W; c < hidden; c += step) {
       Pack<T, W> acc, extra_chunk;
