@@ -27,6 +27,20 @@ struct Pack {
       for (int i = 0; i < W; ++i) v[i] = t.v[i];
     }
   }
+  // the same load with the non-temporal hint: for rows that are read once and never again
+  __device__ __forceinline__ void load_once(const T* p) {
+    if constexpr (W == 8 && sizeof(T) == 2) {
+      typedef unsigned int word4 __attribute__((ext_vector_type(4)));
+      const word4 t = __builtin_nontemporal_load(reinterpret_cast<const word4*>(p));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(t[i] << 16);
+        v[2 * i + 1] = __uint_as_float(t[i] & 0xffff0000u);
+      }
+    } else {
+      load(p);
+    }
+  }
   __device__ __forceinline__ void store(T* p) const {
     if constexpr (W == 1) {
       Elem<T>::store(p, v[0]);
@@ -142,7 +156,7 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
 #pragma unroll
         for (int k = 0; k < kTopK; ++k) {
           if (kDense || valid[k]) {
-            x[k].load(from[k] + c);
+            x[k].load_once(from[k] + c);
           } else {
 #pragma unroll
             for (int i = 0; i < W; ++i) x[k].v[i] = 0.f;
