@@ -170,7 +170,7 @@ __device__ __forceinline__ void lds_load16(u32x4 rsrc, lds_bytes_ptr lds_base, u
                :
                : "s"(uniform(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_base)))), "v"(voffset),
                  "s"(uniform(rsrc)), "s"(uniform(soffset))
-               : "memory");
+               : "memory", "m0");
 }
 
 // Eight bf16 values plus eight more, each sum rounded to bf16: what a bf16 tensor addition does element by element.
@@ -1310,7 +1310,7 @@ __device__ __forceinline__ void lds_load4(u32x4 rsrc, lds_bytes_ptr lds_base, ui
                :
                : "s"(uniform(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_base)))), "v"(voffset),
                  "s"(uniform(rsrc)), "s"(uniform(soffset))
-               : "memory");
+               : "memory", "m0");
 }
 // one byte per lane, which lands zero-extended in the lane's dword
 __device__ __forceinline__ void lds_load1(u32x4 rsrc, lds_bytes_ptr lds_base, uint32_t voffset, uint32_t soffset) {
@@ -1318,7 +1318,7 @@ __device__ __forceinline__ void lds_load1(u32x4 rsrc, lds_bytes_ptr lds_base, ui
                :
                : "s"(uniform(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_base)))), "v"(voffset),
                  "s"(uniform(rsrc)), "s"(uniform(soffset))
-               : "memory");
+               : "memory", "m0");
 }
 
 __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
