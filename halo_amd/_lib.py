@@ -25,6 +25,7 @@ SIGNATURES = {
     "hmoe_status_string": (c_char_p, [I]),
     "hmoe_route_sort_workspace_bytes": (L, [L, I, I]),
     "hmoe_route_sort": (I, [P, I, P, I, L, I, I, L, P, P, P, P, P, P, P, P, P]),
+    "hmoe_route_sort_static": (I, [P, I, P, I, L, I, I, L, P, P, P, P, P, P, P, P]),
     "hmoe_route_sort_bwd": (I, [P, P, L, L, I, P, P]),
     "hmoe_bincount": (I, [P, P, L, I, I, P, P]),
     "hmoe_gather_rows": (I, [P, L, P, L, L, I, P, P]),

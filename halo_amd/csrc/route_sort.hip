@@ -12,8 +12,41 @@
 // is stable and bit-reproducible.
 #include "common.h"
 
+#include <atomic>
+
 namespace hmoe {
 namespace {
+
+// Scratch of hmoe_route_sort_static: the per-block histogram / start table of the sort, held by the library instead of
+// a caller's workspace.  Each GPU the library runs on holds its own copy until the process ends.  In host code the
+// array's name is only a handle: its device address comes from hipGetSymbolAddress (static_scratch below).
+constexpr int64_t kStaticScratchInts = int64_t(1) << 20;  // 4 MiB: n_blocks * num_local_experts entries at most
+// (`used`: no kernel names the array, the sort's kernels take its address as an argument)
+static __device__ __align__(256) __attribute__((used)) int32_t scratch[kStaticScratchInts];
+
+constexpr int kMaxDevices = 64;
+std::atomic<int32_t*> g_scratch_address[kMaxDevices];  // per device, resolved on the first call with that device current
+
+// The address of the current device's copy of `scratch`, or null with `status` set.
+int32_t* static_scratch(int& status) {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+    status = HMOE_UNSUPPORTED;
+    return nullptr;
+  }
+  int32_t* address = g_scratch_address[device].load(std::memory_order_acquire);
+  if (address == nullptr) {
+    void* resolved = nullptr;
+    if (hipGetSymbolAddress(&resolved, HIP_SYMBOL(scratch)) != hipSuccess || resolved == nullptr) {
+      status = HMOE_LAUNCH_FAILED;
+      return nullptr;
+    }
+    address = static_cast<int32_t*>(resolved);
+    g_scratch_address[device].store(address, std::memory_order_release);  // two first callers resolve the same value
+  }
+  status = HMOE_OK;
+  return address;
+}
 
 constexpr int kBlockSlots = 1024;   // slots per sort block (whole rows)
 constexpr int kPlaceThreads = 256;  // 4 wavefronts
@@ -264,6 +297,26 @@ int hmoe_route_sort(const void* experts, int experts_elem_bytes, const void* wei
   }
 #undef HMOE_SORT
   return HMOE_UNSUPPORTED;
+}
+
+int hmoe_route_sort_static(const void* experts, int experts_elem_bytes, const void* weights, int weight_elem_bytes,
+                           int64_t n_rows, int top_k, int num_local_experts, int64_t n_valid,
+                           int64_t* sorted_token_idx, void* sorted_weights, void* sorted_expert_ids, int32_t* offs,
+                           int64_t* inv_map, int32_t* dest, int32_t* ok, void* stream) {
+  using namespace hmoe;
+  if (n_rows < 0 || top_k <= 0 || num_local_experts <= 0 || n_valid < 0) return HMOE_INVALID_ARGUMENT;
+  const int64_t needed = hmoe_route_sort_workspace_bytes(n_rows, top_k, num_local_experts);
+  if (needed < 0) return HMOE_INVALID_ARGUMENT;
+  // the table must fit the library's array: refused, never truncated
+  if (needed > kStaticScratchInts * static_cast<int64_t>(sizeof(int32_t))) return HMOE_UNSUPPORTED;
+  int status = HMOE_OK;
+  int32_t* table = static_scratch(status);
+  if (table == nullptr) return status;
+  // Every entry the scan and the placement read is written by this call's histogram launch first (each sort block
+  // writes its whole row of the table), so what the previous call left in the array is never seen.
+  return hmoe_route_sort(experts, experts_elem_bytes, weights, weight_elem_bytes, n_rows, top_k, num_local_experts,
+                         n_valid, sorted_token_idx, sorted_weights, sorted_expert_ids, offs, inv_map, dest, ok, table,
+                         stream);
 }
 
 int hmoe_route_sort_bwd(const void* grad_sorted, const int32_t* dest, int64_t n_slots, int64_t n_valid,

@@ -11,7 +11,8 @@
  *   - `stream` is a hipStream_t passed as void*; all work is enqueued on it;
  *   - row strides are in elements; `dtype` is an hmoe_dtype;
  *   - return value: 0 on success, a negative hmoe_status otherwise (hmoe_status_string names it);
- *   - re-entrant: no mutable global state, safe to call from autograd's backward thread.
+ *   - re-entrant: no mutable global state, safe to call from autograd's backward thread (the one exception,
+ *     hmoe_route_sort_static, says so where it is declared).
  */
 #ifndef HALO_MOE_H
 #define HALO_MOE_H
@@ -59,6 +60,19 @@ int hmoe_route_sort(const void* experts, int experts_elem_bytes, const void* wei
                     int64_t n_rows, int top_k, int num_local_experts, int64_t n_valid, int64_t* sorted_token_idx,
                     void* sorted_weights, void* sorted_expert_ids, int32_t* offs, int64_t* inv_map, int32_t* dest,
                     int32_t* ok, void* workspace, void* stream);
+
+/* hmoe_route_sort without a workspace argument and without any allocation.  No counterpart in the reference: it is
+ * for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  Same arguments, outputs, launches and bits as hmoe_route_sort; the histogram / start table lives
+ * in a 4 MiB device array inside the library (one copy per GPU, held until the process ends), whose address is looked
+ * up once per device on the first call made with that device current.  A routing whose table does not fit
+ * (hmoe_route_sort_workspace_bytes(...) > 4 MiB, i.e. sort blocks x local experts > 2^20) returns HMOE_UNSUPPORTED.
+ * Calls that overlap on one GPU (two streams, two threads) share the array and race: serialise them per GPU.  Nothing
+ * in the array needs clearing between calls: every entry read is written by the same call first. */
+int hmoe_route_sort_static(const void* experts, int experts_elem_bytes, const void* weights, int weight_elem_bytes,
+                           int64_t n_rows, int top_k, int num_local_experts, int64_t n_valid,
+                           int64_t* sorted_token_idx, void* sorted_weights, void* sorted_expert_ids, int32_t* offs,
+                           int64_t* inv_map, int32_t* dest, int32_t* ok, void* stream);
 
 /* Replaces _CountingSort.backward: halo/kernels/moe_route_sort.py:181-189.
  * grad_weights[slot] = dest[slot] < n_valid ? grad_sorted[dest[slot]] : 0. */
