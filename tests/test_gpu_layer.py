@@ -225,6 +225,54 @@ def test_quantised_weight_forward(device):
     assert torch.equal(two_step, fp8)
 
 
+def test_quantised_weight_layer_against_the_cpu_loop_over_oracle_dequantised_weights(device):
+    """BASELINE config 5, scaled down, against the oracle end to end: the oracle quantises the fp32 weights
+    (numpy, ``oracle.block_fp8``), dequantises them, and runs the fp32 per-expert loop over them; the layer quantises
+    the same weights with the HIP quantiser and runs its W8A16 forward.  Bit-equal codes and scales first, then the
+    output within the bf16 tolerance; with quantised activations within the band stated for that route."""
+    import numpy as np
+
+    from halo_amd.kernels.expert_gemm import BlockFp8Weight
+    from halo_amd.kernels.lowp.block_fp8 import quantize_block_fp8
+    from halo_amd.moe_layer import EPConfig, EPQwen3_5MoELayer
+    from oracle import block_fp8 as fp8_oracle
+    from oracle import moe_layer as oracle
+
+    g = torch.Generator().manual_seed(4)
+    local, top_k, hidden, ffn, rows = 8, 8, 384, 256, 900
+    picks = torch.rand(rows, local * 8, generator=g).argsort(dim=1)[:, :top_k]
+    experts = torch.where(picks < local, picks, -1)
+    experts = experts[(experts >= 0).any(dim=1)]
+    counts = tuple(torch.bincount(experts[experts >= 0], minlength=local).tolist())
+    weights = torch.rand(experts.shape, generator=g)
+    x = torch.randn(experts.shape[0], hidden, generator=g).bfloat16()
+    w1 = torch.randn(local, hidden, 2 * ffn, generator=g) * 0.02
+    w2 = torch.randn(local, ffn, hidden, generator=g) * 0.02
+    device_q, oracle_params = {}, {}
+    for name, w in (("gate_up_proj", w1), ("down_proj", w2)):
+        q, scale = quantize_block_fp8(w.to(device))
+        want_q, want_scale = fp8_oracle.quantize_block_fp8(w.numpy())
+        assert np.array_equal(q.view(torch.uint8).cpu().numpy(), want_q), name
+        assert np.array_equal(scale.cpu().numpy(), want_scale), name
+        device_q[name] = BlockFp8Weight(q, scale)
+        # the reference's dequantised-bf16 path: q * scale in fp32, rounded once to bf16 (exact here)
+        oracle_params[name] = torch.from_numpy(fp8_oracle.dequantize_block_fp8(want_q, want_scale)).bfloat16().float()
+    layer = EPQwen3_5MoELayer.from_weights(router_weight=None, top_k=top_k, ep_config=EPConfig(ep_size=8, ep_rank=0),
+                                           **device_q)
+    want = oracle.compute_experts_loop(x.float(), experts, weights.bfloat16().float(), oracle_params, oracle.Glu(),
+                                       local)
+    with torch.no_grad():
+        got = layer._compute_experts(x.to(device), experts.to(device), weights.to(device), torch.bfloat16,
+                                     recv_counts=counts)
+        _check("W8A16 layer", got, want, 2e-2)
+        layer._lowp_fp8_activations = True
+        fp8 = layer._compute_experts(x.to(device), experts.to(device), weights.to(device), torch.bfloat16,
+                                     recv_counts=counts)
+    rel = ((fp8.double().cpu() - want.double()).norm() / want.double().norm()).item()
+    assert 0.005 < rel < 0.07, rel
+    assert cosine(fp8, want) > 0.997
+
+
 # ------------------------------------------------------------------------------ drop-ins for the Hugging Face blocks
 
 def _hf_config(model_type, **kw):
