@@ -36,6 +36,8 @@ SIGNATURES = {
     "hmoe_expert_colsum": (I, [P, P, L, L, I, I, P, P, P]),
     "hmoe_glu_fwd": (I, [P, P, L, L, L, L, I, I, F, F, I, I, P, P]),
     "hmoe_glu_bwd": (I, [P, P, L, L, P, L, L, I, I, F, F, I, I, P, P, L, L, P]),
+    "hmoe_glu_fwd_weighted": (I, [P, P, L, L, P, L, L, I, I, F, F, I, I, P, P]),
+    "hmoe_glu_bwd_weighted": (I, [P, P, L, L, P, P, L, L, I, I, F, F, I, I, P, P, L, L, P, P]),
     "hmoe_router_topk_fwd": (I, [P, I, L, I, I, I, I, F, P, P, P]),
     "hmoe_router_topk_bwd": (I, [P, I, P, P, L, I, I, I, I, F, P, P]),
     "hmoe_grouped_gemm_fwd": (I, [P, L, P, P, L, I, L, L, I, P, L, P]),
@@ -44,6 +46,8 @@ SIGNATURES = {
     "hmoe_grouped_gemm_wgrad": (I, [P, L, P, L, P, L, I, L, L, I, P, P]),
     "hmoe_grouped_gemm_fwd_gather": (I, [P, L, L, P, P, P, L, I, L, L, I, P, L, P]),
     "hmoe_grouped_gemm_wgrad_gather": (I, [P, L, L, P, P, L, P, L, I, L, L, I, P, P]),
+    "hmoe_grouped_gemm_dgrad_gather": (I, [P, L, L, P, P, P, L, I, L, L, I, P, L, P]),
+    "hmoe_grouped_gemm_wgrad_gather_grad": (I, [P, L, P, L, L, P, P, L, I, L, L, I, P, P]),
     "hmoe_quantize_block_fp8": (I, [P, I, L, L, L, P, P, P]),
     "hmoe_dequantize_block_fp8": (I, [P, P, L, L, L, I, P, P]),
     "hmoe_grouped_gemm_fwd_fp8w": (I, [P, L, P, P, P, L, I, L, L, P, L, P]),

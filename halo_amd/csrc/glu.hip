@@ -152,6 +152,63 @@ glu_bwd_kernel(const T* __restrict__ gate, const T* __restrict__ up, const T* __
   du.store(dup + row * stride_dup + col);
 }
 
+// The combine with the row's gate weight folded in: out[r] = round(w[r] * glu(gate[r], up[r])), the product taken in
+// fp32, so the down projection runs on weighted rows and the combine behind it is a plain sum.
+template <typename T, int W, int kAct, bool kClampAct, bool kPlusOne>
+__global__ void __launch_bounds__(kThreads)
+glu_fwd_weighted_kernel(const T* __restrict__ gate, const T* __restrict__ up, const T* __restrict__ row_weight,
+                        T* __restrict__ out, int64_t stride_gate, int64_t stride_up, int64_t n_rows,
+                        int64_t chunks_per_row, int64_t width, GluParams p) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t row = i / chunks_per_row;
+  if (row >= n_rows) return;
+  const int64_t col = (i - row * chunks_per_row) * W;
+  const float w = Elem<T>::load(row_weight + row);
+  Chunk<T, W> g, u, o;
+  g.load(gate + row * stride_gate + col);
+  u.load(up + row * stride_up + col);
+#pragma unroll
+  for (int k = 0; k < W; ++k) o.v[k] = w * glu_value<kAct, kClampAct, kPlusOne>(g.v[k], u.v[k], p);
+  o.store(out + row * width + col);
+}
+
+// Its gradient.  grad_out is the gradient of the weighted rows; with act = glu(gate, up) recomputed in fp32:
+//   (dgate, dup) = glu_grad(gate, up, w[r] * grad_out[r]),   grad_weight[r] = <grad_out[r], act[r]>.
+// kLanes lanes share a row (a power of two up to the wavefront), each taking every kLanes-th 16-byte chunk; the dot
+// product is summed in fp32 in a fixed order (per lane in chunk order, then a butterfly over the lanes) and stored as
+// fp32.
+template <typename T, int W, int kLanes, int kAct, bool kClampAct, bool kPlusOne>
+__global__ void __launch_bounds__(kThreads)
+glu_bwd_weighted_kernel(const T* __restrict__ gate, const T* __restrict__ up, const T* __restrict__ grad_out,
+                        const T* __restrict__ row_weight, T* __restrict__ dgate, T* __restrict__ dup,
+                        float* __restrict__ grad_weight, int64_t stride_gate, int64_t stride_up, int64_t stride_dgate,
+                        int64_t stride_dup, int64_t n_rows, int chunks_per_row, int64_t width, GluParams p) {
+  const int64_t thread = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t row = thread / kLanes;
+  const int sub = static_cast<int>(thread % kLanes);
+  float dot = 0.f;
+  if (row < n_rows) {
+    const float w = Elem<T>::load(row_weight + row);
+    for (int chunk = sub; chunk < chunks_per_row; chunk += kLanes) {
+      const int64_t col = static_cast<int64_t>(chunk) * W;
+      Chunk<T, W> g, u, d, dg, du;
+      g.load(gate + row * stride_gate + col);
+      u.load(up + row * stride_up + col);
+      d.load(grad_out + row * width + col);
+#pragma unroll
+      for (int k = 0; k < W; ++k) {
+        dot = fmaf(d.v[k], glu_value<kAct, kClampAct, kPlusOne>(g.v[k], u.v[k], p), dot);
+        glu_grad<kAct, kClampAct, kPlusOne>(g.v[k], u.v[k], w * d.v[k], p, dg.v[k], du.v[k]);
+      }
+      dg.store(dgate + row * stride_dgate + col);
+      du.store(dup + row * stride_dup + col);
+    }
+  }
+#pragma unroll
+  for (int off = kLanes / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off, HMOE_WAVE);
+  if (row < n_rows && sub == 0) grad_weight[row] = dot;
+}
+
 struct GluArgs {
   const void *gate, *up, *grad_out;
   void *out, *dgate, *dup;
@@ -162,6 +219,8 @@ struct GluArgs {
   uint8_t* q = nullptr;      // forward only: e4m3 panels and scale exponents instead of `out`
   uint8_t* scale = nullptr;
   int64_t out_rows = 0;
+  const void* row_weight = nullptr;  // the weighted forms: one gate weight per row, in the operands' dtype
+  float* grad_weight = nullptr;      // backward: its gradient, fp32 [n_rows]
 };
 
 template <typename T, int W, int kAct, bool kClampAct, bool kPlusOne>
@@ -174,6 +233,29 @@ void launch(const GluArgs& a) {
       glu_fwd_quant_kernel<kAct, kClampAct, kPlusOne><<<grid, block, 0, a.stream>>>(
           static_cast<const bf16_t*>(a.gate), static_cast<const bf16_t*>(a.up), a.q, a.scale, a.out_rows,
           a.stride_gate, a.stride_up, a.n_rows, chunks, a.p);
+  } else if (a.row_weight && !a.backward) {
+    glu_fwd_weighted_kernel<T, W, kAct, kClampAct, kPlusOne><<<grid, block, 0, a.stream>>>(
+        static_cast<const T*>(a.gate), static_cast<const T*>(a.up), static_cast<const T*>(a.row_weight),
+        static_cast<T*>(a.out), a.stride_gate, a.stride_up, a.n_rows, chunks, a.width, a.p);
+  } else if (a.row_weight) {
+    // lanes per row: the power of two (16, 32 or 64) that leaves the fewest idle lane-iterations, larger on a tie
+    int lanes = 64;
+    int64_t waste = (chunks + 63) / 64 * 64 - chunks;
+    for (int cand : {32, 16}) {
+      const int64_t w = (chunks + cand - 1) / cand * cand - chunks;
+      if (w < waste) lanes = cand, waste = w;
+    }
+    const int64_t threads = a.n_rows * lanes;
+    const dim3 row_grid(static_cast<unsigned>((threads + kThreads - 1) / kThreads));
+#define HMOE_GLU_BWD_W(L)                                                                                        \
+  glu_bwd_weighted_kernel<T, W, L, kAct, kClampAct, kPlusOne><<<row_grid, block, 0, a.stream>>>(                 \
+      static_cast<const T*>(a.gate), static_cast<const T*>(a.up), static_cast<const T*>(a.grad_out),             \
+      static_cast<const T*>(a.row_weight), static_cast<T*>(a.dgate), static_cast<T*>(a.dup), a.grad_weight,      \
+      a.stride_gate, a.stride_up, a.stride_dgate, a.stride_dup, a.n_rows, static_cast<int>(chunks), a.width, a.p)
+    if (lanes == 64) HMOE_GLU_BWD_W(64);
+    else if (lanes == 32) HMOE_GLU_BWD_W(32);
+    else HMOE_GLU_BWD_W(16);
+#undef HMOE_GLU_BWD_W
   } else if (!a.backward)
     glu_fwd_kernel<T, W, kAct, kClampAct, kPlusOne><<<grid, block, 0, a.stream>>>(
         static_cast<const T*>(a.gate), static_cast<const T*>(a.up), static_cast<T*>(a.out), a.stride_gate,
@@ -207,6 +289,8 @@ int run(const GluArgs& a, int dtype, int activation, int clamp_activated, int up
   if (!a.gate || !a.up) return HMOE_INVALID_ARGUMENT;
   if (a.backward ? (!a.grad_out || !a.dgate || !a.dup) : (a.q ? !a.scale : !a.out)) return HMOE_INVALID_ARGUMENT;
   if (a.n_rows * a.width / 1 >= (int64_t(1) << 40)) return HMOE_UNSUPPORTED;
+  if (a.row_weight && a.backward && !a.grad_weight) return HMOE_INVALID_ARGUMENT;
+  if (a.row_weight && a.n_rows >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
   const int64_t w = dtype == HMOE_BF16 ? 8 : 4;
   bool vec = a.width % w == 0 && a.stride_gate % w == 0 && a.stride_up % w == 0 && aligned16(a.gate) &&
              aligned16(a.up);
@@ -259,6 +343,35 @@ int hmoe_glu_fwd_quant_fp8(const void* gate, const void* up, int64_t stride_gate
   a.stream = static_cast<hipStream_t>(stream);
   if (n_rows > 0 && width > 0 && !q) return HMOE_INVALID_ARGUMENT;
   return hmoe::run(a, HMOE_BF16, activation, clamp_activated, up_plus_one);
+}
+
+int hmoe_glu_fwd_weighted(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up,
+                          const void* row_weight, int64_t n_rows, int64_t width, int dtype, int activation,
+                          float alpha, float limit, int clamp_activated, int up_plus_one, void* out, void* stream) {
+  hmoe::GluArgs a{};
+  a.gate = gate; a.up = up; a.out = out; a.row_weight = row_weight;
+  a.stride_gate = stride_gate; a.stride_up = stride_up; a.n_rows = n_rows; a.width = width;
+  a.p = {alpha, limit};
+  a.backward = false;
+  a.stream = static_cast<hipStream_t>(stream);
+  if (n_rows > 0 && width > 0 && !row_weight) return HMOE_INVALID_ARGUMENT;
+  return hmoe::run(a, dtype, activation, clamp_activated, up_plus_one);
+}
+
+int hmoe_glu_bwd_weighted(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up,
+                          const void* grad_out, const void* row_weight, int64_t n_rows, int64_t width, int dtype,
+                          int activation, float alpha, float limit, int clamp_activated, int up_plus_one, void* dgate,
+                          void* dup, int64_t stride_dgate, int64_t stride_dup, float* grad_weight, void* stream) {
+  hmoe::GluArgs a{};
+  a.gate = gate; a.up = up; a.grad_out = grad_out; a.dgate = dgate; a.dup = dup;
+  a.row_weight = row_weight; a.grad_weight = grad_weight;
+  a.stride_gate = stride_gate; a.stride_up = stride_up; a.stride_dgate = stride_dgate; a.stride_dup = stride_dup;
+  a.n_rows = n_rows; a.width = width;
+  a.p = {alpha, limit};
+  a.backward = true;
+  a.stream = static_cast<hipStream_t>(stream);
+  if (n_rows > 0 && width > 0 && (!row_weight || !grad_weight)) return HMOE_INVALID_ARGUMENT;
+  return hmoe::run(a, dtype, activation, clamp_activated, up_plus_one);
 }
 
 int hmoe_glu_bwd(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up, const void* grad_out,

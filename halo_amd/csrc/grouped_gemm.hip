@@ -39,10 +39,12 @@
 // round-robin over all workgroups, neighbouring tiles landed on different XCDs and every operand row was fetched from
 // HBM once per tile that uses it (4x the algorithmic bytes, measured).
 //
-// Gathered operand A (template parameter kGather; fwd and wgrad).  A may be given as (array, row index): logical row
-// r is array[index[r]], which folds the reference's permute by expert (halo/kernels/moe_permute.py:130-141) into the
-// first expert projection and its weight gradient.  The direct-to-LDS load takes a per-lane offset, so a gathered row
-// costs what a contiguous one does; see GatherDirect and GatherTransposed.
+// Gathered operand (template parameter kGather: 1 = A, 2 = wgrad's B).  The operand may be given as (array, row
+// index): logical row r is array[index[r]].  With A gathered in fwd and wgrad this folds the reference's permute by
+// expert (halo/kernels/moe_permute.py:130-141) into the first expert projection and its weight gradient; with the
+// output gradient gathered in dgrad (A) and wgrad (B) the down projection's two gradients read grad_out[token of row]
+// directly, so the combine's backward (moe_permute.py:44-72) writes no [R, H] gradient.  The direct-to-LDS load takes a
+// per-lane offset, so a gathered row costs what a contiguous one does; see GatherDirect and GatherTransposed.
 //
 // Weights in block-scaled fp8 (grouped_gemm_staged_kernel, forward only) take the register-staged variant of the same
 // tiling: global -> registers (dequantised there) -> LDS as [output index][64 contraction], both operands read back
@@ -98,8 +100,11 @@ struct GemmArgs {
   int groups;
   int64_t k, n;
   const float* b_scale;  // kFwdFp8W: [G, ceil(K/128), ceil(N/128)]
-  const int64_t* a_index = nullptr;  // gathered A (fwd, wgrad): logical row r of A is a[a_index[r]]
+  // one operand given as (array, row index): logical row r of it is array[a_index[r]].  A in fwd, dgrad and wgrad;
+  // with gather_b, wgrad's B (the output gradient) instead
+  const int64_t* a_index = nullptr;
   int64_t a_rows = 0;                // rows of the array a_index points into
+  bool gather_b = false;
   const void* bias = nullptr;        // fwd: [G, N] in the operands' dtype, added to group g's output rows
   // kFwdFp8: both operands are e4m3 bytes in panels of 64 contraction values (A [K/64][a_scale_rows][64],
   // B [G][K/64][N][64]); k counts values
@@ -982,11 +987,12 @@ __device__ __forceinline__ void interleave_reads_under_mfmas() {
   }
 }
 
-template <int kMode, typename Cfg, bool kGather = false, bool kBias = false>
+template <int kMode, typename Cfg, int kGather = 0, bool kBias = false>
 __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmArgs p) {
   static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
   static_assert(!kBias || kMode == kFwd, "the expert bias belongs to the forward product");
-  static_assert(!kGather || kMode == kFwd || kMode == kWgrad, "A is gathered in fwd and wgrad");
+  static_assert(kGather >= 0 && kGather <= 2 && (kGather != 2 || kMode == kWgrad), "B is gathered in wgrad only");
+  constexpr bool kGatherA = kGather == 1, kGatherB = kGather == 2;
   constexpr int WM = Cfg::WM, WN = Cfg::WN, BM = Cfg::BM, BN = Cfg::BN;
   constexpr int kWaves = Cfg::GM * Cfg::GN;
   // Wavefronts 0-3 issue all the tile loads and wait for them (16 loads of 1 KB each per step, measured slightly
@@ -996,9 +1002,11 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   constexpr bool kDirectA = kMode != kWgrad, kDirectB = kMode == kDgrad;
   using PlainA = typename std::conditional<kDirectA, SlimDirect<kI>, SlimTransposed<kI>>::type;
   using GatheredA = typename std::conditional<kDirectA, GatherDirect<kI>, GatherTransposed<kI>>::type;
-  using LoaderA = typename std::conditional<kGather, GatheredA, PlainA>::type;
-  using LoaderB = typename std::conditional<kDirectB, SlimDirect<kI>, SlimTransposed<kI>>::type;
-  constexpr bool kRowsPerStep = kGather && !kDirectA;  // the gathered rows are contraction rows: new ones every step
+  using LoaderA = typename std::conditional<kGatherA, GatheredA, PlainA>::type;
+  using PlainB = typename std::conditional<kDirectB, SlimDirect<kI>, SlimTransposed<kI>>::type;
+  using LoaderB = typename std::conditional<kGatherB, GatherTransposed<kI>, PlainB>::type;
+  // the gathered rows are contraction rows (wgrad): new ones every step
+  constexpr bool kRowsPerStep = (kGatherA && !kDirectA) || kGatherB;
   using Sched = TileSchedule<kMode, BM, BN>;
   extern __shared__ __attribute__((aligned(16))) char lds_raw[];  // two stages of (A tile, B tile), 32 KB each
   // tile_start: per group, the prefix of its row tiles (fwd, dgrad) or of its tiles' cost (wgrad: contraction steps
@@ -1048,7 +1056,8 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
 
   LoaderA la;
   LoaderB lb;
-  if constexpr (kRowsPerStep) la.rows_area = lds + 2 * kStageBytes + load_slot * 2048;
+  auto& lg = *[&]() { if constexpr (kGatherB) return &lb; else return &la; }();  // the gathered operand's loader
+  if constexpr (kRowsPerStep) lg.rows_area = lds + 2 * kStageBytes + load_slot * 2048;
   int cursor = 0;
   // describe tile `t`'s operands to the loaders and start its first step into stage 0
   // `rows0_loaded`: the gathered contraction rows of its step 0 were fetched during the previous tile's last step
@@ -1056,7 +1065,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     const bf16_t* a = static_cast<const bf16_t*>(p.a);
     const bf16_t* b = static_cast<const bf16_t*>(p.b);
     const int64_t rows = kMode == kWgrad ? tile.con_lim : tile.a_out_lim;
-    if constexpr (kGather) {
+    if constexpr (kGatherA) {
       if (load_wave)  // the row indices are fetched by the lanes that use them
         la.init(a, p.lda, p.a_rows, p.a_index + tile.row_start, tile.a_out0, tile.a_out_lim, tile.con_lim, load_slot,
                 lane);
@@ -1064,7 +1073,11 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim,
               load_slot, lane);
     }
-    if constexpr (kMode == kWgrad)
+    if constexpr (kGatherB) {
+      if (load_wave)
+        lb.init(b, p.ldb, p.a_rows, p.a_index + tile.row_start, tile.b_out0, tile.b_out_lim, tile.con_lim, load_slot,
+                lane);
+    } else if constexpr (kMode == kWgrad)
       lb.init(b + tile.row_start * p.ldb, p.ldb, rows * p.ldb * 2, tile.b_out0, tile.b_out_lim, tile.con_lim,
               load_slot, lane);
     else
@@ -1072,7 +1085,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     if (load_wave) {
       if constexpr (kRowsPerStep) {
         if (!rows0_loaded) {
-          la.load_rows(0, load_slot, lane);
+          lg.load_rows(0, load_slot, lane);
           wait_loads();
         }
       }
@@ -1080,7 +1093,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         la.issue(lds, 0, load_slot);
         lb.issue(lds + kTileBytes, 0, load_slot);
       }
-      if constexpr (kRowsPerStep) la.load_rows(1, load_slot, lane);
+      if constexpr (kRowsPerStep) lg.load_rows(1, load_slot, lane);
     }
   };
 
@@ -1188,9 +1201,9 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
           // the rows of the step after that: their indices arrive under this step, with its tile loads; in the
           // tile's last step that is the next tile's first
           if constexpr (kRowsPerStep) {
-            if (more) la.load_rows(step + 2, load_slot, lane);
+            if (more) lg.load_rows(step + 2, load_slot, lane);
             else if (has_next)
-              la.load_rows_of(make_rsrc_words(p.a_index + next.row_start, static_cast<uint32_t>(next.con_lim) * 8u),
+              lg.load_rows_of(make_rsrc_words(p.a_index + next.row_start, static_cast<uint32_t>(next.con_lim) * 8u),
                               next.con_lim, 0, load_slot, lane);
           }
         }
@@ -1282,9 +1295,11 @@ HMOE_BF16_INSTANCE(kFwd)
 HMOE_BF16_INSTANCE(kDgrad)
 HMOE_BF16_INSTANCE(kWgrad)
 #undef HMOE_BF16_INSTANCE
-template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, true>(GemmArgs);
-template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, false, true>(GemmArgs);
-template __global__ void grouped_gemm_bf16_kernel<kWgrad, Config<2, 4, 4, 2>, true>(GemmArgs);
+template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, 1>(GemmArgs);
+template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, 0, true>(GemmArgs);
+template __global__ void grouped_gemm_bf16_kernel<kDgrad, Config<2, 4, 4, 2>, 1>(GemmArgs);
+template __global__ void grouped_gemm_bf16_kernel<kWgrad, Config<2, 4, 4, 2>, 1>(GemmArgs);
+template __global__ void grouped_gemm_bf16_kernel<kWgrad, Config<2, 4, 4, 2>, 2>(GemmArgs);
 
 // ------------------------------------------------------------------------------------------------ fp32 path
 // 64x64 tile, contraction step 16, 256 threads each owning a 4x4 block.  grid.x walks row tiles of every group
@@ -1729,7 +1744,7 @@ int launch_staged(const GemmArgs& p, int workgroups_per_cu, hipStream_t stream) 
   return HMOE_OK;
 }
 
-template <int kMode, typename Cfg, bool kGather = false, bool kBias = false>
+template <int kMode, typename Cfg, int kGather = 0, bool kBias = false>
 int launch_direct(const GemmArgs& p, hipStream_t stream) {
   const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
   const int64_t nt = (out_cols + Cfg::BN - 1) / Cfg::BN;
@@ -1758,13 +1773,15 @@ int launch(const GemmArgs& p, int dtype, hipStream_t stream) {
     if constexpr (kMode == kFwdFp8W) {
       rc = launch_staged<kMode, Tile>(p, 1, stream);
     } else if constexpr (kMode == kFwd) {
-      rc = p.a_index ? launch_direct<kMode, Tile, true>(p, stream)
-           : p.bias  ? launch_direct<kMode, Tile, false, true>(p, stream)
+      rc = p.a_index ? launch_direct<kMode, Tile, 1>(p, stream)
+           : p.bias  ? launch_direct<kMode, Tile, 0, true>(p, stream)
                      : launch_direct<kMode, Tile>(p, stream);
     } else if constexpr (kMode == kWgrad) {
-      rc = p.a_index ? launch_direct<kMode, Tile, true>(p, stream) : launch_direct<kMode, Tile>(p, stream);
+      rc = !p.a_index ? launch_direct<kMode, Tile>(p, stream)
+           : p.gather_b ? launch_direct<kMode, Tile, 2>(p, stream)
+                        : launch_direct<kMode, Tile, 1>(p, stream);
     } else {
-      rc = launch_direct<kMode, Tile>(p, stream);
+      rc = p.a_index ? launch_direct<kMode, Tile, 1>(p, stream) : launch_direct<kMode, Tile>(p, stream);
     }
     if (rc) return rc;
   } else if constexpr (kMode != kFwdFp8W) {
@@ -1795,8 +1812,9 @@ int validate(const GemmArgs& p, int dtype) {
     // buffer loads address an operand with 32-bit byte offsets: all rows of an operand and one expert's weight
     // must each stay below 2 GiB
     const int64_t lim = int64_t(1) << 31;
-    const int64_t a_extent = (p.a_index ? p.a_rows : p.total_rows) * p.lda * 2;
-    if (a_extent >= lim || p.total_rows * p.ldb * 2 >= lim || p.total_rows * p.ldc * 2 >= lim || p.k * p.n * 2 >= lim)
+    const int64_t a_extent = (p.a_index && !p.gather_b ? p.a_rows : p.total_rows) * p.lda * 2;
+    const int64_t b_extent = (p.gather_b ? p.a_rows : p.total_rows) * p.ldb * 2;
+    if (a_extent >= lim || b_extent >= lim || p.total_rows * p.ldc * 2 >= lim || p.k * p.n * 2 >= lim)
       return HMOE_UNSUPPORTED;
   }
   return HMOE_OK;
@@ -1853,6 +1871,36 @@ int hmoe_grouped_gemm_wgrad_gather(const void* a, int64_t lda, int64_t a_rows, c
   if (dtype != HMOE_BF16) return HMOE_UNSUPPORTED;
   if (a_rows < 0) return HMOE_INVALID_ARGUMENT;
   GemmArgs p{a, lda, grad_out, ldg, grad_b, n, offs, total_rows, num_groups, k, n, nullptr, row_index, a_rows};
+  if (int rc = validate(p, dtype)) return rc;
+  if (k == 0 || n == 0) return HMOE_OK;
+  if (!grad_b || (total_rows > 0 && (!a || !grad_out || !row_index))) return HMOE_INVALID_ARGUMENT;
+  if (lda < k || ldg < n) return HMOE_INVALID_ARGUMENT;
+  return launch<kWgrad>(p, dtype, static_cast<hipStream_t>(stream));
+}
+
+int hmoe_grouped_gemm_dgrad_gather(const void* grad_out, int64_t ldg, int64_t grad_rows, const int64_t* row_index,
+                                   const void* b, const int32_t* offs, int64_t total_rows, int num_groups, int64_t k,
+                                   int64_t n, int dtype, void* grad_a, int64_t lda, void* stream) {
+  using namespace hmoe;
+  if (dtype != HMOE_BF16) return HMOE_UNSUPPORTED;
+  if (grad_rows < 0) return HMOE_INVALID_ARGUMENT;
+  GemmArgs p{grad_out, ldg, b, n, grad_a, lda, offs, total_rows, num_groups, k, n, nullptr, row_index, grad_rows};
+  if (int rc = validate(p, dtype)) return rc;
+  if (total_rows == 0 || k == 0) return HMOE_OK;
+  if (!grad_out || !b || !grad_a || !row_index) return HMOE_INVALID_ARGUMENT;
+  if (ldg < n || lda < k) return HMOE_INVALID_ARGUMENT;
+  return launch<kDgrad>(p, dtype, static_cast<hipStream_t>(stream));
+}
+
+int hmoe_grouped_gemm_wgrad_gather_grad(const void* a, int64_t lda, const void* grad_out, int64_t ldg,
+                                        int64_t grad_rows, const int64_t* row_index, const int32_t* offs,
+                                        int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype,
+                                        void* grad_b, void* stream) {
+  using namespace hmoe;
+  if (dtype != HMOE_BF16) return HMOE_UNSUPPORTED;
+  if (grad_rows < 0) return HMOE_INVALID_ARGUMENT;
+  GemmArgs p{a, lda, grad_out, ldg, grad_b, n, offs, total_rows, num_groups, k, n, nullptr, row_index, grad_rows};
+  p.gather_b = true;
   if (int rc = validate(p, dtype)) return rc;
   if (k == 0 || n == 0) return HMOE_OK;
   if (!grad_b || (total_rows > 0 && (!a || !grad_out || !row_index))) return HMOE_INVALID_ARGUMENT;

@@ -167,6 +167,52 @@ class _FusedPackedGLU(torch.autograd.Function):
         return grad.view(ctx.shape), None
 
 
+class _WeightedPackedGLU(torch.autograd.Function):
+    """``row_weight[:, None] * combine(gate, up)`` over the halves of a packed ``[R, 2 M]`` tensor, the product taken
+    in fp32 and rounded once: the MoE combine's gate weight applied ahead of the down projection instead of behind it
+    (``sum_k w_k (act_k @ W) = sum_k (w_k act_k) @ W``).  Backward returns the packed gradient and the weights'
+    gradient ``<grad_out[r], combine(gate, up)[r]>`` (fp32 sum, cast to the weights' dtype): what the reference's
+    weighted unpermute computes as ``<grad_out[token], expert_out[r]>`` (``moe_permute.py:44-72``), without the
+    expert outputs."""
+
+    @staticmethod
+    def forward(ctx, gate_up: torch.Tensor, row_weight: torch.Tensor, combine: "GluCombine") -> torch.Tensor:
+        device = _lib.require_device(gate_up, row_weight)
+        packed = _as_rows(gate_up)
+        rows, half = packed.shape[0], packed.shape[1] // 2
+        weight = row_weight.to(packed.dtype).contiguous()
+        ctx.combine, ctx.shape, ctx.weight_dtype = combine, gate_up.shape, row_weight.dtype
+        ctx.save_for_backward(packed, weight)
+        out = packed.new_empty((rows, half))
+        if rows and half:
+            gate, up = packed[:, :half], packed[:, half:]
+            with _lib.on_device(device):
+                _lib.call("hmoe_glu_fwd_weighted", _lib.ptr(gate), _lib.ptr(up), gate.stride(0), up.stride(0),
+                          _lib.ptr(weight), rows, half, _lib.dtype_id(packed.dtype), *_kernel_args(combine),
+                          _lib.ptr(out), _lib.stream_ptr(device))
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out: torch.Tensor):
+        packed, weight = ctx.saved_tensors
+        device = packed.device
+        rows, half = packed.shape[0], packed.shape[1] // 2
+        grad = torch.empty_like(packed, memory_format=torch.contiguous_format)
+        grad_weight = torch.empty(rows, dtype=torch.float32, device=device)
+        if rows and half:
+            grad_out = grad_out.contiguous().view(rows, half)
+            gate, up = packed[:, :half], packed[:, half:]
+            dgate, dup = grad[:, :half], grad[:, half:]
+            with _lib.on_device(device):
+                _lib.call("hmoe_glu_bwd_weighted", _lib.ptr(gate), _lib.ptr(up), gate.stride(0), up.stride(0),
+                          _lib.ptr(grad_out), _lib.ptr(weight), rows, half, _lib.dtype_id(packed.dtype),
+                          *_kernel_args(ctx.combine), _lib.ptr(dgate), _lib.ptr(dup), dgate.stride(0), dup.stride(0),
+                          _lib.ptr(grad_weight), _lib.stream_ptr(device))
+        else:
+            grad_weight.zero_()
+        return (grad.view(ctx.shape), grad_weight.to(ctx.weight_dtype) if ctx.needs_input_grad[1] else None, None)
+
+
 # ---------------------------------------------------------------------------------------------------- combine
 
 @dataclass(frozen=True)
@@ -217,6 +263,14 @@ class GluCombine:
             return _FusedPackedGLU.apply(gate_up, self)
         gate, up = gate_up.chunk(2, dim=-1)
         return self._eager(gate, up)
+
+    def packed_weighted(self, gate_up: torch.Tensor, row_weight: torch.Tensor) -> torch.Tensor:
+        """``row_weight[:, None] * packed(gate_up)`` with one rounding (:class:`_WeightedPackedGLU`); ``gate_up`` is
+        ``[R, 2 M]``, ``row_weight`` ``[R]``."""
+        if _FUSED_GLU_ENABLED:
+            return _WeightedPackedGLU.apply(gate_up, row_weight, self)
+        gate, up = gate_up.chunk(2, dim=-1)
+        return (self._eager(gate, up).float() * row_weight.float().unsqueeze(-1)).to(gate_up.dtype)
 
     def packed_quantized(self, gate_up: torch.Tensor):
         """``packed`` with its output as e4m3 panels and scale exponents for the fp8 expert GEMM

@@ -264,6 +264,86 @@ def gather_grouped_mm(tokens, row_index, inv_map, mat_b, *, offs):
     return _GatherGroupedMM.apply(tokens, row_index, inv_map, mat_b, offs)
 
 
+# ------------------------------------------------------------------------- down projection + plain combine
+
+def combine_fusable(mat_a: torch.Tensor, mat_b, hidden_dtype: torch.dtype) -> bool:
+    """Whether :func:`grouped_mm_combine` can take these operands: bf16 rows of 16-byte multiples on the device and a
+    plain contiguous ``[G, K, N]`` bf16 weight, the layer's output in bf16 as well."""
+    return (isinstance(mat_b, torch.Tensor) and isinstance(mat_a, torch.Tensor) and mat_a.is_cuda
+            and mat_a.dtype == torch.bfloat16 and mat_b.dtype == torch.bfloat16 and hidden_dtype == torch.bfloat16
+            and mat_b.dim() == 3 and mat_b.is_contiguous() and mat_a.dim() == 2 and mat_a.shape[1] == mat_b.shape[1]
+            and mat_b.shape[1] % 8 == 0 and mat_b.shape[2] % 8 == 0)
+
+
+class _GroupedMMCombine(Function):
+    """``out[t] = sum over the sorted rows j of token t of (mat_a @ mat_b)[j]  (+ scale[t] * addend[t])``: a grouped
+    product whose output rows are summed per token through ``inv_map`` without weights (``mat_a``'s rows already
+    carry the gate weights).  One autograd node, so the ``[R, N]`` product is not kept and its gradient never exists:
+    ``grad_a = grad_out[row_index] @ mat_b^T`` and ``grad_b = mat_a^T @ grad_out[row_index]`` fetch the token
+    gradient's rows through ``row_index`` (``hmoe_grouped_gemm_dgrad_gather`` / ``_wgrad_gather_grad``).  Replaces
+    the reference's ``grouped_mm`` (``grouped_mm.py:30-47``) + ``MoEWeightedUnpermute`` (``moe_permute.py:144-189``)
+    pair on the down projection; ``addend`` / ``scale`` as in ``MoEWeightedUnpermuteAdd``."""
+
+    @staticmethod
+    def forward(ctx, mat_a, mat_b, offs, row_index, inv_map, addend, scale):
+        from halo_amd.kernels.moe_permute import gather_reduce_rows
+
+        offs32 = _offs_arg(offs, mat_b.shape[0])
+        row_index = row_index.long().contiguous()
+        product = _forward(mat_a, mat_b, offs32)
+        ctx.scaled = scale is not None
+        ctx.scale_shape = scale.shape if ctx.scaled else None
+        ctx.tokens = inv_map.shape[0]
+        ctx.save_for_backward(mat_a, mat_b, offs32, row_index,
+                              addend if ctx.scaled and ctx.needs_input_grad[6] else None, scale)
+        return gather_reduce_rows(product, inv_map, None, addend=addend, addend_scale=scale)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from halo_amd.kernels.moe_permute import _unpermute_backward
+
+        mat_a, mat_b, offs32, row_index, addend, scale = ctx.saved_tensors
+        device = mat_a.device
+        groups, k, n = mat_b.shape
+        rows = mat_a.shape[0]
+        # under EP the gradient arrives as a row-strided view of the padded transport buffer, read in place
+        if grad_out.stride(-1) != 1 or grad_out.stride(0) % 8 or grad_out.data_ptr() % 16:
+            grad_out = grad_out.contiguous()
+        grad_a = grad_b = grad_addend = grad_scale = None
+        dtype = _lib.dtype_id(mat_a.dtype)
+        with _lib.on_device(device):
+            if ctx.needs_input_grad[0]:
+                grad_a = torch.empty((rows, k), dtype=mat_a.dtype, device=device)
+                if rows and k:
+                    _lib.call("hmoe_grouped_gemm_dgrad_gather", _lib.ptr(grad_out), grad_out.stride(0),
+                              grad_out.shape[0], _lib.ptr(row_index), _lib.ptr(mat_b), _lib.ptr(offs32), rows, groups,
+                              k, n, dtype, _lib.ptr(grad_a), grad_a.stride(0), _lib.stream_ptr(device))
+            if ctx.needs_input_grad[1]:
+                grad_b = torch.empty((groups, k, n), dtype=mat_a.dtype, device=device)
+                a = _rows(mat_a)
+                if k and n:
+                    _lib.call("hmoe_grouped_gemm_wgrad_gather_grad", _lib.ptr(a), a.stride(0) if rows else k,
+                              _lib.ptr(grad_out), grad_out.stride(0) if grad_out.shape[0] else n, grad_out.shape[0],
+                              _lib.ptr(row_index), _lib.ptr(offs32), rows, groups, k, n, dtype, _lib.ptr(grad_b),
+                              _lib.stream_ptr(device))
+        if not ctx.scaled:
+            grad_addend = grad_out if ctx.needs_input_grad[5] else None
+        elif ctx.needs_input_grad[5] or ctx.needs_input_grad[6]:
+            # every row its own token: scale[r] * grad_out[r] and <grad_out[r], addend[r]>
+            own = torch.arange(grad_out.shape[0], device=device)
+            want_scale = ctx.needs_input_grad[6]
+            grad_addend, grad_scale = _unpermute_backward(grad_out, addend, scale.reshape(-1), own, want_scale)
+            if want_scale:
+                grad_scale = grad_scale.to(scale.dtype).view(ctx.scale_shape)
+        return grad_a, grad_b, None, None, None, grad_addend, grad_scale
+
+
+def grouped_mm_combine(mat_a, mat_b, *, offs, row_index, inv_map, addend=None, scale=None):
+    """``gather_reduce_rows(grouped_mm(mat_a, mat_b, offs=offs), inv_map) (+ scale[:, None] * addend)``; see
+    :class:`_GroupedMMCombine`.  The caller checks :func:`combine_fusable` first."""
+    return _GroupedMMCombine.apply(mat_a, mat_b, offs, row_index, inv_map, addend, scale)
+
+
 class GatheredRows:
     """``tokens[row_index]`` that nobody has copied yet: what the sort hands to the first expert projection when that
     projection can fetch the rows itself (:func:`gather_grouped_mm`).  A consumer that cannot calls

@@ -22,7 +22,7 @@ import torch.nn as nn
 
 from halo_amd.kernels.expert_gemm import BlockFp8Weight, expert_gemm, fp8_mfma_usable
 from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled, resolve_fused_glu_mul
-from halo_amd.kernels.grouped_mm import GatheredRows, grouped_mm, grouped_wgrad
+from halo_amd.kernels.grouped_mm import GatheredRows, grouped_mm, grouped_mm_combine, grouped_wgrad
 from halo_amd.kernels.moe_permute import (MoEGatherPermute, MoEWeightedUnpermute, MoEWeightedUnpermuteAdd,
                                           warm_permute_kernels)
 from halo_amd.kernels.moe_route_sort import sort_routing_by_expert, warm_route_sort_kernels
@@ -183,6 +183,9 @@ class EPMoELayerBase(nn.Module, ABC):
         self.fuse_permute_into_gemm = True
         # the shared expert's output joins the routed one in the combine kernel instead of a tensor addition
         self.fuse_shared_into_combine = True
+        # the gate weights multiply the GLU's output instead of the down projection's: the combine becomes a plain
+        # sum and its backward writes no [R, H] gradient (see _compute_experts_weight_folded)
+        self.fold_gate_weight_into_glu = True
         self._fused_glu_mul: Callable | None = None
         # labels the dispatch / expert-compute / combine spans at no device cost (swappable, as in the reference)
         self._perf = torch.profiler.record_function
@@ -288,6 +291,9 @@ class EPMoELayerBase(nn.Module, ABC):
         sorted_tokens, offs, sorted_token_idx, sorted_weights, sorted_expert_ids, inv_map = (
             self._sort_tokens_for_grouped_mm(tokens, experts, weights, recv_counts=recv_counts)
         )
+        if self._folds_gate_weight(sorted_tokens, output_dtype):
+            return self._compute_experts_weight_folded(sorted_tokens, offs, sorted_token_idx, sorted_weights, inv_map,
+                                                       output_dtype, addend)
         expert_out = self._grouped_expert_ffn(sorted_tokens.to(output_dtype), offs, sorted_expert_ids, output_dtype)
         if addend is not None:
             rows, scale = addend
@@ -297,6 +303,39 @@ class EPMoELayerBase(nn.Module, ABC):
         return MoEWeightedUnpermute.apply(
             expert_out.to(output_dtype).contiguous(), sorted_weights.to(output_dtype), sorted_token_idx, inv_map
         )
+
+    def _folds_gate_weight(self, sorted_tokens, output_dtype: torch.dtype) -> bool:
+        """Whether the layer takes :meth:`_compute_experts_weight_folded`: bf16, gate and up stored fused, a fused
+        combine, a plain bf16 down projection without a bias (``(w act) @ W + w b`` is not ``w (act @ W + b)``'s
+        kernel), no adapters and no low-precision route."""
+        down = getattr(self, "down_proj", None)
+        if not (self.fold_gate_weight_into_glu and self._stores_fused_glu and fused_glu_enabled()
+                and isinstance(self._fused_glu_mul, GluCombine) and self._lowp_quant_format is None
+                and not self.has_expert_lora and getattr(self, "down_proj_bias", None) is None
+                and isinstance(self.gate_up_proj, torch.Tensor) and isinstance(down, torch.Tensor)):
+            return False
+        # what combine_fusable asks of the operands, read off the parameter without casting it
+        return (sorted_tokens.dtype == torch.bfloat16 and output_dtype == torch.bfloat16 and down.is_cuda
+                and down.dim() == 3 and (down.dtype != output_dtype or down.is_contiguous())
+                and down.shape[1] % 8 == 0 and down.shape[2] % 8 == 0)
+
+    def _compute_experts_weight_folded(self, sorted_tokens, offs, sorted_token_idx, sorted_weights, inv_map,
+                                       output_dtype, addend):
+        """The same layer with the gate weight moved ahead of the down projection:
+        ``sum_k w_k (act_k @ W_down) = sum_k (w_k act_k) @ W_down``.  The GLU kernel writes ``round(w * act)`` (one
+        rounding, where the reference rounds ``act`` and applies ``w`` in the combine, ``compute.py:222-242`` +
+        ``moe_permute.py:33-41``), the down projection runs on those rows, and the combine is a plain sum per token.
+        In backward the down projection's two gradients fetch ``grad_out[token of row]`` through the sort's index, so
+        the ``[R, H]`` gradient of the expert outputs (``moe_permute.py:44-72``) is never written or re-read, the
+        expert outputs are not kept, and the gate weights' gradient ``<grad_out[token], y_row>`` comes out of the
+        GLU's backward as ``<grad_out[token] @ W_down^T, act_row>``, the same number."""
+        gate_up = self._expert_proj(sorted_tokens.to(output_dtype), "gate_up_proj", offs, output_dtype)
+        weighted = self._fused_glu_mul.packed_weighted(gate_up, sorted_weights.to(output_dtype))
+        rows, scale = addend if addend is not None else (None, None)
+        return grouped_mm_combine(
+            weighted, self._cast_weight("down_proj", output_dtype), offs=offs, row_index=sorted_token_idx,
+            inv_map=inv_map, addend=None if rows is None else rows.to(output_dtype),
+            scale=None if scale is None else scale.to(output_dtype))
 
     def _require_recv_counts(self, recv_counts: tuple[int, ...] | None) -> tuple[int, ...]:
         if recv_counts is not None and len(recv_counts) == self.experts_per_rank:

@@ -136,6 +136,23 @@ int hmoe_glu_bwd(const void* gate, const void* up, int64_t stride_gate, int64_t 
                  int clamp_activated, int up_plus_one, void* dgate, void* dup, int64_t stride_dgate,
                  int64_t stride_dup, void* stream);
 
+/* The same pair with the combine's gate weight folded in (one weight per row, in the operands' dtype):
+ *   fwd:  out[r] = round(w[r] * glu(gate[r], up[r]))             (fp32 product, one rounding)
+ *   bwd:  (dgate, dup) = glu_grad(gate, up, w[r] * grad_out[r]),  grad_weight[r] = <grad_out[r], glu(gate[r], up[r])>
+ * with grad_out the gradient of the weighted rows and grad_weight f32[n_rows], summed in fp32 in a fixed order.
+ * Together with hmoe_grouped_gemm_dgrad_gather / _wgrad_gather_grad they replace the weight's multiply in
+ * _gather_reduce_kernel (halo/kernels/moe_permute.py:33-41) and all of _weighted_unpermute_bwd_kernel (:44-72): since
+ * sum_k w_k (act_k @ W) = sum_k (w_k act_k) @ W, the down projection runs on weighted rows, the combine is a plain
+ * sum, and its backward needs neither the [R, H] gradient of the expert outputs nor the expert outputs themselves
+ * (grad_weight[r] = <grad_out[tok r], y[r]> = <grad_out[tok r] @ W^T, act[r]>). */
+int hmoe_glu_fwd_weighted(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up,
+                          const void* row_weight, int64_t n_rows, int64_t width, int dtype, int activation,
+                          float alpha, float limit, int clamp_activated, int up_plus_one, void* out, void* stream);
+int hmoe_glu_bwd_weighted(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up,
+                          const void* grad_out, const void* row_weight, int64_t n_rows, int64_t width, int dtype,
+                          int activation, float alpha, float limit, int clamp_activated, int up_plus_one, void* dgate,
+                          void* dup, int64_t stride_dgate, int64_t stride_dup, float* grad_weight, void* stream);
+
 /* ------------------------------------------------------------------------------------------------------ router
  * Replaces the softmax / top-k / renormalise / cast sequence of the family routers the layer calls
  * (halo/distributed/expert_parallel/moe_layer/shared_experts_layer.py:44-56; weights as routing.py:110-122 and
@@ -183,6 +200,21 @@ int hmoe_grouped_gemm_fwd_gather(const void* a, int64_t lda, int64_t a_rows, con
 int hmoe_grouped_gemm_wgrad_gather(const void* a, int64_t lda, int64_t a_rows, const int64_t* row_index,
                                    const void* grad_out, int64_t ldg, const int32_t* offs, int64_t total_rows,
                                    int num_groups, int64_t k, int64_t n, int dtype, void* grad_b, void* stream);
+
+/* The two gradients of a product whose OUTPUT rows were then summed per token (the plain combine behind a down
+ * projection on weighted rows): logical row r of the output gradient is grad_out[row_index[r]], grad_out holding
+ * grad_rows rows (the tokens' gradient, read in place: no [R, N] gradient of the expert outputs is written).
+ *   dgrad_gather:       grad_a[s:e] = grad_out[row_index[s:e]] @ b[g]^T
+ *   wgrad_gather_grad:  grad_b[g]   = a[s:e]^T @ grad_out[row_index[s:e]]
+ * Replace F.grouped_mm's two gradients (halo/kernels/grouped_mm.py:25-26) fed by _weighted_unpermute_bwd_kernel
+ * (halo/kernels/moe_permute.py:44-72).  bf16 only. */
+int hmoe_grouped_gemm_dgrad_gather(const void* grad_out, int64_t ldg, int64_t grad_rows, const int64_t* row_index,
+                                   const void* b, const int32_t* offs, int64_t total_rows, int num_groups, int64_t k,
+                                   int64_t n, int dtype, void* grad_a, int64_t lda, void* stream);
+int hmoe_grouped_gemm_wgrad_gather_grad(const void* a, int64_t lda, const void* grad_out, int64_t ldg,
+                                        int64_t grad_rows, const int64_t* row_index, const int32_t* offs,
+                                        int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype,
+                                        void* grad_b, void* stream);
 
 /* ------------------------------------------------------------------------------------------------- block fp8
  * Replaces quantize_block_fp8: halo/kernels/lowp/block_fp8.py:23-34.  w is [batch, rows, cols]; q (e4m3fn bytes)

@@ -360,6 +360,44 @@ def test_glu_matches_oracle_packed_and_separate(device, name, dtype, tol, rows, 
     assert torch.equal(pd.grad[:, :width], gd.grad) and torch.equal(pd.grad[:, width:], ud.grad)
 
 
+@pytest.mark.parametrize("name", ("silu", "gelu_tanh", "gptoss"))
+@pytest.mark.parametrize(("dtype", "tol"), ((torch.float32, 1e-5), (torch.bfloat16, 2e-2)), ids=("fp32", "bf16"))
+@pytest.mark.parametrize(("rows", "width"), ((300, 768), (64, 512), (129, 360), (17, 100), (5, 1025)))
+def test_glu_with_the_gate_weight_folded_in_matches_oracle(device, name, dtype, tol, rows, width):
+    """``w[r] * combine(gate, up)[r]`` and its gradients against the oracle's closed forms in fp64 composed with the
+    product rule: ``d(gate, up) = glu_backward(gate, up, w * dout)`` and ``dw[r] = <dout[r], combine(gate, up)[r]>``.
+    The widths take the three lanes-per-row forms of the backward kernel and the scalar fallback."""
+    from oracle import glu as oracle
+
+    combine = _combines()[name]
+    kw = dict(activation=combine.activation, alpha=combine.alpha, limit=combine.limit,
+              clamp_activated=combine.clamp_activated, up_plus_one=combine.up_plus_one)
+    g = torch.Generator().manual_seed(rows * 11 + width)
+    gate_up = (torch.randn(rows, 2 * width, generator=g) * 3).to(dtype)
+    weight = torch.rand(rows, generator=g).to(dtype)
+    dout = torch.randn(rows, width, generator=g).to(dtype)
+    gate, up, w64 = gate_up[:, :width].double(), gate_up[:, width:].double(), weight.double().unsqueeze(1)
+    act = oracle.glu_forward(gate, up, **kw)
+    want = w64 * act
+    want_dg, want_du = oracle.glu_backward(gate, up, w64 * dout.double(), **kw)
+    want_dw = (dout.double() * act).sum(dim=1)
+    pd = gate_up.to(device).requires_grad_(True)
+    wd = weight.to(device).requires_grad_(True)
+    out = combine.packed_weighted(pd, wd)
+    out.backward(dout.to(device))
+    assert out.dtype == dtype and wd.grad.dtype == dtype and out.shape == (rows, width)
+    assert max_rel(out, want) < tol
+    assert max_rel(pd.grad[:, :width], want_dg) < tol and max_rel(pd.grad[:, width:], want_du) < tol
+    assert max_rel(wd.grad, want_dw) < tol
+    if dtype == torch.bfloat16:  # one rounding of the fp32 product w * act, not a product of two rounded values
+        exact = (weight.float().unsqueeze(1).to(device)
+                 * oracle.glu_forward(gate_up[:, :width].float(), gate_up[:, width:].float(), **kw).to(device))
+        assert fro_rel(out, exact) < 3e-3
+    # a weight of one changes nothing: the plain kernel's bits
+    ones = torch.ones(rows, dtype=dtype, device=device)
+    assert torch.equal(combine.packed_weighted(pd.detach(), ones), combine.packed(pd.detach()))
+
+
 def test_glu_subgradient_at_the_clamp_bound_and_probe_vector(device):
     from halo_amd.kernels.fused_glu import (GluCombine, is_gelu_tanh_activation, is_silu_activation,
                                             resolve_clamped_glu_mul, resolve_fused_glu_mul)
@@ -800,3 +838,71 @@ def test_combine_with_an_added_term_equals_the_tensor_operations(device, dtype, 
     want = combined + (addend if scale is None else scale[:, None] * addend)
     assert torch.equal(got, want)
     assert torch.equal(got[5], want[5]) and combined[5].count_nonzero() == 0
+
+
+@pytest.mark.parametrize(("counts", "k", "n"), (((255, 256, 257, 0, 513, 31), 200, 264), ((64,) * 16, 512, 1536),
+                                                 ((0, 0, 700, 1), 768, 2048),
+                                                 (tuple((37 * i * i + 11 * i) % 91 for i in range(150)), 320, 256)))
+def test_down_projection_with_the_plain_combine_equals_the_separate_operations(device, counts, k, n):
+    """``grouped_mm_combine``: the product's rows summed per token in one autograd node, its backward fetching the
+    token gradient's rows through the index.  Same arithmetic in the same order as ``grouped_mm`` followed by the
+    unweighted gather-reduce, whose backward materialises ``grad_out[row_index]``: output and both gradients are
+    bit-equal, with and without an added term, for contiguous and row-strided token gradients."""
+    from halo_amd.kernels.grouped_mm import combine_fusable, grouped_mm, grouped_mm_combine
+    from halo_amd.kernels.moe_permute import build_inv_map, gather_reduce_rows
+
+    g = torch.Generator().manual_seed(5)
+    rows, n_tokens = sum(counts), max(8, sum(counts) // 3)
+    row_index = torch.randint(0, n_tokens, (rows,), generator=g).to(device)
+    width = int(torch.bincount(row_index.cpu(), minlength=n_tokens).max())
+    inv_map = build_inv_map(row_index, n_tokens, width)
+    a = torch.randn(rows, k, generator=g).bfloat16().to(device)
+    w = (torch.randn(len(counts), k, n, generator=g) * 0.05).bfloat16().to(device)
+    addend = torch.randn(n_tokens, n, generator=g).bfloat16().to(device)
+    padded = torch.zeros(n_tokens, n + 24, dtype=torch.bfloat16, device=device)
+    padded[:, :n] = torch.randn(n_tokens, n, generator=g).bfloat16().to(device)
+    offs = _offsets(counts, device)
+    assert combine_fusable(a, w, torch.bfloat16)
+    for with_addend in (False, True):
+        for dout in (padded[:, :n].contiguous(), padded[:, :n]):
+            results = []
+            for fused in (False, True):
+                ad, wd = a.clone().requires_grad_(True), w.clone().requires_grad_(True)
+                extra = addend.clone().requires_grad_(True) if with_addend else None
+                if fused:
+                    out = grouped_mm_combine(ad, wd, offs=offs, row_index=row_index, inv_map=inv_map, addend=extra)
+                else:
+                    product = grouped_mm(ad, wd, offs=offs)
+                    out = _PlainCombine.apply(product, row_index, inv_map)
+                    if with_addend:
+                        out = out + extra
+                out.backward(dout)
+                results.append((out.detach(), ad.grad, wd.grad) + ((extra.grad,) if with_addend else ()))
+            for name, x, y in zip(("out", "grad_a", "grad_b", "grad_addend"), *results):
+                assert torch.equal(x, y), (name, with_addend, dout.is_contiguous())
+            # the gradients themselves against fp64 products of the same bf16 values
+            gathered = dout.double()[row_index].cpu()
+            ends = [0] + offs.cpu().tolist()
+            for e, (lo, hi) in enumerate(zip(ends[:-1], ends[1:])):
+                if hi > lo:
+                    want = a[lo:hi].double().cpu().t() @ gathered[lo:hi]
+                    assert max_rel(results[1][2][e], want) < 2e-2
+                else:
+                    assert not results[1][2][e].any()
+
+
+class _PlainCombine(torch.autograd.Function):
+    """Unweighted gather-reduce whose backward copies ``grad_out[row_index]`` out: the two-operation reference of the
+    test above."""
+
+    @staticmethod
+    def forward(ctx, rows, row_index, inv_map):
+        from halo_amd.kernels.moe_permute import gather_reduce_rows
+
+        ctx.save_for_backward(row_index)
+        return gather_reduce_rows(rows, inv_map)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (row_index,) = ctx.saved_tensors
+        return grad_out[row_index].contiguous(), None, None

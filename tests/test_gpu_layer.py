@@ -145,6 +145,38 @@ def test_permute_folded_into_the_first_projection_changes_no_bit(device, cfg):
     assert all(torch.equal(a, b) for a, b in zip(*runs))
 
 
+def test_gate_weight_folded_into_the_glu_stays_inside_the_tolerance(device):
+    """By default the fused-GLU bf16 layer multiplies the gate weights into the GLU's output and sums the down
+    projection's rows unweighted (no gradient of the expert outputs is written in backward).  That moves roundings
+    relative to the reference's order (weight applied behind the down projection), so it is checked twice: both
+    orders against the fp32 CPU loop within BASELINE's tolerance (output and every gradient, the router's included,
+    which carries the gate weights' gradient), and against each other."""
+    from halo_amd.kernels.router import fused_topk_gate
+
+    cfg = CONFIG2_SMALL
+    inputs = make_layer_inputs(cfg)
+    runs = {}
+    for fold in (True, False):
+        layer = _build_layer(cfg, inputs, device)
+        assert layer.fold_gate_weight_into_glu
+        layer.fold_gate_weight_into_glu = fold
+        x = inputs["x"].to(device).requires_grad_(True)
+        out = layer(x)
+        out.backward(inputs["grad_out"].to(device))
+        runs[fold] = {"out": out.detach(), "x": x.grad, "router_weight": layer.gate.weight.grad,
+                      "gate_up_proj": layer.gate_up_proj.grad, "down_proj": layer.down_proj.grad}
+    with torch.no_grad():
+        idx, _ = fused_topk_gate(layer._linear_router_logits(x.detach()), cfg.top_k, normalize=True, eps=0.0)
+    want_out, _, want = _oracle_run(cfg, inputs, idx.cpu())
+    want["out"] = want_out
+    for fold, got in runs.items():
+        for name, value in got.items():
+            _check(f"{name} (fold={fold})", value, want[name], 2e-2)
+    for name in runs[True]:
+        assert max_rel(runs[True][name], runs[False][name]) < 2e-2, name
+    assert not torch.equal(runs[True]["out"], runs[False]["out"])  # the two orders do round differently
+
+
 def test_one_gpus_share_of_an_ep_layer(device):
     """Local ids with -1 for other ranks' picks plus host-side receive counts (an EP8 shard's shape, scaled down):
     ``_compute_experts`` against the dense formula over the valid slots, and the count checks."""
@@ -202,6 +234,7 @@ def test_quantised_weight_forward(device):
                                           gate_up_proj=BlockFp8Weight(*q1), down_proj=BlockFp8Weight(*q2))
     ref = EPQwen3_5MoELayer.from_weights(router_weight=None, top_k=top_k, ep_config=EPConfig(ep_size=8, ep_rank=0),
                                          gate_up_proj=dequantize_block_fp8(*q1), down_proj=dequantize_block_fp8(*q2))
+    ref.fold_gate_weight_into_glu = False  # the order of operations the quantised-weight route keeps
     with torch.no_grad():
         got = lowp._compute_experts(x, experts.to(device), weights.to(device), torch.bfloat16, recv_counts=counts)
         want = ref._compute_experts(x, experts.to(device), weights.to(device), torch.bfloat16, recv_counts=counts)
@@ -446,6 +479,7 @@ def test_expert_lora_equals_the_layer_with_merged_weights(device, cfg):
 
     inputs = make_layer_inputs(cfg)
     base = _build_layer(cfg, inputs, device)
+    base.fold_gate_weight_into_glu = False  # a layer with adapters keeps the reference's order of operations
     spec = ExpertLoraSpec(r=16, alpha=32.0)
     # the same construction with adapters asked for
     from halo_amd.moe_layer import EPGptOssMoELayer, EPQwen3_5MoELayer, EPQwen3MoELayer
