@@ -76,6 +76,45 @@ def compute_experts_loop(tokens: torch.Tensor, experts: torch.Tensor, weights: t
     return output
 
 
+class _CpuGroupedMM(torch.autograd.Function):
+    """``F.grouped_mm`` on CPU tensors with the gradients the reference's wrapper takes
+    (``halo/kernels/grouped_mm.py:16-47``): both are grouped products again, over a gradient made dense first
+    (torch's own backward refuses a broadcast one)."""
+
+    @staticmethod
+    def forward(ctx, a, b, offs):
+        ctx.save_for_backward(a, b, offs)
+        return F.grouped_mm(a, b, offs=offs)
+
+    @staticmethod
+    def backward(ctx, grad):
+        a, b, offs = ctx.saved_tensors
+        grad = grad.contiguous() if grad.numel() else grad.new_empty(grad.shape)
+        grad_a = F.grouped_mm(grad, b.transpose(-2, -1), offs=offs) if ctx.needs_input_grad[0] else None
+        grad_b = F.grouped_mm(a.transpose(-2, -1), grad, offs=offs) if ctx.needs_input_grad[1] else None
+        return grad_a, grad_b, None
+
+
+def compute_experts_grouped(tokens: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor, params: dict,
+                            glu: Glu, num_local_experts: int) -> torch.Tensor:
+    """``_compute_experts_grouped`` (``compute.py:222-242``) as it would run on CPU tensors: stable sort of the valid
+    slots by expert (``moe_route_sort.py:201-227``), ``index_select`` (``moe_permute.py:133-136``),
+    ``F.grouped_mm`` for the fused gate/up and the down projection (``compute.py:357-361``), and the weighted rows
+    summed back per token (``moe_permute.py:115-120``).  fp32 only (the reference does not take this path without
+    CUDA: it is timed beside the loop for completeness); fused ``gate_up_proj`` layout, no biases."""
+    top_k = experts.shape[1]
+    flat = experts.reshape(-1)
+    slots = torch.nonzero((flat >= 0) & (flat < num_local_experts)).flatten()
+    order = slots[torch.argsort(flat[slots], stable=True)]
+    token_of = order // top_k
+    offs = torch.bincount(flat[order], minlength=num_local_experts).cumsum(0).to(torch.int32)
+    rows = tokens.index_select(0, token_of)
+    gate, up = _CpuGroupedMM.apply(rows, params["gate_up_proj"], offs).chunk(2, dim=-1)
+    out = _CpuGroupedMM.apply(glu(gate, up), params["down_proj"], offs)
+    gates = weights.reshape(-1)[order].to(out.dtype)
+    return torch.zeros_like(tokens).index_add(0, token_of, out * gates.unsqueeze(-1))
+
+
 def dense_formula(tokens, experts, weights, params, glu, num_local_experts):
     """``out[t] = sum over valid slots of w[t,k] * FFN_{e[t,k]}(x[t])``, slot by slot."""
     out = torch.zeros_like(tokens)

@@ -227,6 +227,32 @@ def test_layer_loop_matches_the_dense_formula(fused, kind):
     assert torch.allclose(got, want, atol=1e-10)
 
 
+def test_layer_grouped_on_cpu_matches_the_loop_and_the_dense_formula():
+    """The grouped-on-CPU variant (sort, ``F.grouped_mm``, weighted sum) against the per-expert loop and the slot-by-
+    slot formula: output and every gradient, with -1 padding, a non-local id and an expert without rows."""
+    g = torch.Generator().manual_seed(6)
+    T, H, E, K, Fw = 24, 16, 4, 3, 8
+    experts = torch.randint(-1, 4, (T, K), generator=g)
+    experts[experts == 2] = 5  # expert 2 gets nothing; 5 is not local
+    weights = torch.rand(T, K, generator=g)
+    base = {"x": torch.randn(T, H, generator=g), "gate_up_proj": torch.randn(E, H, 2 * Fw, generator=g) * 0.3,
+            "down_proj": torch.randn(E, Fw, H, generator=g) * 0.3}
+    upstream = torch.randn(T, H, generator=g)
+    runs = []
+    for fn in (moe_layer.compute_experts_grouped, moe_layer.compute_experts_loop):
+        leaves = {k: v.clone().requires_grad_(True) for k, v in base.items()}
+        params = {k: v for k, v in leaves.items() if k != "x"}
+        out = fn(leaves["x"], experts, weights, params, moe_layer.Glu(), E)
+        out.backward(upstream)
+        runs.append([out.detach()] + [leaves[k].grad for k in ("x", "gate_up_proj", "down_proj")])
+    for a, b in zip(*runs):
+        assert torch.allclose(a, b, atol=1e-5, rtol=1e-5)
+    assert not runs[0][3][2].any()  # the idle expert's weight gradient is exact zeros
+    want = moe_layer.dense_formula(base["x"], experts, weights, {k: v for k, v in base.items() if k != "x"},
+                                   moe_layer.Glu(), E)
+    assert torch.allclose(runs[0][0], want, atol=1e-5)
+
+
 def test_layer_forward_routes_and_adds_the_shared_expert():
     g = torch.Generator().manual_seed(4)
     T, H, E, K, Fw = 16, 8, 4, 2, 6
