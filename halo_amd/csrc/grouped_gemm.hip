@@ -23,7 +23,11 @@
 //    chunks XOR-ed with (con & 3) << 2, and a fragment is two ds_read_b64_tr_b16, the gfx950 transposing LDS read:
 //    within 16 lanes, lane i supplies the address of row (i >> 2), columns 4 (i & 3)..+3 of a 4 x 16 patch and receives
 //    the four rows of column i.
-//  * Two LDS stages; the loads of step k+1 are in flight during step k.  The fragments of sub-step kk+1 are read under
+//  * Two LDS stages of A; the A loads of step k+1 are in flight during step k.  B has two stages in wgrad and three in
+//    fwd and dgrad, where it is the weights, which every launch streams from HBM once: there the B tile of step k+2
+//    is requested near the end of step k, so a weight line has a step and a half to arrive and two B refills are in
+//    flight.  The five stages take all 160 KB of the LDS, so fwd and dgrad keep no tables there (RowTileWalk).
+//    The fragments of sub-step kk+1 are read under
 //    the MFMAs of sub-step kk, and the step's barrier sits in the middle of the last sub-step's MFMAs: the first
 //    fragments of the next step are read behind it, under the rest.  The barrier is a bare s_barrier after an explicit
 //    s_waitcnt: __syncthreads() would fence and drain loads that are meant to stay in flight.
@@ -31,8 +35,9 @@
 //    consecutive columns per accumulator quad.  The epilogue stages 32 rows per wavefront through LDS and writes whole
 //    16-byte chunks with buffer stores; the next tile's first loads are issued before it.
 //
-// Tile schedule.  Every workgroup builds the group bounds and the per-group prefix of row tiles from offs in LDS (no
-// host readback), so ragged and empty groups cost exactly their tiles.  The logical tile order is group-major, then
+// Tile schedule.  Every workgroup derives the group bounds and the per-group prefix of row tiles from offs (wgrad: as
+// tables in LDS; fwd and dgrad: walking offs as the tiles go by), with no host readback, so ragged and empty groups
+// cost exactly their tiles.  The logical tile order is group-major, then
 // column tile, then row tile; it is cut into 8 contiguous chunks, one per XCD (workgroup w runs on XCD w % 8), so the
 // workgroups that share an L2 work on the same expert's weights at the same time, and the tile count per XCD is
 // balanced whatever the skew of the expert loads.  wgrad walks (group, column tile, row tile) the same way: dealt
@@ -730,6 +735,64 @@ struct TileSchedule {
   }
 };
 
+// The tile walk of a fwd / dgrad workgroup without tables: the kernel's LDS is all operand stages there, so the group
+// of a tile is found by walking offs itself (scalar loads) from the previous tile's group.  Same logical order and the
+// same chunks per XCD as TileSchedule; everything uniform across the workgroup.
+template <int kMode, int BM, int BN>
+struct RowTileWalk {
+  const int32_t* offs;
+  int groups, nt, k, n;
+  int64_t total_rows, first, last, stride;
+  int g, ts, mt, s, rows;  // the current group: its index, the row tiles before it, its row tiles, first row, rows
+
+  __device__ __forceinline__ void load_group(int gi) {
+    int64_t s64 = 0, e64 = 0;
+    if (gi < groups) group_bounds(offs, gi, total_rows, s64, e64);
+    s = __builtin_amdgcn_readfirstlane(static_cast<int>(s64));
+    rows = __builtin_amdgcn_readfirstlane(static_cast<int>(e64 - s64));
+    mt = (rows + BM - 1) / BM;
+  }
+  // chunk bounds of this workgroup's XCD, given the number of row tiles over all groups
+  static __device__ __forceinline__ void chunk_of(int64_t total, int64_t& first, int64_t& last) {
+    const int xcd = blockIdx.x % kXcds;
+    const int64_t chunk = (total + kXcds - 1) / kXcds;
+    first = xcd * chunk + blockIdx.x / kXcds;
+    last = xcd * chunk + chunk < total ? xcd * chunk + chunk : total;
+  }
+  __device__ __forceinline__ void init(const GemmArgs& p, int total_row_tiles, int g0, int ts0) {
+    offs = p.offs;
+    groups = p.groups;
+    total_rows = p.total_rows;
+    k = static_cast<int>(p.k);
+    n = static_cast<int>(p.n);
+    const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
+    nt = static_cast<int>((out_cols + BN - 1) / BN);
+    chunk_of(static_cast<int64_t>(total_row_tiles) * nt, first, last);
+    stride = (static_cast<int>(gridDim.x) - static_cast<int>(blockIdx.x % kXcds) + kXcds - 1) / kXcds;
+    g = g0;
+    ts = ts0;
+    load_group(g);
+  }
+  __device__ __forceinline__ TileInfo decode(int64_t t, int& /*cursor*/) {
+    while (g < groups && static_cast<int64_t>(ts + mt) * nt <= t) {  // groups without rows have no tiles
+      ts += mt;
+      ++g;
+      load_group(g);
+    }
+    const int r = static_cast<int>(t - static_cast<int64_t>(ts) * nt);
+    const int n_t = r / mt, m_t = r - n_t * mt;
+    TileInfo tile;
+    tile.g = g;
+    tile.row_start = s;
+    tile.a_out0 = m_t * BM;
+    tile.b_out0 = n_t * BN;
+    tile.a_out_lim = rows;
+    tile.b_out_lim = kMode == kDgrad ? k : n;
+    tile.con_lim = kMode == kDgrad ? n : k;
+    return tile;
+  }
+};
+
 // ------------------------------------------------------------------------------- bf16 kernel, direct to LDS
 
 template <int kI>
@@ -767,6 +830,14 @@ struct SlimDirect {  // element(out, con) = base[out * ld + con]; LDS [256 out][
       for (int t = 0; t < kI; ++t)
         if (t < t_lim) lds_load16(rsrc, tile + (wave * kI + t) * 1024, base + t * t_stride, soff);
     }
+  }
+  // every load of the step, absent rows included (they land as zeros): the same number of loads whatever the tile,
+  // for a loop that waits for its loads by count
+  __device__ __forceinline__ void issue_all(__attribute__((address_space(3))) char* tile, int step, int wave) const {
+    const uint32_t soff = static_cast<uint32_t>(step) * (BK * 2);
+    const uint32_t base = step * BK + con0 < con_lim ? voff : kOutOfRange;
+#pragma unroll
+    for (int t = 0; t < kI; ++t) lds_load16(rsrc, tile + (wave * kI + t) * 1024, base + t * t_stride, soff);
   }
   // per-lane byte address (within the operand tile) of the fragment of sub-step 0, block 0 of the wavefront
   static __device__ __forceinline__ int fragment_base(int row0, int lane) {
@@ -807,6 +878,9 @@ struct SlimTransposed {  // element(out, con) = base[con * ld + out]; LDS [64 co
 #pragma unroll
     for (int t = 0; t < kI; ++t)
       lds_load16(rsrc, tile + (wave * kI + t) * 1024, ((t & 1) ? v1 : v0) + (t >> 1) * pair_stride, soff);
+  }
+  __device__ __forceinline__ void issue_all(__attribute__((address_space(3))) char* tile, int step, int wave) const {
+    issue(tile, step, wave, true);
   }
   // per-lane byte address of the fragment of sub-step 0 for block `block` of the wavefront (blocks do not reduce to
   // an immediate: the XOR reaches the bits the block index occupies)
@@ -1007,13 +1081,19 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   using LoaderB = typename std::conditional<kGatherB, GatherTransposed<kI>, PlainB>::type;
   // the gathered rows are contraction rows (wgrad): new ones every step
   constexpr bool kRowsPerStep = (kGatherA && !kDirectA) || kGatherB;
-  using Sched = TileSchedule<kMode, BM, BN>;
-  extern __shared__ __attribute__((aligned(16))) char lds_raw[];  // two stages of (A tile, B tile), 32 KB each
-  // tile_start: per group, the prefix of its row tiles (fwd, dgrad) or of its tiles' cost (wgrad: contraction steps
-  // + 1 per tile, the same for every tile of a group)
-  __shared__ int32_t grp_s[kMaxGroups], grp_e[kMaxGroups], tile_start[kMaxGroups + 1];
+  // fwd and dgrad keep operand B (the weights, which every launch streams from HBM once) on THREE stages and A on
+  // two: the B tile of step s + 2 is requested while step s runs, so two B refills are in flight and a weight line has
+  // two steps to arrive instead of one.  That takes all 160 KB of the LDS (A0 | B0 | B1 | A1 | B2, 32 KB each), so
+  // these modes hold no tables there: the tile walk reads offs itself.  wgrad keeps two stages of (A, B) and its tables.
+  constexpr bool kRingB = kMode != kWgrad;
+  using Sched = typename std::conditional<kRingB, RowTileWalk<kMode, BM, BN>, TileSchedule<kMode, BM, BN>>::type;
+  extern __shared__ __attribute__((aligned(16))) char lds_raw[];
   auto lds = (__attribute__((address_space(3))) char*)lds_raw;
   constexpr int kTileBytes = 256 * BK * 2, kStageBytes = 2 * kTileBytes;
+  // byte offsets of A stage i (0, 1) and B stage j (0, 1; 2 with the ring)
+  auto a_off = [](int i) { return kRingB ? i * (3 * kTileBytes) : i * kStageBytes; };
+  auto b_off = [](int j) { return kRingB ? (j == 2 ? 4 * kTileBytes : (j + 1) * kTileBytes) : j * kStageBytes + kTileBytes; };
+  constexpr int kEpiBase = kRingB ? 3 * kTileBytes : kStageBytes;  // the epilogue stages through A1 (and B2)
   bf16_t* c = static_cast<bf16_t*>(p.c);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1022,19 +1102,23 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   const bool load_wave = wave < kLoadWaves;
   const int load_slot = wave & (kLoadWaves - 1);
 
-  // ---- group bounds and the row-tile prefix, by wavefront 0
-  if (wave == 0) {
-    const int per = (p.groups + HMOE_WAVE - 1) / HMOE_WAVE;
-    const int g0 = lane * per;
-    int sum = 0;
-    for (int g = g0; g < g0 + per && g < p.groups; ++g) {
-      int64_t s, e;
-      group_bounds(p.offs, g, p.total_rows, s, e);
-      grp_s[g] = static_cast<int32_t>(s);
-      grp_e[g] = static_cast<int32_t>(e);
-      sum += kMode == kWgrad ? static_cast<int>((e - s + BK - 1) / BK) + 1 : static_cast<int>((e - s + BM - 1) / BM);
-    }
-    {
+  Sched sched;
+  if constexpr (!kRingB) {
+    // tile_start: per group, the prefix of its tiles' cost (contraction steps + 1 per tile, the same for every tile
+    // of a group)
+    __shared__ int32_t grp_s[kMaxGroups], grp_e[kMaxGroups], tile_start[kMaxGroups + 1];
+    // ---- group bounds and the cost prefix, by wavefront 0
+    if (wave == 0) {
+      const int per = (p.groups + HMOE_WAVE - 1) / HMOE_WAVE;
+      const int g0 = lane * per;
+      int sum = 0;
+      for (int g = g0; g < g0 + per && g < p.groups; ++g) {
+        int64_t s, e;
+        group_bounds(p.offs, g, p.total_rows, s, e);
+        grp_s[g] = static_cast<int32_t>(s);
+        grp_e[g] = static_cast<int32_t>(e);
+        sum += static_cast<int>((e - s + BK - 1) / BK) + 1;
+      }
       int incl = sum;
 #pragma unroll
       for (int off = 1; off < HMOE_WAVE; off <<= 1) {
@@ -1044,14 +1128,64 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       int running = incl - sum;
       for (int g = g0; g < g0 + per && g < p.groups; ++g) {
         tile_start[g] = running;
-        running += kMode == kWgrad ? (grp_e[g] - grp_s[g] + BK - 1) / BK + 1 : (grp_e[g] - grp_s[g] + BM - 1) / BM;
+        running += (grp_e[g] - grp_s[g] + BK - 1) / BK + 1;
       }
       if (lane == HMOE_WAVE - 1) tile_start[p.groups] = incl;
     }
+    __syncthreads();
+    sched.init(p, grp_s, grp_e, tile_start);
+  } else {
+    // ---- the number of row tiles over all groups and the group of this workgroup's first tile, by wavefront 0;
+    // handed to the other wavefronts through the first words of the (still unused) operand stages
+    int32_t* handoff = reinterpret_cast<int32_t*>(lds_raw);
+    if (wave == 0) {
+      const int per = (p.groups + HMOE_WAVE - 1) / HMOE_WAVE;
+      const int g0 = lane * per;
+      int sum = 0;
+      for (int g = g0; g < g0 + per && g < p.groups; ++g) {
+        int64_t s, e;
+        group_bounds(p.offs, g, p.total_rows, s, e);
+        sum += static_cast<int>((e - s + BM - 1) / BM);
+      }
+      int incl = sum;
+#pragma unroll
+      for (int off = 1; off < HMOE_WAVE; off <<= 1) {
+        const int up = __shfl_up(incl, off, HMOE_WAVE);
+        if (lane >= off) incl += up;
+      }
+      const int total = __shfl(incl, HMOE_WAVE - 1, HMOE_WAVE);
+      const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
+      const int nt = static_cast<int>((out_cols + BN - 1) / BN);
+      int64_t first, last;
+      Sched::chunk_of(static_cast<int64_t>(total) * nt, first, last);
+      const int64_t q = first / nt;  // the row tile (counted over all groups) this workgroup's first tile lies in
+      if (lane == 0) {
+        handoff[0] = total;
+        handoff[1] = p.groups;  // no tile for this workgroup: a walk that starts past the last group
+        handoff[2] = total;
+      }
+      if (q >= incl - sum && q < incl) {  // it lies in one of this lane's groups
+        int running = incl - sum;
+        for (int g = g0; g < g0 + per && g < p.groups; ++g) {
+          int64_t s, e;
+          group_bounds(p.offs, g, p.total_rows, s, e);
+          const int mt = static_cast<int>((e - s + BM - 1) / BM);
+          if (q < running + mt) {
+            handoff[1] = g;
+            handoff[2] = running;
+            break;
+          }
+          running += mt;
+        }
+      }
+    }
+    __syncthreads();
+    const int total = __builtin_amdgcn_readfirstlane(handoff[0]);
+    const int g_first = __builtin_amdgcn_readfirstlane(handoff[1]);
+    const int ts_first = __builtin_amdgcn_readfirstlane(handoff[2]);
+    __syncthreads();  // the words are read before the first tile loads land on them
+    sched.init(p, total, g_first, ts_first);
   }
-  __syncthreads();
-  Sched sched;
-  sched.init(p, grp_s, grp_e, tile_start);
   const int64_t w_elems = p.k * p.n;
 
   LoaderA la;
@@ -1090,8 +1224,13 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         }
       }
       if (tile.con_lim > 0) {
-        la.issue(lds, 0, load_slot);
-        lb.issue(lds + kTileBytes, 0, load_slot);
+        la.issue(lds + a_off(0), 0, load_slot);
+        if constexpr (kRingB) {
+          lb.issue_all(lds + b_off(0), 0, load_slot);
+          if (tile.con_lim > BK) lb.issue_all(lds + b_off(1), 1, load_slot);
+        } else {
+          lb.issue(lds + b_off(0), 0, load_slot);
+        }
       }
       if constexpr (kRowsPerStep) lg.load_rows(1, load_slot, lane);
     }
@@ -1108,9 +1247,9 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
 #pragma unroll
     for (int j = 0; j < WN; ++j) fb_base[j] = LoaderB::fragment_base(row_b + j * 32, lane);
   bf16x8 fa[2][WM], fb[2][WN];
-  auto read_fragments = [&](int stage, int kk, int buf) __attribute__((always_inline)) {
-    const char* ta = lds_raw + stage * kStageBytes;
-    const char* tb = ta + kTileBytes;
+  auto read_fragments = [&](int a_stage, int b_stage, int kk, int buf) __attribute__((always_inline)) {
+    const char* ta = lds_raw + a_off(a_stage);
+    const char* tb = lds_raw + b_off(b_stage);
 #pragma unroll
     for (int j = 0; j < WN; ++j) fb[buf][j] = LoaderB::fragment(tb, fb_base[kDirectB ? 0 : j], j, kk);
 #pragma unroll
@@ -1118,9 +1257,10 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   };
   // the same for a tile whose last rows are missing: only the fragments of the `rows_live` row blocks that hold
   // rows (a short tile's steps are otherwise bound by these reads: 64 per sub-step and CU whatever the row count)
-  auto read_live_fragments = [&](int stage, int kk, int buf, int rows_live) __attribute__((always_inline)) {
-    const char* ta = lds_raw + stage * kStageBytes;
-    const char* tb = ta + kTileBytes;
+  auto read_live_fragments = [&](int a_stage, int b_stage, int kk, int buf, int rows_live)
+                                 __attribute__((always_inline)) {
+    const char* ta = lds_raw + a_off(a_stage);
+    const char* tb = lds_raw + b_off(b_stage);
     if (rows_live > 0) {
 #pragma unroll
       for (int j = 0; j < WN; ++j) fb[buf][j] = LoaderB::fragment(tb, fb_base[kDirectB ? 0 : j], j, kk);
@@ -1139,8 +1279,8 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   constexpr int kLanesPerRow = WN * 4;
   constexpr int kRowsPerPass = 64 / kLanesPerRow;
   static_assert(kEpiRegion * kWaves * 2 <= kStageBytes, "epilogue staging must fit in one stage");
-  const char* stage_rows = lds_raw + kStageBytes + wave * kEpiRegion * 2;
-  const uint32_t stage_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + kStageBytes +
+  const char* stage_rows = lds_raw + kEpiBase + wave * kEpiRegion * 2;
+  const uint32_t stage_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + kEpiBase +
                               static_cast<uint32_t>((wave * kEpiRegion + (lane & 31) * kEpiPitch + ((lane >> 5) << 2)) * 2);
 
   int64_t t = sched.first;
@@ -1176,7 +1316,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     if (load_wave) wait_loads();
     if constexpr (kBias) asm volatile("" : "+v"(bias_chunk));
     workgroup_barrier();  // step 0 of this tile has landed in stage 0
-    if (steps > 0) read_live_fragments(0, 0, 0, live);
+    if (steps > 0) read_live_fragments(0, 0, 0, 0, live);
 
     auto run = [&](auto full_tag) __attribute__((always_inline)) {
       constexpr bool kFull = decltype(full_tag)::value;
@@ -1190,14 +1330,17 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
           }
         }
       };
+      int b_cur = 0;  // operand B's stage of this step: step % 3 with the ring, step & 1 without
       for (int step = 0; step < steps; ++step) {
         const int cur = step & 1;
         const bool more = step + 1 < steps;
-        // the other stage is free since the barrier inside the previous step; past the last step the loads are
-        // issued all the same, out of range, so that the loop has one shape
+        const int b_next = kRingB ? (b_cur == 2 ? 0 : b_cur + 1) : cur ^ 1;
+        const bool more2 = kRingB && step + 2 < steps;
+        // the other A stage is free since the barrier inside the previous step, and so is the B stage that step read;
+        // past the last step the A loads are issued all the same, out of range, so that the loop has one shape
         if (load_wave) {
-          la.issue(lds + (cur ^ 1) * kStageBytes, step + 1, load_slot, more);
-          lb.issue(lds + (cur ^ 1) * kStageBytes + kTileBytes, step + 1, load_slot, more);
+          la.issue(lds + a_off(cur ^ 1), step + 1, load_slot, more);
+          if constexpr (!kRingB) lb.issue(lds + b_off(cur ^ 1), step + 1, load_slot, more);
           // the rows of the step after that: their indices arrive under this step, with its tile loads; in the
           // tile's last step that is the next tile's first
           if constexpr (kRowsPerStep) {
@@ -1210,8 +1353,8 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         if constexpr (kRowsPerStep) next_rows0_loaded = !more && has_next;
 #pragma unroll
         for (int kk = 0; kk < 3; ++kk) {
-          if constexpr (kFull) read_fragments(cur, kk + 1, (kk + 1) & 1);
-          else read_live_fragments(cur, kk + 1, (kk + 1) & 1, live);
+          if constexpr (kFull) read_fragments(cur, b_cur, kk + 1, (kk + 1) & 1);
+          else read_live_fragments(cur, b_cur, kk + 1, (kk + 1) & 1, live);
           mfmas(kk & 1, 0, WM);
           if constexpr (kFull) {
             interleave_reads_under_mfmas<kReads, kMfmas>();
@@ -1219,16 +1362,30 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         }
         mfmas(1, 0, WM / 2);
         __builtin_amdgcn_sched_barrier(0);
-        // lgkmcnt(0): this stage is read out; vmcnt(0) where tile loads were issued: the next step has landed
-        if (load_wave) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        // With the ring, B of the step after next goes out here, into the stage the previous step read: behind this
+        // wavefront's MFMAs rather than ahead of them (a loading wavefront sits in the address unit's queue for the
+        // length of its burst; at the top of the step that delayed its first MFMA by as much, and this burst is
+        // waited for by nobody before the next step's end).
+        if constexpr (kRingB) {
+          if (load_wave && more2) lb.issue_all(lds + b_off(b_next == 2 ? 0 : b_next + 1), step + 2, load_slot);
+        }
+        // lgkmcnt(0): this stage is read out; vmcnt where tile loads were issued: the next step has landed.  The
+        // loads complete in the order they were issued, so with the ring the newest kI (the burst above) may stay
+        // in flight.
+        if (load_wave) {
+          if (more2) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kI) : "memory");
+          else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        } else {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
         workgroup_barrier();
         if (more) {
-          if constexpr (kFull) read_fragments(cur ^ 1, 0, 0);
-          else read_live_fragments(cur ^ 1, 0, 0, live);
+          if constexpr (kFull) read_fragments(cur ^ 1, b_next, 0, 0);
+          else read_live_fragments(cur ^ 1, b_next, 0, 0, live);
         }
         mfmas(1, WM / 2, WM);
         if constexpr (kFull) interleave_reads_under_mfmas<kReads, kMfmas / 2>();
+        b_cur = b_next;
       }
     };
     if (live == WM) run(std::true_type{});
@@ -1755,8 +1912,11 @@ int launch_direct(const GemmArgs& p, hipStream_t stream) {
   if (bound < workers) workers = bound;
   workers = (workers + kXcds - 1) / kXcds * kXcds;
   if (workers <= 0) return HMOE_OK;
-  // two stages; the gathered wgrad keeps 2 x 1 KB of row indices per loading wavefront behind them
-  constexpr size_t lds_bytes = 2 * Cfg::kStage * sizeof(bf16_t) + (kGather && kMode == kWgrad ? 4 * 2048 : 0);
+  // wgrad: two stages; gathered, 2 x 1 KB of row indices per loading wavefront behind them.  fwd, dgrad: two stages
+  // of A and three of B
+  constexpr size_t lds_bytes = kMode == kWgrad
+                                   ? 2 * Cfg::kStage * sizeof(bf16_t) + (kGather ? 4 * 2048 : 0)
+                                   : (2 * Cfg::BM + 3 * Cfg::BN) * BK * sizeof(bf16_t);
   auto kernel = grouped_gemm_bf16_kernel<kMode, Cfg, kGather, kBias>;
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                           static_cast<int>(lds_bytes)) != hipSuccess)
