@@ -27,7 +27,7 @@ SIGNATURES = {
     "hmoe_route_sort": (I, [P, I, P, I, L, I, I, L, P, P, P, P, P, P, P, P, P]),
     "hmoe_route_sort_static": (I, [P, I, P, I, L, I, I, L, P, P, P, P, P, P, P, P]),
     "hmoe_route_sort_bwd": (I, [P, P, L, L, I, P, P]),
-    "hmoe_bincount": (I, [P, P, L, I, I, P, P]),
+    "hmoe_bincount": (I, [P, P, L, L, I, P, P]),
     "hmoe_gather_rows": (I, [P, L, P, L, L, I, P, P]),
     "hmoe_gather_reduce": (I, [P, P, P, L, I, L, L, I, P, P]),
     "hmoe_gather_reduce_add": (I, [P, P, P, L, I, L, L, I, P, L, P, P, P]),

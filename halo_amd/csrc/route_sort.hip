@@ -10,6 +10,9 @@
 // find each other with one ballot per expert-id bit, rank themselves with a popcount of the lower lanes, and the
 // lowest lane advances the expert's running position kept in LDS.  Order within an expert is slot order, so the sort
 // is stable and bit-reproducible.
+//
+// Also here: the sync-free histogram behind hmoe_bincount (halo/kernels/histogram.py:9-18 of the reference), whose
+// many-workgroup form adds per-workgroup counts with vector atomics (integer sums: exact in any order).
 #include "common.h"
 
 #include <atomic>
@@ -224,6 +227,55 @@ bincount_kernel(const int64_t* __restrict__ indices, const float* __restrict__ w
   }
 }
 
+constexpr int64_t kBincountLdsBins = 8192;     // bins a workgroup can count in LDS
+constexpr int64_t kBincountOneBlock = 1 << 16;  // up to this many indices one workgroup does it all
+constexpr int64_t kBincountPerBlock = 1 << 14;  // indices per workgroup beyond that (grid-stride past 2048 workgroups)
+
+__global__ void __launch_bounds__(1024) bincount_clear_kernel(uint32_t* __restrict__ out, int64_t words) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < words;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    out[i] = 0u;
+}
+
+// Each workgroup counts its share of the indices, in LDS first where the bins fit (kLds), and adds what it found to
+// the cleared output.  The output adds are vector atomics on global memory: integer counts come out exact whatever
+// their order; a weighted sum's order is not fixed (as the reference's scatter_add_).
+template <bool kLds>
+__global__ void __launch_bounds__(1024)
+bincount_blocks_kernel(const int64_t* __restrict__ indices, const float* __restrict__ weights, int64_t n, int64_t size,
+                       int out_is_i64, void* __restrict__ out) {
+  extern __shared__ int32_t counts[];
+  float* sums = reinterpret_cast<float*>(counts);
+  if constexpr (kLds) {
+    for (int v = threadIdx.x; v < size; v += blockDim.x) counts[v] = 0;
+    __syncthreads();
+  }
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const int64_t v = indices[i];
+    if (v < 0 || v >= size) continue;
+    if constexpr (kLds) {
+      if (weights) atomicAdd(&sums[v], weights[i]);
+      else atomicAdd(&counts[v], 1);
+    } else {
+      if (weights) atomicAdd(static_cast<float*>(out) + v, weights[i]);
+      else if (out_is_i64) atomicAdd(static_cast<unsigned long long*>(out) + v, 1ull);
+      else atomicAdd(static_cast<float*>(out) + v, 1.0f);
+    }
+  }
+  if constexpr (kLds) {
+    __syncthreads();
+    for (int v = threadIdx.x; v < size; v += blockDim.x) {
+      if (weights) {
+        if (sums[v] != 0.0f) atomicAdd(static_cast<float*>(out) + v, sums[v]);
+      } else if (counts[v] != 0) {
+        if (out_is_i64) atomicAdd(static_cast<unsigned long long*>(out) + v, static_cast<unsigned long long>(counts[v]));
+        else atomicAdd(static_cast<float*>(out) + v, static_cast<float>(counts[v]));
+      }
+    }
+  }
+}
+
 int rows_per_block(int top_k) { return kBlockSlots / top_k > 0 ? kBlockSlots / top_k : 1; }
 
 template <typename IdT, typename WT>
@@ -342,15 +394,34 @@ int hmoe_route_sort_bwd(const void* grad_sorted, const int32_t* dest, int64_t n_
   return HMOE_OK;
 }
 
-int hmoe_bincount(const int64_t* indices, const float* weights, int64_t n, int size, int out_is_i64, void* out,
+int hmoe_bincount(const int64_t* indices, const float* weights, int64_t n, int64_t size, int out_is_i64, void* out,
                   void* stream) {
+  using namespace hmoe;
   if (n < 0 || size < 0) return HMOE_INVALID_ARGUMENT;
   if (size == 0) return HMOE_OK;
   if (!out || (n > 0 && !indices)) return HMOE_INVALID_ARGUMENT;
   if (weights && out_is_i64) return HMOE_INVALID_ARGUMENT;
-  if (size > 8192) return HMOE_UNSUPPORTED;
-  hmoe::bincount_kernel<<<dim3(1), dim3(1024), size * sizeof(int32_t), static_cast<hipStream_t>(stream)>>>(
-      indices, weights, n, size, out_is_i64, out);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (size <= kBincountLdsBins && n <= kBincountOneBlock) {
+    bincount_kernel<<<dim3(1), dim3(1024), size * sizeof(int32_t), s>>>(indices, weights, n, static_cast<int>(size),
+                                                                       out_is_i64, out);
+    HMOE_CHECK_LAUNCH();
+    return HMOE_OK;
+  }
+  // many indices or many bins: the output is cleared by a fill kernel, then every workgroup adds its share
+  const int64_t words = out_is_i64 ? 2 * size : size;
+  bincount_clear_kernel<<<dim3(static_cast<unsigned>((words + 1023) / 1024 < 1024 ? (words + 1023) / 1024 : 1024)),
+                          dim3(1024), 0, s>>>(static_cast<uint32_t*>(out), words);
+  HMOE_CHECK_LAUNCH();
+  if (n == 0) return HMOE_OK;
+  int64_t blocks = (n + kBincountPerBlock - 1) / kBincountPerBlock;
+  if (blocks > 2048) blocks = 2048;
+  if (size <= kBincountLdsBins)
+    bincount_blocks_kernel<true><<<dim3(static_cast<unsigned>(blocks)), dim3(1024), size * sizeof(int32_t), s>>>(
+        indices, weights, n, size, out_is_i64, out);
+  else
+    bincount_blocks_kernel<false><<<dim3(static_cast<unsigned>(blocks)), dim3(1024), 0, s>>>(indices, weights, n, size,
+                                                                                          out_is_i64, out);
   HMOE_CHECK_LAUNCH();
   return HMOE_OK;
 }

@@ -1,7 +1,7 @@
-"""Sync-free histograms for MoE routing (no host readback, no atomics on global memory).
+"""Sync-free histograms for MoE routing (no host readback; counts are exact).
 
-Mirrors the reference's ``halo/kernels/histogram.py:9-26``; the kernel is ``hmoe_bincount`` in
-``csrc/route_sort.hip`` (one workgroup, LDS counters).
+Mirrors the reference's ``halo/kernels/histogram.py:9-26``; the kernels are behind ``hmoe_bincount`` in
+``csrc/route_sort.hip`` (LDS counters; many workgroups for large inputs, any number of bins).
 """
 
 from __future__ import annotations

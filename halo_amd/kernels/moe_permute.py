@@ -11,6 +11,7 @@ from __future__ import annotations
 import torch
 
 from halo_amd import _lib
+from halo_amd.kernels.histogram import sync_free_bincount
 
 
 def _gather_rows(src: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
@@ -83,7 +84,8 @@ def build_inv_map(sorted_token_idx: torch.Tensor, recv_N: int, width: int) -> to
         # token: its index in the grouped order minus the index at which its token's run begins
         by_token = torch.argsort(token_of, stable=True)
         owner = token_of[by_token]
-        per_token = torch.bincount(token_of, minlength=recv_N)
+        # torch.bincount sizes its output from the largest index and reads it back to the host; this one does not
+        per_token = sync_free_bincount(token_of, recv_N, dtype=torch.int64)
         run_start = per_token.cumsum(0) - per_token
         rank = torch.arange(rows, device=device) - run_start[owner]
         result[owner, rank] = by_token

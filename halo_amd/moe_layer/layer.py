@@ -41,17 +41,40 @@ class _RouterProjection(torch.autograd.Function):
     Forward and the input gradient are plain dense products on the library GEMM, as in the reference.  The weight
     gradient ``dlogits^T @ x`` is an ``[E, H]`` output contracted over all T tokens: a handful of output tiles, which
     leaves a dense GEMM (and one grouped-GEMM group) on a few CUs.  The tokens are cut into ``_SPLITS`` slices that
-    the wgrad kernel takes as groups, one partial ``[E, H]`` each, all CUs busy; the partials are summed in fp32 in a
-    fixed order, so the result stays deterministic."""
+    the wgrad kernel takes as groups, one partial ``[E, H]`` each (rounded to the operands' dtype), all CUs busy; the
+    partials are summed in fp32 in a fixed order and rounded once, so the result stays deterministic.  Operands the
+    kernel does not take (rows that are not 16-byte multiples, unaligned views) use the dense product."""
 
     _SPLITS = 32
     _MIN_TOKENS = 2048
-    _slice_ends: ClassVar[dict] = {}  # (device, tokens) -> the slices' row ends
+    _slice_ends: ClassVar[dict] = {}  # (device, tokens) -> the slices' row ends; a handful of sequence lengths at most
+    _SLICE_ENDS_KEPT = 16
+
+    @staticmethod
+    def _slice_ends_for(device: torch.device, tokens: int) -> torch.Tensor:
+        cache, splits = _RouterProjection._slice_ends, _RouterProjection._SPLITS
+        offs = cache.get((device, tokens))
+        if offs is None:
+            if len(cache) >= _RouterProjection._SLICE_ENDS_KEPT:  # varying sequence lengths: start over, never grow
+                cache.clear()
+            offs = torch.arange(1, splits + 1, device=device, dtype=torch.int32) * (tokens // splits)
+            cache[(device, tokens)] = offs
+        return offs
 
     @staticmethod
     def forward(ctx, x, weight):
         ctx.save_for_backward(x, weight)
         return torch.nn.functional.linear(x, weight)
+
+    @staticmethod
+    def _sliced_wgrad_usable(grad_logits: torch.Tensor, x: torch.Tensor) -> bool:
+        tokens, splits = x.shape[0], _RouterProjection._SPLITS
+        return (x.dtype == torch.bfloat16 and grad_logits.dtype == torch.bfloat16
+                and tokens >= _RouterProjection._MIN_TOKENS and tokens % splits == 0
+                # what the grouped kernels ask of bf16 operands: 16-byte rows, 16-byte aligned
+                and grad_logits.shape[1] % 8 == 0 and x.shape[1] % 8 == 0
+                and all(t.stride(-1) == 1 and t.stride(0) % 8 == 0 and t.data_ptr() % 16 == 0
+                        for t in (grad_logits, x)))
 
     @staticmethod
     def backward(ctx, grad_logits):
@@ -60,14 +83,9 @@ class _RouterProjection(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             grad_x = grad_logits @ weight
         if ctx.needs_input_grad[1]:
-            tokens = x.shape[0]
-            splits = _RouterProjection._SPLITS
-            if x.dtype == torch.bfloat16 and tokens >= _RouterProjection._MIN_TOKENS and tokens % splits == 0:
-                key = (x.device, tokens)
-                offs = _RouterProjection._slice_ends.get(key)
-                if offs is None:
-                    offs = torch.arange(1, splits + 1, device=x.device, dtype=torch.int32) * (tokens // splits)
-                    _RouterProjection._slice_ends[key] = offs
+            if _RouterProjection._sliced_wgrad_usable(grad_logits, x):
+                splits = _RouterProjection._SPLITS
+                offs = _RouterProjection._slice_ends_for(x.device, x.shape[0])
                 partial = grouped_wgrad(grad_logits, x, offs, splits)
                 grad_weight = partial.sum(dim=0)  # the reduction accumulates in fp32 and rounds once
             else:

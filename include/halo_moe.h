@@ -81,9 +81,11 @@ int hmoe_route_sort_bwd(const void* grad_sorted, const int32_t* dest, int64_t n_
 
 /* Replaces sync_free_bincount: halo/kernels/histogram.py:9-18.
  * out[v] = number of indices equal to v (weights null) or the sum of their f32 weights, for 0 <= v < size; out is
- * f32 (out_is_i64 == 0) or i64 (counts only).  Indices outside [0, size) are ignored.  One workgroup, counters in
- * LDS; counts are exact, a weighted sum's order is not fixed (as the reference's scatter_add_). */
-int hmoe_bincount(const int64_t* indices, const float* weights, int64_t n, int size, int out_is_i64, void* out,
+ * f32 (out_is_i64 == 0) or i64 (counts only).  Indices outside [0, size) are ignored.  No limit on n or size: up to
+ * 65536 indices and 8192 bins one workgroup counts in LDS; beyond that the output is cleared and many workgroups add
+ * their shares with vector atomics (LDS counters first where the bins fit).  Counts are exact either way; a weighted
+ * sum's order is not fixed (as the reference's scatter_add_), and a float count above 2^24 rounds as float32 does. */
+int hmoe_bincount(const int64_t* indices, const float* weights, int64_t n, int64_t size, int out_is_i64, void* out,
                   void* stream);
 
 /* ------------------------------------------------------------------------------------------- permute / combine

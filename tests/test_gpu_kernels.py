@@ -127,6 +127,63 @@ def test_bincount(device):
     assert torch.equal(counter.cpu(), 2 * want.float())
 
 
+@pytest.mark.parametrize(("n", "size"), ((500_000, 128), (70_000, 8192), (300_000, 65_536), (1000, 100_000),
+                                         (0, 9000)))
+def test_bincount_with_many_indices_and_many_bins(device, n, size):
+    """Beyond one workgroup's reach (65536 indices, 8192 bins) the histogram takes many workgroups: exact counts in
+    int64 and fp32, weighted sums to fp32 rounding, out-of-range indices ignored.  The reference calls it with a
+    token count as ``size`` (``moe_permute.py:75-89``)."""
+    from halo_amd.kernels.histogram import sync_free_bincount
+    from oracle import route_sort as oracle
+
+    g = torch.Generator().manual_seed(n + size)
+    idx = torch.randint(-3, size + 3, (n,), generator=g)  # a few values either side of the range
+    inside = idx[(idx >= 0) & (idx < size)]
+    want = torch.from_numpy(oracle.bincount(inside.numpy(), size, np.int64))
+    got = sync_free_bincount(idx.to(device), size, dtype=torch.long)
+    assert got.dtype == torch.int64 and torch.equal(got.cpu(), want)
+    assert torch.equal(sync_free_bincount(idx.to(device), size).cpu(), want.float())
+    w = torch.rand(n, generator=g)
+    want_w = torch.zeros(size, dtype=torch.float64).scatter_add_(0, inside, w[(idx >= 0) & (idx < size)].double())
+    got_w = sync_free_bincount(idx.to(device), size, weights=w.to(device))
+    assert torch.allclose(got_w.cpu().double(), want_w, rtol=1e-4, atol=1e-4)
+
+
+def test_expert_path_and_inv_map_never_synchronise_the_host(device):
+    """With torch's sync debug mode at ``error`` (the reference's ``cuda_syncs_are_errors``,
+    ``tests/common/harness.py:118-126``) an op that makes the host wait for the device raises.  A layer's forward and
+    backward, ``build_inv_map`` and the histograms run under it; a known synchronising op is checked first, so that a
+    torch build which does not honour the mode fails this test's premise rather than passing it silently."""
+    from halo_amd.kernels.histogram import sync_free_bincount
+    from halo_amd.kernels.moe_permute import build_inv_map
+    from halo_amd.moe_layer import EPQwen3_5MoELayer
+
+    g = torch.Generator().manual_seed(8)
+    tokens, hidden, experts, top_k, ffn = 512, 256, 16, 4, 128
+    x = torch.randn(tokens, hidden, generator=g).bfloat16().to(device).requires_grad_(True)
+    layer = EPQwen3_5MoELayer.from_weights(
+        router_weight=(torch.randn(experts, hidden, generator=g) * 0.02).bfloat16().to(device), top_k=top_k,
+        gate_up_proj=(torch.randn(experts, hidden, 2 * ffn, generator=g) * 0.02).bfloat16().to(device),
+        down_proj=(torch.randn(experts, ffn, hidden, generator=g) * 0.02).bfloat16().to(device))
+    grad = torch.randn(tokens, hidden, generator=g).bfloat16().to(device)
+    sorted_tokens = torch.randint(0, tokens, (3000,), generator=g).to(device)
+    layer(x).backward(grad)  # once outside: allocator warm-up and the library load are not the subject
+    torch.cuda.synchronize()
+    torch.cuda.set_sync_debug_mode("error")
+    try:
+        with pytest.raises(RuntimeError):
+            sorted_tokens.sum().item()  # the premise: a readback is an error in this mode
+        x.grad = None
+        out = layer(x)
+        out.backward(grad)
+        inv_map = build_inv_map(sorted_tokens, tokens, 16)
+        counts = sync_free_bincount(sorted_tokens, 100_000, dtype=torch.long)
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
+    assert out.shape == x.shape and x.grad is not None
+    assert inv_map.shape == (tokens, 16) and int(counts.sum()) == 3000
+
+
 # -------------------------------------------------------------------------------------------- permute / combine
 
 DTYPE_TOLS = ((torch.float32, 1e-5), (torch.bfloat16, 2e-2))

@@ -386,6 +386,23 @@ def test_router_projection_gradients_at_a_token_count_that_splits_the_wgrad(devi
     assert all(torch.equal(a, b) for a, b in zip(results[0], results[1]))
 
 
+def test_router_projection_with_an_expert_count_the_grouped_kernel_does_not_take(device):
+    """60 experts: the logits' rows are not 16-byte multiples, so the sliced weight gradient does not apply and the
+    dense product takes over (it used to raise)."""
+    from halo_amd.moe_layer.layer import _RouterProjection
+
+    tokens, hidden, experts = 2048, 256, 60
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(tokens, hidden, generator=g).bfloat16()
+    w = (torch.randn(experts, hidden, generator=g) * 0.05).bfloat16()
+    dlogits = torch.randn(tokens, experts, generator=g).bfloat16()
+    xd, wd = x.to(device).requires_grad_(True), w.to(device).requires_grad_(True)
+    assert not _RouterProjection._sliced_wgrad_usable(dlogits.to(device), xd)
+    _RouterProjection.apply(xd, wd).backward(dlogits.to(device))
+    _check("dw", wd.grad, dlogits.double().t() @ x.double(), 2e-2)
+    _check("dx", xd.grad, dlogits.double() @ w.double(), 2e-2)
+
+
 class _SharedMlp(torch.nn.Module):
     def __init__(self, hidden, width, dtype, generator):
         super().__init__()
