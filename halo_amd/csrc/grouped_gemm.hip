@@ -849,16 +849,27 @@ struct SlimDirect {  // element(out, con) = base[out * ld + con]; LDS [256 out][
   }
 };
 
-template <int kI>
+template <int kI, bool kRebase = false>
 struct SlimTransposed {  // element(out, con) = base[con * ld + out]; LDS [64 con][256 out], chunk ^= (con & 3) << 2
-  u32x4 rsrc;  // bounded at the operand's last contraction row
+  // With kRebase (wgrad, whose contraction walks every row of a group: more than 32 bits of bytes for a large one)
+  // the descriptor is rebased every step: base + step * step_bytes in 64 bits, bounded at what is left of the operand
+  // (or 2 GiB - 1), so that the per-lane offsets stay inside one step.  Without it (an expert's weight, below 2 GiB)
+  // the descriptor is fixed and the step is a 32-bit offset.
+  u32x4 rsrc;                   // !kRebase: bounded at the operand's last contraction row
+  uint64_t base_address;        // kRebase
+  int64_t extent;               // kRebase: bytes from the base to the operand's last contraction row
   uint32_t voff[2];             // even and odd loads of a step differ in (con & 3); pairs are 4 contraction rows apart
   uint32_t pair_stride, step_bytes;
 
   __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int64_t bytes, int out0, int out_lim,
                                        int /*con_lim*/, int wave, int lane) {
     static_assert(kI % 2 == 0, "loads come in even/odd pairs");
-    rsrc = make_rsrc_words(base, static_cast<uint32_t>(bytes));
+    if constexpr (kRebase) {
+      base_address = reinterpret_cast<uint64_t>(base);
+      extent = bytes;
+    } else {
+      rsrc = make_rsrc_words(base, static_cast<uint32_t>(bytes));
+    }
     step_bytes = BK * static_cast<uint32_t>(ld) * 2u;
     pair_stride = 4u * static_cast<uint32_t>(ld) * 2u;
 #pragma unroll
@@ -871,13 +882,23 @@ struct SlimTransposed {  // element(out, con) = base[con * ld + out]; LDS [64 co
                     : kOutOfRange;
     }
   }
+  // the descriptor of one step
+  __device__ __forceinline__ u32x4 step_rsrc(int step) const {
+    if constexpr (!kRebase) return rsrc;
+    const int64_t offset = static_cast<int64_t>(step) * step_bytes;
+    int64_t left = extent - offset;
+    left = left < 0 ? 0 : (left > 0x7fffffff ? 0x7fffffff : left);  // below kOutOfRange, which must stay out of range
+    return make_rsrc_words(reinterpret_cast<const void*>(base_address + static_cast<uint64_t>(offset)),
+                           static_cast<uint32_t>(left));
+  }
   __device__ __forceinline__ void issue(__attribute__((address_space(3))) char* tile, int step, int wave,
                                         bool live = true) const {
-    const uint32_t soff = live ? static_cast<uint32_t>(step) * step_bytes : 0u;
+    const u32x4 r = step_rsrc(live ? step : 0);
+    const uint32_t soff = !kRebase && live ? static_cast<uint32_t>(step) * step_bytes : 0u;
     const uint32_t v0 = live ? voff[0] : kOutOfRange, v1 = live ? voff[1] : kOutOfRange;
 #pragma unroll
     for (int t = 0; t < kI; ++t)
-      lds_load16(rsrc, tile + (wave * kI + t) * 1024, ((t & 1) ? v1 : v0) + (t >> 1) * pair_stride, soff);
+      lds_load16(r, tile + (wave * kI + t) * 1024, ((t & 1) ? v1 : v0) + (t >> 1) * pair_stride, soff);
   }
   __device__ __forceinline__ void issue_all(__attribute__((address_space(3))) char* tile, int step, int wave) const {
     issue(tile, step, wave, true);
@@ -1074,10 +1095,10 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   constexpr int kLoadWaves = 4;
   constexpr int kI = 32 / kLoadWaves;
   constexpr bool kDirectA = kMode != kWgrad, kDirectB = kMode == kDgrad;
-  using PlainA = typename std::conditional<kDirectA, SlimDirect<kI>, SlimTransposed<kI>>::type;
+  using PlainA = typename std::conditional<kDirectA, SlimDirect<kI>, SlimTransposed<kI, true>>::type;
   using GatheredA = typename std::conditional<kDirectA, GatherDirect<kI>, GatherTransposed<kI>>::type;
   using LoaderA = typename std::conditional<kGatherA, GatheredA, PlainA>::type;
-  using PlainB = typename std::conditional<kDirectB, SlimDirect<kI>, SlimTransposed<kI>>::type;
+  using PlainB = typename std::conditional<kDirectB, SlimDirect<kI>, SlimTransposed<kI, kMode == kWgrad>>::type;
   using LoaderB = typename std::conditional<kGatherB, GatherTransposed<kI>, PlainB>::type;
   // the gathered rows are contraction rows (wgrad): new ones every step
   constexpr bool kRowsPerStep = (kGatherA && !kDirectA) || kGatherB;
@@ -1203,9 +1224,15 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
       if (load_wave)  // the row indices are fetched by the lanes that use them
         la.init(a, p.lda, p.a_rows, p.a_index + tile.row_start, tile.a_out0, tile.a_out_lim, tile.con_lim, load_slot,
                 lane);
-    } else {
+    } else if constexpr (kMode == kWgrad) {
       la.init(a + tile.row_start * p.lda, p.lda, rows * p.lda * 2, tile.a_out0, tile.a_out_lim, tile.con_lim,
               load_slot, lane);
+    } else {
+      // the descriptor starts at the tile's first row and ends at its last, so its 32-bit offsets span one tile
+      // whatever the operand's or the group's size
+      const int rows_left = tile.a_out_lim - tile.a_out0;
+      la.init(a + (tile.row_start + tile.a_out0) * p.lda, p.lda, (rows_left < BM ? rows_left : BM) * p.lda * 2, 0,
+              rows_left, tile.con_lim, load_slot, lane);
     }
     if constexpr (kGatherB) {
       if (load_wave)
@@ -1400,8 +1427,11 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     }
 
     // epilogue through the second stage: 32 rows at a time per wavefront, whole 16-byte chunks out
-    bf16_t* c_base = kMode == kWgrad ? c + done.g * w_elems : c + done.row_start * p.ldc;
-    const int64_t c_rows = kMode == kWgrad ? p.k : done.a_out_lim;
+    // fwd, dgrad: the output descriptor spans this tile's rows only (as the A descriptor does)
+    const int c_row0 = kMode == kWgrad ? 0 : done.a_out0;
+    const int c_row_lim = kMode == kWgrad ? static_cast<int>(p.k) : done.a_out_lim - done.a_out0;
+    bf16_t* c_base = kMode == kWgrad ? c + done.g * w_elems : c + (done.row_start + c_row0) * p.ldc;
+    const int64_t c_rows = kMode == kWgrad ? p.k : (c_row_lim < BM ? c_row_lim : BM);
     const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(c_base, static_cast<uint32_t>(c_rows * p.ldc * 2));
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
@@ -1427,11 +1457,11 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
         for (int pass = 0; pass < 32 / kRowsPerPass; ++pass) {
           const int rr = pass * kRowsPerPass + lane / kLanesPerRow;
           const int cc = (lane % kLanesPerRow) << 3;
-          const int row = done.a_out0 + row_a + i * 32 + rr;
+          const int row = (kMode == kWgrad ? done.a_out0 : 0) + row_a + i * 32 + rr;  // from the descriptor's first row
           const int col = done.b_out0 + row_b + cc;
           u32x4 v = *reinterpret_cast<const u32x4*>(stage_rows + (rr * kEpiPitch + cc) * 2);
           if constexpr (kBias) v = add_bf16x8(v, bias_chunk);
-          const uint32_t off = row < done.a_out_lim && col < done.b_out_lim
+          const uint32_t off = row < c_row_lim && col < done.b_out_lim
                                    ? static_cast<uint32_t>(row) * static_cast<uint32_t>(p.ldc) * 2u + col * 2u
                                    : kOutOfRange;
           // a weight gradient is not read again before the optimizer: stored non-temporally, it leaves the L2's
@@ -1969,13 +1999,16 @@ int validate(const GemmArgs& p, int dtype) {
     // 16-byte rows: the alignment torch's grouped GEMM asks for as well
     if (p.k % 8 || p.n % 8 || p.lda % 8 || p.ldb % 8 || p.ldc % 8) return HMOE_UNSUPPORTED;
     if (!aligned16(p.a) || !aligned16(p.b) || !aligned16(p.c)) return HMOE_UNSUPPORTED;
-    // buffer loads address an operand with 32-bit byte offsets: all rows of an operand and one expert's weight
-    // must each stay below 2 GiB
+    // Buffer loads address memory with 32-bit byte offsets from a descriptor's base.  The kernels base their
+    // descriptors at a tile's first row (activations and outputs) or rebase them every contraction step (wgrad), so
+    // the activation operands and the outputs may be of any size; what must stay below 2 GiB is one expert's weight,
+    // one 256-row tile of any operand, and an array that is gathered from by row index.
     const int64_t lim = int64_t(1) << 31;
-    const int64_t a_extent = (p.a_index && !p.gather_b ? p.a_rows : p.total_rows) * p.lda * 2;
-    const int64_t b_extent = (p.gather_b ? p.a_rows : p.total_rows) * p.ldb * 2;
-    if (a_extent >= lim || b_extent >= lim || p.total_rows * p.ldc * 2 >= lim || p.k * p.n * 2 >= lim)
-      return HMOE_UNSUPPORTED;
+    const int64_t widest = p.lda > p.ldb ? (p.lda > p.ldc ? p.lda : p.ldc) : (p.ldb > p.ldc ? p.ldb : p.ldc);
+    if (widest * 2 * 512 >= lim || p.k * p.n * 2 >= lim) return HMOE_UNSUPPORTED;
+    if (p.a_index && p.a_rows * (p.gather_b ? p.ldb : p.lda) * 2 >= lim) return HMOE_UNSUPPORTED;
+    if (p.b_scale && (p.total_rows * p.lda * 2 >= lim || p.total_rows * p.ldc * 2 >= lim))
+      return HMOE_UNSUPPORTED;  // the register-staged fp8-weight kernel still spans a group per descriptor
   }
   return HMOE_OK;
 }

@@ -97,6 +97,19 @@ def test_bad_arguments_come_back_as_status_codes_before_any_launch():
     assert lib.hmoe_grouped_gemm_fwd_gather(fake, 64, 8, fake, fake, fake, 8, 4, 64, 64, f32, fake, 64, None) == unsupported
     assert lib.hmoe_grouped_gemm_fwd_gather(fake, 64, -3, fake, fake, fake, 8, 4, 64, 64, bf16, fake, 64, None) == invalid
 
+    # what must stay below 2 GiB: an array gathered from by row index, one expert's weight, 512 rows of the widest
+    # operand -- and nothing else (activations and outputs of any size are addressed tile by tile)
+    big_rows = (1 << 31) // (2880 * 2) + 1000  # 2880-wide bf16 rows past 2 GiB
+    gather = lib.hmoe_grouped_gemm_fwd_gather
+    assert gather(fake, 2880, big_rows, fake, fake, fake, 64, 4, 2880, 64, bf16, fake, 64, None) == unsupported
+    assert lib.hmoe_grouped_gemm_dgrad_gather(fake, 2880, big_rows, fake, fake, fake, 64, 4, 64, 2880, bf16, fake, 64,
+                                              None) == unsupported
+    assert lib.hmoe_grouped_gemm_wgrad_gather_grad(fake, 64, fake, 2880, big_rows, fake, fake, 64, 4, 64, 2880, bf16,
+                                                   fake, None) == unsupported
+    assert gemm(fake, 40000, fake, fake, 8, 4, 40000, 40000, bf16, fake, 40000, None) == unsupported  # 3 GB per expert
+    assert gemm(fake, 1 << 22, fake, fake, 8, 4, 64, 64, bf16, fake, 64, None) == unsupported  # 8 MiB between rows
+    assert lib.hmoe_grouped_gemm_fwd_fp8w(fake, 2880, fake, fake, fake, big_rows, 4, 2880, 64, fake, 64, None) == unsupported
+
     # fp8 MFMA product: whole scale blocks along K, 16-byte output rows, a scale row for every row
     fp8 = lib.hmoe_grouped_gemm_fwd_fp8
     assert fp8(fake, fake, 8, fake, fake, fake, 8, 4, 200, 128, fake, 128, None) == unsupported
