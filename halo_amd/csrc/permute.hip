@@ -151,7 +151,31 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
     for (int k = 0; k < kTopK; ++k) all_valid = all_valid && valid[k];
     auto reduce_row = [&](auto dense_tag) __attribute__((always_inline)) {
       constexpr bool kDense = decltype(dense_tag)::value;
-      for (int64_t c = static_cast<int64_t>(lane_id()) * W; c < hidden; c += step) {
+      int64_t c = static_cast<int64_t>(lane_id()) * W;
+      if constexpr (kDense && kTopK <= 8) {
+        // two column chunks per pass while the row has them: 2 * kTopK row fetches in flight per lane
+        for (; c + step < hidden; c += 2 * step) {
+          Pack<T, W> x[2][kTopK], acc[2], extra_chunk[2];
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int k = 0; k < kTopK; ++k) x[h][k].load_once(from[k] + c + h * step);
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            if (extra) extra_chunk[h].load(extra + c + h * step);
+#pragma unroll
+            for (int i = 0; i < W; ++i) acc[h].v[i] = 0.f;
+#pragma unroll
+            for (int k = 0; k < kTopK; ++k) {
+#pragma unroll
+              for (int i = 0; i < W; ++i) acc[h].v[i] += kWeighted ? x[h][k].v[i] * w[k] : x[h][k].v[i];
+            }
+            finish(acc[h], extra_chunk[h]);
+            acc[h].store(to + c + h * step);
+          }
+        }
+      }
+      for (; c < hidden; c += step) {
         Pack<T, W> x[kTopK], acc, extra_chunk;
 #pragma unroll
         for (int k = 0; k < kTopK; ++k) {
