@@ -1,5 +1,6 @@
 """The MoE block (route, sort, grouped GLU FFN, combine, shared expert) on one GPU."""
 
+from halo_amd.moe_layer.balancing import expert_load_token_weights  # noqa: F401
 from halo_amd.moe_layer.config import EPConfig, single_process_ep_config  # noqa: F401
 from halo_amd.moe_layer.families import (  # noqa: F401
     MOE_LAYER_MAP,

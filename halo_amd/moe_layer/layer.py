@@ -13,6 +13,7 @@ dispatch/combine exchange, balancing bias, routing replay and expert TP of the r
 from __future__ import annotations
 
 import logging
+import os
 from abc import ABC, abstractmethod
 from collections.abc import Callable
 from typing import ClassVar
@@ -27,12 +28,18 @@ from halo_amd.kernels.moe_permute import (MoEGatherPermute, MoEWeightedUnpermute
                                           warm_permute_kernels)
 from halo_amd.kernels.moe_route_sort import sort_routing_by_expert, warm_route_sort_kernels
 from halo_amd.kernels.router import SOFTMAX_ALL, fused_topk_gate
+from halo_amd.moe_layer.balancing import ExpertLoadMixin
 from halo_amd.moe_layer.config import EPConfig, MoEFamilySpec
 from halo_amd.moe_layer.expert_lora import EXPERT_LORA_SUFFIXES, init_expert_lora
 
 logger = logging.getLogger(__name__)
 
 ROUTER_TOPK_FIELDS = ("top_k", "num_experts_per_tok", "num_experts_per_token")
+
+# Opt-in: the shared expert's FFN on a second stream (of the same, default priority) beside the routed path, joined
+# before the sum; one stream per device.  The reference's HALO_EP_SHARED_OVERLAP (layer.py:31-33, 284-296).
+_SHARED_OVERLAP_ENABLED = os.environ.get("HALO_EP_SHARED_OVERLAP", "").strip().lower() in ("1", "true", "yes", "on")
+_shared_overlap_streams: dict[int, torch.cuda.Stream] = {}
 
 
 class _RouterProjection(torch.autograd.Function):
@@ -99,7 +106,7 @@ def dense_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return grouped_mm(x, weight.unsqueeze(0).transpose(1, 2), offs=None)
 
 
-class EPMoELayerBase(nn.Module, ABC):
+class EPMoELayerBase(ExpertLoadMixin, nn.Module, ABC):
     """Base class of the per-family MoE blocks.  A family fills in the declarations below, implements ``forward`` and
     overrides the ``_adopt_*`` hooks its expert layout needs.  Built from an HF MoE block
     (``cls(original_layer, ep_config)``, what the reference's ``apply_ep_layers`` does), or directly from tensors with
@@ -295,24 +302,29 @@ class EPMoELayerBase(nn.Module, ABC):
 
     def _compute_experts(self, tokens: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor,
                          output_dtype: torch.dtype, *, recv_counts: tuple[int, ...] | None,
-                         addend: tuple[torch.Tensor, torch.Tensor | None] | None = None) -> torch.Tensor:
+                         addend: tuple[torch.Tensor, torch.Tensor | None] | None = None,
+                         addend_ready: "torch.cuda.Stream | None" = None) -> torch.Tensor:
         """``experts``/``weights`` are ``[T, top_k]`` local ids (``-1`` = not this rank's) and gate weights;
         ``recv_counts`` counts per local expert, None at ``ep_size`` 1.  ``addend = (rows [T, H], scale [T] or None)``
-        (not in the reference's signature) is added to the result, ``scale[:, None] * rows``, by the combine kernel."""
+        (not in the reference's signature) is added to the result, ``scale[:, None] * rows``, by the combine kernel;
+        ``addend_ready`` is the stream that produces it, waited for right ahead of that kernel."""
         if tokens.shape[0] == 0:
             return torch.zeros((0, tokens.shape[-1]), device=tokens.device, dtype=output_dtype)
         return self._compute_experts_grouped(tokens, experts, weights, output_dtype, recv_counts=recv_counts,
-                                             addend=addend)
+                                             addend=addend, addend_ready=addend_ready)
 
-    def _compute_experts_grouped(self, tokens, experts, weights, output_dtype, *, recv_counts, addend=None):
+    def _compute_experts_grouped(self, tokens, experts, weights, output_dtype, *, recv_counts, addend=None,
+                                 addend_ready=None):
         """Sort -> grouped GLU FFN -> weighted unpermute."""
         sorted_tokens, offs, sorted_token_idx, sorted_weights, sorted_expert_ids, inv_map = (
             self._sort_tokens_for_grouped_mm(tokens, experts, weights, recv_counts=recv_counts)
         )
         if self._folds_gate_weight(sorted_tokens, output_dtype):
             return self._compute_experts_weight_folded(sorted_tokens, offs, sorted_token_idx, sorted_weights, inv_map,
-                                                       output_dtype, addend)
+                                                       output_dtype, addend, addend_ready)
         expert_out = self._grouped_expert_ffn(sorted_tokens.to(output_dtype), offs, sorted_expert_ids, output_dtype)
+        if addend_ready is not None:
+            torch.cuda.current_stream(tokens.device).wait_stream(addend_ready)
         if addend is not None:
             rows, scale = addend
             return MoEWeightedUnpermuteAdd.apply(
@@ -338,7 +350,7 @@ class EPMoELayerBase(nn.Module, ABC):
                 and down.shape[1] % 8 == 0 and down.shape[2] % 8 == 0)
 
     def _compute_experts_weight_folded(self, sorted_tokens, offs, sorted_token_idx, sorted_weights, inv_map,
-                                       output_dtype, addend):
+                                       output_dtype, addend, addend_ready=None):
         """The same layer with the gate weight moved ahead of the down projection:
         ``sum_k w_k (act_k @ W_down) = sum_k (w_k act_k) @ W_down``.  The GLU kernel writes ``round(w * act)`` (one
         rounding, where the reference rounds ``act`` and applies ``w`` in the combine, ``compute.py:222-242`` +
@@ -350,6 +362,10 @@ class EPMoELayerBase(nn.Module, ABC):
         gate_up = self._expert_proj(sorted_tokens.to(output_dtype), "gate_up_proj", offs, output_dtype)
         weighted = self._fused_glu_mul.packed_weighted(gate_up, sorted_weights.to(output_dtype))
         rows, scale = addend if addend is not None else (None, None)
+        if addend_ready is not None:
+            # the join: the down projection runs ahead of the sum in the same node, so it waits with it (the gate_up
+            # projection and the GLU have overlapped with the shared expert by now)
+            torch.cuda.current_stream(weighted.device).wait_stream(addend_ready)
         return grouped_mm_combine(
             weighted, self._cast_weight("down_proj", output_dtype), offs=offs, row_index=sorted_token_idx,
             inv_map=inv_map, addend=None if rows is None else rows.to(output_dtype),
@@ -484,7 +500,7 @@ class EPMoELayerBase(nn.Module, ABC):
     # ------------------------------------------------------------------------------- dispatch / compute / combine
 
     def _dispatch_compute_combine(self, flat: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor,
-                                  input_dtype: torch.dtype, addend=None) -> torch.Tensor:
+                                  input_dtype: torch.dtype, addend=None, addend_ready=None) -> torch.Tensor:
         """At ``ep_size`` 1 dispatch and combine are the identity; the spans keep the reference's names."""
         if self.ep_size > 1:
             raise NotImplementedError(
@@ -492,11 +508,12 @@ class EPMoELayerBase(nn.Module, ABC):
                 "received rows to _compute_experts(recv_x, recv_topk_idx, recv_topk_weights, dtype, recv_counts=...)"
             )
         self._warm_expert_kernels(flat.device, input_dtype, flat.shape[-1], experts.shape[1])
+        self._record_expert_load(experts)
         with self._perf("ep.dispatch"):
             recv_x, recv_topk_idx, recv_topk_weights, recv_counts = flat, experts, weights, None
         with self._perf("ep.expert_compute"):
             output = self._compute_experts(recv_x, recv_topk_idx, recv_topk_weights, input_dtype,
-                                           recv_counts=recv_counts, addend=addend)
+                                           recv_counts=recv_counts, addend=addend, addend_ready=addend_ready)
         with self._perf("ep.combine"):
             combined = output
         return combined
@@ -504,8 +521,31 @@ class EPMoELayerBase(nn.Module, ABC):
     def _dispatch_compute_combine_shared(self, flat, experts, weights, input_dtype, orig_shape, shared_fn,
                                          shared_parts_fn=None):
         """``routed + shared``.  With ``shared_parts_fn`` (the shared expert's output as ``(rows [T, H], scale [T] or
-        None)``, ``shared = scale[:, None] * rows``) and tokens to route, the sum is taken by the combine kernel."""
-        if shared_parts_fn is not None and self.fuse_shared_into_combine and flat.shape[0] > 0:
+        None)``, ``shared = scale[:, None] * rows``) and tokens to route, the sum is taken by the combine kernel.
+        Under ``HALO_EP_SHARED_OVERLAP`` the shared expert runs on a side stream beside the routed path and the two
+        are joined before the sum (``layer.py:284-296`` of the reference)."""
+        fused = shared_parts_fn is not None and self.fuse_shared_into_combine and flat.shape[0] > 0
+        if shared_fn is not None and _SHARED_OVERLAP_ENABLED and flat.is_cuda:
+            index = flat.device.index if flat.device.index is not None else torch.cuda.current_device()
+            side = _shared_overlap_streams.get(index)
+            if side is None:
+                side = _shared_overlap_streams[index] = torch.cuda.Stream(device=index)  # default priority
+            current = torch.cuda.current_stream(flat.device)
+            side.wait_stream(current)
+            with torch.cuda.stream(side):
+                shared = shared_parts_fn() if fused else shared_fn()
+            if not fused:
+                routed = self._dispatch_compute_combine(flat, experts, weights, input_dtype).view(*orig_shape)
+                current.wait_stream(side)
+                shared.record_stream(current)  # the side stream's tensor stays alive for the sum
+                return routed + shared
+            # the combine kernel takes the shared rows: everything ahead of it overlaps, the join sits in front of it
+            for part in shared:
+                if part is not None:
+                    part.record_stream(current)
+            return self._dispatch_compute_combine(flat, experts, weights, input_dtype, addend=shared,
+                                                  addend_ready=side).view(*orig_shape)
+        if fused:
             return self._dispatch_compute_combine(flat, experts, weights, input_dtype,
                                                   addend=shared_parts_fn()).view(*orig_shape)
         routed = self._dispatch_compute_combine(flat, experts, weights, input_dtype).view(*orig_shape)

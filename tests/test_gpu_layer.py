@@ -480,6 +480,70 @@ def test_shared_expert_added_in_the_combine_kernel(device, cfg, gated):
     _check("grad shared down_proj", grads_b["shared_expert.down_proj.weight"], shared["down_proj"].grad, check_tol)
 
 
+@pytest.mark.parametrize("fuse", (False, True), ids=("tensor_add", "in_combine"))
+def test_shared_expert_on_a_side_stream_changes_no_bit(device, fuse, monkeypatch):
+    """``HALO_EP_SHARED_OVERLAP``: the shared expert runs on a second stream beside the routed path and is joined
+    ahead of the sum.  Same kernels on the same data: output and every gradient equal the single-stream run bit for
+    bit, three steps in a row (a missing join would show as a stale or half-written shared output)."""
+    from halo_amd.moe_layer import layer as layer_module
+
+    cfg = CONFIG2_SMALL
+    inputs = make_layer_inputs(cfg)
+    runs = {}
+    for overlap in (False, True):
+        monkeypatch.setattr(layer_module, "_SHARED_OVERLAP_ENABLED", overlap)
+        layer = _layer_with_shared_expert(cfg, inputs, device, gated=True, fuse=fuse)
+        steps = []
+        for _ in range(3):
+            for p in layer.parameters():
+                p.grad = None
+            x = inputs["x"].to(device).requires_grad_(True)
+            out = layer(x)
+            out.backward(inputs["grad_out"].to(device))
+            torch.cuda.synchronize()
+            steps.append([out.detach(), x.grad] + [p.grad.clone() for _, p in sorted(layer.named_parameters())])
+        assert all(torch.equal(a, b) for later in steps[1:] for a, b in zip(steps[0], later))
+        runs[overlap] = steps[0]
+    assert len(layer_module._shared_overlap_streams) == 1
+    assert all(torch.equal(a, b) for a, b in zip(runs[False], runs[True]))
+
+
+def test_expert_load_counter(device):
+    """``_record_expert_load`` (reference ``balancing_bias.py:200-207``): once ``balancing_biases`` is attached, every
+    grad-enabled training forward adds the router's selection counts to ``expert_load_counter``; evaluation, a
+    ``no_grad`` forward and a layer without the bias leave it alone; a token-weight scope counts tokens by weight."""
+    from halo_amd.kernels.router import fused_topk_gate
+    from halo_amd.moe_layer import expert_load_token_weights
+
+    cfg = CONFIG2_SMALL
+    inputs = make_layer_inputs(cfg)
+    layer = _build_layer(cfg, inputs, device)
+    x = inputs["x"].to(device)
+    layer.train()
+    layer(x)
+    assert layer.expert_load_counter is None  # no balancing bias attached: nothing is counted
+    layer.balancing_biases = torch.zeros(cfg.experts, device=device)
+    with torch.no_grad():
+        idx, _ = fused_topk_gate(layer._linear_router_logits(x), cfg.top_k, normalize=True, eps=0.0)
+    want = torch.bincount(idx.flatten().cpu(), minlength=cfg.experts).float()
+    layer(x)
+    layer(x)
+    assert torch.equal(layer.expert_load_counter.cpu(), 2 * want)
+    with torch.no_grad():
+        layer(x)
+    layer.eval()
+    layer(x)
+    assert torch.equal(layer.expert_load_counter.cpu(), 2 * want)
+    layer.train()
+    token_weights = torch.arange(cfg.tokens, dtype=torch.float32) % 3
+    with expert_load_token_weights(token_weights):
+        layer(x)
+    weighted = torch.zeros(cfg.experts).index_add_(0, idx.flatten().cpu(), token_weights.repeat_interleave(cfg.top_k))
+    assert torch.allclose(layer.expert_load_counter.cpu(), 2 * want + weighted, rtol=1e-6)
+    with pytest.raises(ValueError, match="do not describe this forward"), expert_load_token_weights(token_weights[:5]):
+        layer(x)
+
+
 # ------------------------------------------------------------------------------------------------- expert LoRA
 
 @pytest.mark.parametrize("cfg", (CONFIG2_SMALL, CONFIG4_SMALL), ids=lambda c: c.name)
