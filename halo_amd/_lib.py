@@ -42,6 +42,7 @@ SIGNATURES = {
     "hmoe_router_topk_bwd": (I, [P, I, P, P, L, I, I, I, I, F, P, P]),
     "hmoe_grouped_gemm_fwd": (I, [P, L, P, P, L, I, L, L, I, P, L, P]),
     "hmoe_grouped_gemm_fwd_bias": (I, [P, L, P, P, P, L, I, L, L, I, P, L, P]),
+    "hmoe_grouped_gemm_fwd_addto": (I, [P, L, P, P, L, I, L, L, I, P, L, F, P, L, P]),
     "hmoe_grouped_gemm_dgrad": (I, [P, L, P, P, L, I, L, L, I, P, L, P]),
     "hmoe_grouped_gemm_wgrad": (I, [P, L, P, L, P, L, I, L, L, I, P, P]),
     "hmoe_grouped_gemm_fwd_gather": (I, [P, L, L, P, P, P, L, I, L, L, I, P, L, P]),

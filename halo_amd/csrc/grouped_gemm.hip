@@ -111,6 +111,11 @@ struct GemmArgs {
   int64_t a_rows = 0;                // rows of the array a_index points into
   bool gather_b = false;
   const void* bias = nullptr;        // fwd: [G, N] in the operands' dtype, added to group g's output rows
+  // fwd: out = addend + addend_scale * product, element by element with the roundings of those tensor operations
+  // (an adapter's low-rank delta joining the base projection); rows ld_addend apart, may be the output itself
+  const void* addend = nullptr;
+  int64_t ld_addend = 0;
+  float addend_scale = 1.f;
   // kFwdFp8: both operands are e4m3 bytes in panels of 64 contraction values (A [K/64][a_scale_rows][64],
   // B [G][K/64][N][64]); k counts values
   const uint8_t* a_scale = nullptr;  // [K / 128][a_scale_rows]: the e8m0 exponent of row r's block b at (b, r)
@@ -191,6 +196,20 @@ __device__ __forceinline__ u32x4 add_bf16x8(u32x4 a, u32x4 b) {
     const float lo = __uint_as_float(a[w] << 16) + __uint_as_float(b[w] << 16);
     const float hi = __uint_as_float(a[w] & 0xffff0000u) + __uint_as_float(b[w] & 0xffff0000u);
     out[w] = pack_bf16x2(lo, hi);
+  }
+  return out;
+}
+
+// base + round(scale * product) per bf16 value, each operation rounded to bf16: `base + scale * product` as two tensor
+// operations compute it.
+__device__ __forceinline__ u32x4 scale_add_bf16x8(u32x4 product, u32x4 base, float scale) {
+  u32x4 out;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float lo = bf16_to_f32(f32_to_bf16(__fmul_rn(scale, __uint_as_float(product[w] << 16))));
+    const float hi = bf16_to_f32(f32_to_bf16(__fmul_rn(scale, __uint_as_float(product[w] & 0xffff0000u))));
+    out[w] = pack_bf16x2(__fadd_rn(__uint_as_float(base[w] << 16), lo),
+                         __fadd_rn(__uint_as_float(base[w] & 0xffff0000u), hi));
   }
   return out;
 }
@@ -1082,8 +1101,9 @@ __device__ __forceinline__ void interleave_reads_under_mfmas() {
   }
 }
 
-template <int kMode, typename Cfg, int kGather = 0, bool kBias = false>
+template <int kMode, typename Cfg, int kGather = 0, bool kBias = false, bool kAddTo = false>
 __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmArgs p) {
+  static_assert(!kAddTo || (kMode == kFwd && !kBias), "the scaled sum into an addend belongs to the plain forward");
   static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
   static_assert(!kBias || kMode == kFwd, "the expert bias belongs to the forward product");
   static_assert(kGather >= 0 && kGather <= 2 && (kGather != 2 || kMode == kWgrad), "B is gathered in wgrad only");
@@ -1433,6 +1453,10 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     bf16_t* c_base = kMode == kWgrad ? c + done.g * w_elems : c + (done.row_start + c_row0) * p.ldc;
     const int64_t c_rows = kMode == kWgrad ? p.k : (c_row_lim < BM ? c_row_lim : BM);
     const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(c_base, static_cast<uint32_t>(c_rows * p.ldc * 2));
+    __amdgpu_buffer_rsrc_t addend_rsrc = c_rsrc;
+    if constexpr (kAddTo)
+      addend_rsrc = make_rsrc(static_cast<const bf16_t*>(p.addend) + (done.row_start + c_row0) * p.ld_addend,
+                              static_cast<uint32_t>(c_rows * p.ld_addend * 2));
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
       if (i < live) {
@@ -1461,6 +1485,13 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
           const int col = done.b_out0 + row_b + cc;
           u32x4 v = *reinterpret_cast<const u32x4*>(stage_rows + (rr * kEpiPitch + cc) * 2);
           if constexpr (kBias) v = add_bf16x8(v, bias_chunk);
+          if constexpr (kAddTo) {
+            const uint32_t from = row < c_row_lim && col < done.b_out_lim
+                                      ? static_cast<uint32_t>(row) * static_cast<uint32_t>(p.ld_addend) * 2u + col * 2u
+                                      : kOutOfRange;
+            const u32x4 base = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(addend_rsrc, from, 0, 0));
+            v = scale_add_bf16x8(v, base, p.addend_scale);
+          }
           const uint32_t off = row < c_row_lim && col < done.b_out_lim
                                    ? static_cast<uint32_t>(row) * static_cast<uint32_t>(p.ldc) * 2u + col * 2u
                                    : kOutOfRange;
@@ -1484,6 +1515,7 @@ HMOE_BF16_INSTANCE(kWgrad)
 #undef HMOE_BF16_INSTANCE
 template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, 1>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, 0, true>(GemmArgs);
+template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, 0, false, true>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kDgrad, Config<2, 4, 4, 2>, 1>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kWgrad, Config<2, 4, 4, 2>, 1>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kWgrad, Config<2, 4, 4, 2>, 2>(GemmArgs);
@@ -1893,6 +1925,12 @@ __global__ void __launch_bounds__(256) grouped_gemm_f32_kernel(GemmArgs p) {
       if (r < rows_out && cc < cols_out) {
         float v = acc[i][j];
         if (kMode == kFwd && p.bias != nullptr) v += static_cast<const float*>(p.bias)[static_cast<int64_t>(g) * p.n + cc];
+        if (kMode == kFwd && p.addend != nullptr) {
+          // two roundings, as the tensor operations have them: the multiply must not contract into the add
+#pragma clang fp contract(off)
+          const float scaled = p.addend_scale * v;
+          v = static_cast<const float*>(p.addend)[(s + r) * p.ld_addend + cc] + scaled;
+        }
         out[r * p.ldc + cc] = v;
       }
     }
@@ -1931,7 +1969,7 @@ int launch_staged(const GemmArgs& p, int workgroups_per_cu, hipStream_t stream) 
   return HMOE_OK;
 }
 
-template <int kMode, typename Cfg, int kGather = 0, bool kBias = false>
+template <int kMode, typename Cfg, int kGather = 0, bool kBias = false, bool kAddTo = false>
 int launch_direct(const GemmArgs& p, hipStream_t stream) {
   const int64_t out_cols = kMode == kDgrad ? p.k : p.n;
   const int64_t nt = (out_cols + Cfg::BN - 1) / Cfg::BN;
@@ -1947,7 +1985,7 @@ int launch_direct(const GemmArgs& p, hipStream_t stream) {
   constexpr size_t lds_bytes = kMode == kWgrad
                                    ? 2 * Cfg::kStage * sizeof(bf16_t) + (kGather ? 4 * 2048 : 0)
                                    : (2 * Cfg::BM + 3 * Cfg::BN) * BK * sizeof(bf16_t);
-  auto kernel = grouped_gemm_bf16_kernel<kMode, Cfg, kGather, kBias>;
+  auto kernel = grouped_gemm_bf16_kernel<kMode, Cfg, kGather, kBias, kAddTo>;
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                           static_cast<int>(lds_bytes)) != hipSuccess)
     return HMOE_LAUNCH_FAILED;
@@ -1963,9 +2001,10 @@ int launch(const GemmArgs& p, int dtype, hipStream_t stream) {
     if constexpr (kMode == kFwdFp8W) {
       rc = launch_staged<kMode, Tile>(p, 1, stream);
     } else if constexpr (kMode == kFwd) {
-      rc = p.a_index ? launch_direct<kMode, Tile, 1>(p, stream)
-           : p.bias  ? launch_direct<kMode, Tile, 0, true>(p, stream)
-                     : launch_direct<kMode, Tile>(p, stream);
+      rc = p.a_index  ? launch_direct<kMode, Tile, 1>(p, stream)
+           : p.bias   ? launch_direct<kMode, Tile, 0, true>(p, stream)
+           : p.addend ? launch_direct<kMode, Tile, 0, false, true>(p, stream)
+                      : launch_direct<kMode, Tile>(p, stream);
     } else if constexpr (kMode == kWgrad) {
       rc = !p.a_index ? launch_direct<kMode, Tile>(p, stream)
            : p.gather_b ? launch_direct<kMode, Tile, 2>(p, stream)
@@ -2040,6 +2079,23 @@ int hmoe_grouped_gemm_fwd_bias(const void* a, int64_t lda, const void* b, const 
   if (!a || !b || !out || !bias) return HMOE_INVALID_ARGUMENT;
   if (lda < k || ldo < n) return HMOE_INVALID_ARGUMENT;
   if (dtype == HMOE_BF16 && !aligned16(bias)) return HMOE_UNSUPPORTED;
+  return launch<kFwd>(p, dtype, static_cast<hipStream_t>(stream));
+}
+
+int hmoe_grouped_gemm_fwd_addto(const void* a, int64_t lda, const void* b, const int32_t* offs, int64_t total_rows,
+                                int num_groups, int64_t k, int64_t n, int dtype, const void* addend,
+                                int64_t ld_addend, float scale, void* out, int64_t ldo, void* stream) {
+  using namespace hmoe;
+  GemmArgs p{a, lda, b, n, out, ldo, offs, total_rows, num_groups, k, n, nullptr};
+  p.addend = addend;
+  p.ld_addend = ld_addend;
+  p.addend_scale = scale;
+  if (int rc = validate(p, dtype)) return rc;
+  if (total_rows == 0 || n == 0) return HMOE_OK;
+  if (!a || !b || !out || !addend) return HMOE_INVALID_ARGUMENT;
+  if (lda < k || ldo < n || ld_addend < n) return HMOE_INVALID_ARGUMENT;
+  if (dtype == HMOE_BF16 && (!aligned16(addend) || ld_addend % 8 || ld_addend * 2 * 512 >= (int64_t(1) << 31)))
+    return HMOE_UNSUPPORTED;
   return launch<kFwd>(p, dtype, static_cast<hipStream_t>(stream));
 }
 

@@ -199,6 +199,63 @@ def grouped_mm_bias(mat_a, mat_b, bias, *, offs, eids):
     return _GroupedMMBias.apply(mat_a, mat_b, bias, offs, eids)
 
 
+# --------------------------------------------------------------------------- a scaled product added to a tensor
+
+class _GroupedMMAddTo(Function):
+    """``addend + scale * grouped_mm(mat_a, mat_b, offs)`` as one node: the product's epilogue multiplies by ``scale``
+    and adds ``addend`` (``hmoe_grouped_gemm_fwd_addto``), rounding where the tensor operations round, so the result
+    carries their bits and neither the product nor its multiple is written.  The adapted expert projection of the
+    reference, ``out + scaling * grouped_mm(hidden, lora_b)`` (``compute.py:283-294``), with ``mat_a`` the adapter's
+    low-rank activations.  The gradients are those operations' own: ``grad_addend = grad_out``, and the product's two
+    gradients over ``scale * grad_out``."""
+
+    @staticmethod
+    def forward(ctx, mat_a, mat_b, addend, scale, offs):
+        device = _lib.require_device(mat_a, mat_b, addend, offs)
+        groups, k, n = mat_b.shape
+        rows = mat_a.shape[0]
+        offs32 = _offs_arg(offs, groups)
+        ctx.scale = float(scale)
+        ctx.save_for_backward(mat_a, mat_b, offs32)
+        out = torch.empty((rows, n), dtype=mat_a.dtype, device=device)
+        if rows == 0 or n == 0:
+            return out
+        a, base = _rows(mat_a), _rows(addend)
+        with _lib.on_device(device):
+            _lib.call("hmoe_grouped_gemm_fwd_addto", _lib.ptr(a), a.stride(0), _lib.ptr(mat_b), _lib.ptr(offs32), rows,
+                      groups, k, n, _lib.dtype_id(mat_a.dtype), _lib.ptr(base), base.stride(0), ctx.scale,
+                      _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        mat_a, mat_b, offs32 = ctx.saved_tensors
+        grad_a = grad_b = None
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            scaled = grad_output * ctx.scale  # the gradient of `scale * product`, rounded as autograd rounds it
+            grad_a, grad_b = grouped_mm_grads(mat_a, mat_b, scaled, offs32, ctx.needs_input_grad[0],
+                                              ctx.needs_input_grad[1])
+        return grad_a, grad_b, grad_output if ctx.needs_input_grad[2] else None, None, None
+
+
+def addto_fusable(mat_a: torch.Tensor, mat_b, addend) -> bool:
+    """Whether :func:`grouped_mm_addto` can take these operands: a plain contiguous ``[G, K, N]`` weight and an
+    ``[R, N]`` addend on the device, all of ``mat_a``'s dtype (bf16 or fp32), rows of 16-byte multiples in bf16."""
+    if not (isinstance(mat_b, torch.Tensor) and isinstance(addend, torch.Tensor) and isinstance(mat_a, torch.Tensor)
+            and mat_a.is_cuda and mat_a.dtype in (torch.bfloat16, torch.float32) and mat_b.dtype == mat_a.dtype
+            and addend.dtype == mat_a.dtype and mat_a.dim() == 2 and mat_b.dim() == 3 and mat_b.is_contiguous()
+            and addend.dim() == 2 and addend.shape == (mat_a.shape[0], mat_b.shape[2])
+            and mat_a.shape[1] == mat_b.shape[1]):
+        return False
+    return mat_a.dtype == torch.float32 or (mat_b.shape[1] % 8 == 0 and mat_b.shape[2] % 8 == 0)
+
+
+def grouped_mm_addto(mat_a, mat_b, addend, scale: float, *, offs):
+    """``addend + scale * grouped_mm(mat_a, mat_b, offs=offs)``; see :class:`_GroupedMMAddTo` and
+    :func:`addto_fusable`."""
+    return _GroupedMMAddTo.apply(mat_a, mat_b, addend, scale, offs)
+
+
 # ------------------------------------------------------------------------------------- permute folded into the GEMM
 
 def gather_fusable(tokens: torch.Tensor, mat_b) -> bool:

@@ -23,7 +23,8 @@ import torch.nn as nn
 
 from halo_amd.kernels.expert_gemm import BlockFp8Weight, expert_gemm, fp8_mfma_usable
 from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled, resolve_fused_glu_mul
-from halo_amd.kernels.grouped_mm import GatheredRows, grouped_mm, grouped_mm_combine, grouped_wgrad
+from halo_amd.kernels.grouped_mm import (GatheredRows, addto_fusable, grouped_mm, grouped_mm_addto,
+                                         grouped_mm_combine, grouped_wgrad)
 from halo_amd.kernels.moe_permute import (MoEGatherPermute, MoEWeightedUnpermute, MoEWeightedUnpermuteAdd,
                                           warm_permute_kernels)
 from halo_amd.kernels.moe_route_sort import sort_routing_by_expert, warm_route_sort_kernels
@@ -208,6 +209,8 @@ class EPMoELayerBase(ExpertLoadMixin, nn.Module, ABC):
         self.fuse_permute_into_gemm = True
         # the shared expert's output joins the routed one in the combine kernel instead of a tensor addition
         self.fuse_shared_into_combine = True
+        # an adapted projection adds its low-rank delta in the second adapter product's epilogue
+        self.fuse_lora_into_gemm = True
         # the gate weights multiply the GLU's output instead of the down projection's: the combine becomes a plain
         # sum and its backward writes no [R, H] gradient (see _compute_experts_weight_folded)
         self.fold_gate_weight_into_glu = True
@@ -410,11 +413,21 @@ class EPMoELayerBase(ExpertLoadMixin, nn.Module, ABC):
         if self._adapted(weight_attr):
             # x @ W + scaling * (dropout(x) @ A) @ B, the adapter products in the activation dtype whatever the
             # base weight is stored in (a scale block along a rank of 8-64 means nothing)
-            rows = x.materialize() if isinstance(x, GatheredRows) else x
-            base = self._grouped_mm(rows, self._cast_weight(weight_attr, out_dtype), offs=offs)
             lora_a = getattr(self, weight_attr + EXPERT_LORA_SUFFIXES[0]).to(out_dtype)
             lora_b = getattr(self, weight_attr + EXPERT_LORA_SUFFIXES[1]).to(out_dtype)
-            low = self._grouped_mm(self.expert_lora_dropout(rows), lora_a, offs=offs, lowp=False)
+            weight = self._cast_weight(weight_attr, out_dtype)
+            base = low = None
+            drops = isinstance(self.expert_lora_dropout, nn.Dropout) and self.training and self.expert_lora_dropout.p > 0
+            if isinstance(x, GatheredRows) and not drops and self._lowp_quant_format is None:
+                # both readers of the rows fetch them through the sort's index: no permuted copy for the adapters
+                base, low = x.grouped_mm(weight, offs=offs), x.grouped_mm(lora_a, offs=offs)
+            if base is None or low is None:
+                rows = x.materialize() if isinstance(x, GatheredRows) else x
+                base = self._grouped_mm(rows, weight, offs=offs)
+                low = self._grouped_mm(self.expert_lora_dropout(rows), lora_a, offs=offs, lowp=False)
+            if self.fuse_lora_into_gemm and addto_fusable(low, lora_b, base):
+                # the delta joins the base projection in the second adapter product's epilogue: the same bits
+                return grouped_mm_addto(low, lora_b, base, self.expert_lora_scaling, offs=offs)
             return base + self.expert_lora_scaling * self._grouped_mm(low, lora_b, offs=offs, lowp=False)
         weight = self._cast_weight(weight_attr, out_dtype)
         if isinstance(x, GatheredRows):

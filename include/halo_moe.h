@@ -191,6 +191,15 @@ int hmoe_grouped_gemm_fwd_bias(const void* a, int64_t lda, const void* b, const 
                                int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype, void* out,
                                int64_t ldo, void* stream);
 
+/* The forward product scaled and added to an existing [total_rows, n] tensor: out = addend + scale * (a[s:e] @ b[g]),
+ * element by element with the roundings of those tensor operations (the product to dtype, its multiple by scale to
+ * dtype, the sum to dtype).  Replaces the `out + scaling * grouped_mm(hidden, lora_b)` of the adapted expert projection
+ * (halo/distributed/expert_parallel/moe_layer/compute.py:283-294): the low-rank delta joins the base projection in the
+ * second adapter product's epilogue, so neither the delta nor its multiple is written.  out may be addend itself. */
+int hmoe_grouped_gemm_fwd_addto(const void* a, int64_t lda, const void* b, const int32_t* offs, int64_t total_rows,
+                                int num_groups, int64_t k, int64_t n, int dtype, const void* addend,
+                                int64_t ld_addend, float scale, void* out, int64_t ldo, void* stream);
+
 /* The same two GEMMs with the rows of A gathered: logical row r of A is a[row_index[r]], a holding a_rows rows; an
  * index outside [0, a_rows) reads as a row of zeros.  This folds MoEGatherPermute.forward
  * (halo/kernels/moe_permute.py:133-136, tokens.index_select(0, sorted_token_idx)) into the first expert GEMM and its

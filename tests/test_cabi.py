@@ -95,6 +95,11 @@ def test_bad_arguments_come_back_as_status_codes_before_any_launch():
     assert gemm(None, 64, None, None, 0, 1, 64, 64, bf16, None, 64, None) == 0  # no rows: nothing to do
     assert lib.hmoe_grouped_gemm_fwd_bias(fake, 64, fake, None, fake, 8, 4, 64, 64, bf16, fake, 64, None) == invalid
     assert lib.hmoe_grouped_gemm_fwd_gather(fake, 64, 8, fake, fake, fake, 8, 4, 64, 64, f32, fake, 64, None) == unsupported
+    addto = lib.hmoe_grouped_gemm_fwd_addto
+    assert addto(fake, 64, fake, fake, 8, 4, 64, 64, bf16, None, 64, 2.0, fake, 64, None) == invalid  # no addend
+    assert addto(fake, 64, fake, fake, 8, 4, 64, 64, bf16, fake, 32, 2.0, fake, 64, None) == invalid  # addend rows overlap
+    assert addto(fake, 64, fake, fake, 8, 4, 64, 64, bf16, fake, 68, 2.0, fake, 64, None) == unsupported  # 136-byte rows
+    assert addto(fake, 64, fake, fake, 8, 4, 64, 64, bf16, fake + 2, 64, 2.0, fake, 64, None) == unsupported
     assert lib.hmoe_grouped_gemm_fwd_gather(fake, 64, -3, fake, fake, fake, 8, 4, 64, 64, bf16, fake, 64, None) == invalid
 
     # what must stay below 2 GiB: an array gathered from by row index, one expert's weight, 512 rows of the widest

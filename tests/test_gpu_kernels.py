@@ -963,3 +963,30 @@ class _PlainCombine(torch.autograd.Function):
     def backward(ctx, grad_out):
         (row_index,) = ctx.saved_tensors
         return grad_out[row_index].contiguous(), None, None
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float32), ids=("bf16", "fp32"))
+@pytest.mark.parametrize(("counts", "k", "n"), (((255, 256, 257, 0, 513, 31), 16, 264), ((64,) * 16, 64, 1536),
+                                                 ((300, 0, 41), 8, 520)))
+def test_grouped_mm_added_to_a_tensor_equals_the_tensor_operations(device, dtype, counts, k, n):
+    """``grouped_mm_addto``: ``addend + scale * grouped_mm(a, b)`` with the product scaled and added in the GEMM's
+    epilogue.  The roundings sit where the tensor operations have them, so the output and all three gradients equal
+    the unfused expression bit for bit; the contraction lengths are adapter ranks."""
+    from halo_amd.kernels.grouped_mm import addto_fusable, grouped_mm, grouped_mm_addto
+
+    g = torch.Generator().manual_seed(17)
+    rows, scale = sum(counts), 32.0 / 24.0  # a scale that is not a power of two: its rounding shows
+    a = torch.randn(rows, k, generator=g).to(dtype).to(device)
+    b = (torch.randn(len(counts), k, n, generator=g) * 0.2).to(dtype).to(device)
+    base = torch.randn(rows, n, generator=g).to(dtype).to(device)
+    dout = torch.randn(rows, n, generator=g).to(dtype).to(device)
+    offs = _offsets(counts, device)
+    assert addto_fusable(a, b, base)
+    results = []
+    for fused in (False, True):
+        ad, bd, cd = (t.clone().requires_grad_(True) for t in (a, b, base))
+        out = grouped_mm_addto(ad, bd, cd, scale, offs=offs) if fused else cd + scale * grouped_mm(ad, bd, offs=offs)
+        out.backward(dout)
+        results.append((out.detach(), ad.grad, bd.grad, cd.grad))
+    for name, x, y in zip(("out", "grad_a", "grad_b", "grad_addend"), *results):
+        assert torch.equal(x, y), name

@@ -630,6 +630,45 @@ def test_expert_lora_equals_the_layer_with_merged_weights(device, cfg):
         assert getattr(layer, attr).grad is None
 
 
+@pytest.mark.parametrize("cfg", (CONFIG2_SMALL, CONFIG4_SMALL), ids=lambda c: c.name)
+def test_expert_lora_delta_added_in_the_gemm_epilogue_changes_no_bit(device, cfg):
+    """With adapters the projection's low-rank delta is added by the second adapter product's epilogue, and on a
+    fused-GLU layer both readers of the token rows fetch them through the sort's index.  Output and every gradient
+    equal the three-products-and-two-tensor-operations form bit for bit."""
+    from halo_amd.moe_layer import EPGptOssMoELayer, EPQwen3_5MoELayer, ExpertLoraSpec
+    from halo_amd.moe_layer.config import EPConfig
+
+    inputs = make_layer_inputs(cfg)
+    runs = []
+    for fuse in (False, True):
+        params = {k: v.to(device) for k, v in inputs["params"].items()}
+        ep = EPConfig(expert_lora=ExpertLoraSpec(r=16, alpha=24.0))
+        if cfg.router == "softmax_topk":
+            params = {k.replace("gate_proj", "gate_proj_gmm").replace("up_proj", "up_proj_gmm"): v
+                      for k, v in params.items()}
+            layer = EPGptOssMoELayer.from_weights(
+                router_weight=inputs["router_weight"].to(device), top_k=cfg.top_k, ep_config=ep,
+                router_bias=inputs.get("router_bias", torch.zeros(cfg.experts)).to(device), **params)
+        else:
+            layer = EPQwen3_5MoELayer.from_weights(router_weight=inputs["router_weight"].to(device), top_k=cfg.top_k,
+                                                   ep_config=ep, **params)
+        g = torch.Generator().manual_seed(5)
+        with torch.no_grad():
+            for attr in sorted(layer._expert_lora_attrs):
+                for suffix in ("_lora_A", "_lora_B"):
+                    p = getattr(layer, attr + suffix)
+                    p.copy_((torch.randn(p.shape, generator=g) * 0.05).to(p.dtype))
+        layer.fuse_lora_into_gemm = fuse
+        x = inputs["x"].to(device).requires_grad_(True)
+        out = layer(x)
+        out = out[0] if isinstance(out, tuple) else out
+        out.backward(inputs["grad_out"].to(device))
+        grads = {name: p.grad for name, p in layer.named_parameters() if p.grad is not None}
+        runs.append({"out": out.detach(), "grad_x": x.grad, **grads})
+    assert runs[0].keys() == runs[1].keys() and len(runs[0]) >= 6
+    assert [name for name in runs[0] if not torch.equal(runs[0][name], runs[1][name])] == []
+
+
 def test_expert_lora_rank_must_span_whole_rows(device):
     from halo_amd.moe_layer import EPQwen3_5MoELayer, ExpertLoraSpec
     from halo_amd.moe_layer.config import EPConfig
