@@ -55,6 +55,10 @@ SIGNATURES = {
     "hmoe_quantize_rows_fp8": (I, [P, L, P, L, L, L, P, P, L, P]),
     "hmoe_glu_fwd_quant_fp8": (I, [P, P, L, L, L, L, I, F, F, I, I, P, P, L, P]),
     "hmoe_grouped_gemm_fwd_fp8": (I, [P, P, L, P, P, P, L, I, L, L, P, L, P]),
+    "hmoe_quantize_rows_mxfp8": (I, [P, I, L, P, L, L, L, P, P, L, P]),
+    "hmoe_dequantize_rows_mxfp8": (I, [P, P, L, L, L, P, L, P]),
+    "hmoe_quantize_weight_mxfp8": (I, [P, I, L, L, L, P, P, P, P]),
+    "hmoe_grouped_gemm_fwd_mxfp8": (I, [P, P, L, P, P, P, L, I, L, L, P, L, P]),
 }
 
 _lib = None

@@ -121,6 +121,9 @@ struct GemmArgs {
   const uint8_t* a_scale = nullptr;  // [K / 128][a_scale_rows]: the e8m0 exponent of row r's block b at (b, r)
   int64_t a_scale_rows = 0;
   int k_blocks = 0, n_blocks = 0;     // the grid of b_scale [G, k_blocks, n_blocks]
+  // kFwdFp8 with one e8m0 exponent per 32 contraction values on both sides (MXFP8): a_scale is [K / 32][a_scale_rows]
+  // and the weights' exponents are bytes [G][K / 32][N]
+  const uint8_t* b_scale_e8m0 = nullptr;
 };
 
 __device__ __forceinline__ int swizzle(int row) { return (row & 7) ^ ((row >> 3) & 7); }
@@ -1534,10 +1537,17 @@ constexpr int kF8Stages = 4;
 constexpr int kF8K = 64;                              // contraction values (bytes) per stage
 constexpr int kF8Tile = 256 * kF8K;                   // one operand's share of a stage
 constexpr int kF8Stage = 2 * kF8Tile;
-constexpr int kF8ScaleA = 256 * 4, kF8ScaleB = 64 * 4;  // a dword per tile row; 64 dwords of weight scales
 constexpr int kF8ScaleBase = kF8Stages * kF8Stage;
-constexpr int kF8Lds = kF8ScaleBase + kF8Stages * (kF8ScaleA + kF8ScaleB);
-constexpr int kF8LoadsPerStage = 10;                  // per loading wavefront: 4 + 4 tile loads, 2 scale loads
+// The scales of a stage.  Block scales (kMx false): a dword per tile row holding the row's exponent for the stage's
+// 128-value block, and 64 dwords of weight scales.  MXFP8 (kMx true): an exponent per 32 values on both sides, so a
+// stage (64 values) carries two planes of 256 dwords per operand, plane h for the stage's contraction half h.
+template <bool kMx>
+struct F8Scales {
+  static constexpr int kA = kMx ? 2 * 256 * 4 : 256 * 4;
+  static constexpr int kB = kMx ? 2 * 256 * 4 : 64 * 4;
+  static constexpr int kLds = kF8ScaleBase + kF8Stages * (kA + kB);
+  static constexpr int kLoads = kMx ? 12 : 10;  // per loading wavefront and stage: 4 + 4 tile loads, then the scales
+};
 
 __device__ __forceinline__ void lds_load4(u32x4 rsrc, lds_bytes_ptr lds_base, uint32_t voffset, uint32_t soffset) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
@@ -1555,8 +1565,10 @@ __device__ __forceinline__ void lds_load1(u32x4 rsrc, lds_bytes_ptr lds_base, ui
                : "memory", "m0");
 }
 
+template <bool kMx>
 __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
   constexpr int WM = 4, WN = 2, BM = 256, BN = 256, kLoadWaves = 4;
+  constexpr int kF8ScaleA = F8Scales<kMx>::kA, kF8ScaleB = F8Scales<kMx>::kB;
   using Sched = TileSchedule<kFwd, BM, BN>;
   extern __shared__ __attribute__((aligned(16))) char lds_raw[];
   __shared__ int32_t grp_s[kMaxGroups], grp_e[kMaxGroups], tile_start[kMaxGroups + 1];
@@ -1616,7 +1628,11 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
       rsrc_a = make_rsrc_words(a, static_cast<uint32_t>(steps) * a_panel - static_cast<uint32_t>(tile.row_start) * kF8K);
       rsrc_b = make_rsrc_words(static_cast<const uint8_t*>(p.b) + tile.g * w_bytes, static_cast<uint32_t>(w_bytes));
       rsrc_sa = make_rsrc_words(p.a_scale, static_cast<uint32_t>(p.k_blocks) * static_cast<uint32_t>(p.a_scale_rows));
-      rsrc_sb = make_rsrc_words(p.b_scale, static_cast<uint32_t>(p.groups) * p.k_blocks * p.n_blocks * 4u);
+      if constexpr (kMx)
+        rsrc_sb = make_rsrc_words(p.b_scale_e8m0 + static_cast<int64_t>(tile.g) * p.k_blocks * p.n,
+                                  static_cast<uint32_t>(p.k_blocks) * static_cast<uint32_t>(p.n));
+      else
+        rsrc_sb = make_rsrc_words(p.b_scale, static_cast<uint32_t>(p.groups) * p.k_blocks * p.n_blocks * 4u);
       voff_a = static_cast<uint32_t>(tile.a_out0 + slot * 64) * kF8K + lane_off;
       voff_b = static_cast<uint32_t>(tile.b_out0 + slot * 64) * kF8K + lane_off;
       // the dword this lane's byte lands in is d = 64 slot + lane; it takes the scale of tile row
@@ -1624,12 +1640,19 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
       // one 16-byte read
       const int d = slot * 64 + lane;
       voff_sa = static_cast<uint32_t>(tile.row_start + tile.a_out0 + (d >> 7) * 128 + (d & 3) * 32 + ((d & 127) >> 2));
-      int nb = (tile.b_out0 >> 7) + (lane & 1);
-      nb = nb < p.n_blocks ? nb : p.n_blocks - 1;
-      voff_sb = (static_cast<uint32_t>(tile.g) * p.k_blocks * p.n_blocks + nb) * 4u;
+      if constexpr (kMx) {
+        // the weights' plane: dword d takes tile column (d >> 6) * 64 + (d & 1) * 32 + ((d & 63) >> 1), so that the two
+        // column blocks of a wavefront's lane lie in one 8-byte read.  A column past N reads another column's
+        // exponent (or zero past the group's end) and reaches only outputs that are not stored.
+        voff_sb = static_cast<uint32_t>(tile.b_out0 + (d >> 6) * 64 + (d & 1) * 32 + ((d & 63) >> 1));
+      } else {
+        int nb = (tile.b_out0 >> 7) + (lane & 1);
+        nb = nb < p.n_blocks ? nb : p.n_blocks - 1;
+        voff_sb = (static_cast<uint32_t>(tile.g) * p.k_blocks * p.n_blocks + nb) * 4u;
+      }
     }
   };
-  // stage `step` of the described tile into buffer step & 3: always kF8LoadsPerStage loads, so that the waits below
+  // stage `step` of the described tile into buffer step & 3: always F8Scales<kMx>::kLoads loads, so that the waits below
   // can count them
   auto issue = [&](int step) __attribute__((always_inline)) {
     const int buf = step & (kF8Stages - 1);
@@ -1640,20 +1663,38 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) lds_load16(rsrc_b, ta + kF8Tile + t * 1024, voff_b + t * 1024, soff_b);
     lds_bytes_ptr sc = lds + kF8ScaleBase + buf * (kF8ScaleA + kF8ScaleB);
-    lds_load1(rsrc_sa, sc + slot * 256, voff_sa, static_cast<uint32_t>(step >> 1) * static_cast<uint32_t>(p.a_scale_rows));
-    lds_load4(rsrc_sb, sc + kF8ScaleA, voff_sb, static_cast<uint32_t>(step >> 1) * static_cast<uint32_t>(p.n_blocks) * 4u);
+    if constexpr (kMx) {
+      const uint32_t rows_a = static_cast<uint32_t>(p.a_scale_rows), cols_b = static_cast<uint32_t>(p.n);
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        lds_load1(rsrc_sa, sc + h * 1024 + slot * 256, voff_sa, static_cast<uint32_t>(2 * step + h) * rows_a);
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        lds_load1(rsrc_sb, sc + kF8ScaleA + h * 1024 + slot * 256, voff_sb, static_cast<uint32_t>(2 * step + h) * cols_b);
+    } else {
+      lds_load1(rsrc_sa, sc + slot * 256, voff_sa, static_cast<uint32_t>(step >> 1) * static_cast<uint32_t>(p.a_scale_rows));
+      lds_load4(rsrc_sb, sc + kF8ScaleA, voff_sb, static_cast<uint32_t>(step >> 1) * static_cast<uint32_t>(p.n_blocks) * 4u);
+    }
   };
 
   // ---- the computing view
-  const int frag_chunk = ((lane >> 5) ^ ((lane >> 1) & 3) ^ ((lane >> 3) & 1)) << 4;
+  // A lane of half h = lane >> 5 holds its row's contraction values [16 h, 16 h + 16) in its first four registers and
+  // [32 + 16 h, 48 + 16 h) in the other four: logical chunks h and h ^ 2.  That is the instruction's own layout, which
+  // shows once a scale differs between the two blocks of 32: registers 0-3 of either half are scaled by the exponent
+  // that the row's lane of half 0 supplies and registers 4-7 by the one the lane of half 1 supplies, so lane
+  // (row, h) must supply the exponent of block h, whatever values it holds itself.
+  const int half = lane >> 5;
+  const int frag_chunk = (half ^ ((lane >> 1) & 3) ^ ((lane >> 3) & 1)) << 4;
+  constexpr int kPartner = 32;
   const int fa0 = (row_a + (lane & 31)) * kF8K + frag_chunk;
   const int fb0 = kF8Tile + (row_b + (lane & 31)) * kF8K + frag_chunk;
-  const int sa_at = kF8ScaleBase + (row_a + (lane & 31) * 4) * 4;
-  const int sb_at = kF8ScaleBase + kF8ScaleA + (gn >> 1) * 4;
+  const int sa_at = kF8ScaleBase + (kMx ? half * 1024 : 0) + (row_a + (lane & 31) * 4) * 4;
+  const int sb_at = kMx ? kF8ScaleBase + kF8ScaleA + half * 1024 + (row_b + (lane & 31) * 2) * 4
+                        : kF8ScaleBase + kF8ScaleA + (gn >> 1) * 4;
   i32x8 fa8[WM], fb8[WN];
   auto fragment = [&](int at) __attribute__((always_inline)) {
     const i32x4 lo = *reinterpret_cast<const i32x4*>(lds_raw + at);
-    const i32x4 hi = *reinterpret_cast<const i32x4*>(lds_raw + (at ^ 32));
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(lds_raw + (at ^ kPartner));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
   // epilogue staging in buffer 3, one 32 x 32 block at a time per wavefront
@@ -1701,7 +1742,12 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
       const char* sc = lds_raw + buf * (kF8ScaleA + kF8ScaleB);
       const u32x4 q = *reinterpret_cast<const u32x4*>(sc + sa_at);
       sa_pack = (q[0] & 0xffu) | ((q[1] & 0xffu) << 8) | ((q[2] & 0xffu) << 16) | (q[3] << 24);
-      sb_bits = *reinterpret_cast<const uint32_t*>(sc + sb_at);
+      if constexpr (kMx) {
+        const u32x2 w = *reinterpret_cast<const u32x2*>(sc + sb_at);
+        sb_bits = (w[0] & 0xffu) | ((w[1] & 0xffu) << 8);  // the lane's exponents for its two column blocks
+      } else {
+        sb_bits = *reinterpret_cast<const uint32_t*>(sc + sb_at);
+      }
     };
     {
 #pragma unroll
@@ -1717,7 +1763,7 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
       auto mfma = [&](auto row_block, auto col_block, int sa, int sb) __attribute__((always_inline)) {
         constexpr int i = decltype(row_block)::value, j = decltype(col_block)::value;
         if (kFull || i < live)
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[j], fa8[i], acc[i][j], 0, 0, 0, sb, i, sa);
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[j], fa8[i], acc[i][j], 0, 0, kMx ? j : 0, sb, i, sa);
       };
       using std::integral_constant;
       const integral_constant<int, 0> b0;
@@ -1728,20 +1774,26 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
         const int buf = step & (kF8Stages - 1), nbuf = (step + 1) & (kF8Stages - 1);
         // the weight scale: exponent to the MFMA, mantissa carried by the accumulators (1 for power-of-two scales);
         // zero or subnormal goes in as 2^-127 with mantissa 1 and contributes nothing either way
-        const uint32_t bits = uniform(sb_bits);
-        const uint32_t sb_exp = bits >> 23;
-        const float mant = sb_exp ? __uint_as_float((bits & 0x007fffffu) | 0x3f800000u) : 1.0f;
-        if (mant != mant_last) {
-          const float ratio = mant_last / mant;
+        int sb;
+        if constexpr (kMx) {
+          sb = static_cast<int>(sb_bits);  // a byte per column block, picked by the instruction's operand select
+        } else {
+          const uint32_t bits = uniform(sb_bits);
+          const uint32_t sb_exp = bits >> 23;
+          const float mant = sb_exp ? __uint_as_float((bits & 0x007fffffu) | 0x3f800000u) : 1.0f;
+          if (mant != mant_last) {
+            const float ratio = mant_last / mant;
 #pragma unroll
-          for (int i = 0; i < WM; ++i)
+            for (int i = 0; i < WM; ++i)
 #pragma unroll
-            for (int j = 0; j < WN; ++j)
+              for (int j = 0; j < WN; ++j)
 #pragma unroll
-              for (int v = 0; v < 16; ++v) acc[i][j][v] *= ratio;
-          mant_last = mant;
+                for (int v = 0; v < 16; ++v) acc[i][j][v] *= ratio;
+            mant_last = mant;
+          }
+          sb = static_cast<int>(sb_exp);
         }
-        const int sa = static_cast<int>(sa_pack), sb = static_cast<int>(sb_exp);
+        const int sa = static_cast<int>(sa_pack);
         __builtin_amdgcn_sched_barrier(0);
         mfma(b0, b0, sa, sb);
         mfma(b1, b0, sa, sb);
@@ -1755,9 +1807,16 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
         // stage step + 1 must be in: the loads of at most two younger stages may still be out
         const int younger = steps - 2 - step;
         if (load_wave) {
-          if (younger >= 2) asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)" ::: "memory");
-          else if (younger == 1) asm volatile("s_waitcnt vmcnt(10) lgkmcnt(0)" ::: "memory");
-          else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+          static_assert(F8Scales<false>::kLoads == 10 && F8Scales<true>::kLoads == 12, "the waits below count them");
+          if (younger >= 2) {
+            if constexpr (kMx) asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)" ::: "memory");
+          } else if (younger == 1) {
+            if constexpr (kMx) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(10) lgkmcnt(0)" ::: "memory");
+          } else {
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+          }
         } else {
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         }
@@ -1787,7 +1846,7 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
     };
     if (live == WM) run(std::true_type{});
     else run(std::false_type{});
-    if (mant_last != 1.0f) {
+    if (!kMx && mant_last != 1.0f) {
 #pragma unroll
       for (int i = 0; i < WM; ++i)
 #pragma unroll
@@ -2052,6 +2111,18 @@ int validate(const GemmArgs& p, int dtype) {
   return HMOE_OK;
 }
 
+template <bool kMx>
+int launch_fp8(const GemmArgs& p, int64_t workers, void* stream) {
+  constexpr int kLds = F8Scales<kMx>::kLds;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_fp8_kernel<kMx>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
+    return HMOE_LAUNCH_FAILED;
+  grouped_gemm_fp8_kernel<kMx><<<dim3(static_cast<unsigned>(workers)), dim3(512), kLds,
+                                static_cast<hipStream_t>(stream)>>>(p);
+  if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
+  return HMOE_OK;
+}
+
 }  // namespace
 }  // namespace hmoe
 
@@ -2206,12 +2277,43 @@ int hmoe_grouped_gemm_fwd_fp8(const uint8_t* a_q, const uint8_t* a_scale, int64_
   int64_t workers = device_cus();
   if (bound < workers) workers = bound;
   workers = (workers + kXcds - 1) / kXcds * kXcds;
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_fp8_kernel),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, kF8Lds) != hipSuccess)
-    return HMOE_LAUNCH_FAILED;
-  grouped_gemm_fp8_kernel<<<dim3(static_cast<unsigned>(workers)), dim3(512), kF8Lds, static_cast<hipStream_t>(stream)>>>(p);
-  if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
-  return HMOE_OK;
+  return launch_fp8<false>(p, workers, stream);
+}
+
+int hmoe_grouped_gemm_fwd_mxfp8(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
+                                const uint8_t* b_scale, const int32_t* offs, int64_t total_rows, int num_groups,
+                                int64_t k, int64_t n, void* out, int64_t ldo, void* stream) {
+  using namespace hmoe;
+  if (total_rows < 0 || num_groups <= 0 || k < 0 || n < 0) return HMOE_INVALID_ARGUMENT;
+  if (offs == nullptr && num_groups != 1) return HMOE_INVALID_ARGUMENT;
+  if (num_groups > kMaxGroups) return HMOE_UNSUPPORTED;
+  // whole panels of 64 values along the contraction; 16-byte rows on both sides
+  if (k % 64 || n % 8 || ldo % 8 || ldo < n || a_rows < total_rows) return HMOE_UNSUPPORTED;
+  if (total_rows == 0 || n == 0) return HMOE_OK;
+  if (k == 0) return HMOE_UNSUPPORTED;
+  if (!a_q || !a_scale || !bq || !b_scale || !out) return HMOE_INVALID_ARGUMENT;
+  if (!aligned16(a_q) || !aligned16(bq) || !aligned16(out)) return HMOE_UNSUPPORTED;
+  const int64_t lim = int64_t(1) << 31;
+  if (a_rows * k >= lim || k * n >= lim || total_rows * ldo * 2 >= lim) return HMOE_UNSUPPORTED;
+  GemmArgs p{};
+  p.a = a_q;
+  p.b = bq;
+  p.c = out;
+  p.ldc = ldo;
+  p.offs = offs;
+  p.total_rows = total_rows;
+  p.groups = num_groups;
+  p.k = k;
+  p.n = n;
+  p.b_scale_e8m0 = b_scale;
+  p.a_scale = a_scale;
+  p.a_scale_rows = a_rows;
+  p.k_blocks = static_cast<int>(k / 32);
+  const int64_t bound = (total_rows / 256 + num_groups) * ((n + 255) / 256);
+  int64_t workers = device_cus();
+  if (bound < workers) workers = bound;
+  workers = (workers + kXcds - 1) / kXcds * kXcds;
+  return launch_fp8<true>(p, workers, stream);
 }
 
 int hmoe_grouped_gemm_dgrad(const void* grad_out, int64_t ldg, const void* b, const int32_t* offs,

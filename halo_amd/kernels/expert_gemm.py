@@ -1,8 +1,9 @@
-"""Grouped GEMM for MoE expert FFNs, by weight format: bf16/fp32 (the training path), or block-fp8 weights (the
+"""Grouped GEMM for MoE expert FFNs, by format: bf16/fp32 (the training path), the MXFP8 quantisation-aware format
+(both operands block-scaled along the contraction, straight-through backward), or block-fp8 weights (the
 quantised-weight serving configuration, forward only).
 
-Mirrors the dispatch seam of the reference's ``halo/kernels/expert_gemm.py:14-38``.  The reference's other
-``quant_format`` values name its fake-quant QAT formats (mxfp8 / mxfp4 / nvfp4), which are not part of this path.
+Mirrors the dispatch seam of the reference's ``halo/kernels/expert_gemm.py:14-38``.  Of its ``quant_format`` values
+``"mxfp8"`` is built here, on the scaled e4m3 matrix instruction; the 4-bit formats (mxfp4 / nvfp4) raise.
 """
 
 from __future__ import annotations
@@ -10,7 +11,8 @@ from __future__ import annotations
 import torch
 
 from halo_amd import _lib
-from halo_amd.kernels.grouped_mm import GatheredRows, _offs_arg, _rows, grouped_mm
+from halo_amd.kernels.grouped_mm import GatheredRows, _forward, _offs_arg, _rows, grouped_mm, grouped_mm_grads
+from halo_amd.kernels.lowp.spec import require_implemented
 
 
 # rows per expert (on average) from which the dequantised-copy route is taken
@@ -86,10 +88,73 @@ def expert_gemm(
                 return grouped_mm(mat_a, weight.dequantized(), offs=offs)
         return _fp8w_forward(mat_a, weight, offs)
     if quant_format is not None:
-        raise NotImplementedError(
-            f"quant_format={quant_format!r}: the reference's fake-quant QAT formats are not part of the expert path"
-        )
+        require_implemented(quant_format)
+        if isinstance(mat_a, GatheredRows):  # the row quantiser fetches the rows itself
+            return _MxFp8ExpertGemm.apply(mat_a.tokens, mat_b, offs, weight_cacheable, mat_a.row_index, mat_a.inv_map)
+        return _MxFp8ExpertGemm.apply(mat_a, mat_b, offs, weight_cacheable, None, None)
     return grouped_mm(mat_a, mat_b, offs=offs)
+
+
+def mxfp8_mfma_usable(mat_a_dtype: torch.dtype, mat_b_dtype: torch.dtype, k: int, n: int) -> bool:
+    """Whether the scaled e4m3 MFMA kernel takes the product: bf16 operands, whole panels of 64 values along K,
+    16-byte output rows.  Anything else multiplies the two round-tripped operands on the bf16 / fp32 kernel, which is
+    the reference's own formulation."""
+    return (mat_a_dtype == torch.bfloat16 and mat_b_dtype == torch.bfloat16 and k > 0 and k % 64 == 0
+            and n % 8 == 0)
+
+
+class _MxFp8ExpertGemm(torch.autograd.Function):
+    """``grouped_mm(fake_quant(mat_a, "mxfp8", axis=-1), cached_fake_quant(mat_b, "mxfp8", axis=1), offs)`` of the
+    reference (``expert_gemm.py:33-38``) as one node.  Forward: the rows are quantised to e4m3 with an e8m0 scale per
+    32 values (one launch, which also fetches them through ``row_index`` when the permuted copy was never made), the
+    weights once per optimizer step, and the product runs on the scaled e4m3 matrix instruction: the same products of
+    dequantised values the reference's bf16 GEMM sums, accumulated in fp32, at twice the bf16 rate and half the
+    operand bytes.  Backward is the fake-quant's straight-through estimator around ``grouped_mm``'s own gradients
+    (``quantization.py:350-360``, ``grouped_mm.py:16-27``): ``grad_a = dO @ fq(B)^T``, ``grad_b = fq(A)^T @ dO`` with
+    the round-tripped operands in bf16, ``fq(A)`` rebuilt from the saved e4m3 rows (half the bytes of a bf16 copy)."""
+
+    @staticmethod
+    def forward(ctx, mat_a, mat_b, offs, weight_cacheable, row_index, inv_map):
+        from halo_amd.kernels.lowp.quantization import (MxRows, dequantize_rows_mxfp8, expert_weight_operand,
+                                                        quantize_rows_mxfp8)
+
+        device = _lib.require_device(mat_a, mat_b, offs, row_index, inv_map)
+        if mat_a.dim() != 2 or mat_b.dim() != 3 or mat_a.shape[1] != mat_b.shape[1]:
+            raise ValueError(f"expected [R, K] x [G, K, N], got {tuple(mat_a.shape)} x {tuple(mat_b.shape)}")
+        groups, k, n = mat_b.shape
+        offs32 = _offs_arg(offs, groups)
+        weight = expert_weight_operand(mat_b, weight_cacheable)
+        rows_q = quantize_rows_mxfp8(mat_a, row_index)
+        rows = rows_q.rows
+        ctx.k, ctx.dtype, ctx.gathered = k, mat_a.dtype, row_index is not None
+        ctx.save_for_backward(rows_q.q, rows_q.scales, weight.dequant, offs32, inv_map)
+        if not mxfp8_mfma_usable(mat_a.dtype, mat_b.dtype, k, n):
+            return _forward(dequantize_rows_mxfp8(rows_q).to(mat_a.dtype), weight.dequant.to(mat_a.dtype), offs32)
+        out = torch.empty((rows, n), dtype=torch.bfloat16, device=device)
+        if rows and n:
+            with _lib.on_device(device):
+                _lib.call("hmoe_grouped_gemm_fwd_mxfp8", _lib.ptr(rows_q.q), _lib.ptr(rows_q.scales), rows,
+                          _lib.ptr(weight.q), _lib.ptr(weight.scales), _lib.ptr(offs32), rows, groups, k, n,
+                          _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from halo_amd.kernels.lowp.quantization import MxRows, dequantize_rows_mxfp8
+        from halo_amd.kernels.moe_permute import gather_reduce_rows
+
+        q, scales, w_dq, offs32, inv_map = ctx.saved_tensors
+        grad_a = grad_b = None
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            if ctx.needs_input_grad[1]:
+                a_dq = dequantize_rows_mxfp8(MxRows(q, scales, ctx.k)).to(ctx.dtype)
+            else:  # the input gradient reads the rows' shape and dtype only
+                a_dq = grad_output.new_empty((1, ctx.k)).expand(q.shape[1], ctx.k).to(ctx.dtype)
+            grad_a, grad_b = grouped_mm_grads(a_dq, w_dq.to(ctx.dtype), grad_output.to(ctx.dtype), offs32,
+                                              ctx.needs_input_grad[0], ctx.needs_input_grad[1])
+            if ctx.gathered and grad_a is not None:
+                grad_a = gather_reduce_rows(grad_a, inv_map)
+        return grad_a, grad_b, None, None, None, None
 
 
 def _fp8w_forward(mat_a: torch.Tensor, weight: BlockFp8Weight, offs: torch.Tensor | None) -> torch.Tensor:

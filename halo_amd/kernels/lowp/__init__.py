@@ -1,1 +1,1 @@
-"""Low-precision weight formats on the expert path (block fp8)."""
+"""Low-precision formats on the expert path: block fp8 served weights and the MXFP8 quantisation-aware format."""

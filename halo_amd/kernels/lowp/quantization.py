@@ -1,0 +1,289 @@
+"""MXFP8 block-scaled quantisation for the expert GEMM: e4m3 elements plus one e8m0 power-of-two scale per 32 values
+along the contraction axis, the straight-through fake-quant, and the per-step weight cache.
+
+Mirrors ``halo/kernels/lowp/quantization.py`` of the reference for its ``mxfp8`` format: ``BlockScaledTensor``
+(:104-117), ``quantize_mxfp8`` (:236-245), ``dequantize`` (:277-297), ``fake_quant`` (:350-365),
+``WeightVersionCache`` / ``cached_fake_quant`` (:368-422).  The kernels are ``csrc/mxfp8.hip``; they write the operands
+in the layout the GEMM kernel loads (:class:`MxRows`, :class:`MxWeight`), and the reference's logical layout is a
+byte permutation of those.
+"""
+
+from __future__ import annotations
+
+import os
+import weakref
+from dataclasses import dataclass
+
+import torch
+
+from halo_amd import _lib
+from halo_amd.kernels.lowp.spec import FORMAT_BLOCK_SIZE, require_implemented
+
+E4M3_MAX = 448.0
+BLOCK = FORMAT_BLOCK_SIZE["mxfp8"]
+PANEL = 64  # contraction values that lie together in the GEMM's operand layout
+
+
+@dataclass(frozen=True)
+class BlockScaledTensor:
+    """``data`` holds ``float8_e4m3fn`` elements in the source's shape; ``scales`` one ``e8m0`` biased exponent
+    (uint8) per block of ``block_size`` along ``axis``.  An element is ``code x 2^(scales - 127)``."""
+
+    data: torch.Tensor
+    scales: torch.Tensor
+    block_size: int
+    axis: int
+    packed: bool = False
+    pow2_scale: bool = True
+    global_scale: torch.Tensor | None = None
+
+
+@dataclass(frozen=True)
+class MxRows:
+    """Activation rows ``[R, K]`` as the GEMM loads them: ``q`` uint8 ``[ceil(K / 64), R, 64]`` (e4m3 codes in panels
+    of 64 contraction values) and ``scales`` uint8 ``[K / 32, R]``."""
+
+    q: torch.Tensor
+    scales: torch.Tensor
+    k: int
+
+    @property
+    def rows(self) -> int:
+        return self.q.shape[1]
+
+
+@dataclass(frozen=True)
+class MxWeight:
+    """Expert weights ``[G, K, N]`` quantised along K: ``q`` uint8 ``[G, ceil(K / 64), N, 64]``, ``scales`` uint8
+    ``[G, K / 32, N]``, and ``dequant`` the round trip's bf16 ``[G, K, N]`` (None unless asked for)."""
+
+    q: torch.Tensor
+    scales: torch.Tensor
+    dequant: torch.Tensor | None
+    k: int
+
+
+def _native_input(t: torch.Tensor) -> torch.Tensor:
+    return t if t.dtype in (torch.bfloat16, torch.float32) else t.float()
+
+
+def quantize_rows_mxfp8(x: torch.Tensor, row_index: torch.Tensor | None = None) -> MxRows:
+    """``x [R, K]`` (bf16 or fp32, K a multiple of 32) to :class:`MxRows`; with ``row_index`` (int64 ``[R']``) the rows
+    quantised are ``x[row_index]``, fetched by the kernel itself."""
+    device = _lib.require_device(x, row_index)
+    if x.dim() != 2:
+        raise ValueError(f"expected [R, K], got {tuple(x.shape)}")
+    x = _native_input(x)
+    k = x.shape[1]
+    if k % BLOCK:
+        raise ValueError(f"axis 1 size {k} not divisible by block_size {BLOCK}")
+    if row_index is not None:
+        row_index = row_index.to(torch.int64).contiguous()
+    rows = x.shape[0] if row_index is None else row_index.numel()
+    if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+        if x.stride(0) % 8:  # a row length that is no multiple of 8 cannot happen (K % 32 == 0); a 1-row view can
+            x = x.clone()
+    q = torch.empty((-(-k // PANEL), rows, PANEL), dtype=torch.uint8, device=device)
+    scales = torch.empty((k // BLOCK, rows), dtype=torch.uint8, device=device)
+    if k % PANEL:
+        q[-1, :, BLOCK:].zero_()  # the half panel no value belongs to
+    with _lib.on_device(device):
+        _lib.call("hmoe_quantize_rows_mxfp8", _lib.ptr(x), _lib.dtype_id(x.dtype), x.stride(0), _lib.ptr(row_index),
+                  x.shape[0], rows, k, _lib.ptr(q), _lib.ptr(scales), rows, _lib.stream_ptr(device))
+    return MxRows(q, scales, k)
+
+
+def dequantize_rows_mxfp8(rows: MxRows) -> torch.Tensor:
+    """bf16 ``[R, K]``: ``code * 2^(scale - 127)`` for every element of an :class:`MxRows`."""
+    device = _lib.require_device(rows.q, rows.scales)
+    out = torch.empty((rows.rows, rows.k), dtype=torch.bfloat16, device=device)
+    with _lib.on_device(device):
+        _lib.call("hmoe_dequantize_rows_mxfp8", _lib.ptr(rows.q), _lib.ptr(rows.scales), rows.rows, rows.rows, rows.k,
+                  _lib.ptr(out), out.stride(0) if rows.rows else rows.k, _lib.stream_ptr(device))
+    return out
+
+
+def quantize_weight_mxfp8(w: torch.Tensor, with_dequant: bool = False) -> MxWeight:
+    """``w [G, K, N]`` (bf16 or fp32, K a multiple of 32) quantised along K to :class:`MxWeight`."""
+    device = _lib.require_device(w)
+    if w.dim() != 3:
+        raise ValueError(f"expected [G, K, N], got {tuple(w.shape)}")
+    w = _native_input(w).contiguous()
+    g, k, n = w.shape
+    if k % BLOCK:
+        raise ValueError(f"axis 1 size {k} not divisible by block_size {BLOCK}")
+    q = torch.empty((g, -(-k // PANEL), n, PANEL), dtype=torch.uint8, device=device)
+    scales = torch.empty((g, k // BLOCK, n), dtype=torch.uint8, device=device)
+    dequant = torch.empty((g, k, n), dtype=torch.bfloat16, device=device) if with_dequant else None
+    if k % PANEL:
+        q[:, -1, :, BLOCK:].zero_()
+    with _lib.on_device(device):
+        _lib.call("hmoe_quantize_weight_mxfp8", _lib.ptr(w), _lib.dtype_id(w.dtype), g, k, n, _lib.ptr(q),
+                  _lib.ptr(scales), _lib.ptr(dequant), _lib.stream_ptr(device))
+    return MxWeight(q, scales, dequant, k)
+
+
+def _axis_layout(t: torch.Tensor, axis: int) -> tuple[str, int]:
+    axis = axis % t.dim()
+    if axis == t.dim() - 1:
+        return "rows", axis
+    if axis == t.dim() - 2:
+        return "weight", axis
+    return "moved", axis
+
+
+def quantize_mxfp8(t: torch.Tensor, axis: int = -1) -> BlockScaledTensor:
+    """The reference's layout (``quantization.py:236-245``): ``data`` float8_e4m3fn of ``t``'s shape, ``scales`` uint8
+    with ``axis`` divided by 32.  Quantised by the same kernels as the GEMM's operands; the panels are unfolded."""
+    if t.dim() == 0:
+        raise ValueError("quantize_mxfp8 expects at least one axis")
+    kind, axis = _axis_layout(t, axis)
+    k = t.shape[axis]
+    if k % BLOCK:
+        raise ValueError(f"axis {axis} size {k} not divisible by block_size {BLOCK}")
+    if kind == "moved":
+        inner = quantize_mxfp8(t.transpose(axis, -1).contiguous(), -1)
+        return BlockScaledTensor(inner.data.transpose(axis, -1).contiguous(),
+                                 inner.scales.transpose(axis, -1).contiguous(), BLOCK, axis)
+    if kind == "rows":
+        lead = t.shape[:-1]
+        rows = quantize_rows_mxfp8(t.reshape(-1, k))
+        data = rows.q.permute(1, 0, 2).reshape(rows.rows, -1)[:, :k].reshape(*lead, k)
+        scales = rows.scales.t().reshape(*lead, k // BLOCK)
+    else:
+        lead, n = t.shape[:-2], t.shape[-1]
+        w = quantize_weight_mxfp8(t.reshape(-1, k, n))
+        data = w.q.permute(0, 1, 3, 2).reshape(w.q.shape[0], -1, n)[:, :k].reshape(*lead, k, n)
+        scales = w.scales.reshape(*lead, k // BLOCK, n)
+    return BlockScaledTensor(data.contiguous().view(torch.float8_e4m3fn), scales.contiguous(), BLOCK, axis)
+
+
+def dequantize(q: BlockScaledTensor) -> torch.Tensor:
+    """bf16 ``code * 2^(scales - 127)`` in ``q.data``'s shape (``quantization.py:277-297``)."""
+    if q.packed or not q.pow2_scale or q.block_size != BLOCK:
+        raise NotImplementedError("only mxfp8 block-scaled tensors are built on this path")
+    data = q.data.view(torch.uint8)
+    axis = q.axis % data.dim()
+    if axis != data.dim() - 1:
+        moved = BlockScaledTensor(data.transpose(axis, -1).contiguous(), q.scales.transpose(axis, -1).contiguous(),
+                                  BLOCK, -1)
+        return dequantize(moved).transpose(axis, -1).contiguous()
+    k = data.shape[-1]
+    flat = data.reshape(-1, k)
+    rows = flat.shape[0]
+    panels = -(-k // PANEL)
+    padded = flat if k % PANEL == 0 else torch.nn.functional.pad(flat, (0, panels * PANEL - k))
+    packed = MxRows(padded.reshape(rows, panels, PANEL).permute(1, 0, 2).contiguous(),
+                    q.scales.reshape(rows, k // BLOCK).t().contiguous(), k)
+    return dequantize_rows_mxfp8(packed).reshape(data.shape)
+
+
+def _round_trip(t: torch.Tensor, axis: int) -> torch.Tensor:
+    """Quantise then dequantise, bf16 (``quantization.py:307-311``): one launch for a weight axis, two for rows."""
+    kind, axis = _axis_layout(t, axis)
+    if t.shape[axis] % BLOCK:
+        raise ValueError(f"axis {axis} size {t.shape[axis]} not divisible by block_size {BLOCK}")
+    if kind == "moved":
+        return _round_trip(t.transpose(axis, -1).contiguous(), -1).transpose(axis, -1).contiguous()
+    if kind == "rows":
+        return dequantize_rows_mxfp8(quantize_rows_mxfp8(t.reshape(-1, t.shape[-1]))).reshape(t.shape)
+    return quantize_weight_mxfp8(t.reshape(-1, *t.shape[-2:]), with_dequant=True).dequant.reshape(t.shape)
+
+
+class _FakeQuant(torch.autograd.Function):
+    """Straight-through estimator: forward quantise -> dequantise, identity backward to the master
+    (``quantization.py:350-360``)."""
+
+    @staticmethod
+    def forward(ctx, t: torch.Tensor, fmt: str, axis: int) -> torch.Tensor:
+        require_implemented(fmt)
+        return _round_trip(t, axis).to(t.dtype)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return grad_output, None, None
+
+
+def fake_quant(t: torch.Tensor, fmt: str = "mxfp8", axis: int = -1) -> torch.Tensor:
+    """The axis must divide by the format's block size.  Expert weights use :func:`cached_fake_quant`."""
+    return _FakeQuant.apply(t, fmt, axis)
+
+
+class WeightVersionCache:
+    """Keyed by tensor identity plus a caller fingerprint, for values derived once per optimizer step.  A ``weakref``
+    finalizer evicts a collected weight's entry, so a reused ``id`` never serves a stale hit
+    (``quantization.py:368-394``)."""
+
+    def __init__(self) -> None:
+        self._entries: dict[int, tuple[weakref.ref, tuple, object]] = {}
+
+    def get(self, weight: torch.Tensor, fingerprint: tuple):
+        entry = self._entries.get(id(weight))
+        if entry is None:
+            return None
+        ref, cached_fingerprint, value = entry
+        if ref() is not weight or cached_fingerprint != fingerprint:
+            return None
+        return value
+
+    def put(self, weight: torch.Tensor, fingerprint: tuple, value) -> None:
+        wid = id(weight)
+        entries = self._entries
+        ref = weakref.ref(weight, lambda _ref, wid=wid: entries.pop(wid, None))
+        entries[wid] = (ref, fingerprint, value)
+
+    def __len__(self) -> int:
+        return len(self._entries)
+
+
+_weight_dequant_cache = WeightVersionCache()
+_weight_operand_cache = WeightVersionCache()
+
+
+def weight_cache_enabled() -> bool:
+    """``HALO_LOWP_WEIGHT_CACHE`` (default on), the reference's switch (``quantization.py:414``)."""
+    return os.environ.get("HALO_LOWP_WEIGHT_CACHE", "1").strip().lower() not in ("0", "false", "no", "off", "")
+
+
+class _CachedFakeQuant(torch.autograd.Function):
+    """Cloned per call so the shared entry never meets autograd's one-grad_fn-per-tensor rule
+    (``quantization.py:397-407``)."""
+
+    @staticmethod
+    def forward(ctx, weight: torch.Tensor, cached_dequant: torch.Tensor) -> torch.Tensor:
+        return cached_dequant.clone()
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return grad_output, None
+
+
+def cached_fake_quant(weight: torch.Tensor, fmt: str = "mxfp8", axis: int = -1) -> torch.Tensor:
+    """:func:`fake_quant` for an expert weight, quantised once per optimizer step (keyed on ``weight._version``); only
+    leaf parameters cache (``quantization.py:410-422``)."""
+    require_implemented(fmt)
+    if not weight.is_leaf or not weight_cache_enabled():
+        return fake_quant(weight, fmt, axis)
+    fingerprint = (weight._version, fmt, axis)
+    dequant = _weight_dequant_cache.get(weight, fingerprint)
+    if dequant is None:
+        with torch.no_grad():
+            dequant = _round_trip(weight, axis).to(weight.dtype)
+        _weight_dequant_cache.put(weight, fingerprint, dequant)
+    return _CachedFakeQuant.apply(weight, dequant)
+
+
+def expert_weight_operand(weight: torch.Tensor, cacheable: bool) -> MxWeight:
+    """``[G, K, N]`` expert weights as the GEMM's MXFP8 operand together with the round trip's bf16 copy (which the
+    backward products read), quantised once per optimizer step for a leaf parameter when ``cacheable``."""
+    if not (cacheable and weight.is_leaf and weight_cache_enabled()):
+        with torch.no_grad():
+            return quantize_weight_mxfp8(weight.detach(), with_dequant=True)
+    fingerprint = (weight._version, "mxfp8", 1)
+    operand = _weight_operand_cache.get(weight, fingerprint)
+    if operand is None:
+        with torch.no_grad():
+            operand = quantize_weight_mxfp8(weight.detach(), with_dequant=True)
+        _weight_operand_cache.put(weight, fingerprint, operand)
+    return operand

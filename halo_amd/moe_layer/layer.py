@@ -434,11 +434,25 @@ class EPMoELayerBase(ExpertLoadMixin, nn.Module, ABC):
             if (isinstance(weight, BlockFp8Weight) and self._lowp_fp8_activations and x.dtype == torch.bfloat16
                     and fp8_mfma_usable(weight.shape[1], weight.shape[2])):
                 return self._grouped_mm(x, weight, offs=offs)  # the row quantiser fetches the rows itself
+            if self._lowp_quant_format is not None and isinstance(weight, torch.Tensor):
+                return self._grouped_mm(x, weight, offs=offs)  # as above: quantised as they are fetched
             fused = x.grouped_mm(weight, offs=offs) if self._lowp_quant_format is None else None
             if fused is not None:
                 return fused
             x = x.materialize()
         return self._grouped_mm(x, weight, offs=offs)
+
+    def set_lowp_compute(self, quant_format, *, weight_cacheable: bool) -> bool:
+        """Set this layer's expert-compute quantisation format (``"mxfp8"``); returns whether it applies (always: the
+        layer runs on the grouped kernels only).  ``weight_cacheable=False`` re-quantises the weights on every call,
+        for parameters whose version counter does not track the optimizer step.  Reference ``compute.py:53-58``."""
+        if quant_format is not None:
+            from halo_amd.kernels.lowp.spec import require_implemented
+
+            require_implemented(quant_format)
+        self._lowp_quant_format = quant_format
+        self._lowp_weight_cacheable = weight_cacheable
+        return self._use_grouped_mm
 
     def _cast_weight(self, weight_attr: str, out_dtype: torch.dtype):
         weight = getattr(self, weight_attr)

@@ -272,6 +272,41 @@ int hmoe_grouped_gemm_fwd_fp8(const uint8_t* a_q, const uint8_t* a_scale, int64_
                               const float* b_scale, const int32_t* offs, int64_t total_rows, int num_groups, int64_t k,
                               int64_t n, void* out, int64_t ldo, void* stream);
 
+/* ------------------------------------------------------------------------------------------------------- MXFP8
+ * The reference's "mxfp8" quant_format (halo/kernels/lowp/spec.py:11): e4m3 elements with one e8m0 power-of-two scale
+ * per 32 values along the contraction axis.  expert_gemm(quant_format="mxfp8") of the reference is the bf16 product of
+ * the two fake-quantised operands (halo/kernels/expert_gemm.py:33-38); here the quantised operands go to the scaled
+ * e4m3 matrix instruction, which applies a scale per 32 values by itself, so the same products are summed in fp32
+ * without the dequantised copies being read.
+ *
+ * hmoe_quantize_rows_mxfp8 replaces quantize_mxfp8(t, axis=-1) (halo/kernels/lowp/quantization.py:154-188, 236-245)
+ * for x [x_rows, k] (HMOE_BF16 or HMOE_F32, row stride ldx): q e4m3fn in panels [ceil(k / 64)][out_rows][64] (values
+ * [64 p, 64 p + 64) of row r at q[(p * out_rows + r) * 64]) and scale u8 [k / 32][out_rows], at
+ * scale[b * out_rows + r] the e8m0 code of row r's block b: the biased exponent e + 127 of the smallest power of two
+ * 2^e >= amax / 448, e clamped to [-127, 127]; 254 for a block holding an inf, 0xFF for one holding a NaN.  Row r is
+ * x[row_index[r]] (an index outside [0, x_rows) gives zeros) or x[r] with row_index NULL.  k must be a multiple of 32.
+ *
+ * hmoe_dequantize_rows_mxfp8 replaces dequantize (quantization.py:277-297) for that pair: out bf16 [rows, k] =
+ * code * 2^(scale - 127), q and scale holding q_rows rows.
+ *
+ * hmoe_quantize_weight_mxfp8 replaces quantize_mxfp8(w, axis=1) for expert weights w [groups, k, n]: q e4m3fn
+ * [groups][ceil(k / 64)][n][64] (value (kk, c) of expert g at q[((g * ceil(k / 64) + kk / 64) * n + c) * 64 + kk % 64])
+ * and scale u8 [groups][k / 32][n]; with dequant not NULL also the round trip's result (quantization.py:307-311) as
+ * bf16 [groups, k, n], which the straight-through backward multiplies by.
+ *
+ * hmoe_grouped_gemm_fwd_mxfp8: out bf16 [total_rows, n] = per group, dequant(a_q, a_scale)[rows, k] @
+ * dequant(bq, b_scale)[g]: operands as the two quantisers write them (a_rows = their out_rows); accumulation in fp32,
+ * one rounding to bf16.  k must be a multiple of 64, n of 8. */
+int hmoe_quantize_rows_mxfp8(const void* x, int dtype, int64_t ldx, const int64_t* row_index, int64_t x_rows,
+                             int64_t rows, int64_t k, uint8_t* q, uint8_t* scale, int64_t out_rows, void* stream);
+int hmoe_dequantize_rows_mxfp8(const uint8_t* q, const uint8_t* scale, int64_t q_rows, int64_t rows, int64_t k,
+                               void* out, int64_t ldo, void* stream);
+int hmoe_quantize_weight_mxfp8(const void* w, int dtype, int64_t groups, int64_t k, int64_t n, uint8_t* q,
+                               uint8_t* scale, void* dequant, void* stream);
+int hmoe_grouped_gemm_fwd_mxfp8(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
+                                const uint8_t* b_scale, const int32_t* offs, int64_t total_rows, int num_groups,
+                                int64_t k, int64_t n, void* out, int64_t ldo, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -45,13 +45,17 @@ class Glu:
         raise ValueError(self.kind)
 
 
-def expert_ffn(x: torch.Tensor, params: dict, e: int, glu: Glu) -> torch.Tensor:
+def expert_ffn(x: torch.Tensor, params: dict, e: int, glu: Glu, quant=None) -> torch.Tensor:
     """One expert's GLU FFN on either stored layout (``compute.py:357-361``; ``families/gpt_oss.py:121-137``).
     ``params`` holds ``gate_up_proj [E,H,2F]`` + ``down_proj [E,F,H]`` or ``gate_proj``/``up_proj [E,H,F]`` +
-    ``down_proj``, each with an optional ``<name>_bias [E, width]``."""
+    ``down_proj``, each with an optional ``<name>_bias [E, width]``.  ``quant(t, axis)``, when given, is applied to both
+    operands of every product along its contraction axis, which is what the grouped path's low-precision dispatch does
+    (``compute.py:306-312`` into ``expert_gemm.py:33-38``: activations along their last axis, ``[E, K, N]`` weights
+    along axis 1; a block lies inside one row or one expert's column, so per expert is the same)."""
 
     def proj(t, name):
-        out = t @ params[name][e]
+        weight = params[name][e]
+        out = t @ weight if quant is None else quant(t, -1) @ quant(weight, 0)
         bias = params.get(name + "_bias")
         return out if bias is None else out + bias[e]
 
@@ -63,7 +67,7 @@ def expert_ffn(x: torch.Tensor, params: dict, e: int, glu: Glu) -> torch.Tensor:
 
 
 def compute_experts_loop(tokens: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor, params: dict, glu: Glu,
-                         num_local_experts: int) -> torch.Tensor:
+                         num_local_experts: int, quant=None) -> torch.Tensor:
     """``_compute_experts_loop`` (``compute.py:314-347``): ids outside ``[0, E)`` (the dispatch's ``-1``) take no
     part."""
     output = torch.zeros_like(tokens)
@@ -71,7 +75,7 @@ def compute_experts_loop(tokens: torch.Tensor, experts: torch.Tensor, weights: t
         top_k_pos, token_idx = torch.where((experts == e).t())
         if token_idx.numel() == 0:
             continue
-        out = expert_ffn(tokens.index_select(0, token_idx), params, e, glu)
+        out = expert_ffn(tokens.index_select(0, token_idx), params, e, glu, quant)
         output = output.index_add(0, token_idx, out * weights[token_idx, top_k_pos].unsqueeze(-1).to(out.dtype))
     return output
 
@@ -138,15 +142,16 @@ def shared_expert(x: torch.Tensor, shared: dict, glu: Glu) -> torch.Tensor:
 def moe_layer_forward(x: torch.Tensor, router_weight: torch.Tensor, params: dict, glu: Glu, top_k: int, *,
                       router_bias: torch.Tensor | None = None, mode: int = router_oracle.SOFTMAX_ALL,
                       normalize: bool = True, eps: float = 0.0, indices: torch.Tensor | None = None,
-                      shared: dict | None = None):
+                      shared: dict | None = None, quant=None):
     """Router -> per-expert loop -> (+ shared expert).  ``indices`` overrides the selection (used to compare an fp32
-    run against a bf16 run that selected on bf16 logits).  Returns ``(out, logits, indices, weights)``."""
+    run against a bf16 run that selected on bf16 logits); ``quant`` as in :func:`expert_ffn` (the routed experts'
+    products only).  Returns ``(out, logits, indices, weights)``."""
     logits = F.linear(x, router_weight, router_bias)
     if indices is None:
         indices = router_oracle.select_topk(logits.detach(), top_k)
     weights = router_oracle.gate_weights(logits, indices, mode, normalize, eps).float()
     num_experts = router_weight.shape[0]
-    out = compute_experts_loop(x, indices, weights.to(x.dtype), params, glu, num_experts)
+    out = compute_experts_loop(x, indices, weights.to(x.dtype), params, glu, num_experts, quant)
     if shared is not None:
         out = out + shared_expert(x, shared, glu)
     return out, logits, indices, weights

@@ -122,6 +122,28 @@ def test_bad_arguments_come_back_as_status_codes_before_any_launch():
     assert fp8(fake, fake, 8, fake, fake, fake, 8, 4, 256, 128, fake, 100, None) == unsupported
     assert fp8(fake, fake, 4, fake, fake, fake, 8, 4, 256, 128, fake, 128, None) == unsupported
     assert fp8(fake, fake, 8, fake, fake, fake, -1, 4, 256, 128, fake, 128, None) == invalid
+
+    # MXFP8: blocks of 32 along the contraction for the quantisers, whole panels of 64 for the product
+    rows_mx = lib.hmoe_quantize_rows_mxfp8
+    assert rows_mx(fake, bf16, 64, None, 8, 8, 48, fake, fake, 8, None) == unsupported      # K % 32
+    assert rows_mx(fake, 77, 64, None, 8, 8, 64, fake, fake, 8, None) == unsupported        # dtype
+    assert rows_mx(fake, bf16, 64, None, 9, 8, 64, fake, fake, 8, None) == invalid          # no index: x_rows == rows
+    assert rows_mx(fake, bf16, 64, None, 8, 8, 64, fake, fake, 4, None) == unsupported      # out_rows < rows
+    assert rows_mx(fake, bf16, 64, None, 8, 8, 64, None, fake, 8, None) == invalid
+    assert rows_mx(None, bf16, 64, None, 0, 0, 64, None, None, 0, None) == 0
+    assert lib.hmoe_dequantize_rows_mxfp8(fake, fake, 4, 8, 64, fake, 64, None) == invalid  # fewer rows than asked for
+    assert lib.hmoe_dequantize_rows_mxfp8(fake, fake, 8, 8, 48, fake, 64, None) == unsupported
+    weight_mx = lib.hmoe_quantize_weight_mxfp8
+    assert weight_mx(fake, bf16, 4, 48, 64, fake, fake, None, None) == unsupported
+    assert weight_mx(fake, bf16, 4, 64, 64, None, fake, None, None) == invalid
+    assert weight_mx(fake, bf16, 0, 64, 64, None, None, None, None) == 0
+    mx = lib.hmoe_grouped_gemm_fwd_mxfp8
+    assert mx(fake, fake, 8, fake, fake, fake, 8, 4, 96, 128, fake, 128, None) == unsupported   # half a panel
+    assert mx(fake, fake, 8, fake, fake, fake, 8, 4, 128, 100, fake, 128, None) == unsupported
+    assert mx(fake, fake, 4, fake, fake, fake, 8, 4, 128, 128, fake, 128, None) == unsupported  # scale rows < rows
+    assert mx(fake, fake, 8, fake, fake, None, 8, 4, 128, 128, fake, 128, None) == invalid      # groups without ends
+    assert mx(fake, fake, 8, fake, None, fake, 8, 4, 128, 128, fake, 128, None) == invalid
+    assert mx(None, None, 0, None, None, None, 0, 1, 128, 128, None, 128, None) == 0
     assert fp8(fake, None, 8, fake, fake, fake, 8, 4, 256, 128, fake, 128, None) == invalid
     assert fp8(None, None, 0, None, None, None, 0, 1, 256, 128, None, 128, None) == 0
     assert lib.hmoe_quantize_rows_fp8(fake, 200, None, 8, 8, 200, fake, fake, 8, None) == unsupported

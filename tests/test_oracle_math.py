@@ -1,4 +1,4 @@
-"""Pins ``oracle.glu``, ``oracle.grouped_mm``, ``oracle.router``, ``oracle.block_fp8`` and ``oracle.moe_layer`` against
+"""Pins ``oracle.glu``, ``oracle.grouped_mm``, ``oracle.router``, ``oracle.block_fp8``, ``oracle.mxfp8`` and ``oracle.moe_layer`` against
 library routines (torch autograd, matmul, softmax, topk, the float8 cast), identities and brute force."""
 
 import numpy as np
@@ -6,7 +6,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from oracle import block_fp8, glu, grouped_mm, moe_layer, router
+from oracle import block_fp8, glu, grouped_mm, moe_layer, mxfp8, router
 
 PROBE = (-64.0, -8.0, -1.0, -0.5, -1e-3, 0.0, 1e-3, 0.5, 1.0, 8.0, 64.0)  # fused_glu.py:33 of the reference
 
@@ -317,4 +317,127 @@ def test_fp8_product_of_the_oracle_is_the_product_of_its_dequantised_operands():
         total = 0.0
         for kk in range(256):
             total += qa[r, kk] * 2.0 ** (int(exps_t[kk // 128, r]) - 127) * qw[expert, kk, c] * float(ws[expert, kk // 128, c // 128])
+        assert abs(got[r, c] - total) <= 1e-12 * max(1.0, abs(total))
+
+
+# ----------------------------------------------------------------------------------------------------------- mxfp8
+def _mx_blocks(seed=21):
+    """bf16-valued blocks over 40 binades, with the boundary cases of the scale rule in the first rows."""
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(96, 256, generator=g) * torch.exp2(torch.randint(-20, 20, (96, 8), generator=g)
+                                                        .repeat_interleave(32, dim=1).float())).bfloat16().float()
+    x[0, :32] = 0                                        # an all-zero block
+    x[1, :32] = 0; x[1, 3] = 448.0                       # exactly the format's maximum: scale 1
+    x[2, :32] = 0; x[2, 3] = -452.0                      # the next bf16 magnitude above: scale 2
+    x[3, :32] = 0; x[3, 3] = 446.0                       # the next below: scale 1
+    x[4, :32] = 0; x[4, 3] = 448.0 * 2.0 ** -30          # a power-of-two multiple of the maximum, far down
+    x[5, :32] = 0; x[5, 0] = 100.0; x[5, 5] = -12.5      # the reference's own first-principles case
+    return x
+
+
+def test_mxfp8_block_exponent_is_the_smallest_power_of_two_that_fits():
+    """Pins ``e8m0_exponent`` by its defining inequality in exact rational arithmetic, 2^(e-1) < amax / 448 <= 2^e,
+    and by the known answers the reference's tests hold: ``ceil(log2(100 / 448)) + 127`` for a block whose amax is 100
+    (``tests/cpu/kernels/test_block_scale_oracle.py:19-23, 40-48``), code 0 for an all-zero block and for one below
+    448 * 2^-127, 254 for a block holding an inf (``tests/cpu/kernels/test_quantization.py:268-301``) and 0xFF for a
+    NaN block (``quantization.py:36``)."""
+    import math
+    from fractions import Fraction
+
+    x = _mx_blocks()
+    amax = x.abs().reshape(96, 8, 32).amax(dim=2).numpy()
+    e, biased = mxfp8.e8m0_exponent(amax)
+    assert biased.dtype == np.uint8 and np.array_equal(biased.astype(np.int64), e + 127)
+    for a, ee in zip(amax.reshape(-1).tolist(), e.reshape(-1).tolist()):
+        if a == 0:
+            assert ee == -127
+            continue
+        ratio = Fraction(a) / 448
+        assert ratio <= Fraction(2) ** ee and (ee == -127 or ratio > Fraction(2) ** (ee - 1)), (a, ee)
+    assert biased[0, 0] == 0 and biased[1, 0] == 127 and biased[2, 0] == 128 and biased[3, 0] == 127
+    assert biased[4, 0] == 97 and biased[5, 0] == math.ceil(math.log2(100.0 / 448.0)) + 127 == 125
+    edge = np.array([3e-38, 1e-36, np.inf, np.nan, 448.0 * 2.0 ** 119, 3.0e38], dtype=np.float32)
+    assert mxfp8.e8m0_exponent(edge)[1].tolist() == [0, 0, 254, 255, 246, 247]
+
+
+def test_mxfp8_codes_are_torchs_e4m3_cast_of_the_scaled_block_and_round_trip_to_e4m3_precision():
+    """Pins ``quantize_mxfp8`` / ``dequantize_mxfp8``: the codes equal torch's own float8_e4m3fn cast of the block
+    divided (exactly, in float64) by its power-of-two scale; ``code * scale`` is within half an e4m3 step of the value
+    (2^-4 relative for normals, 2^-10 of the scale below); shapes and dtypes as the reference's tests state them
+    (``tests/cpu/kernels/test_quantization.py:29-35, 77-82``), along the last axis and along axis 0."""
+    x = _mx_blocks()
+    data, scales = mxfp8.quantize_mxfp8(x.numpy())
+    assert data.shape == (96, 256) and data.dtype == np.uint8 and scales.shape == (96, 8) and scales.dtype == np.uint8
+    scale = np.ldexp(1.0, scales.astype(np.int64) - 127)
+    scaled = (x.double().reshape(96, 8, 32) / torch.from_numpy(scale)[:, :, None]).reshape(96, 256)
+    assert float(scaled.abs().max()) <= 448
+    want = scaled.float().to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    nonzero = (data & 0x7F) != 0
+    assert np.array_equal(data[nonzero], want[nonzero]) and not (want[~nonzero] & 0x7F).any()
+    restored = mxfp8.dequantize_mxfp8(data, scales)
+    assert np.array_equal(restored, torch.from_numpy(restored).bfloat16().float().numpy())  # bf16 values
+    xd = x.double().numpy()
+    step = np.repeat(scale, 32, axis=1) * 2.0 ** -10
+    assert (np.abs(restored - xd) <= np.maximum(np.abs(xd) * 2.0 ** -4, step)).all()
+    # axis 0: the same blocks taken down the columns
+    d0, s0 = mxfp8.quantize_mxfp8(x.numpy().T.copy(), axis=0)
+    assert d0.shape == (256, 96) and s0.shape == (8, 96)
+    assert np.array_equal(d0, data.T) and np.array_equal(s0, scales.T)
+    with pytest.raises(ValueError, match="not divisible"):
+        mxfp8.quantize_mxfp8(np.zeros((8, 30), dtype=np.float32))
+
+
+def test_mxfp8_extreme_blocks_keep_their_codes():
+    """The edges the reference tests (``tests/cpu/kernels/test_quantization.py:87-93, 268-301``): an all-zero tensor
+    round-trips to exact zeros; a block below 448 * 2^-127 clamps to exponent -127 and one holding an inf reaches 127,
+    and both keep nonzero codes (they are scaled by normal powers of two); a NaN poisons its own block only."""
+    zeros = mxfp8.fake_quant_mxfp8(np.zeros((32, 64), dtype=np.float32))
+    assert np.isfinite(zeros).all() and not zeros.any()
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(4, 64, generator=g)
+    sign = torch.where(torch.rand(32, generator=g) < 0.5, -1.0, 1.0)
+    x[1, :32] = (torch.rand(32, generator=g) * 0.5 + 0.5) * 3e-38 * sign
+    x[2, :32] = torch.exp2(torch.rand(32, generator=g) * 19 + 108) * sign
+    x[2, 0] = float("inf")
+    x[3, 40] = float("nan")
+    data, scales = mxfp8.quantize_mxfp8(x.numpy())
+    assert scales[1, 0] == 0 and scales[2, 0] == 254 and scales[3, 1] == 255 and scales[3, 0] != 255
+    assert (data[1, :32] & 0x7F).max() > 0 and (data[2, 1:16] & 0x7F).max() > 0
+    assert data[2, 0] == 0x7E  # the inf itself saturates at 448
+    # 3e-38 * 2^127 = 5.1: every element of the tiny block is a normal e4m3 value after scaling
+    want = (x[1, :32].double() * 2.0 ** 127).float().to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(data[1, :32], want)
+    restored = mxfp8.dequantize_mxfp8(data, scales)
+    assert np.isnan(restored[3, 32:]).all() and np.isfinite(restored[3, :32]).all() and np.isfinite(restored[0]).all()
+
+
+def test_mxfp8_round_trip_and_expert_product_sit_in_the_reference_error_bands():
+    """The reference's tolerance for the round trip (relative Frobenius error below 0.05 on ``randn(64, 256) * 0.5``,
+    ``tests/cpu/kernels/test_quantization.py:24, 57-64``) and its band for the fake-quantised expert product against
+    the bf16 one (between 0.01 and 0.08, about 0.038 measured, ``tests/gpu/kernels/test_expert_gemm.py:55-74``: zero
+    would mean nothing was quantised).  The product is also checked term by term on sampled outputs."""
+    torch.manual_seed(0)
+    x = torch.randn(64, 256) * 0.5
+    recon = mxfp8.fake_quant_mxfp8(x.numpy())
+    assert np.linalg.norm(recon - x.numpy()) / np.linalg.norm(x.numpy()) < 0.05
+    g = torch.Generator().manual_seed(3)
+    counts = (40, 0, 70, 18)
+    a = (torch.randn(sum(counts), 320, generator=g) * 0.3).bfloat16().float().numpy()
+    b = (torch.randn(len(counts), 320, 96, generator=g) * 0.02).bfloat16().float().numpy()
+    offs = np.cumsum(counts)
+    got = mxfp8.expert_gemm_mxfp8(a, b, offs)
+    plain = np.zeros_like(got)
+    start = 0
+    for e, end in enumerate(offs.tolist()):
+        plain[start:end] = a[start:end].astype(np.float64) @ b[e].astype(np.float64)
+        start = end
+    rel = np.linalg.norm(got - plain) / np.linalg.norm(plain)
+    assert 0.01 < rel < 0.08, rel
+    da, sa = mxfp8.quantize_mxfp8(a, -1)
+    db, sb = mxfp8.quantize_mxfp8(b, 1)
+    va, vb = block_fp8.decode_e4m3fn(da).astype(float), block_fp8.decode_e4m3fn(db).astype(float)
+    for r, c in ((0, 0), (39, 95), (40, 3), (127, 50)):
+        e = int(np.searchsorted(offs, r, side="right"))
+        total = sum(va[r, k] * 2.0 ** (int(sa[r, k // 32]) - 127) * vb[e, k, c] * 2.0 ** (int(sb[e, k // 32, c]) - 127)
+                    for k in range(320))
         assert abs(got[r, c] - total) <= 1e-12 * max(1.0, abs(total))
