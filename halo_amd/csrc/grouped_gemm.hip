@@ -1129,7 +1129,10 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   // two: the B tile of step s + 2 is requested while step s runs, so two B refills are in flight and a weight line has
   // two steps to arrive instead of one.  That takes all 160 KB of the LDS (A0 | B0 | B1 | A1 | B2, 32 KB each), so
   // these modes hold no tables there: the tile walk reads offs itself.  wgrad keeps two stages of (A, B) and its tables.
-  constexpr bool kRingB = kMode != kWgrad;
+#ifndef HMOE_RING
+#define HMOE_RING 1
+#endif
+  constexpr bool kRingB = HMOE_RING && kMode != kWgrad;
   using Sched = typename std::conditional<kRingB, RowTileWalk<kMode, BM, BN>, TileSchedule<kMode, BM, BN>>::type;
   extern __shared__ __attribute__((aligned(16))) char lds_raw[];
   auto lds = (__attribute__((address_space(3))) char*)lds_raw;
@@ -2041,7 +2044,7 @@ int launch_direct(const GemmArgs& p, hipStream_t stream) {
   if (workers <= 0) return HMOE_OK;
   // wgrad: two stages; gathered, 2 x 1 KB of row indices per loading wavefront behind them.  fwd, dgrad: two stages
   // of A and three of B
-  constexpr size_t lds_bytes = kMode == kWgrad
+  constexpr size_t lds_bytes = (kMode == kWgrad || !HMOE_RING)
                                    ? 2 * Cfg::kStage * sizeof(bf16_t) + (kGather ? 4 * 2048 : 0)
                                    : (2 * Cfg::BM + 3 * Cfg::BN) * BK * sizeof(bf16_t);
   auto kernel = grouped_gemm_bf16_kernel<kMode, Cfg, kGather, kBias, kAddTo>;
