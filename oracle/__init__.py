@@ -25,5 +25,13 @@ How each function is pinned (tests/test_oracle_*.py):
   it to the lower index.
 * ``block_fp8.*`` -- the ``exp2(ceil(log2(amax/448)))`` diagnostic formula, the ``448*4`` boundary case, padded
   shapes and the zero block of ``tests/cpu/weight_sync/test_block_fp8.py``.
+* ``mxfp8.*`` -- the block exponent by its defining inequality ``2^(e-1) < amax/448 <= 2^e`` in exact rational
+  arithmetic; the codes by torch's own ``float8_e4m3fn`` cast of the exactly scaled blocks; ``code * scale`` within half
+  an e4m3 step of the value; the known answers the reference's tests hold (amax 100 -> code 125 of
+  ``tests/cpu/kernels/test_block_scale_oracle.py:40-48``; zero, sub-2^-127, inf and NaN blocks and the round-trip bound of
+  ``tests/cpu/kernels/test_quantization.py:57-93, 268-301``; the expert product's error band of
+  ``tests/gpu/kernels/test_expert_gemm.py:55-74``) and the product term by term on sampled outputs.  For fp32 inputs
+  whose amax / 448 lies within an ulp of a power of two the reference's exponent depends on the rounding of its
+  ``log2``: "parity unpinned" there (bf16 inputs are never that close).
 * ``moe_layer.*`` -- the dense formula ``out[t] = sum_k w[t,k] * FFN_e(x[t])`` over valid slots.
 """
