@@ -63,6 +63,10 @@
 // fp32 operands take a plain LDS-tiled FMA kernel (the CPU-sized plumbing configuration and tests).
 #include "common.h"
 
+#ifndef HMOE_EVEN_ROWS
+#define HMOE_EVEN_ROWS 0
+#endif
+
 #include <cstdlib>
 #include <type_traits>
 
@@ -806,9 +810,16 @@ struct RowTileWalk {
     TileInfo tile;
     tile.g = g;
     tile.row_start = s;
+#if HMOE_EVEN_ROWS
+    // the group's rows dealt evenly over its row tiles, in whole 32-row blocks: tiles of one group cost the same
+    const int height = (((rows + mt - 1) / mt) + HMOE_EVEN_ROWS - 1) / HMOE_EVEN_ROWS * HMOE_EVEN_ROWS;
+    tile.a_out0 = m_t * height;
+    tile.a_out_lim = (m_t + 1) * height < rows ? (m_t + 1) * height : rows;
+#else
     tile.a_out0 = m_t * BM;
-    tile.b_out0 = n_t * BN;
     tile.a_out_lim = rows;
+#endif
+    tile.b_out0 = n_t * BN;
     tile.b_out_lim = kMode == kDgrad ? k : n;
     tile.con_lim = kMode == kDgrad ? n : k;
     return tile;
