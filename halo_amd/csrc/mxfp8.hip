@@ -15,41 +15,48 @@ namespace {
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 template <typename T>
-__device__ __forceinline__ void load8(const T* p, float (&v)[8]);
+__device__ __forceinline__ void load16(const T* p, float (&v)[16]);
 template <>
-__device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float (&v)[8]) {
-  Vec16<bf16_t> in;
-  in.load(p);
+__device__ __forceinline__ void load16<bf16_t>(const bf16_t* p, float (&v)[16]) {
+  Vec16<bf16_t> lo, hi;
+  lo.load(p);
+  hi.load(p + 8);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) v[i] = in.v[i];
+  for (int i = 0; i < 8; ++i) {
+    v[i] = lo.v[i];
+    v[8 + i] = hi.v[i];
+  }
 }
 template <>
-__device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
-  const float4 lo = *reinterpret_cast<const float4*>(p), hi = *reinterpret_cast<const float4*>(p + 4);
-  v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
-  v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+__device__ __forceinline__ void load16<float>(const float* p, float (&v)[16]) {
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const float4 t = *reinterpret_cast<const float4*>(p + 4 * c);
+    v[4 * c] = t.x; v[4 * c + 1] = t.y; v[4 * c + 2] = t.z; v[4 * c + 3] = t.w;
+  }
 }
 
-// Rows to MXFP8.  Four lanes share a block of 32 values, eight each; with row_index, output row r is
-// x[row_index[r]] (zeros where the index is outside [0, x_rows)): the permute by expert taken on the way.
+// Rows to MXFP8.  grid.y walks the panels of 64 contraction values, a workgroup takes 64 rows of one panel: four lanes
+// per row, sixteen values each, so that a wavefront reads 16 rows x 128 bytes (whole lines) and writes 1 KB of the
+// panel in one piece.  With row_index, output row r is x[row_index[r]] (zeros where the index is outside
+// [0, x_rows)): the permute by expert taken on the way.
 template <typename T>
 __global__ void __launch_bounds__(256)
 quantize_rows_mx_kernel(const T* __restrict__ x, int64_t ldx, const int64_t* __restrict__ row_index, int64_t x_rows,
                         int64_t rows, int k, uint8_t* __restrict__ q, uint8_t* __restrict__ scale, int64_t out_rows) {
-  const int chunks = k >> 3;
-  const int64_t unit = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  const int64_t row = unit / chunks;
-  const int chunk = static_cast<int>(unit - row * chunks);
-  if (row >= rows) return;  // whole groups of four lanes leave together (chunks is a multiple of 4)
-  float v[8];
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 64 + (threadIdx.x >> 2);
+  const int panel = blockIdx.y, sub = threadIdx.x & 3;
+  const int first = panel * 64 + sub * 16;
+  if (row >= rows || first >= k) return;  // lane pairs leave together (k is a multiple of 32)
+  float v[16];
   const int64_t from = row_index ? row_index[row] : row;
   if (from >= 0 && from < x_rows) {
-    load8<T>(x + from * ldx + (chunk << 3), v);
+    load16<T>(x + from * ldx + first, v);
   } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = 0.f;
+    for (int i = 0; i < 16; ++i) v[i] = 0.f;
   }
-  quantize_mx_block_of_row(v, row, chunk, q, scale, out_rows);
+  quantize_mx_half_block(v, row, panel, sub, q, scale, out_rows);
 }
 
 // e8m0 code to its fp32 value: 2^(code - 127), with 2^-127 (a subnormal) for code 0 and NaN for 0xFF.
@@ -58,30 +65,30 @@ __device__ __forceinline__ float e8m0_value(uint32_t code) {
 }
 
 // The rows back as bf16 [R, K]: code value times the block's power of two, rounded to bf16 (exact for every normal
-// result).  One lane per eight values.
+// result).  The same thread layout as the quantiser: 1 KB of the panel read in one piece per wavefront, whole lines
+// written.
 __global__ void __launch_bounds__(256)
 dequantize_rows_mx_kernel(const uint8_t* __restrict__ q, const uint8_t* __restrict__ scale, int64_t q_rows,
                           int64_t rows, int k, bf16_t* __restrict__ out, int64_t ldo) {
-  const int chunks = k >> 3;
-  const int64_t unit = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  const int64_t row = unit / chunks;
-  const int chunk = static_cast<int>(unit - row * chunks);
-  if (row >= rows) return;
-  const uint2 packed = *reinterpret_cast<const uint2*>(q + (static_cast<int64_t>(chunk >> 3) * q_rows + row) * 64 +
-                                                       ((chunk & 7) << 3));
-  const float s = e8m0_value(scale[static_cast<int64_t>(chunk >> 2) * q_rows + row]);
-  Vec16<bf16_t> o;
-  const uint32_t words[2] = {packed.x, packed.y};
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 64 + (threadIdx.x >> 2);
+  const int panel = blockIdx.y, sub = threadIdx.x & 3;
+  const int first = panel * 64 + sub * 16;
+  if (row >= rows || first >= k) return;
+  const uint4 packed = *reinterpret_cast<const uint4*>(q + (static_cast<int64_t>(panel) * q_rows + row) * 64 + sub * 16);
+  const float s = e8m0_value(scale[static_cast<int64_t>(2 * panel + (sub >> 1)) * q_rows + row]);
+  const uint32_t words[4] = {packed.x, packed.y, packed.z, packed.w};
+  Vec16<bf16_t> o[2];
 #pragma unroll
-  for (int w = 0; w < 2; ++w) {
+  for (int w = 0; w < 4; ++w) {
     const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(words[w]), false);
     const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(words[w]), true);
-    o.v[4 * w + 0] = lo.x * s;
-    o.v[4 * w + 1] = lo.y * s;
-    o.v[4 * w + 2] = hi.x * s;
-    o.v[4 * w + 3] = hi.y * s;
+    o[w >> 1].v[4 * (w & 1) + 0] = lo.x * s;
+    o[w >> 1].v[4 * (w & 1) + 1] = lo.y * s;
+    o[w >> 1].v[4 * (w & 1) + 2] = hi.x * s;
+    o[w >> 1].v[4 * (w & 1) + 3] = hi.y * s;
   }
-  o.store(out + row * ldo + (chunk << 3));
+  o[0].store(out + row * ldo + first);
+  o[1].store(out + row * ldo + first + 8);
 }
 
 // Expert weights [G, K, N] to MXFP8 along K.  A workgroup takes one panel (64 contraction values) of 128 columns:
@@ -180,12 +187,11 @@ int hmoe_quantize_rows_mxfp8(const void* x, int dtype, int64_t ldx, const int64_
   if (k % 32 || ldx < k || ldx % 8 || out_rows < rows) return HMOE_UNSUPPORTED;
   if (rows == 0 || k == 0) return HMOE_OK;
   if (!q || !scale || (!x && x_rows > 0)) return HMOE_INVALID_ARGUMENT;
-  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(q) % 8) return HMOE_UNSUPPORTED;
-  const int64_t units = rows * (k / 8);
-  const int64_t blocks = (units + 255) / 256;
-  if (blocks >= (int64_t(1) << 31) || k >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(q) % 16) return HMOE_UNSUPPORTED;
+  const int64_t row_blocks = (rows + 63) / 64, panels = (k + 63) / 64;
+  if (row_blocks >= (int64_t(1) << 31) || panels > 65535) return HMOE_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(static_cast<unsigned>(blocks));
+  const dim3 grid(static_cast<unsigned>(row_blocks), static_cast<unsigned>(panels));
   if (dtype == HMOE_BF16)
     quantize_rows_mx_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(static_cast<const bf16_t*>(x), ldx, row_index, x_rows,
                                                               rows, static_cast<int>(k), q, scale, out_rows);
@@ -203,11 +209,11 @@ int hmoe_dequantize_rows_mxfp8(const uint8_t* q, const uint8_t* scale, int64_t q
   if (k % 32 || ldo < k || ldo % 8) return HMOE_UNSUPPORTED;
   if (rows == 0 || k == 0) return HMOE_OK;
   if (!q || !scale || !out) return HMOE_INVALID_ARGUMENT;
-  if (reinterpret_cast<uintptr_t>(out) % 16 || reinterpret_cast<uintptr_t>(q) % 8) return HMOE_UNSUPPORTED;
-  const int64_t units = rows * (k / 8);
-  const int64_t blocks = (units + 255) / 256;
-  if (blocks >= (int64_t(1) << 31) || k >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
-  dequantize_rows_mx_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+  if (reinterpret_cast<uintptr_t>(out) % 16 || reinterpret_cast<uintptr_t>(q) % 16) return HMOE_UNSUPPORTED;
+  const int64_t row_blocks = (rows + 63) / 64, panels = (k + 63) / 64;
+  if (row_blocks >= (int64_t(1) << 31) || panels > 65535) return HMOE_UNSUPPORTED;
+  dequantize_rows_mx_kernel<<<dim3(static_cast<unsigned>(row_blocks), static_cast<unsigned>(panels)), dim3(256), 0,
+                              static_cast<hipStream_t>(stream)>>>(
       q, scale, q_rows, rows, static_cast<int>(k), static_cast<bf16_t*>(out), ldo);
   HMOE_CHECK_LAUNCH();
   return HMOE_OK;

@@ -103,6 +103,33 @@ def mxfp8_mfma_usable(mat_a_dtype: torch.dtype, mat_b_dtype: torch.dtype, k: int
             and n % 8 == 0)
 
 
+class _SharedRows:
+    """The last activation tensor quantised (forward) and the last e4m3 rows dequantised (backward), each with its
+    result: projections that read the same rows (gate and up stored apart) quantise them once and rebuild them once.
+    An entry is tied to the tensor object by a weak reference and to its version counter, and dies with the tensor."""
+
+    def __init__(self):
+        self._ref, self._key, self._value = None, None, None
+
+    def get(self, tensor: torch.Tensor, key: tuple):
+        if self._ref is not None and self._ref() is tensor and self._key == key:
+            return self._value
+        return None
+
+    def put(self, tensor: torch.Tensor, key: tuple, value) -> None:
+        import weakref
+
+        def drop(ref, self=self):
+            if self._ref is ref:
+                self._ref, self._key, self._value = None, None, None
+
+        self._ref, self._key, self._value = weakref.ref(tensor, drop), key, value
+
+
+_quantised_rows = _SharedRows()
+_dequantised_rows = _SharedRows()
+
+
 class _MxFp8ExpertGemm(torch.autograd.Function):
     """``grouped_mm(fake_quant(mat_a, "mxfp8", axis=-1), cached_fake_quant(mat_b, "mxfp8", axis=1), offs)`` of the
     reference (``expert_gemm.py:33-38``) as one node.  Forward: the rows are quantised to e4m3 with an e8m0 scale per
@@ -124,10 +151,17 @@ class _MxFp8ExpertGemm(torch.autograd.Function):
         groups, k, n = mat_b.shape
         offs32 = _offs_arg(offs, groups)
         weight = expert_weight_operand(mat_b, weight_cacheable)
-        rows_q = quantize_rows_mxfp8(mat_a, row_index)
+        key = (mat_a._version, None if row_index is None else (id(row_index), row_index._version))
+        rows_q = _quantised_rows.get(mat_a, key)
+        if rows_q is None:
+            rows_q = quantize_rows_mxfp8(mat_a, row_index)
+            _quantised_rows.put(mat_a, key, rows_q)
         rows = rows_q.rows
         ctx.k, ctx.dtype, ctx.gathered = k, mat_a.dtype, row_index is not None
-        ctx.save_for_backward(rows_q.q, rows_q.scales, weight.dequant, offs32, inv_map)
+        # the e4m3 rows ride on the node itself: projections that share them must see one object, and they are no
+        # input or output of this node
+        ctx.rows_q = rows_q
+        ctx.save_for_backward(weight.dequant, offs32, inv_map)
         if not mxfp8_mfma_usable(mat_a.dtype, mat_b.dtype, k, n):
             return _forward(dequantize_rows_mxfp8(rows_q).to(mat_a.dtype), weight.dequant.to(mat_a.dtype), offs32)
         out = torch.empty((rows, n), dtype=torch.bfloat16, device=device)
@@ -143,11 +177,15 @@ class _MxFp8ExpertGemm(torch.autograd.Function):
         from halo_amd.kernels.lowp.quantization import MxRows, dequantize_rows_mxfp8
         from halo_amd.kernels.moe_permute import gather_reduce_rows
 
-        q, scales, w_dq, offs32, inv_map = ctx.saved_tensors
+        w_dq, offs32, inv_map = ctx.saved_tensors
+        q, scales = ctx.rows_q.q, ctx.rows_q.scales
         grad_a = grad_b = None
         if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
             if ctx.needs_input_grad[1]:
-                a_dq = dequantize_rows_mxfp8(MxRows(q, scales, ctx.k)).to(ctx.dtype)
+                a_dq = _dequantised_rows.get(q, (q._version, ctx.dtype))
+                if a_dq is None:
+                    a_dq = dequantize_rows_mxfp8(MxRows(q, scales, ctx.k)).to(ctx.dtype)
+                    _dequantised_rows.put(q, (q._version, ctx.dtype), a_dq)
             else:  # the input gradient reads the rows' shape and dtype only
                 a_dq = grad_output.new_empty((1, ctx.k)).expand(q.shape[1], ctx.k).to(ctx.dtype)
             grad_a, grad_b = grouped_mm_grads(a_dq, w_dq.to(ctx.dtype), grad_output.to(ctx.dtype), offs32,
