@@ -264,6 +264,52 @@ def test_mxfp8_expert_gemm_outside_the_matrix_kernel(device):
     assert ((grad_fetched.double() - grad_copied.double()).norm() / grad_copied.double().norm()).item() < 5e-3
 
 
+def test_projections_reading_the_same_rows_quantise_them_once(device, monkeypatch):
+    """Gate and up stored apart read the same sorted rows: the second product takes the first one's e4m3 rows, and in
+    backward the second weight gradient takes the first one's dequantised rows.  A change of the tensor in place (its
+    version moves) or another tensor quantises again; the results equal the unshared ones bit for bit."""
+    from halo_amd.kernels import expert_gemm as eg
+    from halo_amd.kernels.lowp import quantization
+
+    calls = {"quantise": 0, "dequantise": 0}
+    real_q, real_d = quantization.quantize_rows_mxfp8, quantization.dequantize_rows_mxfp8
+
+    def counting_q(*args, **kwargs):
+        calls["quantise"] += 1
+        return real_q(*args, **kwargs)
+
+    def counting_d(*args, **kwargs):
+        calls["dequantise"] += 1
+        return real_d(*args, **kwargs)
+
+    monkeypatch.setattr(quantization, "quantize_rows_mxfp8", counting_q)
+    monkeypatch.setattr(quantization, "dequantize_rows_mxfp8", counting_d)
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(192, 128, generator=g).bfloat16().to(device).requires_grad_(True)
+    w_gate = (torch.randn(3, 128, 64, generator=g) * 0.05).bfloat16().to(device).requires_grad_(True)
+    w_up = (torch.randn(3, 128, 64, generator=g) * 0.05).bfloat16().to(device).requires_grad_(True)
+    offs = torch.tensor([64, 64, 192], dtype=torch.int32, device=device)
+    gate = eg.expert_gemm(x, w_gate, offs=offs, quant_format="mxfp8")
+    up = eg.expert_gemm(x, w_up, offs=offs, quant_format="mxfp8")
+    assert calls["quantise"] == 1
+    (gate * up).sum().backward()
+    assert calls["dequantise"] == 1
+    shared = (gate.detach().clone(), up.detach().clone(), x.grad.clone(), w_gate.grad.clone(), w_up.grad.clone())
+    with torch.no_grad():
+        x.mul_(1.0)  # same values, the version counter moves
+    again = eg.expert_gemm(x, w_up, offs=offs, quant_format="mxfp8")
+    other = eg.expert_gemm(x.detach().clone(), w_up, offs=offs, quant_format="mxfp8")
+    assert calls["quantise"] == 3 and torch.equal(again, up) and torch.equal(other, up)
+    # unshared: every product on a tensor of its own
+    x.grad = w_gate.grad = w_up.grad = None
+    xa, xb = x.detach().clone().requires_grad_(True), x.detach().clone().requires_grad_(True)
+    gate2 = eg.expert_gemm(xa, w_gate, offs=offs, quant_format="mxfp8")
+    up2 = eg.expert_gemm(xb, w_up, offs=offs, quant_format="mxfp8")
+    (gate2 * up2).sum().backward()
+    assert torch.equal(gate2, shared[0]) and torch.equal(up2, shared[1]) and torch.equal(xa.grad + xb.grad, shared[2])
+    assert torch.equal(w_gate.grad, shared[3]) and torch.equal(w_up.grad, shared[4])
+
+
 @pytest.mark.parametrize("name", ("cfg2_small", "cfg4_small"))
 def test_layer_with_mxfp8_experts_against_the_cpu_loop_over_fake_quantised_products(device, name):
     """``set_lowp_compute("mxfp8")`` on the layer (reference ``compute.py:53-58, 306-312``): forward and every
