@@ -1115,8 +1115,15 @@ __device__ __forceinline__ void interleave_reads_under_mfmas() {
   }
 }
 
+#ifdef HMOE_WG_TIMES
+__device__ unsigned long long g_wg_times[2048];
+#endif
+
 template <int kMode, typename Cfg, int kGather = 0, bool kBias = false, bool kAddTo = false>
 __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmArgs p) {
+#ifdef HMOE_WG_TIMES
+  const unsigned long long wg_entered = __builtin_readcyclecounter();
+#endif
   static_assert(!kAddTo || (kMode == kFwd && !kBias), "the scaled sum into an addend belongs to the plain forward");
   static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
   static_assert(!kBias || kMode == kFwd, "the expert bias belongs to the forward product");
@@ -1522,6 +1529,13 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     }
   }
   wait_loads();  // no load may land in LDS after the workgroup has given it back
+#ifdef HMOE_WG_TIMES
+  // timing build: when each workgroup entered and left (cycle counter), read back with hmoe_debug_wg_times
+  if (threadIdx.x == 0) {
+    g_wg_times[blockIdx.x] = wg_entered;
+    g_wg_times[1024 + blockIdx.x] = __builtin_readcyclecounter();
+  }
+#endif
 }
 
 #define HMOE_BF16_INSTANCE(mode) \
@@ -2141,6 +2155,12 @@ int launch_fp8(const GemmArgs& p, int64_t workers, void* stream) {
 }  // namespace hmoe
 
 extern "C" {
+
+#ifdef HMOE_WG_TIMES
+int hmoe_debug_wg_times(unsigned long long* host_out) {
+  return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(hmoe::g_wg_times), sizeof(unsigned long long) * 2048) == hipSuccess ? 0 : -3;
+}
+#endif
 
 int hmoe_grouped_gemm_fwd(const void* a, int64_t lda, const void* b, const int32_t* offs, int64_t total_rows,
                           int num_groups, int64_t k, int64_t n, int dtype, void* out, int64_t ldo, void* stream) {
