@@ -59,6 +59,9 @@ SIGNATURES = {
     "hmoe_dequantize_rows_mxfp8": (I, [P, P, L, L, L, P, L, P]),
     "hmoe_quantize_weight_mxfp8": (I, [P, I, L, L, L, P, P, P, P]),
     "hmoe_grouped_gemm_fwd_mxfp8": (I, [P, P, L, P, P, P, L, I, L, L, P, L, P]),
+    "hmoe_mxfp4_rows": (I, [P, I, L, P, L, L, L, P, P, P, L, P]),
+    "hmoe_mxfp4_weight": (I, [P, I, L, L, L, P, P, P, P]),
+    "hmoe_mxfp4_dequantize_rows": (I, [P, P, L, L, P, L, P]),
 }
 
 _lib = None

@@ -1,9 +1,10 @@
-"""Grouped GEMM for MoE expert FFNs, by format: bf16/fp32 (the training path), the MXFP8 quantisation-aware format
-(both operands block-scaled along the contraction, straight-through backward), or block-fp8 weights (the
-quantised-weight serving configuration, forward only).
+"""Grouped GEMM for MoE expert FFNs, by format: bf16/fp32 (the training path), the MXFP8 and MXFP4
+quantisation-aware formats (both operands block-scaled along the contraction, straight-through backward), or block-fp8
+weights (the quantised-weight serving configuration, forward only).
 
 Mirrors the dispatch seam of the reference's ``halo/kernels/expert_gemm.py:14-38``.  Of its ``quant_format`` values
-``"mxfp8"`` is built here, on the scaled e4m3 matrix instruction; the 4-bit formats (mxfp4 / nvfp4) raise.
+``"mxfp8"`` runs on the scaled e4m3 matrix instruction and ``"mxfp4"`` as the reference's default does, the bf16 product
+of the two round-tripped operands; ``"nvfp4"`` raises.
 """
 
 from __future__ import annotations
@@ -89,9 +90,11 @@ def expert_gemm(
         return _fp8w_forward(mat_a, weight, offs)
     if quant_format is not None:
         require_implemented(quant_format)
-        if isinstance(mat_a, GatheredRows):  # the row quantiser fetches the rows itself
-            return _MxFp8ExpertGemm.apply(mat_a.tokens, mat_b, offs, weight_cacheable, mat_a.row_index, mat_a.inv_map)
-        return _MxFp8ExpertGemm.apply(mat_a, mat_b, offs, weight_cacheable, None, None)
+        gathered = isinstance(mat_a, GatheredRows)  # the row quantiser fetches the rows itself
+        source, row_index, inv_map = (mat_a.tokens, mat_a.row_index, mat_a.inv_map) if gathered else (mat_a, None, None)
+        if quant_format == "mxfp4":
+            return _Mxfp4ExpertGemm.apply(source, mat_b, offs, weight_cacheable, row_index, inv_map)
+        return _MxFp8ExpertGemm.apply(source, mat_b, offs, weight_cacheable, row_index, inv_map)
     return grouped_mm(mat_a, mat_b, offs=offs)
 
 
@@ -189,6 +192,48 @@ class _MxFp8ExpertGemm(torch.autograd.Function):
             else:  # the input gradient reads the rows' shape and dtype only
                 a_dq = grad_output.new_empty((1, ctx.k)).expand(q.shape[1], ctx.k).to(ctx.dtype)
             grad_a, grad_b = grouped_mm_grads(a_dq, w_dq.to(ctx.dtype), grad_output.to(ctx.dtype), offs32,
+                                              ctx.needs_input_grad[0], ctx.needs_input_grad[1])
+            if ctx.gathered and grad_a is not None:
+                grad_a = gather_reduce_rows(grad_a, inv_map)
+        return grad_a, grad_b, None, None, None, None
+
+
+_round_tripped_rows = _SharedRows()
+
+
+class _Mxfp4ExpertGemm(torch.autograd.Function):
+    """``grouped_mm(fake_quant(mat_a, "mxfp4", axis=-1), cached_fake_quant(mat_b, "mxfp4", axis=1), offs)`` of the
+    reference (``expert_gemm.py:33-38``) as one node: the rows go through the e2m1 round trip in one launch (which also
+    fetches them through ``row_index`` when the permuted copy was never made), the weights once per optimizer step,
+    and the product is the bf16 grouped GEMM's.  Backward is the straight-through estimator around ``grouped_mm``'s own
+    gradients (``quantization.py:350-360``, ``grouped_mm.py:16-27``) with the round-tripped operands."""
+
+    @staticmethod
+    def forward(ctx, mat_a, mat_b, offs, weight_cacheable, row_index, inv_map):
+        from halo_amd.kernels.lowp.quantization import expert_weight_round_trip, mxfp4_rows
+
+        _lib.require_device(mat_a, mat_b, offs, row_index, inv_map)
+        if mat_a.dim() != 2 or mat_b.dim() != 3 or mat_a.shape[1] != mat_b.shape[1]:
+            raise ValueError(f"expected [R, K] x [G, K, N], got {tuple(mat_a.shape)} x {tuple(mat_b.shape)}")
+        offs32 = _offs_arg(offs, mat_b.shape[0])
+        w_rt = expert_weight_round_trip(mat_b, "mxfp4", weight_cacheable).to(mat_a.dtype)
+        key = (mat_a._version, None if row_index is None else (id(row_index), row_index._version))
+        a_rt = _round_tripped_rows.get(mat_a, key)
+        if a_rt is None:
+            a_rt = mxfp4_rows(mat_a, row_index, codes=False, round_trip=True)[2].to(mat_a.dtype)
+            _round_tripped_rows.put(mat_a, key, a_rt)
+        ctx.gathered = row_index is not None
+        ctx.save_for_backward(a_rt, w_rt, offs32, inv_map)
+        return _forward(a_rt, w_rt, offs32)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from halo_amd.kernels.moe_permute import gather_reduce_rows
+
+        a_rt, w_rt, offs32, inv_map = ctx.saved_tensors
+        grad_a = grad_b = None
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            grad_a, grad_b = grouped_mm_grads(a_rt, w_rt, grad_output.to(a_rt.dtype), offs32,
                                               ctx.needs_input_grad[0], ctx.needs_input_grad[1])
             if ctx.gathered and grad_a is not None:
                 grad_a = gather_reduce_rows(grad_a, inv_map)

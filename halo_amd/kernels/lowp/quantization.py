@@ -1,11 +1,13 @@
-"""MXFP8 block-scaled quantisation for the expert GEMM: e4m3 elements plus one e8m0 power-of-two scale per 32 values
-along the contraction axis, the straight-through fake-quant, and the per-step weight cache.
+"""MX block-scaled quantisation for the expert GEMM: e4m3 (MXFP8) or e2m1 (MXFP4) elements plus one e8m0 power-of-two
+scale per 32 values along the contraction axis, the straight-through fake-quant, and the per-step weight cache.
 
-Mirrors ``halo/kernels/lowp/quantization.py`` of the reference for its ``mxfp8`` format: ``BlockScaledTensor``
-(:104-117), ``quantize_mxfp8`` (:236-245), ``dequantize`` (:277-297), ``fake_quant`` (:350-365),
-``WeightVersionCache`` / ``cached_fake_quant`` (:368-422).  The kernels are ``csrc/mxfp8.hip``; they write the operands
-in the layout the GEMM kernel loads (:class:`MxRows`, :class:`MxWeight`), and the reference's logical layout is a
-byte permutation of those.
+Mirrors ``halo/kernels/lowp/quantization.py`` of the reference for its ``mxfp8`` and ``mxfp4`` formats:
+``BlockScaledTensor`` (:104-117), ``quantize_mxfp8`` (:236-245), ``quantize_mxfp4`` (:248-266), ``dequantize``
+(:277-297), ``fake_quant`` (:350-365), ``WeightVersionCache`` / ``cached_fake_quant`` (:368-422).  The MXFP8 kernels are
+``csrc/mxfp8.hip``; they write the operands in the layout the GEMM kernel loads (:class:`MxRows`, :class:`MxWeight`),
+and the reference's logical layout is a byte permutation of those.  The MXFP4 kernels are ``csrc/mxfp4.hip``; they
+write the reference's layout (two codes per byte along the quantised axis) and, for the fake-quant route the expert
+GEMM takes with this format, the round trip's bf16 result in the same pass.
 """
 
 from __future__ import annotations
@@ -26,8 +28,9 @@ PANEL = 64  # contraction values that lie together in the GEMM's operand layout
 
 @dataclass(frozen=True)
 class BlockScaledTensor:
-    """``data`` holds ``float8_e4m3fn`` elements in the source's shape; ``scales`` one ``e8m0`` biased exponent
-    (uint8) per block of ``block_size`` along ``axis``.  An element is ``code x 2^(scales - 127)``."""
+    """``data`` holds ``float8_e4m3fn`` elements in the source's shape, or, when ``packed``, two ``e2m1`` codes per byte
+    (uint8, ``axis`` halved, the even element in the low nibble); ``scales`` one ``e8m0`` biased exponent (uint8) per
+    block of ``block_size`` along ``axis``.  An element is ``code x 2^(scales - 127)``."""
 
     data: torch.Tensor
     scales: torch.Tensor
@@ -124,6 +127,63 @@ def quantize_weight_mxfp8(w: torch.Tensor, with_dequant: bool = False) -> MxWeig
     return MxWeight(q, scales, dequant, k)
 
 
+def _aligned_rows(x: torch.Tensor) -> torch.Tensor:
+    if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+        if x.stride(0) % 8:
+            x = x.clone()
+    return x
+
+
+def mxfp4_rows(x: torch.Tensor, row_index: torch.Tensor | None = None, *, codes: bool = True,
+               round_trip: bool = False) -> tuple[torch.Tensor | None, torch.Tensor | None, torch.Tensor | None]:
+    """``x [R, K]`` (bf16 or fp32, K a multiple of 32) along its last axis in one launch: ``(packed uint8 [R, K / 2],
+    scales uint8 [R, K / 32], round trip bf16 [R, K])``, the first two None unless ``codes``, the last unless
+    ``round_trip``.  With ``row_index`` (int64 ``[R']``) the rows taken are ``x[row_index]``, fetched by the kernel."""
+    device = _lib.require_device(x, row_index)
+    if x.dim() != 2:
+        raise ValueError(f"expected [R, K], got {tuple(x.shape)}")
+    if not (codes or round_trip):
+        raise ValueError("nothing to compute: neither codes nor round_trip asked for")
+    x = _aligned_rows(_native_input(x))
+    k = x.shape[1]
+    if k % BLOCK:
+        raise ValueError(f"axis 1 size {k} not divisible by block_size {BLOCK}")
+    if row_index is not None:
+        row_index = row_index.to(torch.int64).contiguous()
+    rows = x.shape[0] if row_index is None else row_index.numel()
+    packed = torch.empty((rows, k // 2), dtype=torch.uint8, device=device) if codes else None
+    scales = torch.empty((rows, k // BLOCK), dtype=torch.uint8, device=device) if codes else None
+    out = torch.empty((rows, k), dtype=torch.bfloat16, device=device) if round_trip else None
+    with _lib.on_device(device):
+        _lib.call("hmoe_mxfp4_rows", _lib.ptr(x), _lib.dtype_id(x.dtype), x.stride(0) if x.shape[0] else k,
+                  _lib.ptr(row_index), x.shape[0], rows, k, _lib.ptr(packed), _lib.ptr(scales), _lib.ptr(out), k,
+                  _lib.stream_ptr(device))
+    return packed, scales, out
+
+
+def mxfp4_weight(w: torch.Tensor, *, codes: bool = True, round_trip: bool = False
+                 ) -> tuple[torch.Tensor | None, torch.Tensor | None, torch.Tensor | None]:
+    """``w [G, K, N]`` (bf16 or fp32, K a multiple of 32) along K in one launch: ``(packed uint8 [G, K / 2, N], scales
+    uint8 [G, K / 32, N], round trip bf16 [G, K, N])``, selected as in :func:`mxfp4_rows`."""
+    device = _lib.require_device(w)
+    if w.dim() != 3:
+        raise ValueError(f"expected [G, K, N], got {tuple(w.shape)}")
+    if not (codes or round_trip):
+        raise ValueError("nothing to compute: neither codes nor round_trip asked for")
+    w = _native_input(w).contiguous()
+    g, k, n = w.shape
+    if k % BLOCK:
+        raise ValueError(f"axis 1 size {k} not divisible by block_size {BLOCK}")
+    packed = torch.empty((g, k // 2, n), dtype=torch.uint8, device=device) if codes else None
+    scales = torch.empty((g, k // BLOCK, n), dtype=torch.uint8, device=device) if codes else None
+    out = torch.empty((g, k, n), dtype=torch.bfloat16, device=device) if round_trip else None
+    with _lib.on_device(device):
+        _lib.call("hmoe_mxfp4_weight", _lib.ptr(w), _lib.dtype_id(w.dtype), g, k, n, _lib.ptr(packed), _lib.ptr(scales),
+                  _lib.ptr(out), _lib.stream_ptr(device))
+    return packed, scales, out
+
+
 def _axis_layout(t: torch.Tensor, axis: int) -> tuple[str, int]:
     axis = axis % t.dim()
     if axis == t.dim() - 1:
@@ -159,10 +219,58 @@ def quantize_mxfp8(t: torch.Tensor, axis: int = -1) -> BlockScaledTensor:
     return BlockScaledTensor(data.contiguous().view(torch.float8_e4m3fn), scales.contiguous(), BLOCK, axis)
 
 
+def quantize_mxfp4(t: torch.Tensor, axis: int = -1) -> BlockScaledTensor:
+    """The reference's layout (``quantization.py:248-266``): ``data`` uint8 with ``axis`` halved (two e2m1 codes per
+    byte, the even element low), ``scales`` uint8 with ``axis`` divided by 32."""
+    if t.dim() == 0:
+        raise ValueError("quantize_mxfp4 expects at least one axis")
+    kind, axis = _axis_layout(t, axis)
+    k = t.shape[axis]
+    if k % BLOCK:
+        raise ValueError(f"axis {axis} size {k} not divisible by block_size {BLOCK}")
+    if kind == "moved":
+        inner = quantize_mxfp4(t.transpose(axis, -1).contiguous(), -1)
+        return BlockScaledTensor(inner.data.transpose(axis, -1).contiguous(),
+                                 inner.scales.transpose(axis, -1).contiguous(), BLOCK, axis, packed=True)
+    if kind == "rows":
+        lead = t.shape[:-1]
+        packed, scales, _ = mxfp4_rows(t.reshape(-1, k))
+        return BlockScaledTensor(packed.reshape(*lead, k // 2), scales.reshape(*lead, k // BLOCK), BLOCK, axis,
+                                 packed=True)
+    lead, n = t.shape[:-2], t.shape[-1]
+    packed, scales, _ = mxfp4_weight(t.reshape(-1, k, n))
+    return BlockScaledTensor(packed.reshape(*lead, k // 2, n), scales.reshape(*lead, k // BLOCK, n), BLOCK, axis,
+                             packed=True)
+
+
+QUANTIZERS = {"mxfp8": quantize_mxfp8, "mxfp4": quantize_mxfp4}
+
+
+def _dequantize_packed(q: BlockScaledTensor) -> torch.Tensor:
+    data, axis = q.data, q.axis % q.data.dim()
+    if axis != data.dim() - 1:
+        moved = BlockScaledTensor(data.transpose(axis, -1).contiguous(), q.scales.transpose(axis, -1).contiguous(),
+                                  BLOCK, -1, packed=True)
+        return _dequantize_packed(moved).transpose(axis, -1).contiguous()
+    device = _lib.require_device(data, q.scales)
+    k = data.shape[-1] * 2
+    if k % BLOCK or q.scales.shape[-1] != k // BLOCK:
+        raise ValueError(f"packed axis of {data.shape[-1]} bytes does not match {q.scales.shape[-1]} scales of {BLOCK}")
+    flat = data.reshape(-1, k // 2).contiguous()
+    scales = q.scales.reshape(-1, k // BLOCK).contiguous()
+    out = torch.empty((flat.shape[0], k), dtype=torch.bfloat16, device=device)
+    with _lib.on_device(device):
+        _lib.call("hmoe_mxfp4_dequantize_rows", _lib.ptr(flat), _lib.ptr(scales), flat.shape[0], k, _lib.ptr(out), k,
+                  _lib.stream_ptr(device))
+    return out.reshape(*data.shape[:-1], k)
+
+
 def dequantize(q: BlockScaledTensor) -> torch.Tensor:
-    """bf16 ``code * 2^(scales - 127)`` in ``q.data``'s shape (``quantization.py:277-297``)."""
-    if q.packed or not q.pow2_scale or q.block_size != BLOCK:
-        raise NotImplementedError("only mxfp8 block-scaled tensors are built on this path")
+    """bf16 ``code * 2^(scales - 127)`` in the source's shape (``quantization.py:277-297``)."""
+    if not q.pow2_scale or q.block_size != BLOCK or q.global_scale is not None:
+        raise NotImplementedError("only MX (power-of-two scale per 32) block-scaled tensors are built on this path")
+    if q.packed:
+        return _dequantize_packed(q)
     data = q.data.view(torch.uint8)
     axis = q.axis % data.dim()
     if axis != data.dim() - 1:
@@ -179,16 +287,23 @@ def dequantize(q: BlockScaledTensor) -> torch.Tensor:
     return dequantize_rows_mxfp8(packed).reshape(data.shape)
 
 
-def _round_trip(t: torch.Tensor, axis: int) -> torch.Tensor:
-    """Quantise then dequantise, bf16 (``quantization.py:307-311``): one launch for a weight axis, two for rows."""
+def _round_trip(t: torch.Tensor, fmt: str, axis: int) -> torch.Tensor:
+    """Quantise then dequantise, bf16 (``quantization.py:307-311``): one launch, except MXFP8 rows, which take two."""
+    require_implemented(fmt)
     kind, axis = _axis_layout(t, axis)
     if t.shape[axis] % BLOCK:
         raise ValueError(f"axis {axis} size {t.shape[axis]} not divisible by block_size {BLOCK}")
     if kind == "moved":
-        return _round_trip(t.transpose(axis, -1).contiguous(), -1).transpose(axis, -1).contiguous()
+        return _round_trip(t.transpose(axis, -1).contiguous(), fmt, -1).transpose(axis, -1).contiguous()
     if kind == "rows":
-        return dequantize_rows_mxfp8(quantize_rows_mxfp8(t.reshape(-1, t.shape[-1]))).reshape(t.shape)
-    return quantize_weight_mxfp8(t.reshape(-1, *t.shape[-2:]), with_dequant=True).dequant.reshape(t.shape)
+        flat = t.reshape(-1, t.shape[-1])
+        if fmt == "mxfp4":
+            return mxfp4_rows(flat, codes=False, round_trip=True)[2].reshape(t.shape)
+        return dequantize_rows_mxfp8(quantize_rows_mxfp8(flat)).reshape(t.shape)
+    banks = t.reshape(-1, *t.shape[-2:])
+    if fmt == "mxfp4":
+        return mxfp4_weight(banks, codes=False, round_trip=True)[2].reshape(t.shape)
+    return quantize_weight_mxfp8(banks, with_dequant=True).dequant.reshape(t.shape)
 
 
 class _FakeQuant(torch.autograd.Function):
@@ -197,8 +312,7 @@ class _FakeQuant(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, t: torch.Tensor, fmt: str, axis: int) -> torch.Tensor:
-        require_implemented(fmt)
-        return _round_trip(t, axis).to(t.dtype)
+        return _round_trip(t, fmt, axis).to(t.dtype)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -238,6 +352,7 @@ class WeightVersionCache:
 
 
 _weight_dequant_cache = WeightVersionCache()
+_weight_round_trip_cache = WeightVersionCache()
 _weight_operand_cache = WeightVersionCache()
 
 
@@ -269,9 +384,26 @@ def cached_fake_quant(weight: torch.Tensor, fmt: str = "mxfp8", axis: int = -1) 
     dequant = _weight_dequant_cache.get(weight, fingerprint)
     if dequant is None:
         with torch.no_grad():
-            dequant = _round_trip(weight, axis).to(weight.dtype)
+            dequant = _round_trip(weight, fmt, axis).to(weight.dtype)
         _weight_dequant_cache.put(weight, fingerprint, dequant)
     return _CachedFakeQuant.apply(weight, dequant)
+
+
+def expert_weight_round_trip(weight: torch.Tensor, fmt: str, cacheable: bool) -> torch.Tensor:
+    """The bf16 round trip of ``[G, K, N]`` expert weights along K, detached: what the fake-quant route multiplies by
+    in the forward and in the input gradient.  Computed once per optimizer step for a leaf parameter when
+    ``cacheable``; the caller must not write to it."""
+    require_implemented(fmt)
+    if not (cacheable and weight.is_leaf and weight_cache_enabled()):
+        with torch.no_grad():
+            return _round_trip(weight.detach(), fmt, 1).to(torch.bfloat16)
+    fingerprint = (weight._version, fmt, 1)
+    value = _weight_round_trip_cache.get(weight, fingerprint)
+    if value is None:
+        with torch.no_grad():
+            value = _round_trip(weight.detach(), fmt, 1).to(torch.bfloat16)
+        _weight_round_trip_cache.put(weight, fingerprint, value)
+    return value
 
 
 def expert_weight_operand(weight: torch.Tensor, cacheable: bool) -> MxWeight:

@@ -2,7 +2,8 @@
 
 Mirrors ``halo/kernels/lowp/spec.py:9-11`` of the reference: ``QuantFormat`` names a block-scaled operand format of
 the expert GEMM.  Of the reference's three (mxfp8 = e4m3 + e8m0 / 32, mxfp4 = e2m1 + e8m0 / 32, nvfp4 = e2m1 +
-e4m3 / 16) this path implements mxfp8, on the scaled e4m3 matrix instruction; the 4-bit formats raise.
+e4m3 / 16) this path implements mxfp8, on the scaled e4m3 matrix instruction, and mxfp4, as the reference's default
+does, by the bf16 product of the two round-tripped operands; nvfp4 raises.
 """
 
 from __future__ import annotations
@@ -10,7 +11,7 @@ from __future__ import annotations
 from typing import Literal
 
 QuantFormat = Literal["mxfp8", "mxfp4", "nvfp4"]
-IMPLEMENTED_FORMATS: tuple[str, ...] = ("mxfp8",)
+IMPLEMENTED_FORMATS: tuple[str, ...] = ("mxfp8", "mxfp4")
 
 # Elements per shared scale along the contraction axis (``halo/kernels/lowp/quantization.py:47``).
 FORMAT_BLOCK_SIZE: dict[str, int] = {"mxfp8": 32, "mxfp4": 32, "nvfp4": 16}
@@ -20,4 +21,4 @@ def require_implemented(fmt: str) -> None:
     if fmt not in FORMAT_BLOCK_SIZE:
         raise ValueError(f"unknown block-scaled format {fmt!r} (expected one of {sorted(FORMAT_BLOCK_SIZE)})")
     if fmt not in IMPLEMENTED_FORMATS:
-        raise NotImplementedError(f"quant_format={fmt!r}: only {', '.join(IMPLEMENTED_FORMATS)} is built on this path")
+        raise NotImplementedError(f"quant_format={fmt!r}: only {', '.join(IMPLEMENTED_FORMATS)} are built on this path")

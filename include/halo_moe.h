@@ -307,6 +307,35 @@ int hmoe_grouped_gemm_fwd_mxfp8(const uint8_t* a_q, const uint8_t* a_scale, int6
                                 const uint8_t* b_scale, const int32_t* offs, int64_t total_rows, int num_groups,
                                 int64_t k, int64_t n, void* out, int64_t ldo, void* stream);
 
+/* ------------------------------------------------------------------------------------------------------- MXFP4
+ * The reference's "mxfp4" quant_format (halo/kernels/lowp/spec.py:11): e2m1 elements (magnitudes 0, 0.5, 1, 1.5, 2, 3,
+ * 4, 6; code = sign << 3 | level) with one e8m0 power-of-two scale per 32 values along the contraction axis.
+ * expert_gemm(quant_format="mxfp4") of the reference is the bf16 grouped product of the two fake-quantised operands
+ * (halo/kernels/expert_gemm.py:33-38), and so it is here: these entries produce the round trip's bf16 result in one pass
+ * (and the packed codes and exponents of the quantiser API), the product is hmoe_grouped_gemm_fwd's.
+ *
+ * hmoe_mxfp4_rows replaces quantize_mxfp4(t, axis=-1), dequantize and their composition the fake-quant round trip
+ * (halo/kernels/lowp/quantization.py:154-180, 191-198, 208-211, 248-266, 277-297, 307-311) for x [x_rows, k] (HMOE_BF16
+ * or HMOE_F32, row stride ldx).  Row r is x[row_index[r]] (an index outside [0, x_rows) gives zeros) or x[r] with
+ * row_index NULL.  The block's scale code is the biased exponent e + 127 of the smallest power of two 2^e >= amax / 6,
+ * e clamped to [-127, 127]; 254 for a block holding an inf, 0xFF for one holding a NaN.  An element's code is the level
+ * nearest to |v| 2^-e (clamped to 6), a tie going to the level with the even code, with the sign of v 2^-e.  Outputs,
+ * each optional (NULL), at least one of packed and round_trip given, scale required with packed: packed u8
+ * [rows, k / 2] (element 2 i in the low nibble of byte i, 2 i + 1 in the high), scale u8 [rows, k / 32], round_trip
+ * bf16 [rows, k] (row stride ldo) = level * sign * 2^(scale - 127).  k must be a multiple of 32.
+ *
+ * hmoe_mxfp4_weight is the same along axis 1 of expert weights w [groups, k, n] (quantize_mxfp4(w, axis=1)): packed u8
+ * [groups, k / 2, n] (rows 2 i and 2 i + 1 of k in byte (i, c), the even one low), scale u8 [groups, k / 32, n],
+ * round_trip bf16 [groups, k, n].
+ *
+ * hmoe_mxfp4_dequantize_rows replaces dequantize (quantization.py:277-297) for the pair hmoe_mxfp4_rows writes. */
+int hmoe_mxfp4_rows(const void* x, int dtype, int64_t ldx, const int64_t* row_index, int64_t x_rows, int64_t rows,
+                    int64_t k, uint8_t* packed, uint8_t* scale, void* round_trip, int64_t ldo, void* stream);
+int hmoe_mxfp4_weight(const void* w, int dtype, int64_t groups, int64_t k, int64_t n, uint8_t* packed, uint8_t* scale,
+                      void* round_trip, void* stream);
+int hmoe_mxfp4_dequantize_rows(const uint8_t* packed, const uint8_t* scale, int64_t rows, int64_t k, void* out,
+                               int64_t ldo, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

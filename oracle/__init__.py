@@ -33,5 +33,12 @@ How each function is pinned (tests/test_oracle_*.py):
   ``tests/gpu/kernels/test_expert_gemm.py:55-74``) and the product term by term on sampled outputs.  For fp32 inputs
   whose amax / 448 lies within an ulp of a power of two the reference's exponent depends on the rounding of its
   ``log2``: "parity unpinned" there (bf16 inputs are never that close).
+* ``mxfp4.*`` -- the block exponent by ``2^(e-1) < amax/6 <= 2^e`` in exact rational arithmetic; the e2m1 rounding by brute
+  force over every multiple of 1/64 in [-7, 7] (a nearest level, the even code on a tie); the known answers the
+  reference's tests hold (amax 6 -> scale 1 and every level its own code, 2.5 down / 2.6 up / 2.4 down of
+  ``tests/cpu/kernels/test_block_scale_oracle.py:60-94``; 0.75, 1.75, 3.5, -0.75 -> 1, 2, 4, -1 and the storage shapes
+  of ``tests/cpu/kernels/test_quantization.py:48-55, 99-113``; zero, sub-2^-127, inf and NaN blocks, the 0.25 round-trip
+  bound, the magnitude independence of ``test_block_scale_oracle.py:118-137``) and the product term by term on sampled
+  outputs.  The same fp32 ``log2`` caveat as ``mxfp8`` at power-of-two multiples of 6: "parity unpinned" there.
 * ``moe_layer.*`` -- the dense formula ``out[t] = sum_k w[t,k] * FFN_e(x[t])`` over valid slots.
 """

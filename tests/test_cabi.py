@@ -144,6 +144,24 @@ def test_bad_arguments_come_back_as_status_codes_before_any_launch():
     assert mx(fake, fake, 8, fake, fake, None, 8, 4, 128, 128, fake, 128, None) == invalid      # groups without ends
     assert mx(fake, fake, 8, fake, None, fake, 8, 4, 128, 128, fake, 128, None) == invalid
     assert mx(None, None, 0, None, None, None, 0, 1, 128, 128, None, 128, None) == 0
+
+    # MXFP4: blocks of 32 along the contraction, at least one output, the scales with the codes
+    rows4 = lib.hmoe_mxfp4_rows
+    assert rows4(fake, bf16, 64, None, 8, 8, 48, fake, fake, None, 64, None) == unsupported   # K % 32
+    assert rows4(fake, 77, 64, None, 8, 8, 64, fake, fake, None, 64, None) == unsupported     # dtype
+    assert rows4(fake, bf16, 64, None, 9, 8, 64, fake, fake, None, 64, None) == invalid       # no index: x_rows == rows
+    assert rows4(fake, bf16, 64, None, 8, 8, 64, None, None, None, 64, None) == invalid       # no output
+    assert rows4(fake, bf16, 64, None, 8, 8, 64, fake, None, None, 64, None) == invalid       # codes without scales
+    assert rows4(fake, bf16, 64, None, 8, 8, 64, None, None, fake, 60, None) == unsupported   # rows that overlap
+    assert rows4(None, bf16, 64, None, 0, 0, 64, None, None, None, 64, None) == 0
+    weight4 = lib.hmoe_mxfp4_weight
+    assert weight4(fake, bf16, 4, 48, 64, fake, fake, None, None) == unsupported
+    assert weight4(fake, bf16, 4, 64, 64, None, None, None, None) == invalid
+    assert weight4(fake, bf16, 4, 64, 64, fake, None, None, None) == invalid
+    assert weight4(fake, bf16, 0, 64, 64, None, None, None, None) == 0
+    assert lib.hmoe_mxfp4_dequantize_rows(fake, fake, 8, 48, fake, 64, None) == unsupported
+    assert lib.hmoe_mxfp4_dequantize_rows(fake, None, 8, 64, fake, 64, None) == invalid
+    assert lib.hmoe_mxfp4_dequantize_rows(None, None, 0, 64, None, 64, None) == 0
     assert fp8(fake, None, 8, fake, fake, fake, 8, 4, 256, 128, fake, 128, None) == invalid
     assert fp8(None, None, 0, None, None, None, 0, 1, 256, 128, None, 128, None) == 0
     assert lib.hmoe_quantize_rows_fp8(fake, 200, None, 8, 8, 200, fake, fake, 8, None) == unsupported

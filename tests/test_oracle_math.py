@@ -1,4 +1,5 @@
-"""Pins ``oracle.glu``, ``oracle.grouped_mm``, ``oracle.router``, ``oracle.block_fp8``, ``oracle.mxfp8`` and ``oracle.moe_layer`` against
+"""Pins ``oracle.glu``, ``oracle.grouped_mm``, ``oracle.router``, ``oracle.block_fp8``, ``oracle.mxfp8``,
+``oracle.mxfp4`` and ``oracle.moe_layer`` against
 library routines (torch autograd, matmul, softmax, topk, the float8 cast), identities and brute force."""
 
 import numpy as np
@@ -6,7 +7,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from oracle import block_fp8, glu, grouped_mm, moe_layer, mxfp8, router
+from oracle import block_fp8, glu, grouped_mm, moe_layer, mxfp4, mxfp8, router
 
 PROBE = (-64.0, -8.0, -1.0, -0.5, -1e-3, 0.0, 1e-3, 0.5, 1.0, 8.0, 64.0)  # fused_glu.py:33 of the reference
 
@@ -440,4 +441,133 @@ def test_mxfp8_round_trip_and_expert_product_sit_in_the_reference_error_bands():
         e = int(np.searchsorted(offs, r, side="right"))
         total = sum(va[r, k] * 2.0 ** (int(sa[r, k // 32]) - 127) * vb[e, k, c] * 2.0 ** (int(sb[e, k // 32, c]) - 127)
                     for k in range(320))
+        assert abs(got[r, c] - total) <= 1e-12 * max(1.0, abs(total))
+
+
+# ----------------------------------------------------------------------------------------------------------- mxfp4
+def test_mxfp4_block_exponent_is_the_smallest_power_of_two_that_fits():
+    """Pins ``mxfp4.e8m0_exponent`` by its defining inequality in exact rational arithmetic, 2^(e-1) < amax / 6 <= 2^e,
+    and by the known answers the reference's tests hold: exponent 0 (code 127) for a block whose amax is 6
+    (``tests/cpu/kernels/test_block_scale_oracle.py:60-70``), code 0 for a block below 6 * 2^-127 and 254 for one
+    holding an inf (``tests/cpu/kernels/test_quantization.py:248-280``), 0xFF for a NaN block."""
+    from fractions import Fraction
+
+    x = _mx_blocks()
+    amax = x.abs().reshape(96, 8, 32).amax(dim=2).numpy()
+    e, biased = mxfp4.e8m0_exponent(amax)
+    assert biased.dtype == np.uint8 and np.array_equal(biased.astype(np.int64), e + 127)
+    for a, ee in zip(amax.reshape(-1).tolist(), e.reshape(-1).tolist()):
+        if a == 0:
+            assert ee == -127
+            continue
+        ratio = Fraction(a) / 6
+        assert ratio <= Fraction(2) ** ee and (ee == -127 or ratio > Fraction(2) ** (ee - 1)), (a, ee)
+    edge = np.array([6.0, 6.03125, 5.96875, 3.0, 3e-38, np.inf, np.nan, 3.0e38, 0.0], dtype=np.float32)
+    assert mxfp4.e8m0_exponent(edge)[1].tolist() == [127, 128, 127, 126, 0, 254, 255, 127 + 126, 0]
+
+
+def test_mxfp4_codes_are_the_nearest_level_with_ties_to_the_even_code():
+    """Pins ``e2m1_round`` / ``quantize_mxfp4`` / ``dequantize_mxfp4``: the reference's known answers -- with amax 6 the
+    scale is 1 and the levels map to their own codes (``tests/cpu/kernels/test_block_scale_oracle.py:60-78``); 2.5 goes
+    down to 2.0, 2.6 up, 2.4 down (``:81-94``); 0.75, 1.75, 3.5 and -0.75 go up to 1, 2, 4 and -1, 0.7 and 0.8 to their
+    nearest (``tests/cpu/kernels/test_quantization.py:99-113``) -- and, for every value of a dense grid, brute force:
+    the chosen level is a nearest one, and on an exact tie it is the one whose code is even."""
+    block = np.zeros(32, dtype=np.float32)
+    vals = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.5, -6.0]
+    block[:len(vals)] = vals
+    data, scales = mxfp4.quantize_mxfp4(block)
+    assert data.shape == (16,) and data.dtype == np.uint8 and scales.shape == (1,) and int(scales[0]) == 127
+    assert mxfp4.unpack_codes(data)[:len(vals)].tolist() == [0, 1, 2, 3, 4, 5, 6, 7, 9, 15]
+    assert data[0] == 0x10 and data[4] == 0xF9  # the even element sits in the low nibble
+    block = np.zeros(32, dtype=np.float32)
+    block[:4] = [6.0, 2.5, 2.6, 2.4]
+    assert mxfp4.unpack_codes(mxfp4.quantize_mxfp4(block)[0])[1:4].tolist() == [4, 5, 4]
+    block = np.zeros((1, 32), dtype=np.float32)
+    block[0, :7] = [6.0, 0.75, 1.75, 3.5, -0.75, 0.7, 0.8]
+    assert mxfp4.fake_quant_mxfp4(block)[0, :7].tolist() == [6.0, 1.0, 2.0, 4.0, -1.0, 0.5, 1.0]
+    grid = np.arange(-7 * 64, 7 * 64 + 1, dtype=np.float32) / 64  # every multiple of 1/64 in [-7, 7]: holds every tie
+    codes = mxfp4.e2m1_round(grid)
+    levels = mxfp4.E2M1_LEVELS.astype(np.float64)
+    for v, c in zip(grid.tolist(), codes.tolist()):
+        mag = min(abs(v), 6.0)
+        dist = np.abs(levels - mag)
+        nearest = np.flatnonzero(dist == dist.min())
+        want = nearest[0] if len(nearest) == 1 else next(i for i in nearest if i % 2 == 0)
+        assert c & 7 == want and (c >> 3) == (1 if v < 0 else 0), (v, c)
+    # shapes along the last axis and along axis 0 (``tests/cpu/kernels/test_quantization.py:48-55``)
+    torch.manual_seed(0)
+    x = (torch.randn(64, 256) * 0.5).numpy()
+    data, scales = mxfp4.quantize_mxfp4(x)
+    assert data.shape == (64, 128) and scales.shape == (64, 8) and data.dtype == scales.dtype == np.uint8
+    d0, s0 = mxfp4.quantize_mxfp4(x.T.copy(), axis=0)
+    assert d0.shape == (128, 64) and s0.shape == (8, 64) and np.array_equal(d0, data.T) and np.array_equal(s0, scales.T)
+    # code * scale is within half a level gap of the value: at most a quarter of the block's scale below 2 * scale,
+    # half of it up to 4, one above
+    restored = mxfp4.dequantize_mxfp4(data, scales)
+    scale = np.repeat(np.ldexp(1.0, scales.astype(np.int64) - 127), 32, axis=1)
+    ratio = np.abs(x.astype(np.float64)) / scale
+    bound = np.where(ratio <= 2, 0.25, np.where(ratio <= 4, 0.5, 1.0)) * scale
+    assert (np.abs(restored - x) <= bound * (1 + 2.0 ** -8)).all()  # 2^-8: the bf16 rounding of the result
+    with pytest.raises(ValueError, match="not divisible"):
+        mxfp4.quantize_mxfp4(np.zeros((8, 30), dtype=np.float32))
+
+
+def test_mxfp4_extreme_blocks_keep_their_codes():
+    """The edges the reference tests (``tests/cpu/kernels/test_quantization.py:82-89, 248-280``;
+    ``tests/cpu/kernels/test_block_scale_oracle.py:175-196``): zeros round-trip to zeros; a block below 6 * 2^-127
+    clamps to exponent -127 and one holding an inf reaches 127, both keeping nonzero codes; an inf or a NaN makes its
+    own block non-finite and no other; a large finite outlier never produces a NaN."""
+    zeros = mxfp4.fake_quant_mxfp4(np.zeros((32, 64), dtype=np.float32))
+    assert np.isfinite(zeros).all() and not zeros.any()
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(4, 64, generator=g)
+    sign = torch.where(torch.rand(32, generator=g) < 0.5, -1.0, 1.0)
+    x[1, :32] = (torch.rand(32, generator=g) * 0.5 + 0.5) * 3e-38 * sign
+    x[2, :32] = torch.exp2(torch.rand(32, generator=g) * 19 + 108) * sign
+    x[2, 0] = float("inf")
+    x[3, 40] = float("nan")
+    x[0, 0] = 5e4
+    data, scales = mxfp4.quantize_mxfp4(x.numpy())
+    assert scales[1, 0] == 0 and scales[2, 0] == 254 and scales[3, 1] == 255 and scales[3, 0] != 255
+    codes = mxfp4.unpack_codes(data)
+    assert (codes[1, :32] & 7).max() > 0 and (codes[2, 1:32] & 7).max() > 0 and codes[2, 0] == 7
+    # 3e-38 * 2^127 = 5.1: the tiny block's codes are those of its values times 2^127
+    assert np.array_equal(codes[1, :32], mxfp4.e2m1_round((x[1, :32].double() * 2.0 ** 127).float().numpy()))
+    restored = mxfp4.dequantize_mxfp4(data, scales)
+    assert np.isnan(restored[3, 32:]).all() and np.isfinite(restored[3, :32]).all() and np.isfinite(restored[0]).all()
+    assert not np.isfinite(restored[2, :32]).all() and np.isfinite(restored[2, 32:]).all()
+
+
+def test_mxfp4_round_trip_and_expert_product_sit_in_the_format_error_bands():
+    """The reference's tolerance for the round trip (relative Frobenius error below 0.25 on ``randn(64, 256) * 0.5``,
+    ``tests/cpu/kernels/test_quantization.py:24, 57-64``) with mxfp8 the more accurate of the two (``:67-70`` states it
+    for fp8 against fp4), the error independent of the magnitude over 32 decades
+    (``tests/cpu/kernels/test_block_scale_oracle.py:118-137``), and the product checked term by term on sampled
+    outputs."""
+    torch.manual_seed(0)
+    x = (torch.randn(64, 256) * 0.5).numpy()
+    err4 = np.linalg.norm(mxfp4.fake_quant_mxfp4(x) - x) / np.linalg.norm(x)
+    err8 = np.linalg.norm(mxfp8.fake_quant_mxfp8(x) - x) / np.linalg.norm(x)
+    assert err8 < err4 < 0.25 and err4 > 0.05
+    base = torch.randn(128, 256).double().numpy()
+    errs = []
+    for exponent in range(4, -32, -4):
+        scaled = (base * 10.0 ** exponent).astype(np.float32)
+        recon = mxfp4.fake_quant_mxfp4(scaled).astype(np.float64)
+        errs.append(np.linalg.norm(recon - scaled) / np.linalg.norm(scaled.astype(np.float64)))
+    assert max(errs) - min(errs) < 0.02
+    g = torch.Generator().manual_seed(3)
+    counts = (40, 0, 70, 18)
+    a = (torch.randn(sum(counts), 320, generator=g) * 0.3).bfloat16().float().numpy()
+    b = (torch.randn(len(counts), 320, 96, generator=g) * 0.02).bfloat16().float().numpy()
+    offs = np.cumsum(counts)
+    got = mxfp4.expert_gemm_mxfp4(a, b, offs)
+    ca, sa = mxfp4.unpack_codes(mxfp4.quantize_mxfp4(a, -1)[0]), mxfp4.quantize_mxfp4(a, -1)[1]
+    cb, sb = mxfp4.unpack_codes(mxfp4.quantize_mxfp4(b, 1)[0], 1), mxfp4.quantize_mxfp4(b, 1)[1]
+    level = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+    value = lambda c: level[c & 7] * (-1.0 if c & 8 else 1.0)
+    for r, c in ((0, 0), (39, 95), (40, 3), (127, 50)):
+        e = int(np.searchsorted(offs, r, side="right"))
+        total = sum(value(int(ca[r, k])) * 2.0 ** (int(sa[r, k // 32]) - 127) *
+                    value(int(cb[e, k, c])) * 2.0 ** (int(sb[e, k // 32, c]) - 127) for k in range(320))
         assert abs(got[r, c] - total) <= 1e-12 * max(1.0, abs(total))
