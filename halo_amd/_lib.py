@@ -62,6 +62,10 @@ SIGNATURES = {
     "hmoe_mxfp4_rows": (I, [P, I, L, P, L, L, L, P, P, P, L, P]),
     "hmoe_mxfp4_weight": (I, [P, I, L, L, L, P, P, P, P]),
     "hmoe_mxfp4_dequantize_rows": (I, [P, P, L, L, P, L, P]),
+    "hmoe_mxfp4_rows_panels": (I, [P, I, L, P, L, L, L, P, P, L, P]),
+    "hmoe_mxfp4_weight_panels": (I, [P, I, L, L, L, P, P, P, P]),
+    "hmoe_mxfp4_dequantize_panels": (I, [P, P, L, L, L, P, L, P]),
+    "hmoe_grouped_gemm_fwd_mxfp4": (I, [P, P, L, P, P, P, L, I, L, L, P, L, P]),
 }
 
 _lib = None

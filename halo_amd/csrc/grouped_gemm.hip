@@ -1569,12 +1569,17 @@ constexpr int kF8ScaleBase = kF8Stages * kF8Stage;
 // The scales of a stage.  Block scales (kMx false): a dword per tile row holding the row's exponent for the stage's
 // 128-value block, and 64 dwords of weight scales.  MXFP8 (kMx true): an exponent per 32 values on both sides, so a
 // stage (64 values) carries two planes of 256 dwords per operand, plane h for the stage's contraction half h.
-template <bool kMx>
+// MXFP4 (kFmt 2): e2m1 elements, 128 values in a panel's 64 bytes, so a stage carries four blocks of 32; their four
+// exponents lie side by side in one dword per tile row and per tile column (the quantisers write them so), one plane
+// of 256 dwords per operand.
+enum F8Format { kBlockFp8 = 0, kMxFp8 = 1, kMxFp4 = 2 };
+template <int kFmt>
 struct F8Scales {
-  static constexpr int kA = kMx ? 2 * 256 * 4 : 256 * 4;
-  static constexpr int kB = kMx ? 2 * 256 * 4 : 64 * 4;
+  static constexpr int kA = kFmt == kMxFp8 ? 2 * 256 * 4 : 256 * 4;
+  static constexpr int kB = kFmt == kMxFp8 ? 2 * 256 * 4 : (kFmt == kMxFp4 ? 256 * 4 : 64 * 4);
   static constexpr int kLds = kF8ScaleBase + kF8Stages * (kA + kB);
-  static constexpr int kLoads = kMx ? 12 : 10;  // per loading wavefront and stage: 4 + 4 tile loads, then the scales
+  // per loading wavefront and stage: 4 + 4 tile loads, then the scales
+  static constexpr int kLoads = kFmt == kMxFp8 ? 12 : 10;
 };
 
 __device__ __forceinline__ void lds_load4(u32x4 rsrc, lds_bytes_ptr lds_base, uint32_t voffset, uint32_t soffset) {
@@ -1593,10 +1598,12 @@ __device__ __forceinline__ void lds_load1(u32x4 rsrc, lds_bytes_ptr lds_base, ui
                : "memory", "m0");
 }
 
-template <bool kMx>
+template <int kFmt>
 __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
+  constexpr bool kMx = kFmt != kBlockFp8;   // an e8m0 exponent per 32 values on both sides
+  constexpr bool kMx8 = kFmt == kMxFp8, kFp4 = kFmt == kMxFp4;
   constexpr int WM = 4, WN = 2, BM = 256, BN = 256, kLoadWaves = 4;
-  constexpr int kF8ScaleA = F8Scales<kMx>::kA, kF8ScaleB = F8Scales<kMx>::kB;
+  constexpr int kF8ScaleA = F8Scales<kFmt>::kA, kF8ScaleB = F8Scales<kFmt>::kB;
   using Sched = TileSchedule<kFwd, BM, BN>;
   extern __shared__ __attribute__((aligned(16))) char lds_raw[];
   __shared__ int32_t grp_s[kMaxGroups], grp_e[kMaxGroups], tile_start[kMaxGroups + 1];
@@ -1636,9 +1643,10 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
   __syncthreads();
   Sched sched;
   sched.init(p, grp_s, grp_e, tile_start);
-  const int steps = static_cast<int>(p.k / kF8K);  // the same for every tile
+  // the same for every tile; an e2m1 panel holds 128 values, its last one zeros past K
+  const int steps = kFp4 ? static_cast<int>((p.k + 127) / 128) : static_cast<int>(p.k / kF8K);
   const uint32_t a_panel = static_cast<uint32_t>(p.a_scale_rows) * kF8K, b_panel = static_cast<uint32_t>(p.n) * kF8K;
-  const int64_t w_bytes = p.k * p.n;
+  const int64_t w_bytes = static_cast<int64_t>(steps) * kF8K * p.n;
 
   // ---- the loading wavefronts' view of a tile
   // A load instruction moves 16 rows of 64 bytes: lane L takes row L >> 2, and the chunk that belongs at its place
@@ -1656,7 +1664,7 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
       rsrc_a = make_rsrc_words(a, static_cast<uint32_t>(steps) * a_panel - static_cast<uint32_t>(tile.row_start) * kF8K);
       rsrc_b = make_rsrc_words(static_cast<const uint8_t*>(p.b) + tile.g * w_bytes, static_cast<uint32_t>(w_bytes));
       rsrc_sa = make_rsrc_words(p.a_scale, static_cast<uint32_t>(p.k_blocks) * static_cast<uint32_t>(p.a_scale_rows));
-      if constexpr (kMx)
+      if constexpr (kMx)  // k_blocks counts the exponent bytes per row or column (MXFP4: four per panel)
         rsrc_sb = make_rsrc_words(p.b_scale_e8m0 + static_cast<int64_t>(tile.g) * p.k_blocks * p.n,
                                   static_cast<uint32_t>(p.k_blocks) * static_cast<uint32_t>(p.n));
       else
@@ -1668,11 +1676,13 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
       // one 16-byte read
       const int d = slot * 64 + lane;
       voff_sa = static_cast<uint32_t>(tile.row_start + tile.a_out0 + (d >> 7) * 128 + (d & 3) * 32 + ((d & 127) >> 2));
+      if constexpr (kFp4) voff_sa *= 4u;  // a dword of four exponents per row
       if constexpr (kMx) {
         // the weights' plane: dword d takes tile column (d >> 6) * 64 + (d & 1) * 32 + ((d & 63) >> 1), so that the two
         // column blocks of a wavefront's lane lie in one 8-byte read.  A column past N reads another column's
         // exponent (or zero past the group's end) and reaches only outputs that are not stored.
         voff_sb = static_cast<uint32_t>(tile.b_out0 + (d >> 6) * 64 + (d & 1) * 32 + ((d & 63) >> 1));
+        if constexpr (kFp4) voff_sb *= 4u;
       } else {
         int nb = (tile.b_out0 >> 7) + (lane & 1);
         nb = nb < p.n_blocks ? nb : p.n_blocks - 1;
@@ -1691,7 +1701,10 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) lds_load16(rsrc_b, ta + kF8Tile + t * 1024, voff_b + t * 1024, soff_b);
     lds_bytes_ptr sc = lds + kF8ScaleBase + buf * (kF8ScaleA + kF8ScaleB);
-    if constexpr (kMx) {
+    if constexpr (kFp4) {
+      lds_load4(rsrc_sa, sc + slot * 256, voff_sa, static_cast<uint32_t>(step) * static_cast<uint32_t>(p.a_scale_rows) * 4u);
+      lds_load4(rsrc_sb, sc + kF8ScaleA + slot * 256, voff_sb, static_cast<uint32_t>(step) * static_cast<uint32_t>(p.n) * 4u);
+    } else if constexpr (kMx) {
       const uint32_t rows_a = static_cast<uint32_t>(p.a_scale_rows), cols_b = static_cast<uint32_t>(p.n);
 #pragma unroll
       for (int h = 0; h < 2; ++h)
@@ -1716,9 +1729,16 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
   constexpr int kPartner = 32;
   const int fa0 = (row_a + (lane & 31)) * kF8K + frag_chunk;
   const int fb0 = kF8Tile + (row_b + (lane & 31)) * kF8K + frag_chunk;
-  const int sa_at = kF8ScaleBase + (kMx ? half * 1024 : 0) + (row_a + (lane & 31) * 4) * 4;
-  const int sb_at = kMx ? kF8ScaleBase + kF8ScaleA + half * 1024 + (row_b + (lane & 31) * 2) * 4
+  const int sa_at = kF8ScaleBase + (kMx8 ? half * 1024 : 0) + (row_a + (lane & 31) * 4) * 4;
+  const int sb_at = kMx ? kF8ScaleBase + kF8ScaleA + (kMx8 ? half * 1024 : 0) + (row_b + (lane & 31) * 2) * 4
                         : kF8ScaleBase + kF8ScaleA + (gn >> 1) * 4;
+  // MXFP4: a stage is two instructions of 64 values; in instruction m the lane of half h holds block 2 m + h of the
+  // stage (32 values, the 16 bytes of chunk 2 m + h) and supplies that block's exponent.  Byte selectors that pull
+  // block c out of two neighbouring dwords of exponents (v_perm_b32: selector bytes 0-3 name the second operand's
+  // bytes, 4-7 the first's):
+  const uint32_t sel_a0 = static_cast<uint32_t>(half) * 0x0101u + 0x0400u;
+  const uint32_t sel_a1 = static_cast<uint32_t>(2 + half) * 0x0101u + 0x0400u;
+  const uint32_t sel_b = static_cast<uint32_t>(half) * 0x01010101u + 0x06020400u;
   i32x8 fa8[WM], fb8[WN];
   auto fragment = [&](int at) __attribute__((always_inline)) {
     const i32x4 lo = *reinterpret_cast<const i32x4*>(lds_raw + at);
@@ -1766,9 +1786,20 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
     if (load_wave && steps > 3) issue(3);
     // stage 0 into registers
     uint32_t sa_pack, sb_bits;
+    uint32_t sa_pack1 = 0;  // MXFP4: the row blocks' exponents for the stage's second instruction
     auto read_scales = [&](int buf) __attribute__((always_inline)) {
       const char* sc = lds_raw + buf * (kF8ScaleA + kF8ScaleB);
       const u32x4 q = *reinterpret_cast<const u32x4*>(sc + sa_at);
+      if constexpr (kFp4) {
+        const u32x2 w = *reinterpret_cast<const u32x2*>(sc + sb_at);
+        sa_pack = __builtin_amdgcn_perm(__builtin_amdgcn_perm(q[3], q[2], sel_a0),
+                                        __builtin_amdgcn_perm(q[1], q[0], sel_a0), 0x05040100u);
+        sa_pack1 = __builtin_amdgcn_perm(__builtin_amdgcn_perm(q[3], q[2], sel_a1),
+                                         __builtin_amdgcn_perm(q[1], q[0], sel_a1), 0x05040100u);
+        // bytes: (instruction 0, column block 0), (0, 1), (1, 0), (1, 1)
+        sb_bits = __builtin_amdgcn_perm(w[1], w[0], sel_b);
+        return;
+      }
       sa_pack = (q[0] & 0xffu) | ((q[1] & 0xffu) << 8) | ((q[2] & 0xffu) << 16) | (q[3] << 24);
       if constexpr (kMx) {
         const u32x2 w = *reinterpret_cast<const u32x2*>(sc + sb_at);
@@ -1790,8 +1821,18 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
       constexpr bool kFull = decltype(full_tag)::value;
       auto mfma = [&](auto row_block, auto col_block, int sa, int sb) __attribute__((always_inline)) {
         constexpr int i = decltype(row_block)::value, j = decltype(col_block)::value;
-        if (kFull || i < live)
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[j], fa8[i], acc[i][j], 0, 0, kMx ? j : 0, sb, i, sa);
+        if (kFull || i < live) {
+          if constexpr (kFp4) {
+            // cbsz = blgp = 4: e2m1 operands, of which the instruction reads the first four registers
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[j], fa8[i], acc[i][j], 4, 4, j, sb, i, sa);
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                __builtin_shufflevector(fb8[j], fb8[j], 4, 5, 6, 7, 4, 5, 6, 7),
+                __builtin_shufflevector(fa8[i], fa8[i], 4, 5, 6, 7, 4, 5, 6, 7), acc[i][j], 4, 4, 2 + j, sb, i,
+                static_cast<int>(sa_pack1));
+          } else {
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[j], fa8[i], acc[i][j], 0, 0, kMx ? j : 0, sb, i, sa);
+          }
+        }
       };
       using std::integral_constant;
       const integral_constant<int, 0> b0;
@@ -1835,12 +1876,13 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
         // stage step + 1 must be in: the loads of at most two younger stages may still be out
         const int younger = steps - 2 - step;
         if (load_wave) {
-          static_assert(F8Scales<false>::kLoads == 10 && F8Scales<true>::kLoads == 12, "the waits below count them");
+          constexpr int kLoads = F8Scales<kFmt>::kLoads;
+          static_assert(kLoads == 10 || kLoads == 12, "the waits below count them");
           if (younger >= 2) {
-            if constexpr (kMx) asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)" ::: "memory");
+            if constexpr (kLoads == 12) asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)" ::: "memory");
             else asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)" ::: "memory");
           } else if (younger == 1) {
-            if constexpr (kMx) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
+            if constexpr (kLoads == 12) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
             else asm volatile("s_waitcnt vmcnt(10) lgkmcnt(0)" ::: "memory");
           } else {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -2139,14 +2181,14 @@ int validate(const GemmArgs& p, int dtype) {
   return HMOE_OK;
 }
 
-template <bool kMx>
+template <int kFmt>
 int launch_fp8(const GemmArgs& p, int64_t workers, void* stream) {
-  constexpr int kLds = F8Scales<kMx>::kLds;
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_fp8_kernel<kMx>),
+  constexpr int kLds = F8Scales<kFmt>::kLds;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_fp8_kernel<kFmt>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
     return HMOE_LAUNCH_FAILED;
-  grouped_gemm_fp8_kernel<kMx><<<dim3(static_cast<unsigned>(workers)), dim3(512), kLds,
-                                static_cast<hipStream_t>(stream)>>>(p);
+  grouped_gemm_fp8_kernel<kFmt><<<dim3(static_cast<unsigned>(workers)), dim3(512), kLds,
+                                 static_cast<hipStream_t>(stream)>>>(p);
   if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
   return HMOE_OK;
 }
@@ -2311,7 +2353,7 @@ int hmoe_grouped_gemm_fwd_fp8(const uint8_t* a_q, const uint8_t* a_scale, int64_
   int64_t workers = device_cus();
   if (bound < workers) workers = bound;
   workers = (workers + kXcds - 1) / kXcds * kXcds;
-  return launch_fp8<false>(p, workers, stream);
+  return launch_fp8<kBlockFp8>(p, workers, stream);
 }
 
 int hmoe_grouped_gemm_fwd_mxfp8(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
@@ -2347,7 +2389,45 @@ int hmoe_grouped_gemm_fwd_mxfp8(const uint8_t* a_q, const uint8_t* a_scale, int6
   int64_t workers = device_cus();
   if (bound < workers) workers = bound;
   workers = (workers + kXcds - 1) / kXcds * kXcds;
-  return launch_fp8<true>(p, workers, stream);
+  return launch_fp8<kMxFp8>(p, workers, stream);
+}
+
+int hmoe_grouped_gemm_fwd_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
+                                const uint8_t* b_scale, const int32_t* offs, int64_t total_rows, int num_groups,
+                                int64_t k, int64_t n, void* out, int64_t ldo, void* stream) {
+  using namespace hmoe;
+  if (total_rows < 0 || num_groups <= 0 || k < 0 || n < 0) return HMOE_INVALID_ARGUMENT;
+  if (offs == nullptr && num_groups != 1) return HMOE_INVALID_ARGUMENT;
+  if (num_groups > kMaxGroups) return HMOE_UNSUPPORTED;
+  // whole blocks of 32 values along the contraction (the operands' last panel is zeros past K); 16-byte rows
+  if (k % 32 || n % 8 || ldo % 8 || ldo < n || a_rows < total_rows) return HMOE_UNSUPPORTED;
+  if (total_rows == 0 || n == 0) return HMOE_OK;
+  if (k == 0) return HMOE_UNSUPPORTED;
+  if (!a_q || !a_scale || !bq || !b_scale || !out) return HMOE_INVALID_ARGUMENT;
+  if (!aligned16(a_q) || !aligned16(bq) || !aligned16(out) || reinterpret_cast<uintptr_t>(a_scale) % 4 ||
+      reinterpret_cast<uintptr_t>(b_scale) % 4)
+    return HMOE_UNSUPPORTED;
+  const int64_t lim = int64_t(1) << 31, panels = (k + 127) / 128;
+  if (a_rows * panels * 64 >= lim || panels * 64 * n >= lim || total_rows * ldo * 2 >= lim) return HMOE_UNSUPPORTED;
+  GemmArgs p{};
+  p.a = a_q;
+  p.b = bq;
+  p.c = out;
+  p.ldc = ldo;
+  p.offs = offs;
+  p.total_rows = total_rows;
+  p.groups = num_groups;
+  p.k = k;
+  p.n = n;
+  p.b_scale_e8m0 = b_scale;
+  p.a_scale = a_scale;
+  p.a_scale_rows = a_rows;
+  p.k_blocks = static_cast<int>(panels * 4);
+  const int64_t bound = (total_rows / 256 + num_groups) * ((n + 255) / 256);
+  int64_t workers = device_cus();
+  if (bound < workers) workers = bound;
+  workers = (workers + kXcds - 1) / kXcds * kXcds;
+  return launch_fp8<kMxFp4>(p, workers, stream);
 }
 
 int hmoe_grouped_gemm_dgrad(const void* grad_out, int64_t ldg, const void* b, const int32_t* offs,

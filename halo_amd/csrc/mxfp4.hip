@@ -4,9 +4,11 @@
 // Replaces quantize_mxfp4 / dequantize / the fake-quant round trip of the reference for this format
 // (halo/kernels/lowp/quantization.py:154-180, 191-198, 208-211, 248-269, 277-297, 307-311).  The reference's
 // expert_gemm(quant_format="mxfp4") multiplies the two round-tripped operands with the bf16 grouped GEMM
-// (halo/kernels/expert_gemm.py:33-38); that is what this build does too, so the kernels here produce the round trip's
-// bf16 result in one pass (and, for the quantiser API, the packed codes and exponents in the reference's layout: two
-// codes per byte along the quantised axis, low nibble first).
+// (halo/kernels/expert_gemm.py:33-38).  Here the quantised operands go to the scaled matrix instruction (the e2m1
+// variant of grouped_gemm_fp8_kernel), which sums the same products in fp32; the kernels of this file write its
+// operands (codes and exponents in panels of 128 contraction values), the reference's logical layout for the quantiser
+// API (two codes per byte along the quantised axis, low nibble first), and the round trip's bf16 result in one pass
+// (the straight-through backward's operands, and the forward's for fp32 inputs).
 #include "common.h"
 #include "fp8_rows.h"
 
@@ -24,43 +26,33 @@ __device__ __forceinline__ uint32_t mx4_block_code(float amax, bool any_nan) {
   return any_nan ? 255u : static_cast<uint32_t>(biased);
 }
 
-// |scaled| (clamped to 6) rounded to the nearest e2m1 magnitude, a tie going to the level with the even code
-// (quantization.py:191-198: bucketize sends a value on a boundary down, the ties-up table lifts 0.75, 1.75 and 3.5).
-// The even code is the even significand, so this is IEEE round-to-nearest-even at e2m1's precision: below 1 the levels
-// are the multiples of 0.5, which adding 2^22 rounds to; from 1 up they keep one mantissa bit.  A NaN clamps to 6, the
-// level bucketize gives it.
-__device__ __forceinline__ float e2m1_round_mag(float scaled) {
-  const float mag = fminf(fabsf(scaled), 6.0f);
-  const uint32_t bits = __float_as_uint(mag);
-  const float one_bit = __uint_as_float((bits + 0x001fffffu + ((bits >> 22) & 1u)) & 0xffc00000u);
-  const float halves = (mag + 4194304.0f) - 4194304.0f;
-  return mag < 1.0f ? halves : one_bit;
+// Two scaled values to two e2m1 codes (sign << 3 | level) in byte `kByte` of `word`, by the conversion instruction:
+// the nearest level, a tie to the level with the even code, magnitudes above 6 (an inf too) to 6.  That is the
+// reference's rule (quantization.py:191-198: bucketize sends a value on a boundary down, the ties-up table lifts 0.75,
+// 1.75 and 3.5; the even code is the even significand, so it is IEEE round-to-nearest-even at e2m1's precision): the
+// instruction gives the reference's code for every multiple of 1/64 in [-7, 7], for infinities and for a positive NaN
+// (code 7, where bucketize puts it).  The sign bit is set for a value below zero and not for -0.0, as `scaled < 0` has
+// it: adding +0.0 turns -0.0 into +0.0 and changes nothing else.
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+template <int kByte>
+__device__ __forceinline__ uint32_t e2m1_pack2(uint32_t word, float lo, float hi) {
+  return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, lo + 0.0f, hi + 0.0f, 1.0f, kByte);
 }
-
-// the level's code: 0.5, 1, 1.5, 2, 3, 4, 6 have the top bits 252, 254, 255 .. 259 (exponent and first mantissa bit)
-__device__ __forceinline__ uint32_t e2m1_level(float rounded_mag) {
-  const int from_bits = static_cast<int>(__float_as_uint(rounded_mag) >> 22) - 252;
-  return static_cast<uint32_t>(max(from_bits, rounded_mag > 0.0f ? 1 : 0));
+__device__ __forceinline__ uint32_t e2m1_pack8(const float* v) {
+  uint32_t word = 0u;
+  word = e2m1_pack2<0>(word, v[0], v[1]);
+  word = e2m1_pack2<1>(word, v[2], v[3]);
+  word = e2m1_pack2<2>(word, v[4], v[5]);
+  word = e2m1_pack2<3>(word, v[6], v[7]);
+  return word;
 }
-
-// e2m1 code (sign << 3 | level) of a scaled value; the sign bit is set for a value below zero (not for -0.0)
-__device__ __forceinline__ uint32_t e2m1_code(float scaled) {
-  return e2m1_level(e2m1_round_mag(scaled)) | (scaled < 0.0f ? 8u : 0u);
-}
-
-// the round trip of a scaled value before the block's scale is put back: the rounded magnitude under that sign
-__device__ __forceinline__ float e2m1_round(float scaled) {
-  const float mag = e2m1_round_mag(scaled);
-  return scaled < 0.0f ? -mag : mag;
-}
-
-// the value of a code: levels 0, 0.5, 1, 1.5, 2, 3, 4, 6 with the sign bit
-__device__ __forceinline__ float e2m1_value(uint32_t code) {
-  const uint32_t level = code & 7u;
-  // level >= 2: (1 + (level & 1) / 2) * 2^((level >> 1) - 1), assembled as fp32 bits
-  const float mag = level < 2u ? 0.5f * static_cast<float>(level)
-                               : __uint_as_float(((126u + (level >> 1)) << 23) | ((level & 1u) << 22));
-  return (code & 8u) ? -mag : mag;
+// the values of the eight codes of a word: levels 0, 0.5, 1, 1.5, 2, 3, 4, 6 under the sign bit
+__device__ __forceinline__ void e2m1_unpack8(uint32_t word, float* v) {
+  const f32x2_t a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 0);
+  const f32x2_t b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 1);
+  const f32x2_t c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 2);
+  const f32x2_t d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 3);
+  v[0] = a.x; v[1] = a.y; v[2] = b.x; v[3] = b.y; v[4] = c.x; v[5] = c.y; v[6] = d.x; v[7] = d.y;
 }
 
 __device__ __forceinline__ float e8m0_to_f32(uint32_t code) {
@@ -93,19 +85,28 @@ __device__ __forceinline__ void load16<float>(const float* p, float (&v)[16]) {
 // an index.  Two lanes hold a block of 32 values, sixteen each.  Outputs, each optional: packed [R, K / 2] (two codes
 // per byte, the even element in the low nibble), scale [R, K / 32], and round_trip bf16 [R, K] (row stride ldo): code
 // value times 2^(scale - 127).
-template <typename T>
+//
+// kPanels: the layout the e2m1 matrix kernel loads instead.  packed [ceil(K / 128)][out_rows][64]: the 128 values of
+// panel p of row r in the 64 bytes at (p * out_rows + r) * 64, value 2 b in the low nibble of byte b; scale
+// [ceil(K / 128)][out_rows][4]: the exponents of the panel's four blocks side by side.  Values past K are zeros (code
+// 0, exponent 0).  Consecutive lanes run along a row (whole lines in); a panel's 64 bytes of a row go out together.
+template <typename T, bool kPanels>
 __global__ void __launch_bounds__(256)
 mxfp4_rows_kernel(const T* __restrict__ x, int64_t ldx, const int64_t* __restrict__ row_index, int64_t x_rows,
                   int64_t rows, int k, uint8_t* __restrict__ packed, uint8_t* __restrict__ scale,
-                  bf16_t* __restrict__ round_trip, int64_t ldo) {
-  const int pieces = k >> 4;  // 16-value pieces per row
+                  bf16_t* __restrict__ round_trip, int64_t ldo, int64_t out_rows) {
   const int64_t unit = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  const int64_t row = unit / pieces;
-  const int piece = static_cast<int>(unit - row * pieces);
-  if (row >= rows) return;  // lane pairs leave together (pieces is even)
+  int64_t row;
+  int piece;  // 16-value piece of the row
+  {
+    const int pieces = kPanels ? ((k + 127) >> 7) * 8 : k >> 4;  // whole panels: the last one's tail is written as zeros
+    row = unit / pieces;
+    piece = static_cast<int>(unit - row * pieces);
+    if (row >= rows) return;  // lane pairs leave together (pieces is even)
+  }
   float v[16];
   const int64_t from = row_index != nullptr ? row_index[row] : row;
-  if (from >= 0 && from < x_rows) {
+  if (from >= 0 && from < x_rows && (piece << 4) < k) {
     load16<T>(x + from * ldx + (piece << 4), v);
   } else {
 #pragma unroll
@@ -125,18 +126,25 @@ mxfp4_rows_kernel(const T* __restrict__ x, int64_t ldx, const int64_t* __restric
   mx_scale_down(biased, pre, inv);
 #pragma unroll
   for (int i = 0; i < 16; ++i) v[i] = nan ? 6.0f : v[i] * pre * inv;  // a NaN block: every code 7, the scale NaN
+  const uint32_t words[2] = {e2m1_pack8(v), e2m1_pack8(v + 8)};
   if (packed != nullptr) {
-    uint32_t words[2] = {0u, 0u};
-#pragma unroll
-    for (int i = 0; i < 16; ++i) words[i >> 3] |= e2m1_code(v[i]) << ((i & 7) * 4);
-    *reinterpret_cast<uint2*>(packed + row * (k >> 1) + (piece << 3)) = make_uint2(words[0], words[1]);
+    const int64_t at = kPanels ? ((piece >> 3) * out_rows + row) * 64 + ((piece & 7) << 3)
+                               : row * (k >> 1) + (piece << 3);
+    *reinterpret_cast<uint2*>(packed + at) = make_uint2(words[0], words[1]);
   }
-  if (scale != nullptr && (piece & 1) == 0) scale[row * (k >> 5) + (piece >> 1)] = static_cast<uint8_t>(biased);
+  if (scale != nullptr && (piece & 1) == 0) {
+    const int64_t at = kPanels ? ((piece >> 3) * out_rows + row) * 4 + ((piece & 7) >> 1) : row * (k >> 5) + (piece >> 1);
+    scale[at] = static_cast<uint8_t>(biased);
+  }
   if (round_trip != nullptr) {
     const float s = e8m0_to_f32(biased);
     Vec16<bf16_t> o[2];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) o[i >> 3].v[i & 7] = e2m1_round(v[i]) * s;
+    for (int h = 0; h < 2; ++h) {
+      e2m1_unpack8(words[h], o[h].v);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[h].v[i] *= s;
+    }
     o[0].store(round_trip + row * ldo + (piece << 4));
     o[1].store(round_trip + row * ldo + (piece << 4) + 8);
   }
@@ -145,9 +153,13 @@ mxfp4_rows_kernel(const T* __restrict__ x, int64_t ldx, const int64_t* __restric
 // Weights [G, K, N] along K (axis 1).  A workgroup takes 64 contraction values of 128 columns through LDS (fp32, pitch
 // 129); thread (column, half) owns the block of 32 down its column.  Outputs, each optional: packed [G, K / 2, N]
 // (rows 2 i and 2 i + 1 of K in one byte, the even one low), scale [G, K / 32, N], round_trip bf16 [G, K, N].
+//
+// kPanels: packed [G][ceil(K / 128)][N][64] (the 128 values of panel p down column c in the 64 bytes at
+// ((g P + p) N + c) * 64) and scale [G][ceil(K / 128)][N][4], as the e2m1 matrix kernel loads them; the grid then covers
+// whole panels, and values past K are zeros (code 0, exponent 0).
 constexpr int kTileK = 64, kTileN = 128, kPitch = kTileN + 1;
 
-template <typename T>
+template <typename T, bool kPanels>
 __global__ void __launch_bounds__(256)
 mxfp4_weight_kernel(const T* __restrict__ w, int64_t k, int64_t n, uint8_t* __restrict__ packed,
                     uint8_t* __restrict__ scale, bf16_t* __restrict__ round_trip) {
@@ -179,7 +191,7 @@ mxfp4_weight_kernel(const T* __restrict__ w, int64_t k, int64_t n, uint8_t* __re
   __syncthreads();
   const int c = threadIdx.x & (kTileN - 1), h = threadIdx.x >> 7;
   const int64_t col = n0 + c, kb = blockIdx.y * 2 + h;
-  if (col >= n || kb * 32 >= k) return;
+  if (col >= n || (!kPanels && kb * 32 >= k)) return;
   float v[32];
   float amax = 0.f;
   bool nan = false;
@@ -193,39 +205,147 @@ mxfp4_weight_kernel(const T* __restrict__ w, int64_t k, int64_t n, uint8_t* __re
   float pre, inv;
   mx_scale_down(biased, pre, inv);
   const float s = e8m0_to_f32(biased);
-  if (scale != nullptr) scale[(g * (k / 32) + kb) * n + col] = static_cast<uint8_t>(biased);
 #pragma unroll
   for (int i = 0; i < 32; ++i) v[i] = nan ? 6.0f : v[i] * pre * inv;
-  if (packed != nullptr) {
+  const uint32_t words[4] = {e2m1_pack8(v), e2m1_pack8(v + 8), e2m1_pack8(v + 16), e2m1_pack8(v + 24)};
+  if constexpr (kPanels) {
+    const int64_t at = (g * ((k + 127) >> 7) + (kb >> 2)) * n + col;  // the column's panel
+    scale[at * 4 + (kb & 3)] = static_cast<uint8_t>(biased);
+    *reinterpret_cast<uint4*>(packed + at * 64 + ((kb & 3) << 4)) = make_uint4(words[0], words[1], words[2], words[3]);
+  } else {
+    if (scale != nullptr) scale[(g * (k / 32) + kb) * n + col] = static_cast<uint8_t>(biased);
+    if (packed != nullptr) {
 #pragma unroll
-    for (int i = 0; i < 32; i += 2)
-      packed[(g * (k / 2) + kb * 16 + (i >> 1)) * n + col] =
-          static_cast<uint8_t>(e2m1_code(v[i]) | (e2m1_code(v[i + 1]) << 4));
+      for (int i = 0; i < 16; ++i)
+        packed[(g * (k / 2) + kb * 16 + i) * n + col] = static_cast<uint8_t>(words[i >> 2] >> ((i & 3) * 8));
+    }
   }
-  if (round_trip != nullptr) {
+  if (round_trip != nullptr && kb * 32 < k) {
     bf16_t* out = round_trip + (g * k + kb * 32) * n + col;
 #pragma unroll
-    for (int i = 0; i < 32; ++i) out[i * n] = f32_to_bf16(e2m1_round(v[i]) * s);
+    for (int q = 0; q < 4; ++q) {
+      float back[8];
+      e2m1_unpack8(words[q], back);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) out[(q * 8 + i) * n] = f32_to_bf16(back[i] * s);
+    }
   }
 }
 
-// packed codes and exponents back to bf16, rows along the last axis (the quantiser API's dequantize)
+// packed codes and exponents back to bf16, rows along the last axis (the quantiser API's dequantize); kPanels: from
+// the matrix kernel's layout (q_rows rows per panel)
+template <bool kPanels>
 __global__ void __launch_bounds__(256)
 mxfp4_dequantize_rows_kernel(const uint8_t* __restrict__ packed, const uint8_t* __restrict__ scale, int64_t rows, int k,
-                             bf16_t* __restrict__ out, int64_t ldo) {
+                             bf16_t* __restrict__ out, int64_t ldo, int64_t q_rows) {
   const int pieces = k >> 4;
   const int64_t unit = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   const int64_t row = unit / pieces;
   const int piece = static_cast<int>(unit - row * pieces);
   if (row >= rows) return;
-  const uint2 words = *reinterpret_cast<const uint2*>(packed + row * (k >> 1) + (piece << 3));
-  const float s = e8m0_to_f32(scale[row * (k >> 5) + (piece >> 1)]);
-  const uint32_t w[2] = {words.x, words.y};
+  const int64_t at = kPanels ? ((piece >> 3) * q_rows + row) * 64 + ((piece & 7) << 3) : row * (k >> 1) + (piece << 3);
+  const int64_t s_at = kPanels ? ((piece >> 3) * q_rows + row) * 4 + ((piece & 7) >> 1) : row * (k >> 5) + (piece >> 1);
+  const uint2 words = *reinterpret_cast<const uint2*>(packed + at);
+  const float s = e8m0_to_f32(scale[s_at]);
   Vec16<bf16_t> o[2];
+  e2m1_unpack8(words.x, o[0].v);
+  e2m1_unpack8(words.y, o[1].v);
 #pragma unroll
-  for (int i = 0; i < 16; ++i) o[i >> 3].v[i & 7] = e2m1_value((w[i >> 3] >> ((i & 7) * 4)) & 15u) * s;
+  for (int i = 0; i < 8; ++i) {
+    o[0].v[i] *= s;
+    o[1].v[i] *= s;
+  }
   o[0].store(out + row * ldo + (piece << 4));
   o[1].store(out + row * ldo + (piece << 4) + 8);
+}
+
+}  // namespace
+}  // namespace hmoe
+
+namespace hmoe {
+namespace {
+
+int launch_rows(const void* x, int dtype, int64_t ldx, const int64_t* row_index, int64_t x_rows, int64_t rows, int64_t k,
+                uint8_t* packed, uint8_t* scale, void* round_trip, int64_t ldo, int64_t out_rows, bool panels,
+                void* stream) {
+  if (rows < 0 || k < 0 || x_rows < 0) return HMOE_INVALID_ARGUMENT;
+  if (!row_index && x_rows != rows) return HMOE_INVALID_ARGUMENT;
+  if (dtype != HMOE_BF16 && dtype != HMOE_F32) return HMOE_UNSUPPORTED;
+  if (k % 32 || ldx < k || ldx % 8) return HMOE_UNSUPPORTED;
+  if (round_trip && (ldo < k || ldo % 8)) return HMOE_UNSUPPORTED;
+  if (panels && out_rows < rows) return HMOE_UNSUPPORTED;
+  if (rows == 0 || k == 0) return HMOE_OK;
+  if ((!x && x_rows > 0) || (!packed && !round_trip) || (packed && !scale)) return HMOE_INVALID_ARGUMENT;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(packed) % 8 ||
+      reinterpret_cast<uintptr_t>(round_trip) % 16)
+    return HMOE_UNSUPPORTED;
+  const int64_t pieces = panels ? (k + 127) / 128 * 8 : k / 16;
+  const int64_t blocks = (rows * pieces + 255) / 256;
+  if (blocks >= (int64_t(1) << 31) || k >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>(blocks));
+  auto launch = [&](auto kernel, auto* typed) {
+    kernel<<<grid, dim3(256), 0, s>>>(typed, ldx, row_index, x_rows, rows, static_cast<int>(k), packed, scale,
+                                      static_cast<bf16_t*>(round_trip), ldo, out_rows);
+  };
+  if (dtype == HMOE_BF16) {
+    if (panels) launch(mxfp4_rows_kernel<bf16_t, true>, static_cast<const bf16_t*>(x));
+    else launch(mxfp4_rows_kernel<bf16_t, false>, static_cast<const bf16_t*>(x));
+  } else {
+    if (panels) launch(mxfp4_rows_kernel<float, true>, static_cast<const float*>(x));
+    else launch(mxfp4_rows_kernel<float, false>, static_cast<const float*>(x));
+  }
+  HMOE_CHECK_LAUNCH();
+  return HMOE_OK;
+}
+
+int launch_weight(const void* w, int dtype, int64_t groups, int64_t k, int64_t n, uint8_t* packed, uint8_t* scale,
+                  void* round_trip, bool panels, void* stream) {
+  if (groups < 0 || k < 0 || n < 0) return HMOE_INVALID_ARGUMENT;
+  if (dtype != HMOE_BF16 && dtype != HMOE_F32) return HMOE_UNSUPPORTED;
+  if (k % 32) return HMOE_UNSUPPORTED;
+  if (groups == 0 || k == 0 || n == 0) return HMOE_OK;
+  if (!w || (!packed && !round_trip) || (packed && !scale) || (panels && !packed)) return HMOE_INVALID_ARGUMENT;
+  if (panels && reinterpret_cast<uintptr_t>(packed) % 16) return HMOE_UNSUPPORTED;
+  const int64_t k_tiles = panels ? (k + 127) / 128 * 2 : (k + kTileK - 1) / kTileK;
+  const int64_t col_tiles = (n + kTileN - 1) / kTileN;
+  if (k_tiles > 65535 || groups > 65535 || col_tiles >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
+  const dim3 grid(static_cast<unsigned>(col_tiles), static_cast<unsigned>(k_tiles), static_cast<unsigned>(groups));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto launch = [&](auto kernel, auto* typed) {
+    kernel<<<grid, dim3(256), 0, s>>>(typed, k, n, packed, scale, static_cast<bf16_t*>(round_trip));
+  };
+  if (dtype == HMOE_BF16) {
+    if (panels) launch(mxfp4_weight_kernel<bf16_t, true>, static_cast<const bf16_t*>(w));
+    else launch(mxfp4_weight_kernel<bf16_t, false>, static_cast<const bf16_t*>(w));
+  } else {
+    if (panels) launch(mxfp4_weight_kernel<float, true>, static_cast<const float*>(w));
+    else launch(mxfp4_weight_kernel<float, false>, static_cast<const float*>(w));
+  }
+  HMOE_CHECK_LAUNCH();
+  return HMOE_OK;
+}
+
+int launch_dequantize(const uint8_t* packed, const uint8_t* scale, int64_t q_rows, int64_t rows, int64_t k, void* out,
+                      int64_t ldo, bool panels, void* stream) {
+  if (rows < 0 || k < 0) return HMOE_INVALID_ARGUMENT;
+  if (k % 32 || ldo < k || ldo % 8) return HMOE_UNSUPPORTED;
+  if (panels && q_rows < rows) return HMOE_INVALID_ARGUMENT;
+  if (rows == 0 || k == 0) return HMOE_OK;
+  if (!packed || !scale || !out) return HMOE_INVALID_ARGUMENT;
+  if (reinterpret_cast<uintptr_t>(packed) % 8 || reinterpret_cast<uintptr_t>(out) % 16) return HMOE_UNSUPPORTED;
+  const int64_t blocks = (rows * (k / 16) + 255) / 256;
+  if (blocks >= (int64_t(1) << 31) || k >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
+  const dim3 grid(static_cast<unsigned>(blocks));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (panels)
+    mxfp4_dequantize_rows_kernel<true><<<grid, dim3(256), 0, s>>>(packed, scale, rows, static_cast<int>(k),
+                                                                 static_cast<bf16_t*>(out), ldo, q_rows);
+  else
+    mxfp4_dequantize_rows_kernel<false><<<grid, dim3(256), 0, s>>>(packed, scale, rows, static_cast<int>(k),
+                                                                  static_cast<bf16_t*>(out), ldo, q_rows);
+  HMOE_CHECK_LAUNCH();
+  return HMOE_OK;
 }
 
 }  // namespace
@@ -235,69 +355,33 @@ extern "C" {
 
 int hmoe_mxfp4_rows(const void* x, int dtype, int64_t ldx, const int64_t* row_index, int64_t x_rows, int64_t rows,
                     int64_t k, uint8_t* packed, uint8_t* scale, void* round_trip, int64_t ldo, void* stream) {
-  using namespace hmoe;
-  if (rows < 0 || k < 0 || x_rows < 0) return HMOE_INVALID_ARGUMENT;
-  if (!row_index && x_rows != rows) return HMOE_INVALID_ARGUMENT;
-  if (dtype != HMOE_BF16 && dtype != HMOE_F32) return HMOE_UNSUPPORTED;
-  if (k % 32 || ldx < k || ldx % 8) return HMOE_UNSUPPORTED;
-  if (round_trip && (ldo < k || ldo % 8)) return HMOE_UNSUPPORTED;
-  if (rows == 0 || k == 0) return HMOE_OK;
-  if ((!x && x_rows > 0) || (!packed && !round_trip) || (packed && !scale)) return HMOE_INVALID_ARGUMENT;
-  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(packed) % 8 ||
-      reinterpret_cast<uintptr_t>(round_trip) % 16)
-    return HMOE_UNSUPPORTED;
-  const int64_t blocks = (rows * (k / 16) + 255) / 256;
-  if (blocks >= (int64_t(1) << 31) || k >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(static_cast<unsigned>(blocks));
-  if (dtype == HMOE_BF16)
-    mxfp4_rows_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(static_cast<const bf16_t*>(x), ldx, row_index, x_rows, rows,
-                                                        static_cast<int>(k), packed, scale,
-                                                        static_cast<bf16_t*>(round_trip), ldo);
-  else
-    mxfp4_rows_kernel<float><<<grid, dim3(256), 0, s>>>(static_cast<const float*>(x), ldx, row_index, x_rows, rows,
-                                                       static_cast<int>(k), packed, scale,
-                                                       static_cast<bf16_t*>(round_trip), ldo);
-  HMOE_CHECK_LAUNCH();
-  return HMOE_OK;
+  return hmoe::launch_rows(x, dtype, ldx, row_index, x_rows, rows, k, packed, scale, round_trip, ldo, rows, false, stream);
 }
 
 int hmoe_mxfp4_weight(const void* w, int dtype, int64_t groups, int64_t k, int64_t n, uint8_t* packed, uint8_t* scale,
                       void* round_trip, void* stream) {
-  using namespace hmoe;
-  if (groups < 0 || k < 0 || n < 0) return HMOE_INVALID_ARGUMENT;
-  if (dtype != HMOE_BF16 && dtype != HMOE_F32) return HMOE_UNSUPPORTED;
-  if (k % 32) return HMOE_UNSUPPORTED;
-  if (groups == 0 || k == 0 || n == 0) return HMOE_OK;
-  if (!w || (!packed && !round_trip) || (packed && !scale)) return HMOE_INVALID_ARGUMENT;
-  const int64_t k_tiles = (k + kTileK - 1) / kTileK, col_tiles = (n + kTileN - 1) / kTileN;
-  if (k_tiles > 65535 || groups > 65535 || col_tiles >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
-  const dim3 grid(static_cast<unsigned>(col_tiles), static_cast<unsigned>(k_tiles), static_cast<unsigned>(groups));
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == HMOE_BF16)
-    mxfp4_weight_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(static_cast<const bf16_t*>(w), k, n, packed, scale,
-                                                          static_cast<bf16_t*>(round_trip));
-  else
-    mxfp4_weight_kernel<float><<<grid, dim3(256), 0, s>>>(static_cast<const float*>(w), k, n, packed, scale,
-                                                         static_cast<bf16_t*>(round_trip));
-  HMOE_CHECK_LAUNCH();
-  return HMOE_OK;
+  return hmoe::launch_weight(w, dtype, groups, k, n, packed, scale, round_trip, false, stream);
 }
 
 int hmoe_mxfp4_dequantize_rows(const uint8_t* packed, const uint8_t* scale, int64_t rows, int64_t k, void* out,
                                int64_t ldo, void* stream) {
-  using namespace hmoe;
-  if (rows < 0 || k < 0) return HMOE_INVALID_ARGUMENT;
-  if (k % 32 || ldo < k || ldo % 8) return HMOE_UNSUPPORTED;
-  if (rows == 0 || k == 0) return HMOE_OK;
-  if (!packed || !scale || !out) return HMOE_INVALID_ARGUMENT;
-  if (reinterpret_cast<uintptr_t>(packed) % 8 || reinterpret_cast<uintptr_t>(out) % 16) return HMOE_UNSUPPORTED;
-  const int64_t blocks = (rows * (k / 16) + 255) / 256;
-  if (blocks >= (int64_t(1) << 31) || k >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
-  mxfp4_dequantize_rows_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
-      packed, scale, rows, static_cast<int>(k), static_cast<bf16_t*>(out), ldo);
-  HMOE_CHECK_LAUNCH();
-  return HMOE_OK;
+  return hmoe::launch_dequantize(packed, scale, rows, rows, k, out, ldo, false, stream);
+}
+
+int hmoe_mxfp4_rows_panels(const void* x, int dtype, int64_t ldx, const int64_t* row_index, int64_t x_rows, int64_t rows,
+                           int64_t k, uint8_t* q, uint8_t* scale, int64_t out_rows, void* stream) {
+  if (rows > 0 && k > 0 && !q) return HMOE_INVALID_ARGUMENT;
+  return hmoe::launch_rows(x, dtype, ldx, row_index, x_rows, rows, k, q, scale, nullptr, 0, out_rows, true, stream);
+}
+
+int hmoe_mxfp4_weight_panels(const void* w, int dtype, int64_t groups, int64_t k, int64_t n, uint8_t* q, uint8_t* scale,
+                             void* round_trip, void* stream) {
+  return hmoe::launch_weight(w, dtype, groups, k, n, q, scale, round_trip, true, stream);
+}
+
+int hmoe_mxfp4_dequantize_panels(const uint8_t* q, const uint8_t* scale, int64_t q_rows, int64_t rows, int64_t k,
+                                 void* out, int64_t ldo, void* stream) {
+  return hmoe::launch_dequantize(q, scale, q_rows, rows, k, out, ldo, true, stream);
 }
 
 }  // extern "C"

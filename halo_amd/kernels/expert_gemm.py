@@ -3,8 +3,8 @@ quantisation-aware formats (both operands block-scaled along the contraction, st
 weights (the quantised-weight serving configuration, forward only).
 
 Mirrors the dispatch seam of the reference's ``halo/kernels/expert_gemm.py:14-38``.  Of its ``quant_format`` values
-``"mxfp8"`` runs on the scaled e4m3 matrix instruction and ``"mxfp4"`` as the reference's default does, the bf16 product
-of the two round-tripped operands; ``"nvfp4"`` raises.
+``"mxfp8"`` and ``"mxfp4"`` run on the scaled matrix instruction (e4m3 / e2m1 operands with an e8m0 exponent per 32
+values); ``"nvfp4"`` raises.
 """
 
 from __future__ import annotations
@@ -198,45 +198,88 @@ class _MxFp8ExpertGemm(torch.autograd.Function):
         return grad_a, grad_b, None, None, None, None
 
 
+def mxfp4_mfma_usable(mat_a_dtype: torch.dtype, mat_b_dtype: torch.dtype, k: int, n: int) -> bool:
+    """Whether the scaled matrix instruction takes the MXFP4 product: bf16 operands, 16-byte output rows.  Anything
+    else multiplies the two round-tripped operands on the bf16 / fp32 kernel, the reference's own formulation."""
+    return mat_a_dtype == torch.bfloat16 and mat_b_dtype == torch.bfloat16 and k > 0 and k % 32 == 0 and n % 8 == 0
+
+
 _round_tripped_rows = _SharedRows()
+_quantised_rows4 = _SharedRows()
+_dequantised_rows4 = _SharedRows()
 
 
 class _Mxfp4ExpertGemm(torch.autograd.Function):
     """``grouped_mm(fake_quant(mat_a, "mxfp4", axis=-1), cached_fake_quant(mat_b, "mxfp4", axis=1), offs)`` of the
-    reference (``expert_gemm.py:33-38``) as one node: the rows go through the e2m1 round trip in one launch (which also
-    fetches them through ``row_index`` when the permuted copy was never made), the weights once per optimizer step,
-    and the product is the bf16 grouped GEMM's.  Backward is the straight-through estimator around ``grouped_mm``'s own
-    gradients (``quantization.py:350-360``, ``grouped_mm.py:16-27``) with the round-tripped operands."""
+    reference (``expert_gemm.py:33-38``) as one node.  Forward: the rows are quantised to e2m1 with an e8m0 scale per 32
+    values (one launch, which also fetches them through ``row_index`` when the permuted copy was never made), the
+    weights once per optimizer step, and the product runs on the scaled matrix instruction with e2m1 operands: the
+    same products of dequantised values the reference's bf16 GEMM sums, accumulated in fp32.  fp32 operands go through
+    the round trip in one launch each and the fp32 grouped GEMM.  Backward is the straight-through estimator around ``grouped_mm``'s own gradients
+    (``quantization.py:350-360``, ``grouped_mm.py:16-27``) with the round-tripped operands, the rows' rebuilt from the
+    saved e2m1 codes (a quarter of the bytes of a bf16 copy)."""
 
     @staticmethod
     def forward(ctx, mat_a, mat_b, offs, weight_cacheable, row_index, inv_map):
-        from halo_amd.kernels.lowp.quantization import expert_weight_round_trip, mxfp4_rows
+        from halo_amd.kernels.lowp.quantization import (expert_weight_operand, expert_weight_round_trip, mxfp4_rows,
+                                                        quantize_rows_mxfp4)
 
-        _lib.require_device(mat_a, mat_b, offs, row_index, inv_map)
+        device = _lib.require_device(mat_a, mat_b, offs, row_index, inv_map)
         if mat_a.dim() != 2 or mat_b.dim() != 3 or mat_a.shape[1] != mat_b.shape[1]:
             raise ValueError(f"expected [R, K] x [G, K, N], got {tuple(mat_a.shape)} x {tuple(mat_b.shape)}")
-        offs32 = _offs_arg(offs, mat_b.shape[0])
-        w_rt = expert_weight_round_trip(mat_b, "mxfp4", weight_cacheable).to(mat_a.dtype)
+        groups, k, n = mat_b.shape
+        offs32 = _offs_arg(offs, groups)
         key = (mat_a._version, None if row_index is None else (id(row_index), row_index._version))
-        a_rt = _round_tripped_rows.get(mat_a, key)
-        if a_rt is None:
-            a_rt = mxfp4_rows(mat_a, row_index, codes=False, round_trip=True)[2].to(mat_a.dtype)
-            _round_tripped_rows.put(mat_a, key, a_rt)
-        ctx.gathered = row_index is not None
-        ctx.save_for_backward(a_rt, w_rt, offs32, inv_map)
-        return _forward(a_rt, w_rt, offs32)
+        ctx.gathered, ctx.k, ctx.dtype = row_index is not None, k, mat_a.dtype
+        ctx.native = mxfp4_mfma_usable(mat_a.dtype, mat_b.dtype, k, n)
+        if not ctx.native:
+            w_rt = expert_weight_round_trip(mat_b, "mxfp4", weight_cacheable).to(mat_a.dtype)
+            a_rt = _round_tripped_rows.get(mat_a, key)
+            if a_rt is None:
+                a_rt = mxfp4_rows(mat_a, row_index, codes=False, round_trip=True)[2].to(mat_a.dtype)
+                _round_tripped_rows.put(mat_a, key, a_rt)
+            ctx.save_for_backward(a_rt, w_rt, offs32, inv_map)
+            return _forward(a_rt, w_rt, offs32)
+        weight = expert_weight_operand(mat_b, weight_cacheable, "mxfp4")
+        rows_q = _quantised_rows4.get(mat_a, key)
+        if rows_q is None:
+            rows_q = quantize_rows_mxfp4(mat_a, row_index)
+            _quantised_rows4.put(mat_a, key, rows_q)
+        rows = rows_q.rows
+        ctx.rows_q = rows_q  # projections that share the rows must see one object
+        ctx.save_for_backward(weight.dequant, offs32, inv_map)
+        out = torch.empty((rows, n), dtype=torch.bfloat16, device=device)
+        if rows and n:
+            with _lib.on_device(device):
+                _lib.call("hmoe_grouped_gemm_fwd_mxfp4", _lib.ptr(rows_q.q), _lib.ptr(rows_q.scales), rows,
+                          _lib.ptr(weight.q), _lib.ptr(weight.scales), _lib.ptr(offs32), rows, groups, k, n,
+                          _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):
+        from halo_amd.kernels.lowp.quantization import dequantize_rows_mxfp4
         from halo_amd.kernels.moe_permute import gather_reduce_rows
 
-        a_rt, w_rt, offs32, inv_map = ctx.saved_tensors
         grad_a = grad_b = None
-        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
-            grad_a, grad_b = grouped_mm_grads(a_rt, w_rt, grad_output.to(a_rt.dtype), offs32,
-                                              ctx.needs_input_grad[0], ctx.needs_input_grad[1])
-            if ctx.gathered and grad_a is not None:
-                grad_a = gather_reduce_rows(grad_a, inv_map)
+        if not (ctx.needs_input_grad[0] or ctx.needs_input_grad[1]):
+            return None, None, None, None, None, None
+        if ctx.native:
+            w_rt, offs32, inv_map = ctx.saved_tensors
+            q = ctx.rows_q.q
+            if ctx.needs_input_grad[1]:
+                a_rt = _dequantised_rows4.get(q, (q._version,))
+                if a_rt is None:
+                    a_rt = dequantize_rows_mxfp4(ctx.rows_q)
+                    _dequantised_rows4.put(q, (q._version,), a_rt)
+            else:  # the input gradient reads the rows' shape and dtype only
+                a_rt = grad_output.new_empty((1, ctx.k)).expand(q.shape[1], ctx.k).to(torch.bfloat16)
+        else:
+            a_rt, w_rt, offs32, inv_map = ctx.saved_tensors
+        grad_a, grad_b = grouped_mm_grads(a_rt, w_rt, grad_output.to(a_rt.dtype), offs32,
+                                          ctx.needs_input_grad[0], ctx.needs_input_grad[1])
+        if ctx.gathered and grad_a is not None:
+            grad_a = gather_reduce_rows(grad_a, inv_map)
         return grad_a, grad_b, None, None, None, None
 
 

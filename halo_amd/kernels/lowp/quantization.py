@@ -6,8 +6,8 @@ Mirrors ``halo/kernels/lowp/quantization.py`` of the reference for its ``mxfp8``
 (:277-297), ``fake_quant`` (:350-365), ``WeightVersionCache`` / ``cached_fake_quant`` (:368-422).  The MXFP8 kernels are
 ``csrc/mxfp8.hip``; they write the operands in the layout the GEMM kernel loads (:class:`MxRows`, :class:`MxWeight`),
 and the reference's logical layout is a byte permutation of those.  The MXFP4 kernels are ``csrc/mxfp4.hip``; they
-write the reference's layout (two codes per byte along the quantised axis) and, for the fake-quant route the expert
-GEMM takes with this format, the round trip's bf16 result in the same pass.
+write the reference's layout (two codes per byte along the quantised axis), the matrix kernel's operands
+(:class:`Mx4Rows`, :class:`Mx4Weight`) and the round trip's bf16 result in one pass.
 """
 
 from __future__ import annotations
@@ -59,6 +59,31 @@ class MxRows:
 class MxWeight:
     """Expert weights ``[G, K, N]`` quantised along K: ``q`` uint8 ``[G, ceil(K / 64), N, 64]``, ``scales`` uint8
     ``[G, K / 32, N]``, and ``dequant`` the round trip's bf16 ``[G, K, N]`` (None unless asked for)."""
+
+    q: torch.Tensor
+    scales: torch.Tensor
+    dequant: torch.Tensor | None
+    k: int
+
+
+@dataclass(frozen=True)
+class Mx4Rows:
+    """Activation rows ``[R, K]`` as the e2m1 matrix kernel loads them: ``q`` uint8 ``[ceil(K / 128), R, 64]`` (two
+    codes per byte, panels of 128 contraction values, zeros past K) and ``scales`` uint8 ``[ceil(K / 128), R, 4]``."""
+
+    q: torch.Tensor
+    scales: torch.Tensor
+    k: int
+
+    @property
+    def rows(self) -> int:
+        return self.q.shape[1]
+
+
+@dataclass(frozen=True)
+class Mx4Weight:
+    """Expert weights ``[G, K, N]`` quantised along K: ``q`` uint8 ``[G, ceil(K / 128), N, 64]``, ``scales`` uint8
+    ``[G, ceil(K / 128), N, 4]``, and ``dequant`` the round trip's bf16 ``[G, K, N]`` (None unless asked for)."""
 
     q: torch.Tensor
     scales: torch.Tensor
@@ -182,6 +207,58 @@ def mxfp4_weight(w: torch.Tensor, *, codes: bool = True, round_trip: bool = Fals
         _lib.call("hmoe_mxfp4_weight", _lib.ptr(w), _lib.dtype_id(w.dtype), g, k, n, _lib.ptr(packed), _lib.ptr(scales),
                   _lib.ptr(out), _lib.stream_ptr(device))
     return packed, scales, out
+
+
+def quantize_rows_mxfp4(x: torch.Tensor, row_index: torch.Tensor | None = None) -> Mx4Rows:
+    """``x [R, K]`` (bf16 or fp32, K a multiple of 32) to :class:`Mx4Rows`; with ``row_index`` (int64 ``[R']``) the rows
+    quantised are ``x[row_index]``, fetched by the kernel itself."""
+    device = _lib.require_device(x, row_index)
+    if x.dim() != 2:
+        raise ValueError(f"expected [R, K], got {tuple(x.shape)}")
+    x = _aligned_rows(_native_input(x))
+    k = x.shape[1]
+    if k % BLOCK:
+        raise ValueError(f"axis 1 size {k} not divisible by block_size {BLOCK}")
+    if row_index is not None:
+        row_index = row_index.to(torch.int64).contiguous()
+    rows = x.shape[0] if row_index is None else row_index.numel()
+    panels = -(-k // 128)
+    q = torch.empty((panels, rows, 64), dtype=torch.uint8, device=device)
+    scales = torch.empty((panels, rows, 4), dtype=torch.uint8, device=device)
+    with _lib.on_device(device):
+        _lib.call("hmoe_mxfp4_rows_panels", _lib.ptr(x), _lib.dtype_id(x.dtype), x.stride(0) if x.shape[0] else k,
+                  _lib.ptr(row_index), x.shape[0], rows, k, _lib.ptr(q), _lib.ptr(scales), rows,
+                  _lib.stream_ptr(device))
+    return Mx4Rows(q, scales, k)
+
+
+def dequantize_rows_mxfp4(rows: Mx4Rows) -> torch.Tensor:
+    """bf16 ``[R, K]``: ``level * sign * 2^(scale - 127)`` for every element of an :class:`Mx4Rows`."""
+    device = _lib.require_device(rows.q, rows.scales)
+    out = torch.empty((rows.rows, rows.k), dtype=torch.bfloat16, device=device)
+    with _lib.on_device(device):
+        _lib.call("hmoe_mxfp4_dequantize_panels", _lib.ptr(rows.q), _lib.ptr(rows.scales), rows.rows, rows.rows,
+                  rows.k, _lib.ptr(out), rows.k, _lib.stream_ptr(device))
+    return out
+
+
+def quantize_weight_mxfp4(w: torch.Tensor, with_dequant: bool = False) -> Mx4Weight:
+    """``w [G, K, N]`` (bf16 or fp32, K a multiple of 32) quantised along K to :class:`Mx4Weight`."""
+    device = _lib.require_device(w)
+    if w.dim() != 3:
+        raise ValueError(f"expected [G, K, N], got {tuple(w.shape)}")
+    w = _native_input(w).contiguous()
+    g, k, n = w.shape
+    if k % BLOCK:
+        raise ValueError(f"axis 1 size {k} not divisible by block_size {BLOCK}")
+    panels = -(-k // 128)
+    q = torch.empty((g, panels, n, 64), dtype=torch.uint8, device=device)
+    scales = torch.empty((g, panels, n, 4), dtype=torch.uint8, device=device)
+    dequant = torch.empty((g, k, n), dtype=torch.bfloat16, device=device) if with_dequant else None
+    with _lib.on_device(device):
+        _lib.call("hmoe_mxfp4_weight_panels", _lib.ptr(w), _lib.dtype_id(w.dtype), g, k, n, _lib.ptr(q),
+                  _lib.ptr(scales), _lib.ptr(dequant), _lib.stream_ptr(device))
+    return Mx4Weight(q, scales, dequant, k)
 
 
 def _axis_layout(t: torch.Tensor, axis: int) -> tuple[str, int]:
@@ -406,16 +483,18 @@ def expert_weight_round_trip(weight: torch.Tensor, fmt: str, cacheable: bool) ->
     return value
 
 
-def expert_weight_operand(weight: torch.Tensor, cacheable: bool) -> MxWeight:
-    """``[G, K, N]`` expert weights as the GEMM's MXFP8 operand together with the round trip's bf16 copy (which the
-    backward products read), quantised once per optimizer step for a leaf parameter when ``cacheable``."""
+def expert_weight_operand(weight: torch.Tensor, cacheable: bool, fmt: str = "mxfp8"):
+    """``[G, K, N]`` expert weights as the matrix kernel's operand in ``fmt`` (:class:`MxWeight` or
+    :class:`Mx4Weight`) together with the round trip's bf16 copy (which the backward products read), quantised once per
+    optimizer step for a leaf parameter when ``cacheable``."""
+    quantise = {"mxfp8": quantize_weight_mxfp8, "mxfp4": quantize_weight_mxfp4}[fmt]
     if not (cacheable and weight.is_leaf and weight_cache_enabled()):
         with torch.no_grad():
-            return quantize_weight_mxfp8(weight.detach(), with_dequant=True)
-    fingerprint = (weight._version, "mxfp8", 1)
+            return quantise(weight.detach(), with_dequant=True)
+    fingerprint = (weight._version, fmt, 1)
     operand = _weight_operand_cache.get(weight, fingerprint)
     if operand is None:
         with torch.no_grad():
-            operand = quantize_weight_mxfp8(weight.detach(), with_dequant=True)
+            operand = quantise(weight.detach(), with_dequant=True)
         _weight_operand_cache.put(weight, fingerprint, operand)
     return operand

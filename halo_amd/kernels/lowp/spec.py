@@ -2,8 +2,8 @@
 
 Mirrors ``halo/kernels/lowp/spec.py:9-11`` of the reference: ``QuantFormat`` names a block-scaled operand format of
 the expert GEMM.  Of the reference's three (mxfp8 = e4m3 + e8m0 / 32, mxfp4 = e2m1 + e8m0 / 32, nvfp4 = e2m1 +
-e4m3 / 16) this path implements mxfp8, on the scaled e4m3 matrix instruction, and mxfp4, as the reference's default
-does, by the bf16 product of the two round-tripped operands; nvfp4 raises.
+e4m3 / 16) this path implements mxfp8 and mxfp4, both on the scaled matrix instruction (e4m3 and e2m1 operands); nvfp4
+raises.
 """
 
 from __future__ import annotations

@@ -328,13 +328,33 @@ int hmoe_grouped_gemm_fwd_mxfp8(const uint8_t* a_q, const uint8_t* a_scale, int6
  * [groups, k / 2, n] (rows 2 i and 2 i + 1 of k in byte (i, c), the even one low), scale u8 [groups, k / 32, n],
  * round_trip bf16 [groups, k, n].
  *
- * hmoe_mxfp4_dequantize_rows replaces dequantize (quantization.py:277-297) for the pair hmoe_mxfp4_rows writes. */
+ * hmoe_mxfp4_dequantize_rows replaces dequantize (quantization.py:277-297) for the pair hmoe_mxfp4_rows writes.
+ *
+ * The same products on the scaled matrix instruction with e2m1 operands (twice the e4m3 rate, a quarter of bf16's
+ * operand bytes): hmoe_mxfp4_rows_panels and hmoe_mxfp4_weight_panels write the operands as the kernel loads them, in
+ * panels of 128 contraction values (64 bytes): rows q [ceil(k / 128)][out_rows][64] (value 2 b of panel p of row r in
+ * the low nibble of q[(p * out_rows + r) * 64 + b]) with scale u8 [ceil(k / 128)][out_rows][4] (the panel's four block
+ * exponents side by side); weights q [groups][ceil(k / 128)][n][64] with scale [groups][ceil(k / 128)][n][4] and, with
+ * round_trip not NULL, the round trip's bf16 [groups, k, n] for the straight-through backward.  Values past k are
+ * zeros (code 0, exponent 0).  hmoe_mxfp4_dequantize_panels gives rows back as bf16 [rows, k] from that layout (q_rows
+ * rows per panel).  hmoe_grouped_gemm_fwd_mxfp4: out bf16 [total_rows, n] = per group, dequant(a)[rows, k] @
+ * dequant(b)[g] with a_rows = the row operand's out_rows; accumulation in fp32, one rounding to bf16; k a multiple of
+ * 32, n of 8. */
 int hmoe_mxfp4_rows(const void* x, int dtype, int64_t ldx, const int64_t* row_index, int64_t x_rows, int64_t rows,
                     int64_t k, uint8_t* packed, uint8_t* scale, void* round_trip, int64_t ldo, void* stream);
 int hmoe_mxfp4_weight(const void* w, int dtype, int64_t groups, int64_t k, int64_t n, uint8_t* packed, uint8_t* scale,
                       void* round_trip, void* stream);
 int hmoe_mxfp4_dequantize_rows(const uint8_t* packed, const uint8_t* scale, int64_t rows, int64_t k, void* out,
                                int64_t ldo, void* stream);
+int hmoe_mxfp4_rows_panels(const void* x, int dtype, int64_t ldx, const int64_t* row_index, int64_t x_rows, int64_t rows,
+                           int64_t k, uint8_t* q, uint8_t* scale, int64_t out_rows, void* stream);
+int hmoe_mxfp4_weight_panels(const void* w, int dtype, int64_t groups, int64_t k, int64_t n, uint8_t* q, uint8_t* scale,
+                             void* round_trip, void* stream);
+int hmoe_mxfp4_dequantize_panels(const uint8_t* q, const uint8_t* scale, int64_t q_rows, int64_t rows, int64_t k,
+                                 void* out, int64_t ldo, void* stream);
+int hmoe_grouped_gemm_fwd_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
+                                const uint8_t* b_scale, const int32_t* offs, int64_t total_rows, int num_groups,
+                                int64_t k, int64_t n, void* out, int64_t ldo, void* stream);
 
 #ifdef __cplusplus
 }

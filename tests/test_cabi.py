@@ -162,6 +162,19 @@ def test_bad_arguments_come_back_as_status_codes_before_any_launch():
     assert lib.hmoe_mxfp4_dequantize_rows(fake, fake, 8, 48, fake, 64, None) == unsupported
     assert lib.hmoe_mxfp4_dequantize_rows(fake, None, 8, 64, fake, 64, None) == invalid
     assert lib.hmoe_mxfp4_dequantize_rows(None, None, 0, 64, None, 64, None) == 0
+    assert lib.hmoe_mxfp4_rows_panels(fake, bf16, 64, None, 8, 8, 64, fake, fake, 4, None) == unsupported  # out_rows < rows
+    assert lib.hmoe_mxfp4_rows_panels(fake, bf16, 64, None, 8, 8, 64, None, fake, 8, None) == invalid
+    assert lib.hmoe_mxfp4_rows_panels(None, bf16, 64, None, 0, 0, 64, None, None, 0, None) == 0
+    assert lib.hmoe_mxfp4_weight_panels(fake, bf16, 4, 64, 64, None, fake, fake, None) == invalid          # no codes
+    assert lib.hmoe_mxfp4_weight_panels(fake, bf16, 4, 48, 64, fake, fake, None, None) == unsupported
+    assert lib.hmoe_mxfp4_dequantize_panels(fake, fake, 4, 8, 64, fake, 64, None) == invalid  # fewer rows than asked for
+    mx4 = lib.hmoe_grouped_gemm_fwd_mxfp4
+    assert mx4(fake, fake, 8, fake, fake, fake, 8, 4, 48, 128, fake, 128, None) == unsupported    # K % 32
+    assert mx4(fake, fake, 8, fake, fake, fake, 8, 4, 128, 100, fake, 128, None) == unsupported
+    assert mx4(fake, fake, 4, fake, fake, fake, 8, 4, 128, 128, fake, 128, None) == unsupported   # scale rows < rows
+    assert mx4(fake, fake, 8, fake, fake, None, 8, 4, 128, 128, fake, 128, None) == invalid       # groups without ends
+    assert mx4(fake, fake, 8, fake, None, fake, 8, 4, 128, 128, fake, 128, None) == invalid
+    assert mx4(None, None, 0, None, None, None, 0, 1, 128, 128, None, 128, None) == 0
     assert fp8(fake, None, 8, fake, fake, fake, 8, 4, 256, 128, fake, 128, None) == invalid
     assert fp8(None, None, 0, None, None, None, 0, 1, 256, 128, None, 128, None) == 0
     assert lib.hmoe_quantize_rows_fp8(fake, 200, None, 8, 8, 200, fake, fake, 8, None) == unsupported
