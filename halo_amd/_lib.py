@@ -66,6 +66,8 @@ SIGNATURES = {
     "hmoe_mxfp4_weight_panels": (I, [P, I, L, L, L, P, P, P, P]),
     "hmoe_mxfp4_dequantize_panels": (I, [P, P, L, L, L, P, L, P]),
     "hmoe_grouped_gemm_fwd_mxfp4": (I, [P, P, L, P, P, P, L, I, L, L, P, L, P]),
+    "hmoe_grouped_gemm_fwd_mxfp8_bias": (I, [P, P, L, P, P, P, P, L, I, L, L, P, L, P]),
+    "hmoe_grouped_gemm_fwd_mxfp4_bias": (I, [P, P, L, P, P, P, P, L, I, L, L, P, L, P]),
 }
 
 _lib = None

@@ -1598,7 +1598,7 @@ __device__ __forceinline__ void lds_load1(u32x4 rsrc, lds_bytes_ptr lds_base, ui
                : "memory", "m0");
 }
 
-template <int kFmt>
+template <int kFmt, bool kBias = false>
 __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
   constexpr bool kMx = kFmt != kBlockFp8;   // an e8m0 exponent per 32 values on both sides
   constexpr bool kMx8 = kFmt == kMxFp8, kFp4 = kFmt == kMxFp4;
@@ -1783,6 +1783,19 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
     else if (stores_out == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     else wait_loads();
     workgroup_barrier();   // and every wavefront is through with that epilogue's use of buffer 3
+    // The expert's bias for this lane's eight output columns in either column block (the same in every store of the
+    // epilogue).  Fetched here and pinned as arrived right behind the main loop, where nothing else is in flight: a wait
+    // placed by the compiler at the first use, in the epilogue, would be for the next tile's first stages as well.
+    u32x4 bias_chunk[WN];
+    if constexpr (kBias) {
+#pragma unroll
+      for (int j = 0; j < WN; ++j) {
+        const int col = tile.b_out0 + row_b + j * 32 + ((lane & 3) << 3);
+        bias_chunk[j] = u32x4{0u, 0u, 0u, 0u};
+        if (col < tile.b_out_lim)
+          bias_chunk[j] = *reinterpret_cast<const u32x4*>(static_cast<const bf16_t*>(p.bias) + tile.g * p.n + col);
+      }
+    }
     if (load_wave && steps > 3) issue(3);
     // stage 0 into registers
     uint32_t sa_pack, sb_bits;
@@ -1925,6 +1938,10 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
           for (int v = 0; v < 16; ++v) acc[i][j][v] *= mant_last;
     }
 
+    if constexpr (kBias) {
+#pragma unroll
+      for (int j = 0; j < WN; ++j) asm volatile("" : "+v"(bias_chunk[j]));
+    }
     // buffers 0-2 are free since the last barrier: the next tile's first stages go out before this tile's epilogue
     const TileInfo done = tile;
     t += sched.stride;
@@ -1958,7 +1975,8 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
             const int cc = (lane & 3) << 3;
             const int row = done.a_out0 + row_a + i * 32 + rr;
             const int col = done.b_out0 + row_b + j * 32 + cc;
-            const u32x4 v = *reinterpret_cast<const u32x4*>(stage_rows + (rr * kEpiPitch + cc) * 2);
+            u32x4 v = *reinterpret_cast<const u32x4*>(stage_rows + (rr * kEpiPitch + cc) * 2);
+            if constexpr (kBias) v = add_bf16x8(v, bias_chunk[j]);
             const uint32_t off = row < done.a_out_lim && col < done.b_out_lim
                                      ? static_cast<uint32_t>(row) * static_cast<uint32_t>(p.ldc) * 2u + col * 2u
                                      : kOutOfRange;
@@ -2181,15 +2199,54 @@ int validate(const GemmArgs& p, int dtype) {
   return HMOE_OK;
 }
 
-template <int kFmt>
+template <int kFmt, bool kBias = false>
 int launch_fp8(const GemmArgs& p, int64_t workers, void* stream) {
   constexpr int kLds = F8Scales<kFmt>::kLds;
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_fp8_kernel<kFmt>),
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_fp8_kernel<kFmt, kBias>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
     return HMOE_LAUNCH_FAILED;
-  grouped_gemm_fp8_kernel<kFmt><<<dim3(static_cast<unsigned>(workers)), dim3(512), kLds,
-                                 static_cast<hipStream_t>(stream)>>>(p);
+  grouped_gemm_fp8_kernel<kFmt, kBias><<<dim3(static_cast<unsigned>(workers)), dim3(512), kLds,
+                                        static_cast<hipStream_t>(stream)>>>(p);
   if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
+  return HMOE_OK;
+}
+
+// The MX products' arguments, checked: `panel_values` contraction values lie in a panel's 64 bytes (64 for e4m3, 128 for
+// e2m1) and `k_multiple` is what k must be a multiple of.
+int mx_args(GemmArgs& p, const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
+            const uint8_t* b_scale, const int32_t* offs, int64_t total_rows, int num_groups, int64_t k, int64_t n,
+            const void* bias, bool with_bias, void* out, int64_t ldo, int panel_values, int k_multiple,
+            int64_t& workers) {
+  if (total_rows < 0 || num_groups <= 0 || k < 0 || n < 0) return HMOE_INVALID_ARGUMENT;
+  if (offs == nullptr && num_groups != 1) return HMOE_INVALID_ARGUMENT;
+  if (num_groups > kMaxGroups) return HMOE_UNSUPPORTED;
+  if (k % k_multiple || n % 8 || ldo % 8 || ldo < n || a_rows < total_rows) return HMOE_UNSUPPORTED;
+  if (total_rows == 0 || n == 0) return 1;  // nothing to do
+  if (k == 0) return HMOE_UNSUPPORTED;
+  if (!a_q || !a_scale || !bq || !b_scale || !out || (with_bias && !bias)) return HMOE_INVALID_ARGUMENT;
+  if (!aligned16(a_q) || !aligned16(bq) || !aligned16(out) || (with_bias && !aligned16(bias))) return HMOE_UNSUPPORTED;
+  if (panel_values == 128 && (reinterpret_cast<uintptr_t>(a_scale) % 4 || reinterpret_cast<uintptr_t>(b_scale) % 4))
+    return HMOE_UNSUPPORTED;
+  const int64_t lim = int64_t(1) << 31, panels = (k + panel_values - 1) / panel_values;
+  if (a_rows * panels * 64 >= lim || panels * 64 * n >= lim || total_rows * ldo * 2 >= lim) return HMOE_UNSUPPORTED;
+  p.a = a_q;
+  p.b = bq;
+  p.c = out;
+  p.ldc = ldo;
+  p.offs = offs;
+  p.total_rows = total_rows;
+  p.groups = num_groups;
+  p.k = k;
+  p.n = n;
+  p.b_scale_e8m0 = b_scale;
+  p.a_scale = a_scale;
+  p.a_scale_rows = a_rows;
+  p.k_blocks = static_cast<int>(panels * (panel_values / 32));
+  p.bias = bias;
+  const int64_t bound = (total_rows / 256 + num_groups) * ((n + 255) / 256);
+  workers = device_cus();
+  if (bound < workers) workers = bound;
+  workers = (workers + kXcds - 1) / kXcds * kXcds;
   return HMOE_OK;
 }
 
@@ -2360,74 +2417,50 @@ int hmoe_grouped_gemm_fwd_mxfp8(const uint8_t* a_q, const uint8_t* a_scale, int6
                                 const uint8_t* b_scale, const int32_t* offs, int64_t total_rows, int num_groups,
                                 int64_t k, int64_t n, void* out, int64_t ldo, void* stream) {
   using namespace hmoe;
-  if (total_rows < 0 || num_groups <= 0 || k < 0 || n < 0) return HMOE_INVALID_ARGUMENT;
-  if (offs == nullptr && num_groups != 1) return HMOE_INVALID_ARGUMENT;
-  if (num_groups > kMaxGroups) return HMOE_UNSUPPORTED;
-  // whole panels of 64 values along the contraction; 16-byte rows on both sides
-  if (k % 64 || n % 8 || ldo % 8 || ldo < n || a_rows < total_rows) return HMOE_UNSUPPORTED;
-  if (total_rows == 0 || n == 0) return HMOE_OK;
-  if (k == 0) return HMOE_UNSUPPORTED;
-  if (!a_q || !a_scale || !bq || !b_scale || !out) return HMOE_INVALID_ARGUMENT;
-  if (!aligned16(a_q) || !aligned16(bq) || !aligned16(out)) return HMOE_UNSUPPORTED;
-  const int64_t lim = int64_t(1) << 31;
-  if (a_rows * k >= lim || k * n >= lim || total_rows * ldo * 2 >= lim) return HMOE_UNSUPPORTED;
   GemmArgs p{};
-  p.a = a_q;
-  p.b = bq;
-  p.c = out;
-  p.ldc = ldo;
-  p.offs = offs;
-  p.total_rows = total_rows;
-  p.groups = num_groups;
-  p.k = k;
-  p.n = n;
-  p.b_scale_e8m0 = b_scale;
-  p.a_scale = a_scale;
-  p.a_scale_rows = a_rows;
-  p.k_blocks = static_cast<int>(k / 32);
-  const int64_t bound = (total_rows / 256 + num_groups) * ((n + 255) / 256);
-  int64_t workers = device_cus();
-  if (bound < workers) workers = bound;
-  workers = (workers + kXcds - 1) / kXcds * kXcds;
+  int64_t workers = 0;
+  // whole panels of 64 values along the contraction; 16-byte rows on both sides
+  const int rc = mx_args(p, a_q, a_scale, a_rows, bq, b_scale, offs, total_rows, num_groups, k, n, nullptr, false, out,
+                         ldo, 64, 64, workers);
+  if (rc) return rc > 0 ? HMOE_OK : rc;
   return launch_fp8<kMxFp8>(p, workers, stream);
+}
+
+int hmoe_grouped_gemm_fwd_mxfp8_bias(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
+                                     const uint8_t* b_scale, const void* bias, const int32_t* offs, int64_t total_rows,
+                                     int num_groups, int64_t k, int64_t n, void* out, int64_t ldo, void* stream) {
+  using namespace hmoe;
+  GemmArgs p{};
+  int64_t workers = 0;
+  const int rc = mx_args(p, a_q, a_scale, a_rows, bq, b_scale, offs, total_rows, num_groups, k, n, bias, true, out, ldo,
+                         64, 64, workers);
+  if (rc) return rc > 0 ? HMOE_OK : rc;
+  return launch_fp8<kMxFp8, true>(p, workers, stream);
 }
 
 int hmoe_grouped_gemm_fwd_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
                                 const uint8_t* b_scale, const int32_t* offs, int64_t total_rows, int num_groups,
                                 int64_t k, int64_t n, void* out, int64_t ldo, void* stream) {
   using namespace hmoe;
-  if (total_rows < 0 || num_groups <= 0 || k < 0 || n < 0) return HMOE_INVALID_ARGUMENT;
-  if (offs == nullptr && num_groups != 1) return HMOE_INVALID_ARGUMENT;
-  if (num_groups > kMaxGroups) return HMOE_UNSUPPORTED;
-  // whole blocks of 32 values along the contraction (the operands' last panel is zeros past K); 16-byte rows
-  if (k % 32 || n % 8 || ldo % 8 || ldo < n || a_rows < total_rows) return HMOE_UNSUPPORTED;
-  if (total_rows == 0 || n == 0) return HMOE_OK;
-  if (k == 0) return HMOE_UNSUPPORTED;
-  if (!a_q || !a_scale || !bq || !b_scale || !out) return HMOE_INVALID_ARGUMENT;
-  if (!aligned16(a_q) || !aligned16(bq) || !aligned16(out) || reinterpret_cast<uintptr_t>(a_scale) % 4 ||
-      reinterpret_cast<uintptr_t>(b_scale) % 4)
-    return HMOE_UNSUPPORTED;
-  const int64_t lim = int64_t(1) << 31, panels = (k + 127) / 128;
-  if (a_rows * panels * 64 >= lim || panels * 64 * n >= lim || total_rows * ldo * 2 >= lim) return HMOE_UNSUPPORTED;
   GemmArgs p{};
-  p.a = a_q;
-  p.b = bq;
-  p.c = out;
-  p.ldc = ldo;
-  p.offs = offs;
-  p.total_rows = total_rows;
-  p.groups = num_groups;
-  p.k = k;
-  p.n = n;
-  p.b_scale_e8m0 = b_scale;
-  p.a_scale = a_scale;
-  p.a_scale_rows = a_rows;
-  p.k_blocks = static_cast<int>(panels * 4);
-  const int64_t bound = (total_rows / 256 + num_groups) * ((n + 255) / 256);
-  int64_t workers = device_cus();
-  if (bound < workers) workers = bound;
-  workers = (workers + kXcds - 1) / kXcds * kXcds;
+  int64_t workers = 0;
+  // whole blocks of 32 values along the contraction (the operands' last panel is zeros past K); 16-byte rows
+  const int rc = mx_args(p, a_q, a_scale, a_rows, bq, b_scale, offs, total_rows, num_groups, k, n, nullptr, false, out,
+                         ldo, 128, 32, workers);
+  if (rc) return rc > 0 ? HMOE_OK : rc;
   return launch_fp8<kMxFp4>(p, workers, stream);
+}
+
+int hmoe_grouped_gemm_fwd_mxfp4_bias(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
+                                     const uint8_t* b_scale, const void* bias, const int32_t* offs, int64_t total_rows,
+                                     int num_groups, int64_t k, int64_t n, void* out, int64_t ldo, void* stream) {
+  using namespace hmoe;
+  GemmArgs p{};
+  int64_t workers = 0;
+  const int rc = mx_args(p, a_q, a_scale, a_rows, bq, b_scale, offs, total_rows, num_groups, k, n, bias, true, out, ldo,
+                         128, 32, workers);
+  if (rc) return rc > 0 ? HMOE_OK : rc;
+  return launch_fp8<kMxFp4, true>(p, workers, stream);
 }
 
 int hmoe_grouped_gemm_dgrad(const void* grad_out, int64_t ldg, const void* b, const int32_t* offs,

@@ -67,12 +67,18 @@ def expert_gemm(
     quant_format=None,
     weight_cacheable: bool = True,
     fp8_activations: bool = False,
+    bias: torch.Tensor | None = None,
+    eids: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """``[total_tokens, K]`` activations stacked by expert times ``[num_experts, K, N]`` weights.  ``mat_b`` may be a
     :class:`BlockFp8Weight` (or ``quant_format == "block_fp8"`` with ``mat_b = (q, scale_inv)``): bf16 activations
     against fp8 weights dequantised on their way into the MFMA tiles, forward only.  ``fp8_activations=True``
     quantises the activations too (per row and 128 values, power-of-two scales) and multiplies on the e4m3 MFMA:
-    twice the bf16 rate and half the bytes, at e4m3 precision on both sides instead of one."""
+    twice the bf16 rate and half the bytes, at e4m3 precision on both sides instead of one.  ``bias [G, N]`` with
+    ``eids`` (the sorted expert id of every row), for the MX formats: ``+ bias[eids]`` joins the product in the
+    kernel's epilogue, rounded as the two tensor operations round (reference ``families/gpt_oss.py:153-159``)."""
+    if bias is not None and (quant_format not in ("mxfp8", "mxfp4") or eids is None):
+        raise ValueError("bias is taken with quant_format 'mxfp8' or 'mxfp4' and needs eids")
     if isinstance(mat_b, BlockFp8Weight) or quant_format == "block_fp8":
         weight = mat_b if isinstance(mat_b, BlockFp8Weight) else BlockFp8Weight(*mat_b)
         if fp8_activations:
@@ -92,9 +98,8 @@ def expert_gemm(
         require_implemented(quant_format)
         gathered = isinstance(mat_a, GatheredRows)  # the row quantiser fetches the rows itself
         source, row_index, inv_map = (mat_a.tokens, mat_a.row_index, mat_a.inv_map) if gathered else (mat_a, None, None)
-        if quant_format == "mxfp4":
-            return _Mxfp4ExpertGemm.apply(source, mat_b, offs, weight_cacheable, row_index, inv_map)
-        return _MxFp8ExpertGemm.apply(source, mat_b, offs, weight_cacheable, row_index, inv_map)
+        node = _Mxfp4ExpertGemm if quant_format == "mxfp4" else _MxFp8ExpertGemm
+        return node.apply(source, mat_b, offs, weight_cacheable, row_index, inv_map, bias, eids)
     return grouped_mm(mat_a, mat_b, offs=offs)
 
 
@@ -104,6 +109,20 @@ def mxfp8_mfma_usable(mat_a_dtype: torch.dtype, mat_b_dtype: torch.dtype, k: int
     the reference's own formulation."""
     return (mat_a_dtype == torch.bfloat16 and mat_b_dtype == torch.bfloat16 and k > 0 and k % 64 == 0
             and n % 8 == 0)
+
+
+def _plus_bias(out: torch.Tensor, bias, eids) -> torch.Tensor:
+    """``out + bias[eids]`` as two tensor operations, for the routes whose kernel has no bias epilogue."""
+    return out if bias is None else out + bias.to(out.dtype).index_select(0, eids.long())
+
+
+def _bias_grad(ctx, grad_output: torch.Tensor, position: int):
+    """The bias gradient of an MX node: per expert, the column sums of the rows' gradient."""
+    if ctx.eids is None or not ctx.needs_input_grad[position]:
+        return None
+    from halo_amd.kernels.moe_permute import expert_bias_grad
+
+    return expert_bias_grad(grad_output, ctx.eids, ctx.groups).to(ctx.bias_dtype)
 
 
 class _SharedRows:
@@ -144,11 +163,12 @@ class _MxFp8ExpertGemm(torch.autograd.Function):
     the round-tripped operands in bf16, ``fq(A)`` rebuilt from the saved e4m3 rows (half the bytes of a bf16 copy)."""
 
     @staticmethod
-    def forward(ctx, mat_a, mat_b, offs, weight_cacheable, row_index, inv_map):
+    def forward(ctx, mat_a, mat_b, offs, weight_cacheable, row_index, inv_map, bias=None, eids=None):
         from halo_amd.kernels.lowp.quantization import (MxRows, dequantize_rows_mxfp8, expert_weight_operand,
                                                         quantize_rows_mxfp8)
 
-        device = _lib.require_device(mat_a, mat_b, offs, row_index, inv_map)
+        device = _lib.require_device(mat_a, mat_b, offs, row_index, inv_map, bias, eids)
+        ctx.eids, ctx.groups, ctx.bias_dtype = eids, mat_b.shape[0], None if bias is None else bias.dtype
         if mat_a.dim() != 2 or mat_b.dim() != 3 or mat_a.shape[1] != mat_b.shape[1]:
             raise ValueError(f"expected [R, K] x [G, K, N], got {tuple(mat_a.shape)} x {tuple(mat_b.shape)}")
         groups, k, n = mat_b.shape
@@ -166,13 +186,20 @@ class _MxFp8ExpertGemm(torch.autograd.Function):
         ctx.rows_q = rows_q
         ctx.save_for_backward(weight.dequant, offs32, inv_map)
         if not mxfp8_mfma_usable(mat_a.dtype, mat_b.dtype, k, n):
-            return _forward(dequantize_rows_mxfp8(rows_q).to(mat_a.dtype), weight.dequant.to(mat_a.dtype), offs32)
+            return _plus_bias(_forward(dequantize_rows_mxfp8(rows_q).to(mat_a.dtype), weight.dequant.to(mat_a.dtype),
+                                       offs32), bias, eids)
         out = torch.empty((rows, n), dtype=torch.bfloat16, device=device)
         if rows and n:
             with _lib.on_device(device):
-                _lib.call("hmoe_grouped_gemm_fwd_mxfp8", _lib.ptr(rows_q.q), _lib.ptr(rows_q.scales), rows,
-                          _lib.ptr(weight.q), _lib.ptr(weight.scales), _lib.ptr(offs32), rows, groups, k, n,
-                          _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
+                if bias is None:
+                    _lib.call("hmoe_grouped_gemm_fwd_mxfp8", _lib.ptr(rows_q.q), _lib.ptr(rows_q.scales), rows,
+                              _lib.ptr(weight.q), _lib.ptr(weight.scales), _lib.ptr(offs32), rows, groups, k, n,
+                              _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
+                else:
+                    bias16 = bias.to(torch.bfloat16).contiguous()
+                    _lib.call("hmoe_grouped_gemm_fwd_mxfp8_bias", _lib.ptr(rows_q.q), _lib.ptr(rows_q.scales), rows,
+                              _lib.ptr(weight.q), _lib.ptr(weight.scales), _lib.ptr(bias16), _lib.ptr(offs32), rows,
+                              groups, k, n, _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
         return out
 
     @staticmethod
@@ -195,7 +222,7 @@ class _MxFp8ExpertGemm(torch.autograd.Function):
                                               ctx.needs_input_grad[0], ctx.needs_input_grad[1])
             if ctx.gathered and grad_a is not None:
                 grad_a = gather_reduce_rows(grad_a, inv_map)
-        return grad_a, grad_b, None, None, None, None
+        return grad_a, grad_b, None, None, None, None, _bias_grad(ctx, grad_output, 6), None
 
 
 def mxfp4_mfma_usable(mat_a_dtype: torch.dtype, mat_b_dtype: torch.dtype, k: int, n: int) -> bool:
@@ -220,11 +247,12 @@ class _Mxfp4ExpertGemm(torch.autograd.Function):
     saved e2m1 codes (a quarter of the bytes of a bf16 copy)."""
 
     @staticmethod
-    def forward(ctx, mat_a, mat_b, offs, weight_cacheable, row_index, inv_map):
+    def forward(ctx, mat_a, mat_b, offs, weight_cacheable, row_index, inv_map, bias=None, eids=None):
         from halo_amd.kernels.lowp.quantization import (expert_weight_operand, expert_weight_round_trip, mxfp4_rows,
                                                         quantize_rows_mxfp4)
 
-        device = _lib.require_device(mat_a, mat_b, offs, row_index, inv_map)
+        device = _lib.require_device(mat_a, mat_b, offs, row_index, inv_map, bias, eids)
+        ctx.eids, ctx.groups, ctx.bias_dtype = eids, mat_b.shape[0], None if bias is None else bias.dtype
         if mat_a.dim() != 2 or mat_b.dim() != 3 or mat_a.shape[1] != mat_b.shape[1]:
             raise ValueError(f"expected [R, K] x [G, K, N], got {tuple(mat_a.shape)} x {tuple(mat_b.shape)}")
         groups, k, n = mat_b.shape
@@ -239,7 +267,7 @@ class _Mxfp4ExpertGemm(torch.autograd.Function):
                 a_rt = mxfp4_rows(mat_a, row_index, codes=False, round_trip=True)[2].to(mat_a.dtype)
                 _round_tripped_rows.put(mat_a, key, a_rt)
             ctx.save_for_backward(a_rt, w_rt, offs32, inv_map)
-            return _forward(a_rt, w_rt, offs32)
+            return _plus_bias(_forward(a_rt, w_rt, offs32), bias, eids)
         weight = expert_weight_operand(mat_b, weight_cacheable, "mxfp4")
         rows_q = _quantised_rows4.get(mat_a, key)
         if rows_q is None:
@@ -251,9 +279,15 @@ class _Mxfp4ExpertGemm(torch.autograd.Function):
         out = torch.empty((rows, n), dtype=torch.bfloat16, device=device)
         if rows and n:
             with _lib.on_device(device):
-                _lib.call("hmoe_grouped_gemm_fwd_mxfp4", _lib.ptr(rows_q.q), _lib.ptr(rows_q.scales), rows,
-                          _lib.ptr(weight.q), _lib.ptr(weight.scales), _lib.ptr(offs32), rows, groups, k, n,
-                          _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
+                if bias is None:
+                    _lib.call("hmoe_grouped_gemm_fwd_mxfp4", _lib.ptr(rows_q.q), _lib.ptr(rows_q.scales), rows,
+                              _lib.ptr(weight.q), _lib.ptr(weight.scales), _lib.ptr(offs32), rows, groups, k, n,
+                              _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
+                else:
+                    bias16 = bias.to(torch.bfloat16).contiguous()
+                    _lib.call("hmoe_grouped_gemm_fwd_mxfp4_bias", _lib.ptr(rows_q.q), _lib.ptr(rows_q.scales), rows,
+                              _lib.ptr(weight.q), _lib.ptr(weight.scales), _lib.ptr(bias16), _lib.ptr(offs32), rows,
+                              groups, k, n, _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
         return out
 
     @staticmethod
@@ -262,8 +296,9 @@ class _Mxfp4ExpertGemm(torch.autograd.Function):
         from halo_amd.kernels.moe_permute import gather_reduce_rows
 
         grad_a = grad_b = None
+        grad_bias = _bias_grad(ctx, grad_output, 6)
         if not (ctx.needs_input_grad[0] or ctx.needs_input_grad[1]):
-            return None, None, None, None, None, None
+            return None, None, None, None, None, None, grad_bias, None
         if ctx.native:
             w_rt, offs32, inv_map = ctx.saved_tensors
             q = ctx.rows_q.q
@@ -280,7 +315,7 @@ class _Mxfp4ExpertGemm(torch.autograd.Function):
                                           ctx.needs_input_grad[0], ctx.needs_input_grad[1])
         if ctx.gathered and grad_a is not None:
             grad_a = gather_reduce_rows(grad_a, inv_map)
-        return grad_a, grad_b, None, None, None, None
+        return grad_a, grad_b, None, None, None, None, grad_bias, None
 
 
 def _fp8w_forward(mat_a: torch.Tensor, weight: BlockFp8Weight, offs: torch.Tensor | None) -> torch.Tensor:

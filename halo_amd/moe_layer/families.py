@@ -140,6 +140,14 @@ class EPGptOssMoELayer(EPMoELayerBase):
             weight, bias_cast = weight.to(out_dtype), bias.to(out_dtype)
             if bias_fusable(x, weight, bias_cast):  # the projection and its bias in one kernel, the same bits
                 return grouped_mm_bias(x, weight, bias_cast, offs=offs, eids=eids)
+        if (bias is not None and getattr(self, "fuse_bias_into_gemm", True)
+                and self._lowp_quant_format in ("mxfp8", "mxfp4") and not self._adapted(weight_attr)
+                and isinstance(weight, torch.Tensor) and out_dtype == torch.bfloat16):
+            # the MX products add the bias row in their epilogue too, with the roundings of the two tensor operations
+            from halo_amd.kernels.expert_gemm import expert_gemm
+
+            return expert_gemm(x, weight.to(out_dtype), offs=offs, quant_format=self._lowp_quant_format,
+                               weight_cacheable=self._lowp_weight_cacheable, bias=bias.to(out_dtype), eids=eids)
         out = self._expert_proj(x, weight_attr, offs, out_dtype)
         return out if bias is None else out + MoEExpertBiasGather.apply(bias.to(out_dtype), eids)
 

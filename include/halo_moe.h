@@ -355,6 +355,15 @@ int hmoe_mxfp4_dequantize_panels(const uint8_t* q, const uint8_t* scale, int64_t
 int hmoe_grouped_gemm_fwd_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
                                 const uint8_t* b_scale, const int32_t* offs, int64_t total_rows, int num_groups,
                                 int64_t k, int64_t n, void* out, int64_t ldo, void* stream);
+/* The two MX products with an expert bias row added in the epilogue: out = bf16(product) + bias[g] per row of group g,
+ * each of the two rounded to bf16 as the reference's two tensor operations round (_expert_proj, then
+ * + MoEExpertBiasGather.apply(bias, eids): halo/moe_layer/families/gpt_oss.py:153-159).  bias bf16 [num_groups, n]. */
+int hmoe_grouped_gemm_fwd_mxfp8_bias(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
+                                     const uint8_t* b_scale, const void* bias, const int32_t* offs, int64_t total_rows,
+                                     int num_groups, int64_t k, int64_t n, void* out, int64_t ldo, void* stream);
+int hmoe_grouped_gemm_fwd_mxfp4_bias(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
+                                     const uint8_t* b_scale, const void* bias, const int32_t* offs, int64_t total_rows,
+                                     int num_groups, int64_t k, int64_t n, void* out, int64_t ldo, void* stream);
 
 #ifdef __cplusplus
 }

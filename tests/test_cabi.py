@@ -175,6 +175,11 @@ def test_bad_arguments_come_back_as_status_codes_before_any_launch():
     assert mx4(fake, fake, 8, fake, fake, None, 8, 4, 128, 128, fake, 128, None) == invalid       # groups without ends
     assert mx4(fake, fake, 8, fake, None, fake, 8, 4, 128, 128, fake, 128, None) == invalid
     assert mx4(None, None, 0, None, None, None, 0, 1, 128, 128, None, 128, None) == 0
+    for with_bias in (lib.hmoe_grouped_gemm_fwd_mxfp8_bias, lib.hmoe_grouped_gemm_fwd_mxfp4_bias):
+        assert with_bias(fake, fake, 8, fake, fake, None, fake, 8, 4, 128, 128, fake, 128, None) == invalid  # no bias
+        assert with_bias(fake, fake, 8, fake, fake, fake + 2, fake, 8, 4, 128, 128, fake, 128, None) == unsupported
+        assert with_bias(fake, fake, 8, fake, fake, fake, fake, 8, 4, 128, 100, fake, 128, None) == unsupported
+        assert with_bias(None, None, 0, None, None, None, None, 0, 1, 128, 128, None, 128, None) == 0
     assert fp8(fake, None, 8, fake, fake, fake, 8, 4, 256, 128, fake, 128, None) == invalid
     assert fp8(None, None, 0, None, None, None, 0, 1, 256, 128, None, 128, None) == 0
     assert lib.hmoe_quantize_rows_fp8(fake, 200, None, 8, 8, 200, fake, fake, 8, None) == unsupported

@@ -390,6 +390,37 @@ def test_mxfp4_rows_fetched_through_the_sorts_index_and_shared_between_projectio
     assert calls["weight"] == 4
 
 
+@pytest.mark.parametrize("fmt", ("mxfp8", "mxfp4"))
+def test_expert_bias_joins_the_mx_products_in_the_epilogue(device, fmt):
+    """``expert_gemm(..., bias=, eids=)`` for the MX formats (reference ``families/gpt_oss.py:153-159``: the projection,
+    then ``+ bias[eids]``): bit-equal to the product followed by the tensor addition, a partial column tile and an empty
+    group included; the bias gradient is the per-expert column sum of the rows' gradient (exact zeros for the empty
+    group), the other gradients are unchanged; fp32 operands (outside the matrix kernel) take the addition unfused."""
+    from halo_amd.kernels.expert_gemm import expert_gemm
+
+    g = torch.Generator().manual_seed(53)
+    counts = (255, 0, 257, 40, 513, 31)
+    offs = torch.tensor(counts).cumsum(0).int().to(device)
+    eids = torch.repeat_interleave(torch.arange(len(counts)), torch.tensor(counts)).to(device)
+    for dtype, k, n in ((torch.bfloat16, 192, 264), (torch.bfloat16, 2880, 136), (torch.float32, 96, 72)):
+        a = (torch.randn(sum(counts), k, generator=g) * 0.5).to(dtype).to(device).requires_grad_(True)
+        b = (torch.randn(len(counts), k, n, generator=g) * 0.05).to(dtype).to(device).requires_grad_(True)
+        bias = torch.randn(len(counts), n, generator=g).to(dtype).to(device).requires_grad_(True)
+        upstream = torch.randn(sum(counts), n, generator=g).to(dtype).to(device)
+        fused = expert_gemm(a, b, offs=offs, quant_format=fmt, weight_cacheable=False, bias=bias, eids=eids)
+        grads_fused = torch.autograd.grad(fused, (a, b, bias), upstream)
+        plain = expert_gemm(a, b, offs=offs, quant_format=fmt, weight_cacheable=False) + bias[eids]
+        grads_plain = torch.autograd.grad(plain, (a, b, bias), upstream)
+        assert fused.dtype == dtype and torch.equal(fused, plain)
+        assert torch.equal(grads_fused[0], grads_plain[0]) and torch.equal(grads_fused[1], grads_plain[1])
+        want = torch.zeros(len(counts), n, dtype=torch.float64, device=device).index_add_(0, eids, upstream.double())
+        assert not grads_fused[2][1].any()
+        tol = 2.0 ** -8 if dtype == torch.bfloat16 else 1e-5
+        assert ((grads_fused[2].double() - want).abs() <= tol * want.abs() + tol).all()
+    with pytest.raises(ValueError, match="bias is taken"):
+        expert_gemm(a, b, offs=offs, bias=bias, eids=eids)
+
+
 @pytest.mark.parametrize("name", ("cfg2_small", "cfg4_small"))
 def test_layer_with_mxfp4_experts_against_the_cpu_loop_over_fake_quantised_products(device, name):
     """``set_lowp_compute("mxfp4")`` on the layer (reference ``compute.py:53-58, 306-312``): forward and every
