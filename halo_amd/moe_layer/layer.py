@@ -102,9 +102,14 @@ class _RouterProjection(torch.autograd.Function):
 
 
 def dense_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """``x @ weight^T`` for an ``F.linear``-convention ``weight [out, in]`` on the grouped kernel with one group (the
-    router projection and the shared expert); differentiable in both operands."""
-    return grouped_mm(x, weight.unsqueeze(0).transpose(1, 2), offs=None)
+    """``x @ weight^T`` for an ``F.linear``-convention ``weight [out, in]`` (the shared expert's projections, which are
+    ``nn.Linear`` modules in the reference: ``families/qwen3_5.py:41-42``); differentiable in both operands.  A plain
+    dense product, so the library's: the grouped kernel with one group has 64 output tiles for 256 compute units at
+    8192 tokens x 512 columns and 16 for the weight gradient, whose contraction over the tokens it cannot split
+    (147 us against the library's 20 for that one product)."""
+    if not x.is_cuda:
+        raise RuntimeError("halo_amd ops run on the GPU: got a CPU tensor")
+    return torch.nn.functional.linear(x, weight)
 
 
 class EPMoELayerBase(ExpertLoadMixin, nn.Module, ABC):
