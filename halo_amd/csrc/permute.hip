@@ -201,8 +201,78 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
         acc.store(to + c);
       }
     };
-    if (all_valid) reduce_row(std::true_type{});
-    else reduce_row(std::false_type{});
+    if (all_valid) {
+      reduce_row(std::true_type{});
+      return;
+    }
+    // Some slots are not this rank's (most of them on one GPU's share of an expert-parallel layer).  The valid ones are
+    // moved to the front, in slot order (the sum keeps its order; a slot left out adds the +0.0f it added before), and
+    // the row is reduced by the loop written for that many sources: every fetch of a pass goes out before the first is
+    // used, and a row with few sources takes more column chunks per pass, so that 8 to 12 fetches are in flight per
+    // lane whatever the count.  Everything here is the same for the whole wavefront (scalar registers, one branch).
+    const T* live_from[kTopK];
+    float live_w[kTopK];
+    int n_live = 0;
+#pragma unroll
+    for (int k = 0; k < kTopK; ++k) {
+      live_from[k] = src;
+      live_w[k] = 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < kTopK; ++k) {
+      if (valid[k]) {
+#pragma unroll
+        for (int i = 0; i <= k; ++i) {  // slot k lands at position n_live <= k
+          if (i == n_live) {
+            live_from[i] = from[k];
+            live_w[i] = w[k];
+          }
+        }
+        ++n_live;
+      }
+    }
+    auto reduce_live = [&](auto count_tag, auto chunks_tag) __attribute__((always_inline)) {
+      constexpr int kLive = decltype(count_tag)::value, kChunks = decltype(chunks_tag)::value;
+      int64_t c = static_cast<int64_t>(lane_id()) * W;
+      auto pass = [&](auto width_tag) __attribute__((always_inline)) {
+        constexpr int kWide = decltype(width_tag)::value;
+        Pack<T, W> x[kWide][kLive > 0 ? kLive : 1], acc[kWide], extra_chunk[kWide];
+#pragma unroll
+        for (int h = 0; h < kWide; ++h)
+#pragma unroll
+          for (int k = 0; k < kLive; ++k) x[h][k].load_once(live_from[k] + c + h * step);
+#pragma unroll
+        for (int h = 0; h < kWide; ++h) {
+          if (extra) extra_chunk[h].load(extra + c + h * step);
+#pragma unroll
+          for (int i = 0; i < W; ++i) acc[h].v[i] = 0.f;
+#pragma unroll
+          for (int k = 0; k < kLive; ++k) {
+#pragma unroll
+            for (int i = 0; i < W; ++i) acc[h].v[i] += kWeighted ? x[h][k].v[i] * live_w[k] : x[h][k].v[i];
+          }
+          finish(acc[h], extra_chunk[h]);
+          acc[h].store(to + c + h * step);
+        }
+      };
+      for (; c + (kChunks - 1) * step < hidden; c += kChunks * step) pass(std::integral_constant<int, kChunks>{});
+      if constexpr (kChunks > 2) {
+        for (; c + step < hidden; c += 2 * step) pass(std::integral_constant<int, 2>{});
+      }
+      for (; c < hidden; c += step) pass(std::integral_constant<int, 1>{});
+    };
+    using std::integral_constant;
+    switch (n_live) {
+      case 0: reduce_live(integral_constant<int, 0>{}, integral_constant<int, 4>{}); break;
+      case 1: reduce_live(integral_constant<int, 1>{}, integral_constant<int, 4>{}); break;
+      case 2: reduce_live(integral_constant<int, 2>{}, integral_constant<int, 4>{}); break;
+      case 3: reduce_live(integral_constant<int, (kTopK >= 3 ? 3 : 1)>{}, integral_constant<int, 4>{}); break;
+      case 4: reduce_live(integral_constant<int, (kTopK >= 4 ? 4 : 1)>{}, integral_constant<int, 2>{}); break;
+      case 5: reduce_live(integral_constant<int, (kTopK >= 5 ? 5 : 1)>{}, integral_constant<int, 2>{}); break;
+      case 6: reduce_live(integral_constant<int, (kTopK >= 6 ? 6 : 1)>{}, integral_constant<int, 2>{}); break;
+      case 7: reduce_live(integral_constant<int, (kTopK >= 7 ? 7 : 1)>{}, integral_constant<int, 2>{}); break;
+      default: reduce_row(std::false_type{}); break;
+    }
   } else {
     for (int64_t c = static_cast<int64_t>(lane_id()) * W; c < hidden; c += step) {
       Pack<T, W> acc, extra_chunk;
