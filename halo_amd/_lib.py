@@ -68,6 +68,9 @@ SIGNATURES = {
     "hmoe_grouped_gemm_fwd_mxfp4": (I, [P, P, L, P, P, P, L, I, L, L, P, L, P]),
     "hmoe_grouped_gemm_fwd_mxfp8_bias": (I, [P, P, L, P, P, P, P, L, I, L, L, P, L, P]),
     "hmoe_grouped_gemm_fwd_mxfp4_bias": (I, [P, P, L, P, P, P, P, L, I, L, L, P, L, P]),
+    "hmoe_nvfp4_rows": (I, [P, I, L, P, L, L, L, P, P, P, P, L, P, P]),
+    "hmoe_nvfp4_weight": (I, [P, I, L, L, L, P, P, P, P, P, P]),
+    "hmoe_nvfp4_dequantize_rows": (I, [P, P, P, L, L, P, L, P]),
 }
 
 _lib = None

@@ -4,7 +4,8 @@ weights (the quantised-weight serving configuration, forward only).
 
 Mirrors the dispatch seam of the reference's ``halo/kernels/expert_gemm.py:14-38``.  Of its ``quant_format`` values
 ``"mxfp8"`` and ``"mxfp4"`` run on the scaled matrix instruction (e4m3 / e2m1 operands with an e8m0 exponent per 32
-values); ``"nvfp4"`` raises.
+values); ``"nvfp4"`` (e4m3 scales, which the instruction cannot take) is the bf16 product of the two round-tripped
+operands, the reference's own formulation.
 """
 
 from __future__ import annotations
@@ -98,6 +99,10 @@ def expert_gemm(
         require_implemented(quant_format)
         gathered = isinstance(mat_a, GatheredRows)  # the row quantiser fetches the rows itself
         source, row_index, inv_map = (mat_a.tokens, mat_a.row_index, mat_a.inv_map) if gathered else (mat_a, None, None)
+        if quant_format == "nvfp4":
+            # one scale for the whole activation tensor: the rows are gathered first, then round-tripped as one tensor
+            return _RoundTripExpertGemm.apply(mat_a.materialize() if gathered else mat_a, mat_b, offs, weight_cacheable,
+                                              quant_format)
         node = _Mxfp4ExpertGemm if quant_format == "mxfp4" else _MxFp8ExpertGemm
         return node.apply(source, mat_b, offs, weight_cacheable, row_index, inv_map, bias, eids)
     return grouped_mm(mat_a, mat_b, offs=offs)
@@ -223,6 +228,39 @@ class _MxFp8ExpertGemm(torch.autograd.Function):
             if ctx.gathered and grad_a is not None:
                 grad_a = gather_reduce_rows(grad_a, inv_map)
         return grad_a, grad_b, None, None, None, None, _bias_grad(ctx, grad_output, 6), None
+
+
+class _RoundTripExpertGemm(torch.autograd.Function):
+    """``grouped_mm(fake_quant(mat_a, fmt, axis=-1), cached_fake_quant(mat_b, fmt, axis=1), offs)`` of the reference
+    (``expert_gemm.py:33-38``) as one node, for a format the matrix instruction has no operand type for (NVFP4): both
+    operands through their round trip (the weights' kept per optimizer step), the product and, straight through
+    (``quantization.py:350-360``), the gradients on the bf16 / fp32 grouped kernels."""
+
+    @staticmethod
+    def forward(ctx, mat_a, mat_b, offs, weight_cacheable, fmt):
+        from halo_amd.kernels.lowp.quantization import _round_trip, expert_weight_round_trip
+
+        _lib.require_device(mat_a, mat_b, offs)
+        if mat_a.dim() != 2 or mat_b.dim() != 3 or mat_a.shape[1] != mat_b.shape[1]:
+            raise ValueError(f"expected [R, K] x [G, K, N], got {tuple(mat_a.shape)} x {tuple(mat_b.shape)}")
+        offs32 = _offs_arg(offs, mat_b.shape[0])
+        w_rt = expert_weight_round_trip(mat_b, fmt, weight_cacheable).to(mat_a.dtype)
+        key = (mat_a._version, fmt)
+        a_rt = _round_tripped_rows.get(mat_a, key)
+        if a_rt is None:
+            a_rt = _round_trip(mat_a.detach(), fmt, -1).to(mat_a.dtype)
+            _round_tripped_rows.put(mat_a, key, a_rt)
+        ctx.save_for_backward(a_rt, w_rt, offs32)
+        return _forward(a_rt, w_rt, offs32)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        a_rt, w_rt, offs32 = ctx.saved_tensors
+        grad_a = grad_b = None
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            grad_a, grad_b = grouped_mm_grads(a_rt, w_rt, grad_output.to(a_rt.dtype), offs32, ctx.needs_input_grad[0],
+                                              ctx.needs_input_grad[1])
+        return grad_a, grad_b, None, None, None
 
 
 def mxfp4_mfma_usable(mat_a_dtype: torch.dtype, mat_b_dtype: torch.dtype, k: int, n: int) -> bool:

@@ -1,5 +1,6 @@
-"""MX block-scaled quantisation for the expert GEMM: e4m3 (MXFP8) or e2m1 (MXFP4) elements plus one e8m0 power-of-two
-scale per 32 values along the contraction axis, the straight-through fake-quant, and the per-step weight cache.
+"""Block-scaled quantisation for the expert GEMM: e4m3 (MXFP8) or e2m1 (MXFP4) elements plus one e8m0 power-of-two
+scale per 32 values along the contraction axis, or e2m1 elements with an e4m3 scale per 16 values and one fp32 scale
+per tensor (NVFP4); the straight-through fake-quant, and the per-step weight cache.
 
 Mirrors ``halo/kernels/lowp/quantization.py`` of the reference for its ``mxfp8`` and ``mxfp4`` formats:
 ``BlockScaledTensor`` (:104-117), ``quantize_mxfp8`` (:236-245), ``quantize_mxfp4`` (:248-266), ``dequantize``
@@ -7,7 +8,9 @@ Mirrors ``halo/kernels/lowp/quantization.py`` of the reference for its ``mxfp8``
 ``csrc/mxfp8.hip``; they write the operands in the layout the GEMM kernel loads (:class:`MxRows`, :class:`MxWeight`),
 and the reference's logical layout is a byte permutation of those.  The MXFP4 kernels are ``csrc/mxfp4.hip``; they
 write the reference's layout (two codes per byte along the quantised axis), the matrix kernel's operands
-(:class:`Mx4Rows`, :class:`Mx4Weight`) and the round trip's bf16 result in one pass.
+(:class:`Mx4Rows`, :class:`Mx4Weight`) and the round trip's bf16 result in one pass.  The NVFP4 kernels are
+``csrc/nvfp4.hip`` (``quantize_nvfp4``, :209-226, :269-270): the reference's layout and the round trip, after a
+reduction of the tensor's largest magnitude.
 """
 
 from __future__ import annotations
@@ -29,8 +32,9 @@ PANEL = 64  # contraction values that lie together in the GEMM's operand layout
 @dataclass(frozen=True)
 class BlockScaledTensor:
     """``data`` holds ``float8_e4m3fn`` elements in the source's shape, or, when ``packed``, two ``e2m1`` codes per byte
-    (uint8, ``axis`` halved, the even element in the low nibble); ``scales`` one ``e8m0`` biased exponent (uint8) per
-    block of ``block_size`` along ``axis``.  An element is ``code x 2^(scales - 127)``."""
+    (uint8, ``axis`` halved, the even element in the low nibble); ``scales`` one entry per block of ``block_size`` along
+    ``axis``: an ``e8m0`` biased exponent (uint8) when ``pow2_scale`` (MX), an ``e4m3`` value otherwise (NVFP4).  An
+    element is ``code x 2^(scales - 127)``, or ``code x scales x global_scale`` for NVFP4."""
 
     data: torch.Tensor
     scales: torch.Tensor
@@ -261,6 +265,112 @@ def quantize_weight_mxfp4(w: torch.Tensor, with_dequant: bool = False) -> Mx4Wei
     return Mx4Weight(q, scales, dequant, k)
 
 
+NVFP4_BLOCK = FORMAT_BLOCK_SIZE["nvfp4"]
+
+
+def _tensor_amax(t: torch.Tensor) -> torch.Tensor:
+    """The largest magnitude of ``t`` as one fp32 value on the device (NaN if ``t`` holds one): the reduction NVFP4's
+    per-tensor scale needs before any block can be scaled."""
+    if t.numel() == 0:
+        return torch.zeros((), dtype=torch.float32, device=t.device)
+    return t.detach().abs().amax().float()
+
+
+def nvfp4_rows(x: torch.Tensor, *, codes: bool = True, round_trip: bool = False, amax: torch.Tensor | None = None):
+    """``x [R, K]`` (bf16 or fp32, K a multiple of 16) along its last axis in one launch: ``(packed uint8 [R, K / 2],
+    scales float8_e4m3fn [R, K / 16], round trip bf16 [R, K], global scale fp32 [])``, the first two None unless
+    ``codes``, the third unless ``round_trip``.  ``amax``: the tensor's largest magnitude when the caller has it."""
+    device = _lib.require_device(x, amax)
+    if x.dim() != 2:
+        raise ValueError(f"expected [R, K], got {tuple(x.shape)}")
+    if not (codes or round_trip):
+        raise ValueError("nothing to compute: neither codes nor round_trip asked for")
+    x = _aligned_rows(_native_input(x))
+    rows, k = x.shape
+    if k % NVFP4_BLOCK:
+        raise ValueError(f"axis 1 size {k} not divisible by block_size {NVFP4_BLOCK}")
+    amax = _tensor_amax(x) if amax is None else amax.float().reshape(())
+    packed = torch.empty((rows, k // 2), dtype=torch.uint8, device=device) if codes else None
+    scales = torch.empty((rows, k // NVFP4_BLOCK), dtype=torch.uint8, device=device) if codes else None
+    out = torch.empty((rows, k), dtype=torch.bfloat16, device=device) if round_trip else None
+    global_scale = torch.ones((), dtype=torch.float32, device=device)
+    with _lib.on_device(device):
+        _lib.call("hmoe_nvfp4_rows", _lib.ptr(x), _lib.dtype_id(x.dtype), x.stride(0) if rows else k, None, rows, rows,
+                  k, _lib.ptr(amax), _lib.ptr(packed), _lib.ptr(scales), _lib.ptr(out), k, _lib.ptr(global_scale),
+                  _lib.stream_ptr(device))
+    return packed, None if scales is None else scales.view(torch.float8_e4m3fn), out, global_scale
+
+
+def nvfp4_weight(w: torch.Tensor, *, codes: bool = True, round_trip: bool = False):
+    """``w [G, K, N]`` (bf16 or fp32, K a multiple of 16) along K under one scale for the whole bank: ``(packed uint8
+    [G, K / 2, N], scales float8_e4m3fn [G, K / 16, N], round trip bf16 [G, K, N], global scale fp32 [])``."""
+    device = _lib.require_device(w)
+    if w.dim() != 3:
+        raise ValueError(f"expected [G, K, N], got {tuple(w.shape)}")
+    if not (codes or round_trip):
+        raise ValueError("nothing to compute: neither codes nor round_trip asked for")
+    w = _native_input(w).contiguous()
+    g, k, n = w.shape
+    if k % NVFP4_BLOCK:
+        raise ValueError(f"axis 1 size {k} not divisible by block_size {NVFP4_BLOCK}")
+    amax = _tensor_amax(w)
+    packed = torch.empty((g, k // 2, n), dtype=torch.uint8, device=device) if codes else None
+    scales = torch.empty((g, k // NVFP4_BLOCK, n), dtype=torch.uint8, device=device) if codes else None
+    out = torch.empty((g, k, n), dtype=torch.bfloat16, device=device) if round_trip else None
+    global_scale = torch.ones((), dtype=torch.float32, device=device)
+    with _lib.on_device(device):
+        _lib.call("hmoe_nvfp4_weight", _lib.ptr(w), _lib.dtype_id(w.dtype), g, k, n, _lib.ptr(amax), _lib.ptr(packed),
+                  _lib.ptr(scales), _lib.ptr(out), _lib.ptr(global_scale), _lib.stream_ptr(device))
+    return packed, None if scales is None else scales.view(torch.float8_e4m3fn), out, global_scale
+
+
+def quantize_nvfp4(t: torch.Tensor, axis: int = -1) -> BlockScaledTensor:
+    """The reference's layout (``quantization.py:218-226, 248-270``): ``data`` uint8 with ``axis`` halved, ``scales``
+    float8_e4m3fn with ``axis`` divided by 16, ``global_scale`` a 0-dim fp32 tensor."""
+    if t.dim() == 0:
+        raise ValueError("quantize_nvfp4 expects at least one axis")
+    kind, axis = _axis_layout(t, axis)
+    k = t.shape[axis]
+    if k % NVFP4_BLOCK:
+        raise ValueError(f"axis {axis} size {k} not divisible by block_size {NVFP4_BLOCK}")
+    if kind == "moved":
+        inner = quantize_nvfp4(t.transpose(axis, -1).contiguous(), -1)
+        return BlockScaledTensor(inner.data.transpose(axis, -1).contiguous(),
+                                 inner.scales.view(torch.uint8).transpose(axis, -1).contiguous().view(torch.float8_e4m3fn),
+                                 NVFP4_BLOCK, axis, packed=True, pow2_scale=False, global_scale=inner.global_scale)
+    if kind == "rows":
+        lead = t.shape[:-1]
+        packed, scales, _, gs = nvfp4_rows(t.reshape(-1, k))
+        return BlockScaledTensor(packed.reshape(*lead, k // 2), scales.reshape(*lead, k // NVFP4_BLOCK), NVFP4_BLOCK,
+                                 axis, packed=True, pow2_scale=False, global_scale=gs)
+    lead, n = t.shape[:-2], t.shape[-1]
+    packed, scales, _, gs = nvfp4_weight(t.reshape(-1, k, n))
+    return BlockScaledTensor(packed.reshape(*lead, k // 2, n), scales.reshape(*lead, k // NVFP4_BLOCK, n), NVFP4_BLOCK,
+                             axis, packed=True, pow2_scale=False, global_scale=gs)
+
+
+def _dequantize_nvfp4(q: BlockScaledTensor) -> torch.Tensor:
+    data, axis = q.data, q.axis % q.data.dim()
+    scales = q.scales.view(torch.uint8)
+    if axis != data.dim() - 1:
+        moved = BlockScaledTensor(data.transpose(axis, -1).contiguous(),
+                                  scales.transpose(axis, -1).contiguous().view(torch.float8_e4m3fn), NVFP4_BLOCK, -1,
+                                  packed=True, pow2_scale=False, global_scale=q.global_scale)
+        return _dequantize_nvfp4(moved).transpose(axis, -1).contiguous()
+    device = _lib.require_device(data, scales, q.global_scale)
+    k = data.shape[-1] * 2
+    if k % NVFP4_BLOCK or scales.shape[-1] != k // NVFP4_BLOCK:
+        raise ValueError(f"packed axis of {data.shape[-1]} bytes does not match {scales.shape[-1]} scales of {NVFP4_BLOCK}")
+    flat = data.reshape(-1, k // 2).contiguous()
+    flat_scales = scales.reshape(-1, k // NVFP4_BLOCK).contiguous()
+    gs = q.global_scale.float().reshape(()).contiguous()
+    out = torch.empty((flat.shape[0], k), dtype=torch.bfloat16, device=device)
+    with _lib.on_device(device):
+        _lib.call("hmoe_nvfp4_dequantize_rows", _lib.ptr(flat), _lib.ptr(flat_scales), _lib.ptr(gs), flat.shape[0], k,
+                  _lib.ptr(out), k, _lib.stream_ptr(device))
+    return out.reshape(*data.shape[:-1], k)
+
+
 def _axis_layout(t: torch.Tensor, axis: int) -> tuple[str, int]:
     axis = axis % t.dim()
     if axis == t.dim() - 1:
@@ -320,7 +430,7 @@ def quantize_mxfp4(t: torch.Tensor, axis: int = -1) -> BlockScaledTensor:
                              packed=True)
 
 
-QUANTIZERS = {"mxfp8": quantize_mxfp8, "mxfp4": quantize_mxfp4}
+QUANTIZERS = {"mxfp8": quantize_mxfp8, "mxfp4": quantize_mxfp4, "nvfp4": quantize_nvfp4}
 
 
 def _dequantize_packed(q: BlockScaledTensor) -> torch.Tensor:
@@ -343,9 +453,12 @@ def _dequantize_packed(q: BlockScaledTensor) -> torch.Tensor:
 
 
 def dequantize(q: BlockScaledTensor) -> torch.Tensor:
-    """bf16 ``code * 2^(scales - 127)`` in the source's shape (``quantization.py:277-297``)."""
+    """bf16 ``code * 2^(scales - 127)`` (MX) or ``code * scales * global_scale`` (NVFP4) in the source's shape
+    (``quantization.py:277-297``)."""
+    if not q.pow2_scale and q.packed and q.block_size == NVFP4_BLOCK and q.global_scale is not None:
+        return _dequantize_nvfp4(q)
     if not q.pow2_scale or q.block_size != BLOCK or q.global_scale is not None:
-        raise NotImplementedError("only MX (power-of-two scale per 32) block-scaled tensors are built on this path")
+        raise NotImplementedError("only the MX formats and NVFP4 are built on this path")
     if q.packed:
         return _dequantize_packed(q)
     data = q.data.view(torch.uint8)
@@ -368,16 +481,20 @@ def _round_trip(t: torch.Tensor, fmt: str, axis: int) -> torch.Tensor:
     """Quantise then dequantise, bf16 (``quantization.py:307-311``): one launch, except MXFP8 rows, which take two."""
     require_implemented(fmt)
     kind, axis = _axis_layout(t, axis)
-    if t.shape[axis] % BLOCK:
-        raise ValueError(f"axis {axis} size {t.shape[axis]} not divisible by block_size {BLOCK}")
+    if t.shape[axis] % FORMAT_BLOCK_SIZE[fmt]:
+        raise ValueError(f"axis {axis} size {t.shape[axis]} not divisible by block_size {FORMAT_BLOCK_SIZE[fmt]}")
     if kind == "moved":
         return _round_trip(t.transpose(axis, -1).contiguous(), fmt, -1).transpose(axis, -1).contiguous()
     if kind == "rows":
         flat = t.reshape(-1, t.shape[-1])
+        if fmt == "nvfp4":
+            return nvfp4_rows(flat, codes=False, round_trip=True)[2].reshape(t.shape)
         if fmt == "mxfp4":
             return mxfp4_rows(flat, codes=False, round_trip=True)[2].reshape(t.shape)
         return dequantize_rows_mxfp8(quantize_rows_mxfp8(flat)).reshape(t.shape)
     banks = t.reshape(-1, *t.shape[-2:])
+    if fmt == "nvfp4":
+        return nvfp4_weight(banks, codes=False, round_trip=True)[2].reshape(t.shape)
     if fmt == "mxfp4":
         return mxfp4_weight(banks, codes=False, round_trip=True)[2].reshape(t.shape)
     return quantize_weight_mxfp8(banks, with_dequant=True).dequant.reshape(t.shape)

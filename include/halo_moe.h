@@ -365,6 +365,31 @@ int hmoe_grouped_gemm_fwd_mxfp4_bias(const uint8_t* a_q, const uint8_t* a_scale,
                                      const uint8_t* b_scale, const void* bias, const int32_t* offs, int64_t total_rows,
                                      int num_groups, int64_t k, int64_t n, void* out, int64_t ldo, void* stream);
 
+/* ------------------------------------------------------------------------------------------------------- NVFP4
+ * The reference's "nvfp4" quant_format (halo/kernels/lowp/spec.py:11): e2m1 elements, two per byte, with one e4m3
+ * scale per 16 values along the contraction axis and one fp32 power-of-two scale per tensor
+ * (halo/kernels/lowp/quantization.py:209-226: global = the smallest power of two >= amax_tensor / 2688, scale =
+ * e4m3(min(amax_block / 6 / global, 448)), code = e2m1(value / (f32(scale) * global)), a zero divisor taken as 1).
+ * expert_gemm(quant_format="nvfp4") of the reference is the bf16 grouped product of the two fake-quantised operands
+ * (halo/kernels/expert_gemm.py:33-38), and so it is here: the scaled matrix instruction takes power-of-two scales only.
+ *
+ * tensor_amax: one float in device memory, the largest magnitude of the whole tensor (NaN if it holds one), reduced by
+ * the caller.  hmoe_nvfp4_rows replaces quantize_nvfp4(t, axis=-1), dequantize and the round trip
+ * (quantization.py:248-270, 277-297, 307-311) for x [x_rows, k] (HMOE_BF16 or HMOE_F32, row stride ldx; row r is
+ * x[row_index[r]], zeros for an index outside [0, x_rows), or x[r] with row_index NULL).  Outputs, each optional (NULL),
+ * at least one of packed and round_trip given, scale required with packed: packed u8 [rows, k / 2] (element 2 i in the
+ * low nibble of byte i), scale u8 [rows, k / 16] (e4m3fn bits), round_trip bf16 [rows, k] (row stride ldo), global_out
+ * (one float: the tensor's scale).  k must be a multiple of 16.  hmoe_nvfp4_weight is the same along axis 1 of
+ * w [groups, k, n] under one scale for the whole bank: packed [groups, k / 2, n], scale [groups, k / 16, n], round_trip
+ * bf16 [groups, k, n].  hmoe_nvfp4_dequantize_rows gives rows back as bf16 = level * sign * (f32(scale) * global). */
+int hmoe_nvfp4_rows(const void* x, int dtype, int64_t ldx, const int64_t* row_index, int64_t x_rows, int64_t rows,
+                    int64_t k, const float* tensor_amax, uint8_t* packed, uint8_t* scale, void* round_trip, int64_t ldo,
+                    float* global_out, void* stream);
+int hmoe_nvfp4_weight(const void* w, int dtype, int64_t groups, int64_t k, int64_t n, const float* tensor_amax,
+                      uint8_t* packed, uint8_t* scale, void* round_trip, float* global_out, void* stream);
+int hmoe_nvfp4_dequantize_rows(const uint8_t* packed, const uint8_t* scale, const float* global_scale, int64_t rows,
+                               int64_t k, void* out, int64_t ldo, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

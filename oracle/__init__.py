@@ -40,5 +40,12 @@ How each function is pinned (tests/test_oracle_*.py):
   of ``tests/cpu/kernels/test_quantization.py:48-55, 99-113``; zero, sub-2^-127, inf and NaN blocks, the 0.25 round-trip
   bound, the magnitude independence of ``test_block_scale_oracle.py:118-137``) and the product term by term on sampled
   outputs.  The same fp32 ``log2`` caveat as ``mxfp8`` at power-of-two multiples of 6: "parity unpinned" there.
+* ``nvfp4.*`` -- the global scale by ``2^(e-1) < amax/2688 <= 2^e`` in exact rational arithmetic; the block scales by
+  torch's own ``float8_e4m3fn`` cast of ``amax / 6 / global``; the codes by brute force (a nearest level of the fp32
+  quotient, the even code on a tie); the known answers the reference's tests hold (amax 30 -> global 2^-6, scale 320,
+  value 30 of ``tests/cpu/kernels/test_block_scale_oracle.py:97-116``; the storage shapes, the outlier of 5000, the
+  0.25 bound and "fp8 beats fp4" of ``tests/cpu/kernels/test_quantization.py:37-45, 58-71, 116-124``; magnitude
+  independence, shard against bank, non-finite inputs of ``test_block_scale_oracle.py:118-196``) and the product term by
+  term.  A tensor whose amax / 2688 lies within an ulp of a power of two: "parity unpinned" (``log2`` rounding).
 * ``moe_layer.*`` -- the dense formula ``out[t] = sum_k w[t,k] * FFN_e(x[t])`` over valid slots.
 """

@@ -175,6 +175,18 @@ def test_bad_arguments_come_back_as_status_codes_before_any_launch():
     assert mx4(fake, fake, 8, fake, fake, None, 8, 4, 128, 128, fake, 128, None) == invalid       # groups without ends
     assert mx4(fake, fake, 8, fake, None, fake, 8, 4, 128, 128, fake, 128, None) == invalid
     assert mx4(None, None, 0, None, None, None, 0, 1, 128, 128, None, 128, None) == 0
+    # NVFP4: blocks of 16, the tensor's amax required, at least one output, the scales with the codes
+    nv = lib.hmoe_nvfp4_rows
+    assert nv(fake, bf16, 64, None, 8, 8, 40, fake, fake, fake, None, 64, None, None) == unsupported   # K % 16
+    assert nv(fake, bf16, 64, None, 8, 8, 64, None, fake, fake, None, 64, None, None) == invalid       # no amax
+    assert nv(fake, bf16, 64, None, 8, 8, 64, fake, None, None, None, 64, None, None) == invalid       # no output
+    assert nv(fake, bf16, 64, None, 8, 8, 64, fake, fake, None, None, 64, None, None) == invalid       # codes, no scales
+    assert nv(None, bf16, 64, None, 0, 0, 64, None, None, None, None, 64, None, None) == 0
+    assert lib.hmoe_nvfp4_weight(fake, bf16, 4, 40, 64, fake, fake, fake, None, None, None) == unsupported
+    assert lib.hmoe_nvfp4_weight(fake, bf16, 4, 64, 64, None, fake, fake, None, None, None) == invalid
+    assert lib.hmoe_nvfp4_weight(fake, bf16, 0, 64, 64, None, None, None, None, None, None) == 0
+    assert lib.hmoe_nvfp4_dequantize_rows(fake, fake, None, 8, 64, fake, 64, None) == invalid
+    assert lib.hmoe_nvfp4_dequantize_rows(fake, fake, fake, 8, 40, fake, 64, None) == unsupported
     for with_bias in (lib.hmoe_grouped_gemm_fwd_mxfp8_bias, lib.hmoe_grouped_gemm_fwd_mxfp4_bias):
         assert with_bias(fake, fake, 8, fake, fake, None, fake, 8, 4, 128, 128, fake, 128, None) == invalid  # no bias
         assert with_bias(fake, fake, 8, fake, fake, fake + 2, fake, 8, 4, 128, 128, fake, 128, None) == unsupported

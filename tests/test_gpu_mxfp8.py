@@ -129,8 +129,8 @@ def test_fake_quant_api_as_the_reference_tests_state_it(device):
     assert large > small and large == 125
     with pytest.raises(ValueError, match="not divisible"):
         quantize_mxfp8(torch.randn(8, 30, device=device))
-    with pytest.raises(NotImplementedError):
-        fake_quant(x, "nvfp4")
+    with pytest.raises(ValueError, match="unknown block-scaled format"):
+        fake_quant(x, "fp3")
     leaf = (torch.randn(64, 256) * 0.3).to(device).requires_grad_(True)
     y = fake_quant(leaf, "mxfp8", axis=-1)
     assert fro(y.detach(), leaf.detach()) < 0.05
@@ -341,8 +341,8 @@ def test_layer_with_mxfp8_experts_against_the_cpu_loop_over_fake_quantised_produ
     inputs = cases.make_layer_inputs(cfg)
     layer = _build_layer(cfg, inputs, device)
     assert layer.set_lowp_compute("mxfp8", weight_cacheable=True) is True
-    with pytest.raises(NotImplementedError):
-        layer.set_lowp_compute("nvfp4", weight_cacheable=True)
+    with pytest.raises(ValueError, match="unknown block-scaled format"):
+        layer.set_lowp_compute("fp3", weight_cacheable=True)
     x = inputs["x"].to(device).requires_grad_(True)
     result = layer(x)
     out = result[0] if isinstance(result, tuple) else result

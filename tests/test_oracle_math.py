@@ -1,5 +1,5 @@
 """Pins ``oracle.glu``, ``oracle.grouped_mm``, ``oracle.router``, ``oracle.block_fp8``, ``oracle.mxfp8``,
-``oracle.mxfp4`` and ``oracle.moe_layer`` against
+``oracle.mxfp4``, ``oracle.nvfp4`` and ``oracle.moe_layer`` against
 library routines (torch autograd, matmul, softmax, topk, the float8 cast), identities and brute force."""
 
 import numpy as np
@@ -7,7 +7,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from oracle import block_fp8, glu, grouped_mm, moe_layer, mxfp4, mxfp8, router
+from oracle import block_fp8, glu, grouped_mm, moe_layer, mxfp4, mxfp8, nvfp4, router
 
 PROBE = (-64.0, -8.0, -1.0, -0.5, -1e-3, 0.0, 1e-3, 0.5, 1.0, 8.0, 64.0)  # fused_glu.py:33 of the reference
 
@@ -571,3 +571,139 @@ def test_mxfp4_round_trip_and_expert_product_sit_in_the_format_error_bands():
         total = sum(value(int(ca[r, k])) * 2.0 ** (int(sa[r, k // 32]) - 127) *
                     value(int(cb[e, k, c])) * 2.0 ** (int(sb[e, k // 32, c]) - 127) for k in range(320))
         assert abs(got[r, c] - total) <= 1e-12 * max(1.0, abs(total))
+
+
+# ----------------------------------------------------------------------------------------------------------- nvfp4
+def test_nvfp4_global_scale_is_the_smallest_power_of_two_that_lifts_the_amax_into_range():
+    """Pins ``nvfp4.global_scale`` by its defining inequality in exact rational arithmetic, 2^(e-1) < amax / 2688 <=
+    2^e, and by the reference's known answer: amax 30 gives 2^ceil(log2(30 / 2688)) = 2^-6, the block's e4m3 scale is
+    then 30 / 6 / 2^-6 = 320 exactly, and the value comes back as 30
+    (``tests/cpu/kernels/test_block_scale_oracle.py:97-116``)."""
+    import math
+    from fractions import Fraction
+
+    g = torch.Generator().manual_seed(5)
+    values = (torch.rand(200, generator=g) + 0.5) * torch.exp2(torch.randint(-100, 100, (200,), generator=g).float())
+    for a in values.tolist() + [2688.0, 2688.0 * 2.0 ** -20, 2689.0, 2687.0, 1e-38, 3e38]:
+        e = int(math.log2(float(nvfp4.global_scale(a))))
+        assert float(nvfp4.global_scale(a)) == 2.0 ** e
+        ratio = Fraction(max(np.float32(a).item(), float(np.finfo(np.float32).tiny))) / 2688
+        assert ratio <= Fraction(2) ** e and ratio > Fraction(2) ** (e - 1), (a, e)
+    assert nvfp4.global_scale(0.0) == np.float32(2.0 ** -137) and np.isnan(nvfp4.global_scale(np.nan))
+    block = np.zeros(16, dtype=np.float32)
+    block[0] = 30.0
+    data, scales, gs = nvfp4.quantize_nvfp4(block)
+    assert gs == 2.0 ** math.ceil(math.log2(30.0 / 2688.0)) == 2.0 ** -6
+    assert block_fp8.decode_e4m3fn(scales)[0] == 320.0 and scales.dtype == np.uint8 and scales.shape == (1,)
+    assert data.shape == (8,) and data[0] == 7 and not data[1:].any()
+    assert nvfp4.dequantize_nvfp4(data, scales, gs)[0] == 30.0
+
+
+def test_nvfp4_scales_are_torchs_e4m3_cast_and_codes_the_nearest_level_of_the_fp32_quotient():
+    """Pins ``quantize_nvfp4`` / ``dequantize_nvfp4`` by library routines and brute force: the block scales equal
+    torch's own float8_e4m3fn cast of ``amax / 6 / global`` (fp32 operations, as the reference's); every code is a
+    level nearest to the fp32 quotient ``value / (scale * global)``, the even code on a tie; the round trip is within
+    half a level gap of the value in units of the block's scale; storage shapes as the reference's tests state them
+    (``tests/cpu/kernels/test_quantization.py:37-45``), along the last axis and along axis 0."""
+    x = _mx_blocks().numpy()[6:]  # finite rows over 40 binades
+    data, scales, gs = nvfp4.quantize_nvfp4(x)
+    rows = x.shape[0]
+    assert data.shape == (rows, 128) and scales.shape == (rows, 16) and data.dtype == scales.dtype == np.uint8
+    xt = torch.from_numpy(x)
+    amax = xt.abs().reshape(rows, 16, 16).amax(dim=2)
+    want_scales = (amax / 6.0 / float(gs)).clamp(max=448.0).to(torch.float8_e4m3fn)
+    assert np.array_equal(scales, want_scales.view(torch.uint8).numpy())
+    divisor = want_scales.float() * float(gs)
+    divisor = torch.where(divisor == 0, torch.ones_like(divisor), divisor)
+    quotient = (xt.reshape(rows, 16, 16) / divisor[:, :, None]).reshape(rows, 256).double().numpy()
+    codes = mxfp4.unpack_codes(data)
+    levels = mxfp4.E2M1_LEVELS.astype(np.float64)
+    mag = np.minimum(np.abs(quotient), 6.0)
+    dist = np.abs(mag[..., None] - levels)
+    chosen = np.take_along_axis(dist, (codes & 7)[..., None].astype(np.int64), axis=-1)[..., 0]
+    assert (chosen == dist.min(axis=-1)).all()
+    tie = (dist == dist.min(axis=-1, keepdims=True)).sum(axis=-1) > 1
+    assert tie.any() and ((codes & 7)[tie] % 2 == 0).all()
+    assert np.array_equal(codes >> 3, (quotient < 0).astype(np.uint8))
+    restored = nvfp4.dequantize_nvfp4(data, scales, gs)
+    assert np.array_equal(restored, torch.from_numpy(restored).bfloat16().float().numpy())
+    # within half a level gap in units of the block's scale; a quotient above 6 (the e4m3 scale was rounded down)
+    # saturates at 6 scales exactly, and a block whose scale underflows e4m3 (the tensor spans 40 binades under one
+    # global scale) comes back as zeros: the format's own behaviour, asserted as such
+    unit = np.repeat((want_scales.float() * float(gs)).double().numpy(), 16, axis=1)
+    bound = np.where(mag <= 2, 0.25, np.where(mag <= 4, 0.5, 1.0)) * unit
+    inside, dead = (np.abs(quotient) <= 6) & (unit > 0), unit == 0
+    assert inside.sum() > 5000 and dead.any() and (~inside & ~dead).any()
+    assert (np.abs(restored - x)[inside] <= (bound * (1 + 2.0 ** -8))[inside]).all()
+    assert np.array_equal(np.abs(restored)[~inside & ~dead], (6 * unit)[~inside & ~dead].astype(np.float32))
+    assert not restored[dead].any()
+    d0, s0, g0 = nvfp4.quantize_nvfp4(x.T.copy(), axis=0)
+    assert d0.shape == (128, rows) and s0.shape == (16, rows) and g0 == gs
+    assert np.array_equal(d0, data.T) and np.array_equal(s0, scales.T)
+    with pytest.raises(ValueError, match="not divisible"):
+        nvfp4.quantize_nvfp4(np.zeros((8, 24), dtype=np.float32))
+
+
+def test_nvfp4_edges_and_error_bands_as_the_reference_tests_state_them():
+    """Zeros round-trip to zeros (``tests/cpu/kernels/test_quantization.py:82-89``); an outlier above 6 * 448 keeps every
+    scale and value finite (``:116-124``); the round trip is inside 0.25 and worse than MXFP8's (``:58-71``); the error
+    does not depend on the magnitude over 32 decades (``tests/cpu/kernels/test_block_scale_oracle.py:118-137``); a shard
+    quantised alone equals its slice of the bank although their global scales differ (``:157-172``); an inf or a NaN is
+    never absorbed and finite input never gives a NaN (``:175-196``); the product term by term on sampled outputs."""
+    zeros = nvfp4.fake_quant_nvfp4(np.zeros((32, 64), dtype=np.float32))
+    assert np.isfinite(zeros).all() and not zeros.any()
+    torch.manual_seed(0)
+    x = (torch.randn(16, 64) * 0.1).numpy()
+    x[0, 0] = 5000.0
+    data, scales, gs = nvfp4.quantize_nvfp4(x)
+    assert np.isfinite(block_fp8.decode_e4m3fn(scales)).all() and ((scales & 0x7F) != 0x7F).all()
+    assert np.isfinite(nvfp4.dequantize_nvfp4(data, scales, gs)).all()
+    torch.manual_seed(0)
+    x = (torch.randn(64, 256) * 0.5).numpy()
+    err4 = np.linalg.norm(nvfp4.fake_quant_nvfp4(x) - x) / np.linalg.norm(x)
+    err8 = np.linalg.norm(mxfp8.fake_quant_mxfp8(x) - x) / np.linalg.norm(x)
+    assert err8 < err4 < 0.25 and err4 > 0.04
+    base = torch.randn(128, 256).double().numpy()
+    errs = []
+    for exponent in range(4, -32, -4):
+        scaled = (base * 10.0 ** exponent).astype(np.float32)
+        recon = nvfp4.fake_quant_nvfp4(scaled).astype(np.float64)
+        errs.append(np.linalg.norm(recon - scaled) / np.linalg.norm(scaled.astype(np.float64)))
+    assert max(errs) - min(errs) < 0.02
+    bank = (torch.randn(8, 64, 256) * 0.02).numpy()
+    bank[0] *= 1e-3
+    whole = nvfp4.fake_quant_nvfp4(bank)
+    assert nvfp4.quantize_nvfp4(bank[:1])[2] != nvfp4.quantize_nvfp4(bank)[2]  # the small expert alone scales lower
+    for lo in range(0, 8, 2):
+        assert np.array_equal(nvfp4.fake_quant_nvfp4(bank[lo:lo + 2]), whole[lo:lo + 2])
+    for poison in (np.nan, np.inf, -np.inf):
+        bad = (torch.randn(4, 64) * 0.3).numpy()
+        bad[1, 7] = poison
+        assert not np.isfinite(nvfp4.fake_quant_nvfp4(bad)).all()
+    fine = (torch.randn(4, 64) * 0.3).numpy()
+    fine[0, 0] = 5e4
+    fine[2, :] = 0.0
+    assert np.isfinite(nvfp4.fake_quant_nvfp4(fine)).all()
+    g = torch.Generator().manual_seed(3)
+    counts = (40, 0, 70, 18)
+    a = (torch.randn(sum(counts), 320, generator=g) * 0.3).bfloat16().float().numpy()
+    b = (torch.randn(len(counts), 320, 96, generator=g) * 0.02).bfloat16().float().numpy()
+    offs = np.cumsum(counts)
+    got = nvfp4.expert_gemm_nvfp4(a, b, offs)
+    da, sa, ga = nvfp4.quantize_nvfp4(a, -1)
+    db, sb, gb = nvfp4.quantize_nvfp4(b, 1)
+    ca, cb = mxfp4.unpack_codes(da), mxfp4.unpack_codes(db, 1)
+    va, vb = block_fp8.decode_e4m3fn(sa).astype(float) * float(ga), block_fp8.decode_e4m3fn(sb).astype(float) * float(gb)
+    level = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+    value = lambda c: level[c & 7] * (-1.0 if c & 8 else 1.0)
+    for r, c in ((0, 0), (39, 95), (40, 3), (127, 50)):
+        e = int(np.searchsorted(offs, r, side="right"))
+        total = sum(value(int(ca[r, k])) * va[r, k // 16] * value(int(cb[e, k, c])) * vb[e, k // 16, c] for k in range(320))
+        assert abs(got[r, c] - total) <= 1e-12 * max(1.0, abs(total))
+    plain = np.zeros_like(got)
+    start = 0
+    for e, end in enumerate(offs.tolist()):
+        plain[start:end] = a[start:end].astype(np.float64) @ b[e].astype(np.float64)
+        start = end
+    rel = np.linalg.norm(got - plain) / np.linalg.norm(plain)
+    assert 0.04 < rel < 0.25, rel  # the reference's band for this format (tests/gpu/kernels/test_expert_gemm.py:55-74)
