@@ -136,21 +136,23 @@ class _SharedRows:
     An entry is tied to the tensor object by a weak reference and to its version counter, and dies with the tensor."""
 
     def __init__(self):
-        self._ref, self._key, self._value = None, None, None
+        self._ref, self._key, self._value, self._hold = None, None, None, None
 
     def get(self, tensor: torch.Tensor, key: tuple):
         if self._ref is not None and self._ref() is tensor and self._key == key:
             return self._value
         return None
 
-    def put(self, tensor: torch.Tensor, key: tuple, value) -> None:
+    def put(self, tensor: torch.Tensor, key: tuple, value, hold=None) -> None:
+        """``hold``: an object the key names by ``id`` (the row index); kept alive with the entry, so that the id
+        cannot pass to another object while the entry can still be hit."""
         import weakref
 
         def drop(ref, self=self):
             if self._ref is ref:
-                self._ref, self._key, self._value = None, None, None
+                self._ref, self._key, self._value, self._hold = None, None, None, None
 
-        self._ref, self._key, self._value = weakref.ref(tensor, drop), key, value
+        self._ref, self._key, self._value, self._hold = weakref.ref(tensor, drop), key, value, hold
 
 
 _quantised_rows = _SharedRows()
@@ -183,7 +185,7 @@ class _MxFp8ExpertGemm(torch.autograd.Function):
         rows_q = _quantised_rows.get(mat_a, key)
         if rows_q is None:
             rows_q = quantize_rows_mxfp8(mat_a, row_index)
-            _quantised_rows.put(mat_a, key, rows_q)
+            _quantised_rows.put(mat_a, key, rows_q, hold=row_index)
         rows = rows_q.rows
         ctx.k, ctx.dtype, ctx.gathered = k, mat_a.dtype, row_index is not None
         # the e4m3 rows ride on the node itself: projections that share them must see one object, and they are no
@@ -303,14 +305,14 @@ class _Mxfp4ExpertGemm(torch.autograd.Function):
             a_rt = _round_tripped_rows.get(mat_a, key)
             if a_rt is None:
                 a_rt = mxfp4_rows(mat_a, row_index, codes=False, round_trip=True)[2].to(mat_a.dtype)
-                _round_tripped_rows.put(mat_a, key, a_rt)
+                _round_tripped_rows.put(mat_a, key, a_rt, hold=row_index)
             ctx.save_for_backward(a_rt, w_rt, offs32, inv_map)
             return _plus_bias(_forward(a_rt, w_rt, offs32), bias, eids)
         weight = expert_weight_operand(mat_b, weight_cacheable, "mxfp4")
         rows_q = _quantised_rows4.get(mat_a, key)
         if rows_q is None:
             rows_q = quantize_rows_mxfp4(mat_a, row_index)
-            _quantised_rows4.put(mat_a, key, rows_q)
+            _quantised_rows4.put(mat_a, key, rows_q, hold=row_index)
         rows = rows_q.rows
         ctx.rows_q = rows_q  # projections that share the rows must see one object
         ctx.save_for_backward(weight.dequant, offs32, inv_map)
