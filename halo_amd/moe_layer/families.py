@@ -15,7 +15,7 @@ from halo_amd.kernels.grouped_mm import bias_fusable, grouped_mm_bias
 from halo_amd.kernels.moe_permute import MoEExpertBiasGather
 from halo_amd.kernels.router import SOFTMAX_TOPK, fused_topk_gate
 from halo_amd.moe_layer.config import GPT_OSS, QWEN3, QWEN3_5
-from halo_amd.moe_layer.layer import EPMoELayerBase, EPSharedExpertsMoELayerBase, dense_mm
+from halo_amd.moe_layer.layer import EPMoELayerBase, EPSharedExpertsMoELayerBase
 
 
 def split_interleaved_gate_up(interleaved: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:

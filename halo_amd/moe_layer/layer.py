@@ -23,8 +23,8 @@ import torch.nn as nn
 
 from halo_amd.kernels.expert_gemm import BlockFp8Weight, expert_gemm, fp8_mfma_usable
 from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled, resolve_fused_glu_mul
-from halo_amd.kernels.grouped_mm import (GatheredRows, addto_fusable, grouped_mm, grouped_mm_addto,
-                                         grouped_mm_combine, grouped_wgrad)
+from halo_amd.kernels.grouped_mm import (GatheredRows, addto_fusable, grouped_mm_addto, grouped_mm_combine,
+                                         grouped_wgrad)
 from halo_amd.kernels.moe_permute import (MoEGatherPermute, MoEWeightedUnpermute, MoEWeightedUnpermuteAdd,
                                           warm_permute_kernels)
 from halo_amd.kernels.moe_route_sort import sort_routing_by_expert, warm_route_sort_kernels
