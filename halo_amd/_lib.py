@@ -44,8 +44,10 @@ SIGNATURES = {
     "hmoe_grouped_gemm_fwd_bias": (I, [P, L, P, P, P, L, I, L, L, I, P, L, P]),
     "hmoe_grouped_gemm_fwd_addto": (I, [P, L, P, P, L, I, L, L, I, P, L, F, P, L, P]),
     "hmoe_grouped_gemm_dgrad": (I, [P, L, P, P, L, I, L, L, I, P, L, P]),
+    "hmoe_grouped_gemm_dgrad_addto": (I, [P, L, P, P, L, I, L, L, I, P, L, P, L, P]),
     "hmoe_grouped_gemm_wgrad": (I, [P, L, P, L, P, L, I, L, L, I, P, P]),
     "hmoe_grouped_gemm_fwd_gather": (I, [P, L, L, P, P, P, L, I, L, L, I, P, L, P]),
+    "hmoe_grouped_gemm_fwd_gather_bias": (I, [P, L, L, P, P, P, P, L, I, L, L, I, P, L, P]),
     "hmoe_grouped_gemm_wgrad_gather": (I, [P, L, L, P, P, L, P, L, I, L, L, I, P, P]),
     "hmoe_grouped_gemm_dgrad_gather": (I, [P, L, L, P, P, P, L, I, L, L, I, P, L, P]),
     "hmoe_grouped_gemm_wgrad_gather_grad": (I, [P, L, P, L, L, P, P, L, I, L, L, I, P, P]),

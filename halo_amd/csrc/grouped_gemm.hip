@@ -115,8 +115,9 @@ struct GemmArgs {
   int64_t a_rows = 0;                // rows of the array a_index points into
   bool gather_b = false;
   const void* bias = nullptr;        // fwd: [G, N] in the operands' dtype, added to group g's output rows
-  // fwd: out = addend + addend_scale * product, element by element with the roundings of those tensor operations
-  // (an adapter's low-rank delta joining the base projection); rows ld_addend apart, may be the output itself
+  // fwd, dgrad: out = addend + addend_scale * product, element by element with the roundings of those tensor
+  // operations (an adapter's low-rank delta joining the base projection; the input gradient of a second projection
+  // of the same rows joining the first's); rows ld_addend apart, may be the output itself
   const void* addend = nullptr;
   int64_t ld_addend = 0;
   float addend_scale = 1.f;
@@ -1124,7 +1125,8 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
 #ifdef HMOE_WG_TIMES
   const unsigned long long wg_entered = __builtin_readcyclecounter();
 #endif
-  static_assert(!kAddTo || (kMode == kFwd && !kBias), "the scaled sum into an addend belongs to the plain forward");
+  static_assert(!kAddTo || ((kMode == kFwd || kMode == kDgrad) && !kBias && !kGather),
+                "the scaled sum into an addend belongs to the plain forward and the plain input gradient");
   static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
   static_assert(!kBias || kMode == kFwd, "the expert bias belongs to the forward product");
   static_assert(kGather >= 0 && kGather <= 2 && (kGather != 2 || kMode == kWgrad), "B is gathered in wgrad only");
@@ -1547,6 +1549,8 @@ HMOE_BF16_INSTANCE(kWgrad)
 template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, 1>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, 0, true>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, 0, false, true>(GemmArgs);
+template __global__ void grouped_gemm_bf16_kernel<kFwd, Config<2, 4, 4, 2>, 1, true>(GemmArgs);
+template __global__ void grouped_gemm_bf16_kernel<kDgrad, Config<2, 4, 4, 2>, 0, false, true>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kDgrad, Config<2, 4, 4, 2>, 1>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kWgrad, Config<2, 4, 4, 2>, 1>(GemmArgs);
 template __global__ void grouped_gemm_bf16_kernel<kWgrad, Config<2, 4, 4, 2>, 2>(GemmArgs);
@@ -2072,7 +2076,7 @@ __global__ void __launch_bounds__(256) grouped_gemm_f32_kernel(GemmArgs p) {
       if (r < rows_out && cc < cols_out) {
         float v = acc[i][j];
         if (kMode == kFwd && p.bias != nullptr) v += static_cast<const float*>(p.bias)[static_cast<int64_t>(g) * p.n + cc];
-        if (kMode == kFwd && p.addend != nullptr) {
+        if ((kMode == kFwd || kMode == kDgrad) && p.addend != nullptr) {
           // two roundings, as the tensor operations have them: the multiply must not contract into the add
 #pragma clang fp contract(off)
           const float scaled = p.addend_scale * v;
@@ -2148,7 +2152,7 @@ int launch(const GemmArgs& p, int dtype, hipStream_t stream) {
     if constexpr (kMode == kFwdFp8W) {
       rc = launch_staged<kMode, Tile>(p, 1, stream);
     } else if constexpr (kMode == kFwd) {
-      rc = p.a_index  ? launch_direct<kMode, Tile, 1>(p, stream)
+      rc = p.a_index  ? (p.bias ? launch_direct<kMode, Tile, 1, true>(p, stream) : launch_direct<kMode, Tile, 1>(p, stream))
            : p.bias   ? launch_direct<kMode, Tile, 0, true>(p, stream)
            : p.addend ? launch_direct<kMode, Tile, 0, false, true>(p, stream)
                       : launch_direct<kMode, Tile>(p, stream);
@@ -2157,7 +2161,9 @@ int launch(const GemmArgs& p, int dtype, hipStream_t stream) {
            : p.gather_b ? launch_direct<kMode, Tile, 2>(p, stream)
                         : launch_direct<kMode, Tile, 1>(p, stream);
     } else {
-      rc = p.a_index ? launch_direct<kMode, Tile, 1>(p, stream) : launch_direct<kMode, Tile>(p, stream);
+      rc = p.a_index  ? launch_direct<kMode, Tile, 1>(p, stream)
+           : p.addend ? launch_direct<kMode, Tile, 0, false, true>(p, stream)
+                      : launch_direct<kMode, Tile>(p, stream);
     }
     if (rc) return rc;
   } else if constexpr (kMode != kFwdFp8W) {
@@ -2317,6 +2323,23 @@ int hmoe_grouped_gemm_fwd_gather(const void* a, int64_t lda, int64_t a_rows, con
   return launch<kFwd>(p, dtype, static_cast<hipStream_t>(stream));
 }
 
+int hmoe_grouped_gemm_fwd_gather_bias(const void* a, int64_t lda, int64_t a_rows, const int64_t* row_index,
+                                      const void* b, const void* bias, const int32_t* offs, int64_t total_rows,
+                                      int num_groups, int64_t k, int64_t n, int dtype, void* out, int64_t ldo,
+                                      void* stream) {
+  using namespace hmoe;
+  if (dtype != HMOE_BF16) return HMOE_UNSUPPORTED;
+  if (a_rows < 0) return HMOE_INVALID_ARGUMENT;
+  GemmArgs p{a, lda, b, n, out, ldo, offs, total_rows, num_groups, k, n, nullptr, row_index, a_rows};
+  p.bias = bias;
+  if (int rc = validate(p, dtype)) return rc;
+  if (total_rows == 0 || n == 0) return HMOE_OK;
+  if (!a || !b || !out || !row_index || !bias) return HMOE_INVALID_ARGUMENT;
+  if (lda < k || ldo < n) return HMOE_INVALID_ARGUMENT;
+  if (!aligned16(bias)) return HMOE_UNSUPPORTED;
+  return launch<kFwd>(p, dtype, static_cast<hipStream_t>(stream));
+}
+
 int hmoe_grouped_gemm_wgrad_gather(const void* a, int64_t lda, int64_t a_rows, const int64_t* row_index,
                                    const void* grad_out, int64_t ldg, const int32_t* offs, int64_t total_rows,
                                    int num_groups, int64_t k, int64_t n, int dtype, void* grad_b, void* stream) {
@@ -2472,6 +2495,23 @@ int hmoe_grouped_gemm_dgrad(const void* grad_out, int64_t ldg, const void* b, co
   if (total_rows == 0 || k == 0) return HMOE_OK;
   if (!grad_out || !b || !grad_a) return HMOE_INVALID_ARGUMENT;
   if (ldg < n || lda < k) return HMOE_INVALID_ARGUMENT;
+  return launch<kDgrad>(p, dtype, static_cast<hipStream_t>(stream));
+}
+
+int hmoe_grouped_gemm_dgrad_addto(const void* grad_out, int64_t ldg, const void* b, const int32_t* offs,
+                                  int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype,
+                                  const void* addend, int64_t ld_addend, void* grad_a, int64_t lda, void* stream) {
+  using namespace hmoe;
+  GemmArgs p{grad_out, ldg, b, n, grad_a, lda, offs, total_rows, num_groups, k, n, nullptr};
+  p.addend = addend;
+  p.ld_addend = ld_addend;
+  p.addend_scale = 1.f;
+  if (int rc = validate(p, dtype)) return rc;
+  if (total_rows == 0 || k == 0) return HMOE_OK;
+  if (!grad_out || !b || !grad_a || !addend) return HMOE_INVALID_ARGUMENT;
+  if (ldg < n || lda < k || ld_addend < k) return HMOE_INVALID_ARGUMENT;
+  if (dtype == HMOE_BF16 && (!aligned16(addend) || ld_addend % 8 || ld_addend * 2 * 512 >= (int64_t(1) << 31)))
+    return HMOE_UNSUPPORTED;
   return launch<kDgrad>(p, dtype, static_cast<hipStream_t>(stream));
 }
 

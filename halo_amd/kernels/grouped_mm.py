@@ -267,6 +267,39 @@ def gather_fusable(tokens: torch.Tensor, mat_b) -> bool:
             and mat_b.shape[2] % 8 == 0 and tokens.shape[1] == mat_b.shape[1])
 
 
+def _gather_forward(tokens, row_index, mat_b, bias, offs32) -> torch.Tensor:
+    """``tokens[row_index] @ mat_b (+ bias row of the row's group)`` through the gathering forward kernel."""
+    device = tokens.device
+    groups, k, n = mat_b.shape
+    rows = row_index.shape[0]
+    out = torch.empty((rows, n), dtype=tokens.dtype, device=device)
+    if rows and n:
+        with _lib.on_device(device):
+            if bias is None:
+                _lib.call("hmoe_grouped_gemm_fwd_gather", _lib.ptr(tokens), tokens.stride(0), tokens.shape[0],
+                          _lib.ptr(row_index), _lib.ptr(mat_b), _lib.ptr(offs32), rows, groups, k, n,
+                          _lib.dtype_id(tokens.dtype), _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
+            else:
+                _lib.call("hmoe_grouped_gemm_fwd_gather_bias", _lib.ptr(tokens), tokens.stride(0), tokens.shape[0],
+                          _lib.ptr(row_index), _lib.ptr(mat_b), _lib.ptr(bias), _lib.ptr(offs32), rows, groups, k, n,
+                          _lib.dtype_id(tokens.dtype), _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
+    return out
+
+
+def _gather_wgrad(tokens, row_index, grad_output, offs32, groups: int) -> torch.Tensor:
+    """``[groups, K, N]``: ``tokens[row_index][s:e]^T @ grad_output[s:e]`` per group, the rows fetched by index."""
+    device = tokens.device
+    rows, k, n = row_index.shape[0], tokens.shape[1], grad_output.shape[1]
+    grad_b = torch.empty((groups, k, n), dtype=tokens.dtype, device=device)
+    if k and n:
+        with _lib.on_device(device):
+            _lib.call("hmoe_grouped_gemm_wgrad_gather", _lib.ptr(tokens), tokens.stride(0), tokens.shape[0],
+                      _lib.ptr(row_index), _lib.ptr(grad_output), grad_output.stride(0) if rows else n,
+                      _lib.ptr(offs32), rows, groups, k, n, _lib.dtype_id(tokens.dtype), _lib.ptr(grad_b),
+                      _lib.stream_ptr(device))
+    return grad_b
+
+
 class _GatherGroupedMM(Function):
     """``grouped_mm(tokens[row_index], mat_b, offs)`` without the permuted copy: the GEMM's loader and its weight
     gradient's fetch the rows through ``row_index`` (``hmoe_grouped_gemm_fwd_gather`` / ``_wgrad_gather``).  This is
@@ -276,26 +309,17 @@ class _GatherGroupedMM(Function):
 
     @staticmethod
     def forward(ctx, tokens, row_index, inv_map, mat_b, offs):
-        device = _lib.require_device(tokens, row_index, inv_map, mat_b, offs)
-        groups, k, n = mat_b.shape
-        rows = row_index.shape[0]
+        _lib.require_device(tokens, row_index, inv_map, mat_b, offs)
         row_index = row_index.long().contiguous()
-        offs32 = _offs_arg(offs, groups)
-        out = torch.empty((rows, n), dtype=tokens.dtype, device=device)
-        if rows and n:
-            with _lib.on_device(device):
-                _lib.call("hmoe_grouped_gemm_fwd_gather", _lib.ptr(tokens), tokens.stride(0), tokens.shape[0],
-                          _lib.ptr(row_index), _lib.ptr(mat_b), _lib.ptr(offs32), rows, groups, k, n,
-                          _lib.dtype_id(tokens.dtype), _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
+        offs32 = _offs_arg(offs, mat_b.shape[0])
         ctx.save_for_backward(tokens, row_index, inv_map, mat_b, offs32)
-        return out
+        return _gather_forward(tokens, row_index, mat_b, None, offs32)
 
     @staticmethod
     def backward(ctx, grad_output):
         from halo_amd.kernels.moe_permute import gather_reduce_rows
 
         tokens, row_index, inv_map, mat_b, offs32 = ctx.saved_tensors
-        device = tokens.device
         groups, k, n = mat_b.shape
         rows = row_index.shape[0]
         grad_output = _rows(grad_output) if grad_output.numel() else grad_output.new_empty(grad_output.shape)
@@ -305,13 +329,7 @@ class _GatherGroupedMM(Function):
             grad_sorted, _ = grouped_mm_grads(shape_only, mat_b, grad_output, offs32, True, False)
             grad_tokens = gather_reduce_rows(grad_sorted, inv_map)
         if ctx.needs_input_grad[3]:
-            grad_b = torch.empty((groups, k, n), dtype=tokens.dtype, device=device)
-            if k and n:
-                with _lib.on_device(device):
-                    _lib.call("hmoe_grouped_gemm_wgrad_gather", _lib.ptr(tokens), tokens.stride(0), tokens.shape[0],
-                              _lib.ptr(row_index), _lib.ptr(grad_output), grad_output.stride(0) if rows else n,
-                              _lib.ptr(offs32), rows, groups, k, n, _lib.dtype_id(tokens.dtype), _lib.ptr(grad_b),
-                              _lib.stream_ptr(device))
+            grad_b = _gather_wgrad(tokens, row_index, grad_output, offs32, groups)
         return grad_tokens, None, None, grad_b, None
 
 
@@ -319,6 +337,71 @@ def gather_grouped_mm(tokens, row_index, inv_map, mat_b, *, offs):
     """``grouped_mm(tokens[row_index], mat_b, offs=offs)``; see :class:`_GatherGroupedMM`.  The caller checks
     :func:`gather_fusable` first."""
     return _GatherGroupedMM.apply(tokens, row_index, inv_map, mat_b, offs)
+
+
+def pair_fusable(tokens: torch.Tensor, mat_b1, bias1, mat_b2, bias2) -> bool:
+    """Whether :func:`gather_grouped_mm_pair` can take these operands: both weights as :func:`gather_fusable` asks,
+    and both biases either absent or ``[G, N]`` of the rows' dtype."""
+    def bias_ok(bias, mat_b):
+        return bias is None or (isinstance(bias, torch.Tensor) and bias.dtype == tokens.dtype and bias.is_cuda
+                                and bias.dim() == 2 and bias.shape == (mat_b.shape[0], mat_b.shape[2]))
+
+    return (gather_fusable(tokens, mat_b1) and gather_fusable(tokens, mat_b2) and mat_b1.shape[0] == mat_b2.shape[0]
+            and bias_ok(bias1, mat_b1) and bias_ok(bias2, mat_b2))
+
+
+class _GatherGroupedMMPair(Function):
+    """Two projections of the same gathered rows as one node: ``(tokens[row_index] @ w1 + b1[eids],
+    tokens[row_index] @ w2 + b2[eids])``, the gate and up projections of a layer that stores them apart (reference
+    ``families/gpt_oss.py:139-160``).  Both fetch the rows through ``row_index`` and add their bias in the epilogue, so
+    the permuted copy is never written.  In backward the reference's autograd adds the two projections' input
+    gradients at the rows' node and then scatters the sum back (``moe_permute.py:138-141``); here the second input
+    gradient joins the first in its epilogue (``hmoe_grouped_gemm_dgrad_addto``: each product rounded, then the sum,
+    as the tensor addition rounds), and one gather-reduce follows: the same bits without the ``[R, K]`` pass that adds
+    them."""
+
+    @staticmethod
+    def forward(ctx, tokens, row_index, inv_map, w1, b1, w2, b2, offs, eids):
+        _lib.require_device(tokens, row_index, inv_map, w1, b1, w2, b2, offs, eids)
+        row_index = row_index.long().contiguous()
+        offs32 = _offs_arg(offs, w1.shape[0])
+        ctx.save_for_backward(tokens, row_index, inv_map, w1, w2, offs32, eids)
+        return (_gather_forward(tokens, row_index, w1, None if b1 is None else b1.contiguous(), offs32),
+                _gather_forward(tokens, row_index, w2, None if b2 is None else b2.contiguous(), offs32))
+
+    @staticmethod
+    def backward(ctx, grad1, grad2):
+        from halo_amd.kernels.moe_permute import expert_bias_grad, gather_reduce_rows
+
+        tokens, row_index, inv_map, w1, w2, offs32, eids = ctx.saved_tensors
+        device = tokens.device
+        groups, k = w1.shape[0], w1.shape[1]
+        rows = row_index.shape[0]
+        grad1 = _rows(grad1) if grad1.numel() else grad1.new_empty(grad1.shape)
+        grad2 = _rows(grad2) if grad2.numel() else grad2.new_empty(grad2.shape)
+        need = ctx.needs_input_grad
+        grad_tokens = None
+        if need[0]:
+            shape_only = grad1.new_empty((1, k)).expand(rows, k)  # dgrad reads mat_a's shape and dtype only
+            grad_sorted, _ = grouped_mm_grads(shape_only, w1, grad1, offs32, True, False)
+            if rows and k:
+                with _lib.on_device(device):
+                    _lib.call("hmoe_grouped_gemm_dgrad_addto", _lib.ptr(grad2), grad2.stride(0), _lib.ptr(w2),
+                              _lib.ptr(offs32), rows, groups, k, w2.shape[2], _lib.dtype_id(tokens.dtype),
+                              _lib.ptr(grad_sorted), grad_sorted.stride(0), _lib.ptr(grad_sorted),
+                              grad_sorted.stride(0), _lib.stream_ptr(device))
+            grad_tokens = gather_reduce_rows(grad_sorted, inv_map)
+        grad_w1 = _gather_wgrad(tokens, row_index, grad1, offs32, groups) if need[3] else None
+        grad_w2 = _gather_wgrad(tokens, row_index, grad2, offs32, groups) if need[5] else None
+        grad_b1 = expert_bias_grad(grad1, eids, groups) if need[4] else None
+        grad_b2 = expert_bias_grad(grad2, eids, groups) if need[6] else None
+        return grad_tokens, None, None, grad_w1, grad_b1, grad_w2, grad_b2, None, None
+
+
+def gather_grouped_mm_pair(tokens, row_index, inv_map, mat_b1, bias1, mat_b2, bias2, *, offs, eids):
+    """``(grouped_mm(tokens[row_index], mat_b1) + bias1[eids], grouped_mm(tokens[row_index], mat_b2) + bias2[eids])``
+    (a bias may be None); see :class:`_GatherGroupedMMPair`.  The caller checks :func:`pair_fusable` first."""
+    return _GatherGroupedMMPair.apply(tokens, row_index, inv_map, mat_b1, bias1, mat_b2, bias2, offs, eids)
 
 
 # ------------------------------------------------------------------------- down projection + plain combine
@@ -437,4 +520,12 @@ class GatheredRows:
         if not gather_fusable(self.tokens, mat_b):
             return None
         return gather_grouped_mm(self.tokens, self.row_index, self.inv_map, mat_b, offs=offs)
+
+    def grouped_mm_pair(self, mat_b1, bias1, mat_b2, bias2, *, offs, eids):
+        """Two biased projections of these rows through the gathering kernels as one node, or None when the operands
+        do not qualify."""
+        if not pair_fusable(self.tokens, mat_b1, bias1, mat_b2, bias2):
+            return None
+        return gather_grouped_mm_pair(self.tokens, self.row_index, self.inv_map, mat_b1, bias1, mat_b2, bias2,
+                                      offs=offs, eids=eids)
 

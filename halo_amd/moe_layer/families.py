@@ -121,15 +121,16 @@ class EPGptOssMoELayer(EPMoELayerBase):
         result = self._dispatch_compute_combine(flat, experts, weights.float(), input_dtype)
         return result.view(shape), logits.to(input_dtype)
 
+    def _gate_up_attrs(self) -> tuple[str, str]:
+        return ("gate_proj_gmm", "up_proj_gmm") if hasattr(self, "gate_proj_gmm") else ("gate_proj", "up_proj")
+
     def _grouped_expert_ffn(self, sorted_tokens, offs, sorted_expert_ids, output_dtype):
         """Three grouped GEMMs (gate, up, down) on de-interleaved weights, each plus its expert bias."""
-        gate_attr, up_attr = ("gate_proj_gmm", "up_proj_gmm") if hasattr(self, "gate_proj_gmm") else (
-            "gate_proj", "up_proj")
         def project(x, weight_attr):
             return self._grouped_proj_with_bias(x, weight_attr, offs, output_dtype, sorted_expert_ids)
 
-        hidden = self._gptoss_glu(project(sorted_tokens, gate_attr), project(sorted_tokens, up_attr))
-        return project(hidden.to(output_dtype), "down_proj")
+        gate, up = self._project_gate_up(sorted_tokens, offs, output_dtype, sorted_expert_ids, project, with_bias=True)
+        return project(self._gptoss_glu(gate, up).to(output_dtype), "down_proj")
 
     def _grouped_proj_with_bias(self, x, weight_attr, offs, out_dtype, eids):
         bias = getattr(self, f"{weight_attr}_bias", None)

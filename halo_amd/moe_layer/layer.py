@@ -393,15 +393,61 @@ class EPMoELayerBase(ExpertLoadMixin, nn.Module, ABC):
             experts, weights, self.experts_per_rank, counts
         )
         # The permuted copy is left to the first expert projection, whose loader can fetch the rows through the index
-        # (one pass over the tokens saved each way); a projection that cannot asks for the copy.  Only where one
-        # projection reads the rows (gate and up stored fused): two readers would each scatter a gradient back.
-        fuse = self.fuse_permute_into_gemm and self._stores_fused_glu
+        # (one pass over the tokens saved each way); a projection that cannot asks for the copy.  Only where one node
+        # reads the rows (gate and up stored fused, or apart and run as a pair): two nodes would each scatter a
+        # gradient back.
+        fuse = self.fuse_permute_into_gemm and (self._stores_fused_glu or self._pairs_gate_up())
         sorted_tokens = (GatheredRows(tokens, sorted_token_idx, inv_map) if fuse
                          else MoEGatherPermute.apply(tokens, sorted_token_idx, inv_map))
         return sorted_tokens, offs, sorted_token_idx, sorted_weights, sorted_expert_ids, inv_map
 
     def _grouped_expert_ffn(self, sorted_tokens, offs, sorted_expert_ids, output_dtype):
-        return self._glu_ffn(sorted_tokens, lambda x, attr: self._expert_proj(x, attr, offs, output_dtype))
+        def proj(x, attr):
+            return self._expert_proj(x, attr, offs, output_dtype)
+
+        if self._stores_fused_glu:
+            return self._glu_ffn(sorted_tokens, proj)
+        gate, up = self._project_gate_up(sorted_tokens, offs, output_dtype, None, proj, with_bias=False)
+        return proj(self._glu_combine(gate, up), "down_proj")
+
+    def _gate_up_attrs(self) -> tuple[str, str] | None:
+        """The attribute names of the gate and up weights where the layer stores them apart."""
+        return None if self._stores_fused_glu else ("gate_proj", "up_proj")
+
+    def _pairs_gate_up(self) -> bool:
+        """Whether gate and up, stored apart, run as one node over rows fetched through the sort's index
+        (``GatheredRows.grouped_mm_pair``): plain weights, no adapters on either, no low-precision route, and a bias
+        only where the GEMM's epilogue adds it."""
+        attrs = self._gate_up_attrs()
+        if attrs is None or self._lowp_quant_format is not None:
+            return False
+        for attr in attrs:
+            if self._adapted(attr) or not isinstance(getattr(self, attr, None), torch.Tensor):
+                return False
+            if getattr(self, f"{attr}_bias", None) is not None and not getattr(self, "fuse_bias_into_gemm", True):
+                return False
+        return True
+
+    def _project_gate_up(self, x, offs, out_dtype, eids, proj, *, with_bias: bool):
+        """``(gate, up)`` of rows ``x``.  Rows nobody has copied yet go through the pair node when the operands
+        qualify (both projections fetch them by index, their two input gradients are summed in the second one's
+        epilogue); otherwise the rows are copied once and ``proj`` runs twice, as the reference has it
+        (``compute.py:222-242``, ``families/gpt_oss.py:139-152``)."""
+        gate_attr, up_attr = self._gate_up_attrs()
+        if isinstance(x, GatheredRows):
+            pair = None
+            if self._pairs_gate_up():
+                def operand(name):
+                    tensor = getattr(self, name, None)
+                    return None if tensor is None else tensor.to(out_dtype)
+
+                biases = [operand(f"{attr}_bias") if with_bias else None for attr in (gate_attr, up_attr)]
+                pair = x.grouped_mm_pair(operand(gate_attr), biases[0], operand(up_attr), biases[1], offs=offs,
+                                         eids=eids)
+            if pair is not None:
+                return pair
+            x = x.materialize()
+        return proj(x, gate_attr), proj(x, up_attr)
 
     @property
     def has_expert_lora(self) -> bool:

@@ -200,6 +200,16 @@ int hmoe_grouped_gemm_fwd_addto(const void* a, int64_t lda, const void* b, const
                                 int num_groups, int64_t k, int64_t n, int dtype, const void* addend,
                                 int64_t ld_addend, float scale, void* out, int64_t ldo, void* stream);
 
+/* The input gradient added to an existing [total_rows, k] tensor: grad_a = addend + grad_out[s:e] @ b[g]^T, element by
+ * element with the roundings of the two tensor operations (the product to dtype, the sum to dtype).  Where two
+ * projections read the same rows (gate and up stored apart, halo/distributed/expert_parallel/families/gpt_oss.py:
+ * 139-152), autograd adds their two input gradients (the sum the engine forms at the rows' node); here the second
+ * projection's input gradient joins the first's in its epilogue, so neither the second product nor the pass that adds
+ * the two exists.  grad_a may be addend itself. */
+int hmoe_grouped_gemm_dgrad_addto(const void* grad_out, int64_t ldg, const void* b, const int32_t* offs,
+                                  int64_t total_rows, int num_groups, int64_t k, int64_t n, int dtype,
+                                  const void* addend, int64_t ld_addend, void* grad_a, int64_t lda, void* stream);
+
 /* The same two GEMMs with the rows of A gathered: logical row r of A is a[row_index[r]], a holding a_rows rows; an
  * index outside [0, a_rows) reads as a row of zeros.  This folds MoEGatherPermute.forward
  * (halo/kernels/moe_permute.py:133-136, tokens.index_select(0, sorted_token_idx)) into the first expert GEMM and its
@@ -211,6 +221,13 @@ int hmoe_grouped_gemm_fwd_gather(const void* a, int64_t lda, int64_t a_rows, con
 int hmoe_grouped_gemm_wgrad_gather(const void* a, int64_t lda, int64_t a_rows, const int64_t* row_index,
                                    const void* grad_out, int64_t ldg, const int32_t* offs, int64_t total_rows,
                                    int num_groups, int64_t k, int64_t n, int dtype, void* grad_b, void* stream);
+/* hmoe_grouped_gemm_fwd_gather with the expert's bias row added in the epilogue as hmoe_grouped_gemm_fwd_bias adds it
+ * (halo/distributed/expert_parallel/families/gpt_oss.py:154-160 over the rows of halo/kernels/moe_permute.py:133-136):
+ * a biased projection that fetches its rows through the sort's index.  bf16 only. */
+int hmoe_grouped_gemm_fwd_gather_bias(const void* a, int64_t lda, int64_t a_rows, const int64_t* row_index,
+                                      const void* b, const void* bias, const int32_t* offs, int64_t total_rows,
+                                      int num_groups, int64_t k, int64_t n, int dtype, void* out, int64_t ldo,
+                                      void* stream);
 
 /* The two gradients of a product whose OUTPUT rows were then summed per token (the plain combine behind a down
  * projection on weighted rows): logical row r of the output gradient is grad_out[row_index[r]], grad_out holding

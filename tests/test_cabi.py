@@ -101,6 +101,17 @@ def test_bad_arguments_come_back_as_status_codes_before_any_launch():
     assert addto(fake, 64, fake, fake, 8, 4, 64, 64, bf16, fake, 68, 2.0, fake, 64, None) == unsupported  # 136-byte rows
     assert addto(fake, 64, fake, fake, 8, 4, 64, 64, bf16, fake + 2, 64, 2.0, fake, 64, None) == unsupported
     assert lib.hmoe_grouped_gemm_fwd_gather(fake, 64, -3, fake, fake, fake, 8, 4, 64, 64, bf16, fake, 64, None) == invalid
+    gather_bias = lib.hmoe_grouped_gemm_fwd_gather_bias
+    assert gather_bias(fake, 64, 8, fake, fake, None, fake, 8, 4, 64, 64, bf16, fake, 64, None) == invalid  # no bias
+    assert gather_bias(fake, 64, 8, fake, fake, fake, fake, 8, 4, 64, 64, f32, fake, 64, None) == unsupported
+    assert gather_bias(fake, 64, 8, fake, fake, fake + 4, fake, 8, 4, 64, 64, bf16, fake, 64, None) == unsupported
+    assert gather_bias(None, 64, 8, None, None, None, None, 0, 1, 64, 64, bf16, None, 64, None) == 0
+    dgrad_addto = lib.hmoe_grouped_gemm_dgrad_addto
+    assert dgrad_addto(fake, 64, fake, fake, 8, 4, 64, 64, bf16, None, 64, fake, 64, None) == invalid  # no addend
+    assert dgrad_addto(fake, 64, fake, fake, 8, 4, 64, 64, bf16, fake, 32, fake, 64, None) == invalid  # addend rows overlap
+    assert dgrad_addto(fake, 64, fake, fake, 8, 4, 64, 64, bf16, fake, 68, fake, 64, None) == unsupported
+    assert dgrad_addto(fake, 64, fake, fake, 8, 4, 64, 64, bf16, fake + 2, 64, fake, 64, None) == unsupported
+    assert dgrad_addto(None, 64, None, None, 0, 1, 64, 64, bf16, None, 64, None, 64, None) == 0
 
     # what must stay below 2 GiB: an array gathered from by row index, one expert's weight, 512 rows of the widest
     # operand -- and nothing else (activations and outputs of any size are addressed tile by tile)

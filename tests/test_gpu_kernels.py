@@ -990,3 +990,79 @@ def test_grouped_mm_added_to_a_tensor_equals_the_tensor_operations(device, dtype
         results.append((out.detach(), ad.grad, bd.grad, cd.grad))
     for name, x, y in zip(("out", "grad_a", "grad_b", "grad_addend"), *results):
         assert torch.equal(x, y), name
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float32), ids=("bf16", "fp32"))
+@pytest.mark.parametrize(("counts", "k", "n"), (((255, 256, 257, 0, 513, 31), 200, 264), ((64,) * 16, 1536, 512),
+                                                 ((0, 0, 700, 1, 0), 2880, 2880), ((5,), 8, 64)))
+def test_input_gradient_added_into_a_tensor_equals_the_two_operations(device, dtype, counts, k, n):
+    """``hmoe_grouped_gemm_dgrad_addto`` returns the bits of ``addend + grad @ W^T``: the product rounded, then the
+    sum, as the tensor addition of two input gradients rounds.  A row-strided addend, and the output written over the
+    addend itself."""
+    from halo_amd import _lib
+    from halo_amd.kernels.grouped_mm import grouped_mm_grads
+
+    g = torch.Generator().manual_seed(21)
+    rows, groups = sum(counts), len(counts)
+    grad = torch.randn(rows, n, generator=g).to(dtype).to(device)
+    w = (torch.randn(groups, k, n, generator=g) * 0.05).to(dtype).to(device)
+    padded = torch.randn(rows, k + 16, generator=g).to(dtype).to(device)
+    addend = padded[:, :k]
+    offs = _offsets(counts, device)
+    shape_only = grad.new_empty((1, k)).expand(rows, k)
+    product, _ = grouped_mm_grads(shape_only, w, grad, offs, True, False)
+    want = addend + product
+
+    def run(base, out):
+        with _lib.on_device(device):
+            _lib.call("hmoe_grouped_gemm_dgrad_addto", _lib.ptr(grad), grad.stride(0), _lib.ptr(w), _lib.ptr(offs), rows,
+                      groups, k, n, _lib.dtype_id(dtype), _lib.ptr(base), base.stride(0), _lib.ptr(out), out.stride(0),
+                      _lib.stream_ptr(device))
+        return out
+
+    assert torch.equal(run(addend, torch.empty(rows, k, dtype=dtype, device=device)), want)
+    in_place = addend.contiguous()
+    assert torch.equal(run(in_place, in_place), want)
+
+
+@pytest.mark.parametrize("biased", (True, False), ids=("biased", "plain"))
+@pytest.mark.parametrize(("counts", "k", "n"), (((255, 256, 257, 0, 513, 31), 200, 264), ((64,) * 16, 512, 768),
+                                                 (tuple((37 * i * i + 11 * i) % 91 for i in range(150)), 320, 256)))
+def test_two_projections_of_gathered_rows_as_one_node_equal_the_separate_operations(device, counts, k, n, biased):
+    """``gather_grouped_mm_pair`` = the permute followed by two (biased) grouped products: both outputs, the token
+    gradient (the two input gradients added, then scattered back), both weight gradients and both bias gradients are
+    bit-equal to the operations the reference runs one by one."""
+    from halo_amd.kernels.grouped_mm import gather_grouped_mm_pair, grouped_mm, pair_fusable
+    from halo_amd.kernels.moe_permute import MoEExpertBiasGather, MoEGatherPermute, build_inv_map
+
+    g = torch.Generator().manual_seed(23)
+    rows, groups, n_tokens = sum(counts), len(counts), max(8, sum(counts) // 3)
+    row_index = torch.randint(0, n_tokens, (rows,), generator=g).to(device)
+    width = int(torch.bincount(row_index.cpu(), minlength=n_tokens).max())
+    inv_map = build_inv_map(row_index, n_tokens, width)
+    tokens = torch.randn(n_tokens, k, generator=g).bfloat16().to(device)
+    w1, w2 = ((torch.randn(groups, k, n, generator=g) * 0.05).bfloat16().to(device) for _ in range(2))
+    b1, b2 = (torch.randn(groups, n, generator=g).bfloat16().to(device) if biased else None for _ in range(2))
+    d1, d2 = (torch.randn(rows, n, generator=g).bfloat16().to(device) for _ in range(2))
+    offs = _offsets(counts, device)
+    eids = torch.repeat_interleave(torch.arange(groups), torch.tensor(counts)).to(device)
+    assert pair_fusable(tokens, w1, b1, w2, b2)
+    results = []
+    for fused in (False, True):
+        leaves = [t.clone().requires_grad_(True) for t in (tokens, w1, w2)]
+        biases = [b.clone().requires_grad_(True) for b in (b1, b2)] if biased else [None, None]
+        t, wa, wb = leaves
+        if fused:
+            out1, out2 = gather_grouped_mm_pair(t, row_index, inv_map, wa, biases[0], wb, biases[1], offs=offs, eids=eids)
+        else:
+            permuted = MoEGatherPermute.apply(t, row_index, inv_map)
+            out1, out2 = grouped_mm(permuted, wa, offs=offs), grouped_mm(permuted, wb, offs=offs)
+            if biased:
+                out1 = out1 + MoEExpertBiasGather.apply(biases[0], eids)
+                out2 = out2 + MoEExpertBiasGather.apply(biases[1], eids)
+        torch.autograd.backward([out1, out2], [d1, d2])
+        results.append([out1.detach(), out2.detach(), *(leaf.grad for leaf in leaves),
+                        *(b.grad for b in biases if b is not None)])
+    names = ("out1", "out2", "grad_tokens", "grad_w1", "grad_w2", "grad_b1", "grad_b2")
+    for name, a, b in zip(names, *results):
+        assert torch.equal(a, b), name

@@ -124,12 +124,20 @@ def test_layer_is_bit_reproducible(device):
     assert all(torch.equal(a, b) for a, b in zip(*runs))
 
 
-@pytest.mark.parametrize("cfg", (CONFIG1, CONFIG2_SMALL), ids=lambda c: c.name)
-def test_permute_folded_into_the_first_projection_changes_no_bit(device, cfg):
+@pytest.mark.parametrize("cfg", (CONFIG1, CONFIG2_SMALL, CONFIG2_SMALL._replace(name="cfg2_small_apart", fused=False),
+                                 CONFIG4_SMALL), ids=lambda c: c.name)
+def test_permute_folded_into_the_first_projection_changes_no_bit(device, cfg, monkeypatch):
     """By default the first expert projection fetches its rows through the sort's index instead of reading a permuted
     copy; the output and every gradient must equal the permute-then-GEMM path's bit for bit (the products and their
-    summation order are the same, only the addressing differs).  The fp32 configuration does not qualify for the gathering
-    kernels and takes the copy either way."""
+    summation order are the same, only the addressing differs).  Where gate and up are stored apart (Qwen3; gpt-oss,
+    with biases) the two projections run as one node that also sums their two input gradients in the second one's
+    epilogue, where autograd adds them as tensors.  The fp32 configuration does not qualify for the gathering kernels
+    and takes the copy either way."""
+    from halo_amd.kernels import grouped_mm as gmm
+
+    pairs = []
+    real_pair = gmm.gather_grouped_mm_pair
+    monkeypatch.setattr(gmm, "gather_grouped_mm_pair", lambda *a, **k: pairs.append(1) or real_pair(*a, **k))
     inputs = make_layer_inputs(cfg)
     runs = []
     for fuse in (True, False):
@@ -143,6 +151,7 @@ def test_permute_folded_into_the_first_projection_changes_no_bit(device, cfg):
         runs.append([out.detach(), x.grad] + [p.grad for _, p in sorted(layer.named_parameters())])
     assert len(runs[0]) >= 4 and all(g is not None for g in runs[0])
     assert all(torch.equal(a, b) for a, b in zip(*runs))
+    assert len(pairs) == (0 if cfg.fused or cfg.dtype != torch.bfloat16 else 1)
 
 
 def test_gate_weight_folded_into_the_glu_stays_inside_the_tolerance(device):
