@@ -12,11 +12,19 @@ namespace hmoe {
 // 1.75 and 3.5; the even code is the even significand, so it is IEEE round-to-nearest-even at e2m1's precision): the
 // instruction gives the reference's code for every multiple of 1/64 in [-7, 7], for infinities and for a positive NaN
 // (code 7, where bucketize puts it).  The sign bit is set for a value below zero and not for -0.0, as `scaled < 0` has
-// it: adding +0.0 turns -0.0 into +0.0 and changes nothing else.
+// it: adding +0.0 turns -0.0 into +0.0 and changes nothing else.  The addition must stay an operation of its own
+// (contraction off): fused into the multiplication that scaled the value it would see the exact product, and a negative
+// value that the fp32 product rounds to -0.0 (a block holding an inf, or one spanning more than 150 binades) would
+// keep its sign where the reference's two operations drop it.
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float without_negative_zero(float x) {
+#pragma clang fp contract(off)
+  return x + 0.0f;
+}
 template <int kByte>
 __device__ __forceinline__ uint32_t e2m1_pack2(uint32_t word, float lo, float hi) {
-  return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, lo + 0.0f, hi + 0.0f, 1.0f, kByte);
+  return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, without_negative_zero(lo), without_negative_zero(hi), 1.0f,
+                                                  kByte);
 }
 __device__ __forceinline__ uint32_t e2m1_pack8(const float* v) {
   uint32_t word = 0u;

@@ -120,6 +120,7 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
   const T* extra = addend ? addend + row * addend_stride : nullptr;
   const float extra_scale = addend_scale ? Elem<T>::load(addend_scale + row) : 1.f;
   auto finish = [&](Pack<T, W>& acc, const Pack<T, W>& term) {
+#pragma clang fp contract(off)  // fp32: the multiple and the sum round separately, as the tensor operations do
     if (extra) {
 #pragma unroll
       for (int i = 0; i < W; ++i) {

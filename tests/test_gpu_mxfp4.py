@@ -68,6 +68,36 @@ def test_row_quantiser_dequantiser_and_round_trip_equal_the_oracle_bit_for_bit(d
     _equal_with_nan(fused, want)
 
 
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float32), ids=("bf16", "fp32"))
+def test_negative_values_that_the_scaling_rounds_to_zero_take_the_code_of_zero(device, dtype):
+    """A negative value whose scaled fp32 product underflows (beside an inf, or more than 150 binades below its block's
+    largest magnitude) is -0.0 by then, which the reference's ``scaled < 0`` does not count as negative: code 0, not 8
+    (``quantization.py:166-177, 191-198``).  Rows and weights, against the oracle's codes."""
+    from halo_amd.kernels.lowp.quantization import quantize_mxfp4
+    from oracle import mxfp4 as oracle
+
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(6, 64, generator=g)
+    x[0, :32] = -torch.rand(32, generator=g) * 1e-11
+    x[0, 5] = float("inf")                                   # scale 254: everything finite underflows
+    x[1, :32] = -torch.rand(32, generator=g) * 1e-20
+    x[1, 9] = 1e30                                           # 166 binades above the rest
+    x[2, 32:] = torch.rand(32, generator=g) * 1e-20 * torch.where(torch.rand(32, generator=g) < 0.5, -1.0, 1.0)
+    x[2, 40] = -3e29
+    x[3, :32] = -torch.rand(32, generator=g) * 2.0 ** -20    # a span that does not underflow: the sign stays
+    x[3, 0] = 2.0 ** 100
+    x = x.to(dtype)
+    want_data, want_scales = oracle.quantize_mxfp4(x.float().numpy())
+    codes = oracle.unpack_codes(want_data)
+    assert (codes[0, :32] == 0).sum() == 31 and (codes[1, :32] == 0).sum() == 31 and (codes[3, 1:32] == 8).all()
+    q = quantize_mxfp4(x.to(device))
+    assert np.array_equal(q.scales.cpu().numpy(), want_scales) and np.array_equal(q.data.cpu().numpy(), want_data)
+    w = x.t().contiguous().view(1, 64, 6).repeat(2, 1, 1)    # the same blocks down the columns of a weight
+    want_data, want_scales = oracle.quantize_mxfp4(w.float().numpy(), axis=1)
+    q = quantize_mxfp4(w.to(device), axis=1)
+    assert np.array_equal(q.scales.cpu().numpy(), want_scales) and np.array_equal(q.data.cpu().numpy(), want_data)
+
+
 def test_row_round_trip_fetches_rows_through_an_index(device):
     from halo_amd.kernels.lowp.quantization import mxfp4_rows
 
