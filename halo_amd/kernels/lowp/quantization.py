@@ -2,7 +2,7 @@
 scale per 32 values along the contraction axis, or e2m1 elements with an e4m3 scale per 16 values and one fp32 scale
 per tensor (NVFP4); the straight-through fake-quant, and the per-step weight cache.
 
-Mirrors ``halo/kernels/lowp/quantization.py`` of the reference for its ``mxfp8`` and ``mxfp4`` formats:
+Mirrors ``halo/kernels/lowp/quantization.py`` of the reference for its three formats:
 ``BlockScaledTensor`` (:104-117), ``quantize_mxfp8`` (:236-245), ``quantize_mxfp4`` (:248-266), ``dequantize``
 (:277-297), ``fake_quant`` (:350-365), ``WeightVersionCache`` / ``cached_fake_quant`` (:368-422).  The MXFP8 kernels are
 ``csrc/mxfp8.hip``; they write the operands in the layout the GEMM kernel loads (:class:`MxRows`, :class:`MxWeight`),
