@@ -43,30 +43,33 @@ _SHARED_OVERLAP_ENABLED = os.environ.get("HALO_EP_SHARED_OVERLAP", "").strip().l
 _shared_overlap_streams: dict[int, torch.cuda.Stream] = {}
 
 
-class _RouterProjection(torch.autograd.Function):
-    """``F.linear(x, weight)`` for the router's logits ``[T, E]`` with the weight gradient on the grouped wgrad kernel.
+class _SlicedWgradLinear(torch.autograd.Function):
+    """``F.linear(x, weight)`` for a dense projection of all tokens (the router's logits ``[T, E]``, the shared expert's
+    three projections) with the weight gradient on the grouped wgrad kernel.
 
     Forward and the input gradient are plain dense products on the library GEMM, as in the reference.  The weight
-    gradient ``dlogits^T @ x`` is an ``[E, H]`` output contracted over all T tokens: a handful of output tiles, which
-    leaves a dense GEMM (and one grouped-GEMM group) on a few CUs.  The tokens are cut into ``_SPLITS`` slices that
-    the wgrad kernel takes as groups, one partial ``[E, H]`` each (rounded to the operands' dtype), all CUs busy; the
-    partials are summed in fp32 in a fixed order and rounded once, so the result stays deterministic.  Operands the
-    kernel does not take (rows that are not 16-byte multiples, unaligned views) use the dense product."""
+    gradient ``dout^T @ x`` is an ``[out, in]`` output contracted over all T tokens: a handful of output tiles, which
+    leaves a dense GEMM (and one grouped-GEMM group) on a few CUs (the library takes 57 us for the shared expert's
+    ``[512, 2048]`` over 8192 tokens, 70 us for the router's ``[128, 2048]``).  The tokens are cut into slices that the
+    wgrad kernel takes as groups, one partial ``[out, in]`` each (rounded to the operands' dtype), as many as bring
+    the launch to about one tile per CU (32 and 22 us for those two); the partials are summed in fp32 in a fixed order
+    and rounded once, so the result stays deterministic.  Operands the kernel does not take (rows that are not
+    16-byte multiples, unaligned views, few tokens) use the dense product."""
 
-    _SPLITS = 32
+    _SPLITS = 32  # at most
     _MIN_TOKENS = 2048
-    _slice_ends: ClassVar[dict] = {}  # (device, tokens) -> the slices' row ends; a handful of sequence lengths at most
+    _slice_ends: ClassVar[dict] = {}  # (device, tokens, splits) -> the slices' row ends; a handful of shapes at most
     _SLICE_ENDS_KEPT = 16
 
     @staticmethod
-    def _slice_ends_for(device: torch.device, tokens: int) -> torch.Tensor:
-        cache, splits = _RouterProjection._slice_ends, _RouterProjection._SPLITS
-        offs = cache.get((device, tokens))
+    def _slice_ends_for(device: torch.device, tokens: int, splits: int) -> torch.Tensor:
+        cache = _SlicedWgradLinear._slice_ends
+        offs = cache.get((device, tokens, splits))
         if offs is None:
-            if len(cache) >= _RouterProjection._SLICE_ENDS_KEPT:  # varying sequence lengths: start over, never grow
+            if len(cache) >= _SlicedWgradLinear._SLICE_ENDS_KEPT:  # varying sequence lengths: start over, never grow
                 cache.clear()
             offs = torch.arange(1, splits + 1, device=device, dtype=torch.int32) * (tokens // splits)
-            cache[(device, tokens)] = offs
+            cache[(device, tokens, splits)] = offs
         return offs
 
     @staticmethod
@@ -75,40 +78,54 @@ class _RouterProjection(torch.autograd.Function):
         return torch.nn.functional.linear(x, weight)
 
     @staticmethod
-    def _sliced_wgrad_usable(grad_logits: torch.Tensor, x: torch.Tensor) -> bool:
-        tokens, splits = x.shape[0], _RouterProjection._SPLITS
-        return (x.dtype == torch.bfloat16 and grad_logits.dtype == torch.bfloat16
-                and tokens >= _RouterProjection._MIN_TOKENS and tokens % splits == 0
-                # what the grouped kernels ask of bf16 operands: 16-byte rows, 16-byte aligned
-                and grad_logits.shape[1] % 8 == 0 and x.shape[1] % 8 == 0
-                and all(t.stride(-1) == 1 and t.stride(0) % 8 == 0 and t.data_ptr() % 16 == 0
-                        for t in (grad_logits, x)))
+    def _splits_for(grad_out: torch.Tensor, x: torch.Tensor) -> int:
+        """How many token slices the weight gradient is cut into: the power of two that brings the launch nearest to
+        256 output tiles of 256 x 256 without passing it, at most 32, slices of equal whole numbers of tokens."""
+        tiles = -(-grad_out.shape[1] // 256) * -(-x.shape[1] // 256)
+        splits = _SlicedWgradLinear._SPLITS
+        while splits > 1 and (splits * tiles > 256 or x.shape[0] % splits):
+            splits //= 2
+        return splits
 
     @staticmethod
-    def backward(ctx, grad_logits):
+    def _sliced_wgrad_usable(grad_out: torch.Tensor, x: torch.Tensor) -> bool:
+        return (x.dtype == torch.bfloat16 and grad_out.dtype == torch.bfloat16
+                and x.shape[0] >= _SlicedWgradLinear._MIN_TOKENS and _SlicedWgradLinear._splits_for(grad_out, x) >= 4
+                # what the grouped kernels ask of bf16 operands: 16-byte rows, 16-byte aligned
+                and grad_out.shape[1] % 8 == 0 and x.shape[1] % 8 == 0
+                and all(t.stride(-1) == 1 and t.stride(0) % 8 == 0 and t.data_ptr() % 16 == 0
+                        for t in (grad_out, x)))
+
+    @staticmethod
+    def backward(ctx, grad_out):
         x, weight = ctx.saved_tensors
         grad_x = grad_weight = None
         if ctx.needs_input_grad[0]:
-            grad_x = grad_logits @ weight
+            grad_x = grad_out @ weight
         if ctx.needs_input_grad[1]:
-            if _RouterProjection._sliced_wgrad_usable(grad_logits, x):
-                splits = _RouterProjection._SPLITS
-                offs = _RouterProjection._slice_ends_for(x.device, x.shape[0])
-                partial = grouped_wgrad(grad_logits, x, offs, splits)
+            if _SlicedWgradLinear._sliced_wgrad_usable(grad_out, x):
+                splits = _SlicedWgradLinear._splits_for(grad_out, x)
+                offs = _SlicedWgradLinear._slice_ends_for(x.device, x.shape[0], splits)
+                partial = grouped_wgrad(grad_out, x, offs, splits)
                 grad_weight = partial.sum(dim=0)  # the reduction accumulates in fp32 and rounds once
             else:
-                grad_weight = grad_logits.t() @ x
+                grad_weight = grad_out.t() @ x
         return grad_x, grad_weight
+
+
+_RouterProjection = _SlicedWgradLinear  # the router's logits were its first use
 
 
 def dense_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``x @ weight^T`` for an ``F.linear``-convention ``weight [out, in]`` (the shared expert's projections, which are
-    ``nn.Linear`` modules in the reference: ``families/qwen3_5.py:41-42``); differentiable in both operands.  A plain
-    dense product, so the library's: the grouped kernel with one group has 64 output tiles for 256 compute units at
-    8192 tokens x 512 columns and 16 for the weight gradient, whose contraction over the tokens it cannot split
-    (147 us against the library's 20 for that one product)."""
+    ``nn.Linear`` modules in the reference: ``families/qwen3_5.py:41-42``); differentiable in both operands.  Forward
+    and input gradient are the library's dense products (the grouped kernel with one group has 64 output tiles for 256
+    compute units at 8192 tokens x 512 columns); the weight gradient is cut into token slices for the grouped kernel
+    (:class:`_SlicedWgradLinear`)."""
     if not x.is_cuda:
         raise RuntimeError("halo_amd ops run on the GPU: got a CPU tensor")
+    if x.dim() == 2 and weight.dim() == 2 and x.dtype == weight.dtype == torch.bfloat16:
+        return _SlicedWgradLinear.apply(x, weight)
     return torch.nn.functional.linear(x, weight)
 
 
@@ -571,7 +588,7 @@ class EPMoELayerBase(ExpertLoadMixin, nn.Module, ABC):
         router = getattr(self, self._ROUTER_ATTR)
         x = self._router_input(flat)
         # A plain dense projection with a tiny output ([T, E]): the library GEMM, as in the reference (F.linear).
-        logits = _RouterProjection.apply(x, router.weight.to(x.dtype))
+        logits = _SlicedWgradLinear.apply(x, router.weight.to(x.dtype))
         bias = getattr(router, "bias", None)
         return logits if bias is None else logits + bias.to(logits.dtype)
 

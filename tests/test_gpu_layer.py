@@ -412,6 +412,31 @@ def test_router_projection_with_an_expert_count_the_grouped_kernel_does_not_take
     _check("dx", xd.grad, dlogits.double() @ w.double(), 2e-2)
 
 
+@pytest.mark.parametrize(("tokens", "width", "hidden"), ((8192, 512, 2048), (4096, 2048, 512), (2048, 264, 1000)))
+def test_dense_projection_weight_gradient_in_token_slices(device, tokens, width, hidden):
+    """``dense_mm`` (the shared expert's projections): forward and input gradient are the library's, the weight
+    gradient is summed from token slices on the grouped kernel (16, 16 and 32 of them here).  Against the fp64
+    products over the same bf16 inputs (BASELINE tolerance) and for run-to-run bit equality."""
+    from halo_amd.moe_layer.layer import _SlicedWgradLinear, dense_mm
+
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(tokens, hidden, generator=g).bfloat16()
+    w = (torch.randn(width, hidden, generator=g) * hidden ** -0.5).bfloat16()
+    dout = torch.randn(tokens, width, generator=g).bfloat16()
+    assert _SlicedWgradLinear._sliced_wgrad_usable(dout.to(device), x.to(device))
+    results = []
+    for _ in range(2):
+        xd, wd = x.to(device).requires_grad_(True), w.to(device).requires_grad_(True)
+        out = dense_mm(xd, wd)
+        out.backward(dout.to(device))
+        results.append((out.detach(), xd.grad, wd.grad))
+    out, dx, dw = results[0]
+    assert torch.equal(out, torch.nn.functional.linear(x.to(device), w.to(device)))
+    _check("dx", dx, dout.double() @ w.double(), 2e-2)
+    _check("dw", dw, dout.double().t() @ x.double(), 2e-2)
+    assert all(torch.equal(a, b) for a, b in zip(results[0], results[1]))
+
+
 class _SharedMlp(torch.nn.Module):
     def __init__(self, hidden, width, dtype, generator):
         super().__init__()
