@@ -33,6 +33,7 @@ class _FusedTopKGate(torch.autograd.Function):
         ctx.save_for_backward(logits, indices)
         ctx.args = (top_k, mode, int(normalize), float(eps))
         ctx.mark_non_differentiable(indices)
+        ctx.set_materialize_grads(False)  # no zero tensor made for the indices' gradient on the way back
         return indices, weights
 
     @staticmethod
