@@ -19,6 +19,36 @@ GROUPED_MM_STRIDE_ALIGNMENT_BYTES = 16
 GROUPED_MM_SMALL_TILE_DIM = 128
 
 
+_GEMM_TILES = {"auto": 0, "mono": 1, "duo": 2, "small": 3}
+
+
+class gemm_tile:
+    """Forces one of the bf16 grouped GEMM's three tile configurations for every product of the process, as a context
+    manager or by ``gemm_tile.set(name)``: ``"mono"`` is the 256 x 256 tile on one workgroup per compute unit, ``"duo"``
+    the 128 x 256 tile on two, ``"small"`` the 128 x 128 tile on three, ``"auto"`` (the default) the largest of which
+    the product has a tile per compute unit.  All give the same bits; a
+    tuning and test switch with no counterpart in the reference (``HALO_GEMM_TILE`` sets the initial value)."""
+
+    def __init__(self, name: str):
+        self.name = name
+        self.before = None
+
+    @staticmethod
+    def set(name: str) -> str:
+        if name not in _GEMM_TILES:
+            raise ValueError(f"unknown tile configuration {name!r}; expected one of {sorted(_GEMM_TILES)}")
+        before = _lib.load().hmoe_set_gemm_tile(_GEMM_TILES[name])
+        return next(k for k, v in _GEMM_TILES.items() if v == before)
+
+    def __enter__(self):
+        self.before = gemm_tile.set(self.name)
+        return self
+
+    def __exit__(self, *exc):
+        gemm_tile.set(self.before)
+        return False
+
+
 def _rows(t: torch.Tensor) -> torch.Tensor:
     """A 2-D operand with unit inner stride (row stride free)."""
     return t if t.stride(-1) == 1 and t.stride(0) >= t.shape[1] else t.contiguous()
@@ -62,6 +92,9 @@ def _forward(mat_a: torch.Tensor, mat_b: torch.Tensor, offs: torch.Tensor | None
             _lib.call("hmoe_grouped_gemm_fwd", _lib.ptr(mat_a), mat_a.stride(0), _lib.ptr(w), _lib.ptr(offs32),
                       rows, groups, k, n, dtype, _lib.ptr(out), out.stride(0), _lib.stream_ptr(device))
     return out
+
+
+grouped_mm_forward = _forward  # the forward product alone (no autograd node), for callers that build their own
 
 
 def grouped_wgrad(mat_a: torch.Tensor, grad_output: torch.Tensor, offs: torch.Tensor | None,

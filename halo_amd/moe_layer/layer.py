@@ -24,7 +24,7 @@ import torch.nn as nn
 from halo_amd.kernels.expert_gemm import BlockFp8Weight, expert_gemm, fp8_mfma_usable
 from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled, resolve_fused_glu_mul
 from halo_amd.kernels.grouped_mm import (GatheredRows, addto_fusable, grouped_mm_addto, grouped_mm_combine,
-                                         grouped_wgrad)
+                                         grouped_mm_forward, grouped_wgrad)
 from halo_amd.kernels.moe_permute import (MoEGatherPermute, MoEWeightedUnpermute, MoEWeightedUnpermuteAdd,
                                           warm_permute_kernels)
 from halo_amd.kernels.moe_route_sort import sort_routing_by_expert, warm_route_sort_kernels
@@ -43,18 +43,20 @@ _SHARED_OVERLAP_ENABLED = os.environ.get("HALO_EP_SHARED_OVERLAP", "").strip().l
 _shared_overlap_streams: dict[int, torch.cuda.Stream] = {}
 
 
-class _SlicedWgradLinear(torch.autograd.Function):
+class _DenseLinear(torch.autograd.Function):
     """``F.linear(x, weight)`` for a dense projection of all tokens (the router's logits ``[T, E]``, the shared expert's
-    three projections) with the weight gradient on the grouped wgrad kernel.
+    three projections, ``nn.Linear`` modules in the reference: ``families/qwen3_5.py:41-42``) on this build's grouped
+    GEMM kernels with one group.
 
-    Forward and the input gradient are plain dense products on the library GEMM, as in the reference.  The weight
-    gradient ``dout^T @ x`` is an ``[out, in]`` output contracted over all T tokens: a handful of output tiles, which
-    leaves a dense GEMM (and one grouped-GEMM group) on a few CUs (the library takes 57 us for the shared expert's
-    ``[512, 2048]`` over 8192 tokens, 70 us for the router's ``[128, 2048]``).  The tokens are cut into slices that the
-    wgrad kernel takes as groups, one partial ``[out, in]`` each (rounded to the operands' dtype), as many as bring
-    the launch to about one tile per CU (32 and 22 us for those two); the partials are summed in fp32 in a fixed order
-    and rounded once, so the result stays deterministic.  Operands the kernel does not take (rows that are not
-    16-byte multiples, unaligned views, few tokens) use the dense product."""
+    Forward ``x @ weight^T`` is the input-gradient kernel's form (both operands contraction-contiguous), the input
+    gradient ``grad_out @ weight`` the forward kernel's; each launch takes the largest of the kernels' three tile
+    configurations that still gives every compute unit a tile (``csrc/grouped_gemm.hip``: 8192 tokens x 512 columns
+    are 64 tiles of 256 x 256 but 256 of 128 x 128).  The weight gradient ``grad_out^T @ x`` is an ``[out, in]`` output
+    contracted over all T tokens, a handful of output tiles however small the tile: the tokens are cut into slices
+    that the weight-gradient kernel takes as groups, one partial ``[out, in]`` each (rounded to the operands' dtype),
+    as many as bring the launch to about one tile per compute unit; the partials are summed in fp32 in a fixed order
+    and rounded once, so the result stays deterministic.  Operands the kernels do not take (fp32 under
+    ``fp32_router``, rows that are not 16-byte multiples, unaligned views) use the library's dense product."""
 
     _SPLITS = 32  # at most
     _MIN_TOKENS = 2048
@@ -63,18 +65,26 @@ class _SlicedWgradLinear(torch.autograd.Function):
 
     @staticmethod
     def _slice_ends_for(device: torch.device, tokens: int, splits: int) -> torch.Tensor:
-        cache = _SlicedWgradLinear._slice_ends
+        cache = _DenseLinear._slice_ends
         offs = cache.get((device, tokens, splits))
         if offs is None:
-            if len(cache) >= _SlicedWgradLinear._SLICE_ENDS_KEPT:  # varying sequence lengths: start over, never grow
+            if len(cache) >= _DenseLinear._SLICE_ENDS_KEPT:  # varying sequence lengths: start over, never grow
                 cache.clear()
             offs = torch.arange(1, splits + 1, device=device, dtype=torch.int32) * (tokens // splits)
             cache[(device, tokens, splits)] = offs
         return offs
 
     @staticmethod
+    def _kernel_usable(*operands: torch.Tensor) -> bool:
+        """What the grouped kernels ask of their operands: bf16, 16-byte rows, 16-byte aligned."""
+        return all(t.dtype == torch.bfloat16 and t.dim() == 2 and t.shape[0] > 0 and t.shape[1] % 8 == 0
+                   and t.stride(-1) == 1 and t.stride(0) % 8 == 0 and t.data_ptr() % 16 == 0 for t in operands)
+
+    @staticmethod
     def forward(ctx, x, weight):
         ctx.save_for_backward(x, weight)
+        if _DenseLinear._kernel_usable(x, weight) and weight.is_contiguous() and weight.shape[0] % 8 == 0:
+            return grouped_mm_forward(x, weight.t().unsqueeze(0), None)  # a transposed view: the kernel reads [out, in]
         return torch.nn.functional.linear(x, weight)
 
     @staticmethod
@@ -82,30 +92,29 @@ class _SlicedWgradLinear(torch.autograd.Function):
         """How many token slices the weight gradient is cut into: the power of two that brings the launch nearest to
         256 output tiles of 256 x 256 without passing it, at most 32, slices of equal whole numbers of tokens."""
         tiles = -(-grad_out.shape[1] // 256) * -(-x.shape[1] // 256)
-        splits = _SlicedWgradLinear._SPLITS
+        splits = _DenseLinear._SPLITS
         while splits > 1 and (splits * tiles > 256 or x.shape[0] % splits):
             splits //= 2
         return splits
 
     @staticmethod
     def _sliced_wgrad_usable(grad_out: torch.Tensor, x: torch.Tensor) -> bool:
-        return (x.dtype == torch.bfloat16 and grad_out.dtype == torch.bfloat16
-                and x.shape[0] >= _SlicedWgradLinear._MIN_TOKENS and _SlicedWgradLinear._splits_for(grad_out, x) >= 4
-                # what the grouped kernels ask of bf16 operands: 16-byte rows, 16-byte aligned
-                and grad_out.shape[1] % 8 == 0 and x.shape[1] % 8 == 0
-                and all(t.stride(-1) == 1 and t.stride(0) % 8 == 0 and t.data_ptr() % 16 == 0
-                        for t in (grad_out, x)))
+        return (_DenseLinear._kernel_usable(grad_out, x) and x.shape[0] >= _DenseLinear._MIN_TOKENS
+                and _DenseLinear._splits_for(grad_out, x) >= 4)
 
     @staticmethod
     def backward(ctx, grad_out):
         x, weight = ctx.saved_tensors
         grad_x = grad_weight = None
         if ctx.needs_input_grad[0]:
-            grad_x = grad_out @ weight
+            if _DenseLinear._kernel_usable(grad_out, weight) and weight.is_contiguous():
+                grad_x = grouped_mm_forward(grad_out, weight.unsqueeze(0), None)
+            else:
+                grad_x = grad_out @ weight
         if ctx.needs_input_grad[1]:
-            if _SlicedWgradLinear._sliced_wgrad_usable(grad_out, x):
-                splits = _SlicedWgradLinear._splits_for(grad_out, x)
-                offs = _SlicedWgradLinear._slice_ends_for(x.device, x.shape[0], splits)
+            if _DenseLinear._sliced_wgrad_usable(grad_out, x):
+                splits = _DenseLinear._splits_for(grad_out, x)
+                offs = _DenseLinear._slice_ends_for(x.device, x.shape[0], splits)
                 partial = grouped_wgrad(grad_out, x, offs, splits)
                 grad_weight = partial.sum(dim=0)  # the reduction accumulates in fp32 and rounds once
             else:
@@ -113,19 +122,13 @@ class _SlicedWgradLinear(torch.autograd.Function):
         return grad_x, grad_weight
 
 
-_RouterProjection = _SlicedWgradLinear  # the router's logits were its first use
-
-
 def dense_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """``x @ weight^T`` for an ``F.linear``-convention ``weight [out, in]`` (the shared expert's projections, which are
-    ``nn.Linear`` modules in the reference: ``families/qwen3_5.py:41-42``); differentiable in both operands.  Forward
-    and input gradient are the library's dense products (the grouped kernel with one group has 64 output tiles for 256
-    compute units at 8192 tokens x 512 columns); the weight gradient is cut into token slices for the grouped kernel
-    (:class:`_SlicedWgradLinear`)."""
+    """``x @ weight^T`` for an ``F.linear``-convention ``weight [out, in]`` (the shared expert's projections);
+    differentiable in both operands.  See :class:`_DenseLinear`."""
     if not x.is_cuda:
-        raise RuntimeError("halo_amd ops run on the GPU: got a CPU tensor")
+        return torch.nn.functional.linear(x, weight)
     if x.dim() == 2 and weight.dim() == 2 and x.dtype == weight.dtype == torch.bfloat16:
-        return _SlicedWgradLinear.apply(x, weight)
+        return _DenseLinear.apply(x, weight)
     return torch.nn.functional.linear(x, weight)
 
 
@@ -587,8 +590,7 @@ class EPMoELayerBase(ExpertLoadMixin, nn.Module, ABC):
         """The router's logits at the input dtype (fp32 under ``fp32_router``), fp32 accumulation, one rounding."""
         router = getattr(self, self._ROUTER_ATTR)
         x = self._router_input(flat)
-        # A plain dense projection with a tiny output ([T, E]): the library GEMM, as in the reference (F.linear).
-        logits = _SlicedWgradLinear.apply(x, router.weight.to(x.dtype))
+        logits = _DenseLinear.apply(x, router.weight.to(x.dtype))
         bias = getattr(router, "bias", None)
         return logits if bias is None else logits + bias.to(logits.dtype)
 

@@ -173,7 +173,17 @@ int hmoe_router_topk_bwd(const void* logits, int dtype, const int64_t* indices, 
  * offs i32[num_groups] are inclusive row ends (null: one group holding every row).  b is [num_groups, K, N]
  * contiguous.  fp32 accumulate, one rounding to dtype.  Rows past offs[num_groups-1] are not written by
  * fwd/dgrad.  An empty group's wgrad is exact zeros.  Deterministic (no split accumulation across workgroups).
+ * The bf16 products exist in three tile configurations with the same bits: a 256 x 256 output tile on one workgroup
+ * per compute unit, a 128 x 256 tile on two and a 128 x 128 tile on three; each call takes the largest of which the
+ * product has at least one tile per compute unit.
  */
+
+/* Forces a tile configuration for every later bf16 product of the process: 0 = by size (the default), 1 = 256 x 256,
+ * 2 = 128 x 256, 3 = 128 x 128; the environment variable HALO_GEMM_TILE=mono|duo|small sets the initial value.
+ * Returns the previous setting, or HMOE_INVALID_ARGUMENT.  A tuning and test switch with no counterpart in the
+ * reference; the one piece of process-wide state besides hmoe_route_sort_static's table, and harmless to race on
+ * (all tiles give the same bits). */
+int hmoe_set_gemm_tile(int tile);
 int hmoe_grouped_gemm_fwd(const void* a, int64_t lda, const void* b, const int32_t* offs, int64_t total_rows,
                           int num_groups, int64_t k, int64_t n, int dtype, void* out, int64_t ldo, void* stream);
 int hmoe_grouped_gemm_dgrad(const void* grad_out, int64_t ldg, const void* b, const int32_t* offs,

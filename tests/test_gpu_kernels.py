@@ -533,6 +533,15 @@ def _offsets(counts, device):
     return torch.cumsum(torch.tensor(counts), 0).to(torch.int32).to(device)
 
 
+@pytest.fixture(params=("mono", "duo", "small"))
+def tile(request, device):
+    """Runs a test once per tile configuration of the bf16 grouped GEMM (fp32 products ignore it)."""
+    from halo_amd.kernels.grouped_mm import gemm_tile
+
+    with gemm_tile(request.param):
+        yield request.param
+
+
 GEMM_CASES = (
     # counts per group, K, N
     ((7, 33, 0, 1, 64, 0), 128, 96),       # the reference's empty-group roster
@@ -548,7 +557,7 @@ GEMM_CASES = (
 
 @pytest.mark.parametrize(("counts", "k", "n"), GEMM_CASES)
 @pytest.mark.parametrize(("dtype", "tol"), ((torch.bfloat16, 2e-2), (torch.float32, 1e-5)), ids=("bf16", "fp32"))
-def test_grouped_mm_forward_and_gradients_match_oracle(device, counts, k, n, dtype, tol):
+def test_grouped_mm_forward_and_gradients_match_oracle(device, counts, k, n, dtype, tol, tile):
     from halo_amd.kernels.grouped_mm import grouped_mm
     from oracle import grouped_mm as oracle
 
@@ -578,7 +587,7 @@ def test_grouped_mm_forward_and_gradients_match_oracle(device, counts, k, n, dty
         assert (c == 0) == (not wd.grad[e].any()), f"expert {e}: an empty group's weight gradient must be exact zeros"
 
 
-def test_grouped_mm_takes_int64_offsets_transposed_weights_and_strided_rows(device):
+def test_grouped_mm_takes_int64_offsets_transposed_weights_and_strided_rows(device, tile):
     from halo_amd.kernels.grouped_mm import grouped_mm
     from oracle import grouped_mm as oracle
 
@@ -602,7 +611,7 @@ def test_grouped_mm_takes_int64_offsets_transposed_weights_and_strided_rows(devi
     assert wd.grad.shape == w_nk.shape and max_rel(wd.grad, want_dw) < 2e-2
 
 
-def test_grouped_mm_is_bit_reproducible_and_zero_rows(device):
+def test_grouped_mm_is_bit_reproducible_and_zero_rows(device, tile):
     from halo_amd.kernels.grouped_mm import grouped_mm
 
     counts = (100, 3, 0, 500, 77)
@@ -622,6 +631,39 @@ def test_grouped_mm_is_bit_reproducible_and_zero_rows(device):
                        offs=torch.zeros(5, dtype=torch.int32, device=device))
     assert empty.shape == (0, 512)
     empty.sum().backward()
+
+
+@pytest.mark.parametrize(("counts", "k", "n"), (((255, 256, 257, 0, 513, 31, 128, 129, 1), 200, 264),
+                                                 ((300, 0, 45), 2880, 360), ((700,), 96, 1000)))
+def test_both_tile_configurations_give_the_same_bits(device, counts, k, n):
+    """The 256 x 256, 128 x 256 and 128 x 128 tiles sum every contraction in the same order (sixteen values at a time, in
+    sequence), so the plain and the gathered products and all their gradients are bit-equal between them, and the
+    choice by size (``auto``) is one of them."""
+    from halo_amd.kernels.grouped_mm import gather_grouped_mm, gemm_tile, grouped_mm
+    from halo_amd.kernels.moe_permute import build_inv_map
+
+    g = torch.Generator().manual_seed(11)
+    rows, n_tokens = sum(counts), max(8, sum(counts) // 3)
+    row_index = torch.randint(0, n_tokens, (rows,), generator=g).to(device)
+    inv_map = build_inv_map(row_index, n_tokens, int(torch.bincount(row_index.cpu(), minlength=n_tokens).max()))
+    tokens = torch.randn(n_tokens, k, generator=g).bfloat16().to(device)
+    x = torch.randn(rows, k, generator=g).bfloat16().to(device)
+    w = (torch.randn(len(counts), k, n, generator=g) * 0.05).bfloat16().to(device)
+    dout = torch.randn(rows, n, generator=g).bfloat16().to(device)
+    offs = _offsets(counts, device)
+    results = {}
+    for name in ("mono", "duo", "small", "auto"):
+        with gemm_tile(name):
+            xd, t, wd, wg = (v.clone().requires_grad_(True) for v in (x, tokens, w, w))
+            out = grouped_mm(xd, wd, offs=offs)
+            out.backward(dout)
+            gathered = gather_grouped_mm(t, row_index, inv_map, wg, offs=offs)
+            gathered.backward(dout)
+            results[name] = (out.detach(), xd.grad, wd.grad, gathered.detach(), t.grad, wg.grad)
+    for other in ("duo", "small", "auto"):
+        for i, (a, b) in enumerate(zip(results["mono"], results[other])):
+            assert torch.equal(a, b), (other, i)
+    assert gemm_tile.set("auto") == "auto"  # the context managers restored the default
 
 
 # ---------------------------------------------------------------------------------------------------- block fp8
@@ -804,7 +846,7 @@ def test_fp8_mfma_path_against_the_dequantised_bf16_path(device):
 
 @pytest.mark.parametrize(("counts", "k", "n"), (((255, 256, 257, 0, 513, 31), 200, 264), ((64,) * 16, 512, 1536),
                                                  (tuple((37 * i * i + 11 * i) % 91 for i in range(150)), 320, 256)))
-def test_gather_grouped_mm_equals_permute_then_grouped_mm(device, counts, k, n):
+def test_gather_grouped_mm_equals_permute_then_grouped_mm(device, counts, k, n, tile):
     """The GEMM that gathers its A rows through the sorted token index does the same arithmetic in the same order as
     the permute followed by the plain GEMM: outputs and all gradients are bit-equal.  Tokens are drawn so that rows
     repeat (top-k) and some tokens are never picked."""
@@ -837,7 +879,7 @@ def test_gather_grouped_mm_equals_permute_then_grouped_mm(device, counts, k, n):
 @pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float32), ids=("bf16", "fp32"))
 @pytest.mark.parametrize(("counts", "k", "n"), (((255, 256, 257, 0, 513, 31), 200, 264), ((64,) * 16, 512, 1536),
                                                  ((0, 0, 700, 1, 0), 2880, 2880), ((5,), 64, 8)))
-def test_grouped_mm_with_the_bias_in_its_epilogue_equals_the_two_operations(device, dtype, counts, k, n):
+def test_grouped_mm_with_the_bias_in_its_epilogue_equals_the_two_operations(device, dtype, counts, k, n, tile):
     """``grouped_mm_bias`` = ``grouped_mm`` followed by ``+ MoEExpertBiasGather.apply(bias, eids)``: the product is
     rounded, the bias row of the row's expert is added, the sum is rounded again.  Output and the three gradients
     are bit-equal to the two-operation path; the output also matches the fp64 loop."""
@@ -900,7 +942,7 @@ def test_combine_with_an_added_term_equals_the_tensor_operations(device, dtype, 
 @pytest.mark.parametrize(("counts", "k", "n"), (((255, 256, 257, 0, 513, 31), 200, 264), ((64,) * 16, 512, 1536),
                                                  ((0, 0, 700, 1), 768, 2048),
                                                  (tuple((37 * i * i + 11 * i) % 91 for i in range(150)), 320, 256)))
-def test_down_projection_with_the_plain_combine_equals_the_separate_operations(device, counts, k, n):
+def test_down_projection_with_the_plain_combine_equals_the_separate_operations(device, counts, k, n, tile):
     """``grouped_mm_combine``: the product's rows summed per token in one autograd node, its backward fetching the
     token gradient's rows through the index.  Same arithmetic in the same order as ``grouped_mm`` followed by the
     unweighted gather-reduce, whose backward materialises ``grad_out[row_index]``: output and both gradients are
@@ -968,7 +1010,7 @@ class _PlainCombine(torch.autograd.Function):
 @pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float32), ids=("bf16", "fp32"))
 @pytest.mark.parametrize(("counts", "k", "n"), (((255, 256, 257, 0, 513, 31), 16, 264), ((64,) * 16, 64, 1536),
                                                  ((300, 0, 41), 8, 520)))
-def test_grouped_mm_added_to_a_tensor_equals_the_tensor_operations(device, dtype, counts, k, n):
+def test_grouped_mm_added_to_a_tensor_equals_the_tensor_operations(device, dtype, counts, k, n, tile):
     """``grouped_mm_addto``: ``addend + scale * grouped_mm(a, b)`` with the product scaled and added in the GEMM's
     epilogue.  The roundings sit where the tensor operations have them, so the output and all three gradients equal
     the unfused expression bit for bit; the contraction lengths are adapter ranks."""
@@ -995,7 +1037,7 @@ def test_grouped_mm_added_to_a_tensor_equals_the_tensor_operations(device, dtype
 @pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float32), ids=("bf16", "fp32"))
 @pytest.mark.parametrize(("counts", "k", "n"), (((255, 256, 257, 0, 513, 31), 200, 264), ((64,) * 16, 1536, 512),
                                                  ((0, 0, 700, 1, 0), 2880, 2880), ((5,), 8, 64)))
-def test_input_gradient_added_into_a_tensor_equals_the_two_operations(device, dtype, counts, k, n):
+def test_input_gradient_added_into_a_tensor_equals_the_two_operations(device, dtype, counts, k, n, tile):
     """``hmoe_grouped_gemm_dgrad_addto`` returns the bits of ``addend + grad @ W^T``: the product rounded, then the
     sum, as the tensor addition of two input gradients rounds.  A row-strided addend, and the output written over the
     addend itself."""
@@ -1028,7 +1070,7 @@ def test_input_gradient_added_into_a_tensor_equals_the_two_operations(device, dt
 @pytest.mark.parametrize("biased", (True, False), ids=("biased", "plain"))
 @pytest.mark.parametrize(("counts", "k", "n"), (((255, 256, 257, 0, 513, 31), 200, 264), ((64,) * 16, 512, 768),
                                                  (tuple((37 * i * i + 11 * i) % 91 for i in range(150)), 320, 256)))
-def test_two_projections_of_gathered_rows_as_one_node_equal_the_separate_operations(device, counts, k, n, biased):
+def test_two_projections_of_gathered_rows_as_one_node_equal_the_separate_operations(device, counts, k, n, biased, tile):
     """``gather_grouped_mm_pair`` = the permute followed by two (biased) grouped products: both outputs, the token
     gradient (the two input gradients added, then scattered back), both weight gradients and both bias gradients are
     bit-equal to the operations the reference runs one by one."""
