@@ -1,7 +1,8 @@
 """ctypes binding of ``libhalo_moe.so`` (``include/halo_moe.h``).
 
-The library is the only compute path of this package: if it is missing or fails to load, importing an op raises.
-There is no eager or CPU fallback.  Torch supplies device memory and the current HIP stream, nothing else.
+The library is the only compute path for device tensors: if it is missing or fails to load, an op on a device tensor
+raises; there is no fallback for it.  (CPU tensors take plain torch operations, as they do in the reference:
+``halo_amd/kernels/_cpu.py``.)  Torch supplies device memory and the current HIP stream, nothing else.
 """
 
 from __future__ import annotations
@@ -104,7 +105,7 @@ def dtype_id(dtype: torch.dtype) -> int:
 
 
 def require_device(*tensors: torch.Tensor) -> torch.device:
-    """All tensors on one GPU; a CPU tensor is refused (no CPU path here)."""
+    """All tensors on one GPU; a CPU tensor among device tensors is refused."""
     device = None
     for t in tensors:
         if t is None:
@@ -112,7 +113,7 @@ def require_device(*tensors: torch.Tensor) -> torch.device:
         if not t.is_cuda:
             raise RuntimeError(
                 "halo_amd kernels run on MI355X device tensors only; got a tensor on "
-                f"{t.device} (this package has no CPU or eager fallback)"
+                f"{t.device} among the operands of a device call"
             )
         if device is None:
             device = t.device

@@ -8,9 +8,10 @@
 //
 // bf16 kernel (grouped_gemm_bf16_kernel).  One persistent launch; a workgroup of 8 wavefronts owns a 256 x 256 output
 // tile and walks the contraction in steps of 64; each wavefront owns 4 x 2 accumulator blocks of 32 x 32
-// (v_mfma_f32_32x32x16_bf16).  The tile is as large as the accumulators allow because LDS is the scarce resource here
-// (one ds_read per 8 cycles per CU whatever its width, measured): per contraction element a wavefront reads
-// (4 + 2) * 32 operand values for 4 * 2 * 1024 multiply-adds.
+// (v_mfma_f32_32x32x16_bf16).  The tile is as large as the accumulators allow: the operand bytes that have to reach a
+// compute unit per multiply-add fall with the tile's size, and the rate at which they arrive is what bounds these
+// kernels; per contraction element a wavefront reads (4 + 2) * 32 operand values from LDS for 4 * 2 * 1024
+// multiply-adds.
 //  * Operand tiles go from global memory straight into LDS (buffer_load ... lds, 16 bytes per lane): no staging
 //    registers, no ds_write, no register transposes.  Rows past a group's end and columns past an operand's edge come
 //    back as zeros from the buffer bounds check, with no branches in the loop.  The loads are issued through inline
@@ -908,15 +909,9 @@ __device__ __forceinline__ void interleave_reads_under_mfmas() {
   }
 }
 
-#ifdef HMOE_WG_TIMES
-__device__ unsigned long long g_wg_times[2048];
-#endif
 
 template <int kMode, typename Cfg, int kGather = 0, bool kBias = false, bool kAddTo = false>
 __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmArgs p) {
-#ifdef HMOE_WG_TIMES
-  const unsigned long long wg_entered = __builtin_readcyclecounter();
-#endif
   static_assert(!kAddTo || ((kMode == kFwd || kMode == kDgrad) && !kBias && !kGather),
                 "the scaled sum into an addend belongs to the plain forward and the plain input gradient");
   static_assert(Cfg::BM == 256 && Cfg::BN == 256, "the direct-to-LDS loaders move 256-row tiles");
@@ -941,10 +936,7 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
   // two: the B tile of step s + 2 is requested while step s runs, so two B refills are in flight and a weight line has
   // two steps to arrive instead of one.  That takes all 160 KB of the LDS (A0 | B0 | B1 | A1 | B2, 32 KB each), so
   // these modes hold no tables there: the tile walk reads offs itself.  wgrad keeps two stages of (A, B) and its tables.
-#ifndef HMOE_RING
-#define HMOE_RING 1
-#endif
-  constexpr bool kRingB = HMOE_RING && kMode != kWgrad;
+  constexpr bool kRingB = kMode != kWgrad;
   using Sched = typename std::conditional<kRingB, RowTileWalk<kMode, BM, BN>, TileSchedule<kMode, BM, BN>>::type;
   extern __shared__ __attribute__((aligned(16))) char lds_raw[];
   auto lds = (__attribute__((address_space(3))) char*)lds_raw;
@@ -1323,13 +1315,6 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     }
   }
   wait_loads();  // no load may land in LDS after the workgroup has given it back
-#ifdef HMOE_WG_TIMES
-  // timing build: when each workgroup entered and left (cycle counter), read back with hmoe_debug_wg_times
-  if (threadIdx.x == 0) {
-    g_wg_times[blockIdx.x] = wg_entered;
-    g_wg_times[1024 + blockIdx.x] = __builtin_readcyclecounter();
-  }
-#endif
 }
 
 #define HMOE_BF16_INSTANCE(mode) \
@@ -1925,7 +1910,7 @@ int launch_direct(const GemmArgs& p, hipStream_t stream) {
   if (workers <= 0) return HMOE_OK;
   // wgrad: two stages; gathered, 2 x 1 KB of row indices per loading wavefront behind them.  fwd, dgrad: two stages
   // of A and three of B
-  constexpr size_t lds_bytes = (kMode == kWgrad || !HMOE_RING)
+  constexpr size_t lds_bytes = kMode == kWgrad
                                    ? 2 * Cfg::kStage * sizeof(bf16_t) + (kGather ? 4 * 2048 : 0)
                                    : (2 * Cfg::BM + 3 * Cfg::BN) * BK * sizeof(bf16_t);
   auto kernel = grouped_gemm_bf16_kernel<kMode, Cfg, kGather, kBias, kAddTo>;
@@ -2104,11 +2089,6 @@ int hmoe_set_gemm_tile(int tile) {
   return before;
 }
 
-#ifdef HMOE_WG_TIMES
-int hmoe_debug_wg_times(unsigned long long* host_out) {
-  return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(hmoe::g_wg_times), sizeof(unsigned long long) * 2048) == hipSuccess ? 0 : -3;
-}
-#endif
 
 int hmoe_grouped_gemm_fwd(const void* a, int64_t lda, const void* b, const int32_t* offs, int64_t total_rows,
                           int num_groups, int64_t k, int64_t n, int dtype, void* out, int64_t ldo, void* stream) {

@@ -219,7 +219,8 @@ class _WeightedPackedGLU(torch.autograd.Function):
 class GluCombine:
     """One of the fused ``activation(gate) * up`` forms; frozen, so two combines with the same numbers are equal and a
     combine can key a cache.  Calling it (or ``packed``) runs the HIP kernel pair, or the eager form when
-    ``HALO_FUSED_GLU`` turns the kernels off."""
+    ``HALO_FUSED_GLU`` turns the kernels off or the tensors live on the CPU (``fused_glu.py:352-361`` of the
+    reference)."""
 
     activation: int
     alpha: float = 1.0
@@ -256,10 +257,10 @@ class GluCombine:
         return ("silu", "gelu_tanh")[self.activation == _GELU_TANH]
 
     def __call__(self, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-        return _FusedGLU.apply(gate, up, self) if _FUSED_GLU_ENABLED else self._eager(gate, up)
+        return _FusedGLU.apply(gate, up, self) if _FUSED_GLU_ENABLED and gate.is_cuda else self._eager(gate, up)
 
     def packed(self, gate_up: torch.Tensor) -> torch.Tensor:
-        if _FUSED_GLU_ENABLED:
+        if _FUSED_GLU_ENABLED and gate_up.is_cuda:
             return _FusedPackedGLU.apply(gate_up, self)
         gate, up = gate_up.chunk(2, dim=-1)
         return self._eager(gate, up)
@@ -267,7 +268,7 @@ class GluCombine:
     def packed_weighted(self, gate_up: torch.Tensor, row_weight: torch.Tensor) -> torch.Tensor:
         """``row_weight[:, None] * packed(gate_up)`` with one rounding (:class:`_WeightedPackedGLU`); ``gate_up`` is
         ``[R, 2 M]``, ``row_weight`` ``[R]``."""
-        if _FUSED_GLU_ENABLED:
+        if _FUSED_GLU_ENABLED and gate_up.is_cuda:
             return _WeightedPackedGLU.apply(gate_up, row_weight, self)
         gate, up = gate_up.chunk(2, dim=-1)
         return (self._eager(gate, up).float() * row_weight.float().unsqueeze(-1)).to(gate_up.dtype)
@@ -279,7 +280,7 @@ class GluCombine:
         switched off, not bf16, a half width that is not a multiple of 128, rows that are not 16-byte aligned)."""
         from halo_amd.kernels.lowp.block_fp8 import QuantizedRows
 
-        if not _FUSED_GLU_ENABLED or gate_up.dtype != torch.bfloat16 or gate_up.dim() != 2:
+        if not _FUSED_GLU_ENABLED or not gate_up.is_cuda or gate_up.dtype != torch.bfloat16 or gate_up.dim() != 2:
             return None
         if gate_up.requires_grad and torch.is_grad_enabled():
             return None

@@ -12,6 +12,7 @@ import torch
 from torch.autograd import Function
 
 from halo_amd import _lib
+from halo_amd.kernels import _cpu
 
 # Every operand row must start on a 16-byte boundary (8 bf16), as for torch's grouped GEMM.
 GROUPED_MM_STRIDE_ALIGNMENT_BYTES = 16
@@ -65,11 +66,13 @@ def _offs_arg(offs: torch.Tensor | None, groups: int):
 
 
 def _forward(mat_a: torch.Tensor, mat_b: torch.Tensor, offs: torch.Tensor | None) -> torch.Tensor:
-    device = _lib.require_device(mat_a, mat_b, offs)
     if mat_a.dtype != mat_b.dtype:
         raise TypeError(f"grouped_mm operands must share a dtype, got {mat_a.dtype} and {mat_b.dtype}")
     if mat_a.dim() != 2 or mat_b.dim() != 3 or mat_a.shape[1] != mat_b.shape[1]:
         raise ValueError(f"expected [R, K] x [G, K, N], got {tuple(mat_a.shape)} x {tuple(mat_b.shape)}")
+    if not mat_a.is_cuda:
+        return _cpu.grouped_forward(mat_a, mat_b, _offs_arg(offs, mat_b.shape[0]))
+    device = _lib.require_device(mat_a, mat_b, offs)
     groups, k, n = mat_b.shape
     rows = mat_a.shape[0]
     out = torch.empty((rows, n), dtype=mat_a.dtype, device=device)
@@ -100,9 +103,11 @@ grouped_mm_forward = _forward  # the forward product alone (no autograd node), f
 def grouped_wgrad(mat_a: torch.Tensor, grad_output: torch.Tensor, offs: torch.Tensor | None,
                   groups: int) -> torch.Tensor:
     """``[groups, K, N]``: ``A[s:e]^T @ dO[s:e]`` per group, contiguous; an empty group's slice is exact zeros."""
-    device = _lib.require_device(mat_a, grad_output, offs)
     if grad_output.dtype != mat_a.dtype:
         raise TypeError("grouped_wgrad operands must share a dtype")
+    if not mat_a.is_cuda:
+        return _cpu.grouped_wgrad(mat_a, grad_output, _offs_arg(offs, groups), groups)
+    device = _lib.require_device(mat_a, grad_output, offs)
     rows, k = mat_a.shape
     n = grad_output.shape[1]
     a = _rows(mat_a)
@@ -121,9 +126,13 @@ def grouped_mm_grads(mat_a, mat_b, grad_output, offs, needs_a: bool, needs_b: bo
     """``(grad_a, grad_b)``: ``dO @ B^T`` per group and ``A^T @ dO`` per group (an empty group's weight gradient is
     exact zeros).  ``grad_output`` and the operands must share a dtype.  A broadcast (zero-stride) gradient is
     materialised first."""
-    device = _lib.require_device(mat_a, mat_b, grad_output, offs)
     if grad_output.dtype != mat_a.dtype or mat_b.dtype != mat_a.dtype:
         raise TypeError("grouped_mm_grads operands must share a dtype")
+    if not mat_a.is_cuda:
+        offs32 = _offs_arg(offs, mat_b.shape[0])
+        return (_cpu.grouped_dgrad(grad_output, mat_b, offs32) if needs_a else None,
+                _cpu.grouped_wgrad(mat_a, grad_output, offs32, mat_b.shape[0]) if needs_b else None)
+    device = _lib.require_device(mat_a, mat_b, grad_output, offs)
     groups, k, n = mat_b.shape
     rows = mat_a.shape[0]
     grad_output = _rows(grad_output) if grad_output.numel() else grad_output.new_empty(grad_output.shape)

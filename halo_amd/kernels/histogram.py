@@ -9,6 +9,7 @@ from __future__ import annotations
 import torch
 
 from halo_amd import _lib
+from halo_amd.kernels import _cpu
 
 
 def sync_free_bincount(
@@ -16,6 +17,8 @@ def sync_free_bincount(
 ) -> torch.Tensor:
     """Counts (or weight sums) of each value in ``[0, size)``; values outside the range are ignored.  ``dtype`` is
     fp32 where counts feed metric math, int64 where they become offsets."""
+    if not indices.is_cuda:
+        return _cpu.bincount(indices, size, dtype, weights)
     device = _lib.require_device(indices, weights)
     flat = indices.flatten().long().contiguous()
     native = torch.int64 if (weights is None and not dtype.is_floating_point) else torch.float32

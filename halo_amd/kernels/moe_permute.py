@@ -11,14 +11,17 @@ from __future__ import annotations
 import torch
 
 from halo_amd import _lib
+from halo_amd.kernels import _cpu
 from halo_amd.kernels.histogram import sync_free_bincount
 
 
 def _gather_rows(src: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
     """``src[index]`` for a 2-D ``src`` whose rows may be strided (a ``[:, :H]`` view of a padded buffer)."""
-    device = _lib.require_device(src, index)
     if src.dim() != 2:
         raise ValueError(f"expected [rows, hidden], got {tuple(src.shape)}")
+    if not src.is_cuda:
+        return src.index_select(0, index.long())
+    device = _lib.require_device(src, index)
     if src.stride(1) != 1:
         src = src.contiguous()
     index = index.long().contiguous()
@@ -36,6 +39,8 @@ def gather_reduce_rows(src: torch.Tensor, inv_map: torch.Tensor, weight: torch.T
     """``out[r] = sum_k w[j] * src[j]`` over ``j = inv_map[r, k] < len(src)``; ``w = 1`` without a weight.  The sum is
     taken in fp32 and rounded once to ``src``'s dtype.  With ``addend [len(out), hidden]`` (and ``addend_scale
     [len(out)]``) the same pass returns ``out + addend_scale[:, None] * addend`` with that expression's roundings."""
+    if not src.is_cuda:
+        return _cpu.gather_reduce(src, inv_map, weight, addend, addend_scale)
     device = _lib.require_device(src, inv_map, weight, addend, addend_scale)
     n_out, top_k = inv_map.shape
     hidden = src.shape[-1]
@@ -66,7 +71,8 @@ def gather_reduce_rows(src: torch.Tensor, inv_map: torch.Tensor, weight: torch.T
 
 
 def padded_gather_reduce(src: torch.Tensor, inv_map: torch.Tensor, weight: torch.Tensor | None = None) -> torch.Tensor:
-    """The reference keeps this name for its CPU twin (``moe_permute.py:115-120``); here it is the same kernel."""
+    """The reference keeps this name for its CPU twin (``moe_permute.py:115-120``); here it is the same operator (the
+    kernel for device tensors, the padded gather-sum in fp32 for CPU tensors)."""
     return gather_reduce_rows(src, inv_map, weight)
 
 
@@ -75,7 +81,7 @@ def build_inv_map(sorted_token_idx: torch.Tensor, recv_N: int, width: int) -> to
     sentinel ``len(sorted_token_idx)``.  Auxiliary: the routing sort already returns this map, so the expert path
     never calls this; it serves callers holding only ``sorted_token_idx`` and is a handful of device-side torch ops
     with no host readback (stable argsort, counts, exclusive cumsum, one scatter)."""
-    device = _lib.require_device(sorted_token_idx)
+    device = sorted_token_idx.device
     token_of = sorted_token_idx.to(torch.int64)
     rows = token_of.numel()
     result = token_of.new_full((recv_N, width), rows)  # every slot the sentinel until a row claims it
@@ -130,6 +136,8 @@ class MoEWeightedUnpermute(torch.autograd.Function):
 
 def _unpermute_backward(grad_out, expert_out, weights, sorted_token_idx, weight_grad: bool):
     """``(w[j] * grad_out[tok[j]], <grad_out[tok[j]], expert_out[j]>)``; the second only when ``weight_grad``."""
+    if not grad_out.is_cuda:
+        return _cpu.unpermute_backward(grad_out, expert_out, weights, sorted_token_idx, weight_grad)
     device = _lib.require_device(grad_out, weights, sorted_token_idx)
     n_sorted, hidden = sorted_token_idx.shape[0], grad_out.shape[-1]
     # Under EP the gradient arrives as a row-strided view of the padded transport buffer, read in place.
@@ -190,6 +198,8 @@ def expert_bias_grad(grad_out: torch.Tensor, eids: torch.Tensor, num_experts: in
     """``[num_experts, width]``: per expert, the sum of the rows of ``grad_out`` that belong to it (``eids`` sorted),
     accumulated in fp32 in a fixed order and rounded once; an expert without rows gets exact zeros.  What the
     reference computes as ``onehot(eids)^T @ grad_out`` (``moe_permute.py:202-208``)."""
+    if not grad_out.is_cuda:
+        return _cpu.expert_bias_grad(grad_out, eids, num_experts)
     device = _lib.require_device(grad_out, eids)
     grad_out = grad_out.contiguous()
     eids = eids.long().contiguous()

@@ -10,6 +10,7 @@ from __future__ import annotations
 import torch
 
 from halo_amd import _lib
+from halo_amd.kernels import _cpu
 
 RECEIVE_COUNTS_DISAGREE = "DeepEP receive counts disagree with the received expert ids"
 # At ep_size 1 no dispatch pads, so an id outside the local range came from the routing itself.
@@ -100,6 +101,9 @@ def sort_routing_by_expert(
     ``halo.kernels.moe_route_sort.sort_routing_by_expert``."""
     if counts is not None and len(counts) != num_local_experts:
         raise ValueError(f"{len(counts)} receive counts for {num_local_experts} local experts")
+    if not experts.is_cuda:  # CPU tensors: a stable argsort, as the reference's _argsort_routing (:201-227)
+        return _cpu.sort_routing(experts, weights, num_local_experts, counts, RECEIVE_COUNTS_DISAGREE,
+                                 NONLOCAL_EXPERT_ID_MESSAGE)
     return _CountingSort.apply(weights, experts, num_local_experts, counts)
 
 

@@ -11,6 +11,7 @@ from __future__ import annotations
 import torch
 
 from halo_amd import _lib
+from halo_amd.kernels import _cpu
 
 SOFTMAX_ALL = 0  # softmax over every expert, gather the picks, optionally renormalise by (sum + eps)
 SOFTMAX_TOPK = 1  # softmax over the k selected logits
@@ -57,4 +58,6 @@ def fused_topk_gate(logits: torch.Tensor, top_k: int, *, mode: int = SOFTMAX_ALL
                     eps: float = 0.0) -> tuple[torch.Tensor, torch.Tensor]:
     """``(indices i64[T, k], weights f32[T, k])``: the router's picks and gate weights, the weights rounded to the
     logits' dtype and held in fp32 (what the layer gets after the router's cast and its own ``.float()``)."""
+    if not logits.is_cuda:
+        return _cpu.topk_gate(logits, top_k, mode == SOFTMAX_TOPK, normalize, eps)
     return _FusedTopKGate.apply(logits, top_k, mode, normalize, eps)
