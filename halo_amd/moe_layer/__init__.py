@@ -4,6 +4,7 @@ from halo_amd.moe_layer.balancing import expert_load_token_weights  # noqa: F401
 from halo_amd.moe_layer.config import EPConfig, single_process_ep_config  # noqa: F401
 from halo_amd.moe_layer.families import (  # noqa: F401
     MOE_LAYER_MAP,
+    EPGemma4MoELayer,
     EPGptOssMoELayer,
     EPQwen3_5MoELayer,
     EPQwen3MoELayer,

@@ -72,6 +72,8 @@ class MoEFamilySpec:
 
 QWEN3 = MoEFamilySpec("qwen3_moe", expert_layout="separate_glu")
 QWEN3_5 = MoEFamilySpec("qwen3_5_moe", expert_layout="fused", shared_expert_attrs=("shared_expert",))
+# Gemma-4: the wrapped HF module is the expert container itself; its router is a sibling module of the decoder layer
+GEMMA4 = MoEFamilySpec("gemma4", expert_layout="fused", experts_container_attrs=())
 GPT_OSS = MoEFamilySpec(
     "gpt_oss",
     expert_layout="interleaved_glu",

@@ -1,8 +1,9 @@
 """Per-family glue over :class:`EPMoELayerBase`: Qwen3 (gate and up stored apart), Qwen3.5 / Qwen3.6 (fused experts and
-a sigmoid-gated shared expert) and gpt-oss (interleaved fused experts with biases, clamped SwiGLU, logit-space router
-bias).
+a sigmoid-gated shared expert), gpt-oss (interleaved fused experts with biases, clamped SwiGLU, logit-space router
+bias) and Gemma-4 (the experts alone: the routing decision arrives with the call).
 
-Mirrors the reference's ``halo/distributed/expert_parallel/families/qwen3.py``, ``qwen3_5.py`` and ``gpt_oss.py``.
+Mirrors the reference's ``halo/distributed/expert_parallel/families/qwen3.py``, ``qwen3_5.py``, ``gpt_oss.py`` and
+``gemma4.py``.
 """
 
 from __future__ import annotations
@@ -14,7 +15,7 @@ from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled
 from halo_amd.kernels.grouped_mm import bias_fusable, grouped_mm_bias
 from halo_amd.kernels.moe_permute import MoEExpertBiasGather
 from halo_amd.kernels.router import SOFTMAX_TOPK, fused_topk_gate
-from halo_amd.moe_layer.config import GPT_OSS, QWEN3, QWEN3_5
+from halo_amd.moe_layer.config import GEMMA4, GPT_OSS, QWEN3, QWEN3_5
 from halo_amd.moe_layer.layer import EPMoELayerBase, EPSharedExpertsMoELayerBase
 
 
@@ -153,7 +154,39 @@ class EPGptOssMoELayer(EPMoELayerBase):
         return out if bias is None else out + MoEExpertBiasGather.apply(bias.to(out_dtype), eids)
 
 
-MOE_LAYER_MAP = {name: cls for cls in (EPQwen3MoELayer, EPQwen3_5MoELayer, EPGptOssMoELayer)
+class EPGemma4MoELayer(EPMoELayerBase):
+    """``Gemma4TextExperts``: Gemma-4 computes its router in the decoder layer, so only the expert container is
+    replaced and ``forward`` takes the routing decision as made: ``(hidden [T, H], top_k_index [T, k], top_k_weights
+    [T, k])``, tokens already flat, the result ``[T, H]`` (``families/gemma4.py:12-39`` of the reference).  The
+    experts-only seam: sort, two grouped GEMMs around the fused tanh-GELU combine, weighted combine; the gate weights
+    carry a gradient back to the caller's router."""
+
+    HF_MODULE_NAMES = ("Gemma4TextExperts",)
+    FAMILY = GEMMA4
+    _ROUTER_ATTR = None  # the router is a sibling module of the decoder layer
+
+    @classmethod
+    def _find_experts_container(cls, layer: nn.Module) -> nn.Module:
+        return layer  # the wrapped module holds gate_up_proj / down_proj itself
+
+    def _adopt_routing(self, original_layer: nn.Module) -> None:
+        """Nothing to adopt: indices and weights come with every call."""
+        self.top_k = None
+
+    @classmethod
+    def from_weights(cls, *, gelu: bool = True, **kwargs):
+        self = super().from_weights(router_weight=None, top_k=kwargs.pop("top_k", None), **kwargs)
+        if gelu:  # Gemma-4's hidden activation, gelu_pytorch_tanh
+            self._fused_glu_mul = GluCombine.gelu_tanh()
+        return self
+
+    def forward(self, hidden_states: torch.Tensor, top_k_index: torch.Tensor,  # type: ignore[override]
+                top_k_weights: torch.Tensor) -> torch.Tensor:
+        return self._dispatch_compute_combine(hidden_states, top_k_index.long(), top_k_weights.float(),
+                                              hidden_states.dtype)
+
+
+MOE_LAYER_MAP = {name: cls for cls in (EPQwen3MoELayer, EPQwen3_5MoELayer, EPGptOssMoELayer, EPGemma4MoELayer)
                  for name in cls.HF_MODULE_NAMES}
 
 

@@ -168,6 +168,13 @@ int hmoe_router_topk_bwd(const void* logits, int dtype, const int64_t* indices, 
                          int64_t n_tokens, int num_experts, int top_k, int mode, int normalize, float eps,
                          void* grad_logits, void* stream);
 
+/* ------------------------------------------------------------------------------------------------ device probe
+ * No counterpart in the reference: a measuring stick for benchmarks.  Runs `iterations` rounds of eight independent
+ * v_mfma_f32_32x32x16_bf16 per wavefront on register operands, two wavefronts per SIMD on every compute unit, and
+ * returns the floating-point operations the launch performs (time it with events on `stream`), or a negative
+ * hmoe_status.  `sink` is a device buffer of at least one float per compute unit (never written in practice). */
+int64_t hmoe_probe_mfma_bf16(int64_t iterations, void* sink, void* stream);
+
 /* ------------------------------------------------------------------------------------------------ grouped GEMM
  * Replace F.grouped_mm as called by halo/kernels/grouped_mm.py:16-47 (forward :39, dgrad :25, wgrad :26).
  * offs i32[num_groups] are inclusive row ends (null: one group holding every row).  b is [num_groups, K, N]

@@ -203,3 +203,32 @@ def test_cpu_layer_forward_backward_matches_the_per_expert_loop(cfg_name):
         attr = name.replace("gate_proj", "gate_proj_gmm").replace("up_proj", "up_proj_gmm") \
             if cfg.router == "softmax_topk" else name
         _check(f"grad {name}", getattr(layer, attr).grad, want_grads[name], tol)
+
+
+def test_cpu_gemma4_experts_drop_in_matches_the_hf_module():
+    """``EPGemma4MoELayer`` wraps transformers' ``Gemma4TextExperts`` (experts only, routing handed in) and returns its
+    output and gradients, the gate weights' included, in fp32 on the CPU."""
+    from transformers.models.gemma4.configuration_gemma4 import Gemma4TextConfig
+    from transformers.models.gemma4.modeling_gemma4 import Gemma4TextExperts
+
+    from halo_amd.moe_layer import MOE_LAYER_MAP, EPGemma4MoELayer, single_process_ep_config
+
+    torch.manual_seed(0)
+    config = Gemma4TextConfig(hidden_size=64, moe_intermediate_size=48, num_experts=8, top_k_experts=2,
+                              hidden_activation="gelu_pytorch_tanh", num_hidden_layers=1)
+    hf = Gemma4TextExperts(config)
+    with torch.no_grad():
+        hf.gate_up_proj.normal_(0, 0.1)
+        hf.down_proj.normal_(0, 0.1)
+    assert MOE_LAYER_MAP["Gemma4TextExperts"] is EPGemma4MoELayer
+    layer = EPGemma4MoELayer(hf, single_process_ep_config())
+    assert layer._glu_combine_name() == "gelu_tanh" and layer.gate_up_proj.shape == (8, 64, 96)
+    assert {n for n, _ in layer.expert_named_params()} == {"gate_up_proj", "down_proj"}
+    x = torch.randn(40, 64, requires_grad=True)
+    probs, idx = torch.topk(torch.softmax(torch.randn(40, 8), -1), 2, dim=-1)
+    w = (probs / probs.sum(-1, keepdim=True)).requires_grad_()
+    out, want = layer(x, idx, w), hf(x, idx, w)
+    torch.testing.assert_close(out, want, rtol=1e-5, atol=1e-6)
+    upstream = torch.randn_like(out)
+    for got, ref in zip(torch.autograd.grad(out, (x, w), upstream), torch.autograd.grad(want, (x, w), upstream)):
+        torch.testing.assert_close(got, ref, rtol=1e-4, atol=1e-6)

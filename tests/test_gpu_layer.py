@@ -370,6 +370,42 @@ def test_drop_in_for_hf_gpt_oss_block(device):
     assert logits.shape == (40, 8) and layer._glu_combine_name() == "gptoss"
 
 
+def test_drop_in_for_hf_gemma4_experts(device):
+    """The experts-only entry (``families/gemma4.py:30-39``): routing decided outside, ``forward(hidden, top_k_index,
+    top_k_weights)``.  bf16 on the device against transformers' ``Gemma4TextExperts`` in fp32 on the CPU: output,
+    input gradient and the gate weights' gradient within BASELINE's tolerance."""
+    from transformers.models.gemma4.configuration_gemma4 import Gemma4TextConfig
+    from transformers.models.gemma4.modeling_gemma4 import Gemma4TextExperts
+
+    from halo_amd.moe_layer import EPGemma4MoELayer, single_process_ep_config
+
+    torch.manual_seed(2)
+    config = Gemma4TextConfig(hidden_size=256, moe_intermediate_size=88, num_experts=16, top_k_experts=4,
+                              hidden_activation="gelu_pytorch_tanh", num_hidden_layers=1)
+    hf = Gemma4TextExperts(config)
+    with torch.no_grad():
+        hf.gate_up_proj.normal_(0, 0.05)
+        hf.down_proj.normal_(0, 0.05)
+    x = torch.randn(300, 256).bfloat16().float().requires_grad_(True)
+    probs, idx = torch.topk(torch.softmax(torch.randn(300, 16), -1), 4, dim=-1)
+    w = (probs / probs.sum(-1, keepdim=True)).bfloat16().float().requires_grad_(True)
+    upstream = torch.randn(300, 256).bfloat16().float()
+    for p in (hf.gate_up_proj, hf.down_proj):
+        p.data = p.data.bfloat16().float()
+    want = hf(x, idx, w)
+    want_gx, want_gw = torch.autograd.grad(want, (x, w), upstream)
+    layer = EPGemma4MoELayer(hf.to(device).to(torch.bfloat16), single_process_ep_config())
+    assert layer._glu_combine_name() == "gelu_tanh"
+    xd = x.detach().bfloat16().to(device).requires_grad_(True)
+    wd = w.detach().to(device).requires_grad_(True)
+    got = layer(xd, idx.to(device), wd)
+    assert got.dtype == torch.bfloat16 and got.shape == (300, 256)
+    got_gx, got_gw = torch.autograd.grad(got, (xd, wd), upstream.bfloat16().to(device))
+    _check("gemma4 out", got, want, 2e-2)
+    _check("gemma4 grad x", got_gx, want_gx, 2e-2)
+    _check("gemma4 grad gate weights", got_gw, want_gw, 2e-2)
+
+
 def test_router_projection_gradients_at_a_token_count_that_splits_the_wgrad(device):
     """The router's weight gradient goes through the grouped wgrad kernel in 32 token slices once there are enough
     tokens; the layer configurations above are too small to take that path.  Checked against the fp64 product over
