@@ -43,6 +43,7 @@ SIGNATURES = {
     "hmoe_router_topk_bwd": (I, [P, I, P, P, L, I, I, I, I, F, P, P]),
     "hmoe_probe_mfma_bf16": (L, [L, P, P]),
     "hmoe_set_gemm_tile": (I, [I]),
+    "hmoe_grouped_gemm_mx_fits": (I, [L, L, L, L, L, I]),
     "hmoe_grouped_gemm_fwd": (I, [P, L, P, P, L, I, L, L, I, P, L, P]),
     "hmoe_grouped_gemm_fwd_bias": (I, [P, L, P, P, P, L, I, L, L, I, P, L, P]),
     "hmoe_grouped_gemm_fwd_addto": (I, [P, L, P, P, L, I, L, L, I, P, L, F, P, L, P]),

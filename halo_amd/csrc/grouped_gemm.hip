@@ -2038,6 +2038,17 @@ int launch_fp8(const GemmArgs& p, int64_t workers, void* stream) {
   return HMOE_OK;
 }
 
+// Whether the scaled-MFMA kernel can address the operands of an MX product: it bases its buffer descriptors at the
+// arrays' starts, so every array must stay below 2 GiB (the bf16 kernels rebase theirs per tile and have no such
+// limit; a caller with larger operands multiplies the round-tripped operands there).
+bool mx_product_fits(int64_t a_rows, int64_t total_rows, int64_t k, int64_t n, int64_t ldo, int panel_values) {
+  if (a_rows < 0 || total_rows < 0 || k < 0 || n < 0 || ldo < 0 || (panel_values != 64 && panel_values != 128)) return false;
+  const int64_t lim = int64_t(1) << 31, panels = (k + panel_values - 1) / panel_values;
+  // products of two values below 2^31 each stay inside int64
+  if (a_rows >= lim || total_rows >= lim || panels >= lim || n >= lim || ldo >= lim) return false;
+  return a_rows * panels < lim / 64 && panels * n < lim / 64 && total_rows * ldo < lim / 2;
+}
+
 // The MX products' arguments, checked: `panel_values` contraction values lie in a panel's 64 bytes (64 for e4m3, 128 for
 // e2m1) and `k_multiple` is what k must be a multiple of.
 int mx_args(GemmArgs& p, const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
@@ -2054,8 +2065,8 @@ int mx_args(GemmArgs& p, const uint8_t* a_q, const uint8_t* a_scale, int64_t a_r
   if (!aligned16(a_q) || !aligned16(bq) || !aligned16(out) || (with_bias && !aligned16(bias))) return HMOE_UNSUPPORTED;
   if (panel_values == 128 && (reinterpret_cast<uintptr_t>(a_scale) % 4 || reinterpret_cast<uintptr_t>(b_scale) % 4))
     return HMOE_UNSUPPORTED;
-  const int64_t lim = int64_t(1) << 31, panels = (k + panel_values - 1) / panel_values;
-  if (a_rows * panels * 64 >= lim || panels * 64 * n >= lim || total_rows * ldo * 2 >= lim) return HMOE_UNSUPPORTED;
+  const int64_t panels = (k + panel_values - 1) / panel_values;
+  if (!mx_product_fits(a_rows, total_rows, k, n, ldo, panel_values)) return HMOE_UNSUPPORTED;
   p.a = a_q;
   p.b = bq;
   p.c = out;
@@ -2081,6 +2092,11 @@ int mx_args(GemmArgs& p, const uint8_t* a_q, const uint8_t* a_scale, int64_t a_r
 }  // namespace hmoe
 
 extern "C" {
+
+int hmoe_grouped_gemm_mx_fits(int64_t a_rows, int64_t total_rows, int64_t k, int64_t n, int64_t ldo,
+                              int panel_values) {
+  return hmoe::mx_product_fits(a_rows, total_rows, k, n, ldo, panel_values) ? 1 : 0;
+}
 
 int hmoe_set_gemm_tile(int tile) {
   if (tile < 0 || tile > 3) return HMOE_INVALID_ARGUMENT;

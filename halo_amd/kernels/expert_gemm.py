@@ -108,12 +108,13 @@ def expert_gemm(
     return grouped_mm(mat_a, mat_b, offs=offs)
 
 
-def mxfp8_mfma_usable(mat_a_dtype: torch.dtype, mat_b_dtype: torch.dtype, k: int, n: int) -> bool:
+def mxfp8_mfma_usable(mat_a_dtype: torch.dtype, mat_b_dtype: torch.dtype, k: int, n: int, rows: int = 0) -> bool:
     """Whether the scaled e4m3 MFMA kernel takes the product: bf16 operands, whole panels of 64 values along K,
-    16-byte output rows.  Anything else multiplies the two round-tripped operands on the bf16 / fp32 kernel, which is
-    the reference's own formulation."""
+    16-byte output rows, and ``rows`` activation rows whose quantised panels and output the kernel can address (each
+    array below 2 GiB: the library's own check, ``hmoe_grouped_gemm_mx_fits``).  Anything else multiplies the two
+    round-tripped operands on the bf16 / fp32 kernel, which is the reference's own formulation."""
     return (mat_a_dtype == torch.bfloat16 and mat_b_dtype == torch.bfloat16 and k > 0 and k % 64 == 0
-            and n % 8 == 0)
+            and n % 8 == 0 and bool(_lib.load().hmoe_grouped_gemm_mx_fits(rows, rows, k, n, n, 64)))
 
 
 def _plus_bias(out: torch.Tensor, bias, eids) -> torch.Tensor:
@@ -133,14 +134,26 @@ def _bias_grad(ctx, grad_output: torch.Tensor, position: int):
 class _SharedRows:
     """The last activation tensor quantised (forward) and the last e4m3 rows dequantised (backward), each with its
     result: projections that read the same rows (gate and up stored apart) quantise them once and rebuild them once.
-    An entry is tied to the tensor object by a weak reference and to its version counter, and dies with the tensor."""
+    An entry is tied to the tensor object by a weak reference, to its version counter, its storage address and its
+    shape, and dies with the tensor; the slot is read and written under a lock (autograd's backward thread shares it
+    with the forward thread).  What the key cannot see is a write that leaves the version counter alone (``.data``
+    assignments into the same storage, a kernel writing through a raw pointer): such writes between two projections
+    of the same rows are not supported."""
 
     def __init__(self):
+        import threading
+
         self._ref, self._key, self._value, self._hold = None, None, None, None
+        self._lock = threading.Lock()
+
+    @staticmethod
+    def _full_key(tensor: torch.Tensor, key: tuple) -> tuple:
+        return (key, tensor.data_ptr(), tuple(tensor.shape), tuple(tensor.stride()))
 
     def get(self, tensor: torch.Tensor, key: tuple):
-        if self._ref is not None and self._ref() is tensor and self._key == key:
-            return self._value
+        with self._lock:
+            if self._ref is not None and self._ref() is tensor and self._key == self._full_key(tensor, key):
+                return self._value
         return None
 
     def put(self, tensor: torch.Tensor, key: tuple, value, hold=None) -> None:
@@ -149,10 +162,13 @@ class _SharedRows:
         import weakref
 
         def drop(ref, self=self):
-            if self._ref is ref:
-                self._ref, self._key, self._value, self._hold = None, None, None, None
+            with self._lock:
+                if self._ref is ref:
+                    self._ref, self._key, self._value, self._hold = None, None, None, None
 
-        self._ref, self._key, self._value, self._hold = weakref.ref(tensor, drop), key, value, hold
+        with self._lock:
+            self._ref, self._key, self._value, self._hold = (weakref.ref(tensor, drop), self._full_key(tensor, key),
+                                                             value, hold)
 
 
 _quantised_rows = _SharedRows()
@@ -192,7 +208,7 @@ class _MxFp8ExpertGemm(torch.autograd.Function):
         # input or output of this node
         ctx.rows_q = rows_q
         ctx.save_for_backward(weight.dequant, offs32, inv_map)
-        if not mxfp8_mfma_usable(mat_a.dtype, mat_b.dtype, k, n):
+        if not mxfp8_mfma_usable(mat_a.dtype, mat_b.dtype, k, n, rows):
             return _plus_bias(_forward(dequantize_rows_mxfp8(rows_q).to(mat_a.dtype), weight.dequant.to(mat_a.dtype),
                                        offs32), bias, eids)
         out = torch.empty((rows, n), dtype=torch.bfloat16, device=device)
@@ -265,10 +281,12 @@ class _RoundTripExpertGemm(torch.autograd.Function):
         return grad_a, grad_b, None, None, None
 
 
-def mxfp4_mfma_usable(mat_a_dtype: torch.dtype, mat_b_dtype: torch.dtype, k: int, n: int) -> bool:
-    """Whether the scaled matrix instruction takes the MXFP4 product: bf16 operands, 16-byte output rows.  Anything
+def mxfp4_mfma_usable(mat_a_dtype: torch.dtype, mat_b_dtype: torch.dtype, k: int, n: int, rows: int = 0) -> bool:
+    """Whether the scaled matrix instruction takes the MXFP4 product: bf16 operands, 16-byte output rows, and ``rows``
+    activation rows whose quantised panels and output the kernel can address (``hmoe_grouped_gemm_mx_fits``).  Anything
     else multiplies the two round-tripped operands on the bf16 / fp32 kernel, the reference's own formulation."""
-    return mat_a_dtype == torch.bfloat16 and mat_b_dtype == torch.bfloat16 and k > 0 and k % 32 == 0 and n % 8 == 0
+    return (mat_a_dtype == torch.bfloat16 and mat_b_dtype == torch.bfloat16 and k > 0 and k % 32 == 0 and n % 8 == 0
+            and bool(_lib.load().hmoe_grouped_gemm_mx_fits(rows, rows, k, n, n, 128)))
 
 
 _round_tripped_rows = _SharedRows()
@@ -299,7 +317,8 @@ class _Mxfp4ExpertGemm(torch.autograd.Function):
         offs32 = _offs_arg(offs, groups)
         key = (mat_a._version, None if row_index is None else (id(row_index), row_index._version))
         ctx.gathered, ctx.k, ctx.dtype = row_index is not None, k, mat_a.dtype
-        ctx.native = mxfp4_mfma_usable(mat_a.dtype, mat_b.dtype, k, n)
+        ctx.native = mxfp4_mfma_usable(mat_a.dtype, mat_b.dtype, k, n,
+                                       mat_a.shape[0] if row_index is None else row_index.shape[0])
         if not ctx.native:
             w_rt = expert_weight_round_trip(mat_b, "mxfp4", weight_cacheable).to(mat_a.dtype)
             a_rt = _round_tripped_rows.get(mat_a, key)

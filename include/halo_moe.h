@@ -68,7 +68,9 @@ int hmoe_route_sort(const void* experts, int experts_elem_bytes, const void* wei
  * up once per device on the first call made with that device current.  A routing whose table does not fit
  * (hmoe_route_sort_workspace_bytes(...) > 4 MiB, i.e. sort blocks x local experts > 2^20) returns HMOE_UNSUPPORTED.
  * Calls that overlap on one GPU (two streams, two threads) share the array and race: serialise them per GPU.  Nothing
- * in the array needs clearing between calls: every entry read is written by the same call first. */
+ * in the array needs clearing between calls: every entry read is written by the same call first.  The first call made
+ * with a device current looks the array's address up (hipGetSymbolAddress, which may load the library's code object on
+ * that device): make that call outside any stream capture; every later call on the device only launches kernels. */
 int hmoe_route_sort_static(const void* experts, int experts_elem_bytes, const void* weights, int weight_elem_bytes,
                            int64_t n_rows, int top_k, int num_local_experts, int64_t n_valid,
                            int64_t* sorted_token_idx, void* sorted_weights, void* sorted_expert_ids, int32_t* offs,
@@ -340,6 +342,13 @@ int hmoe_quantize_weight_mxfp8(const void* w, int dtype, int64_t groups, int64_t
 int hmoe_grouped_gemm_fwd_mxfp8(const uint8_t* a_q, const uint8_t* a_scale, int64_t a_rows, const uint8_t* bq,
                                 const uint8_t* b_scale, const int32_t* offs, int64_t total_rows, int num_groups,
                                 int64_t k, int64_t n, void* out, int64_t ldo, void* stream);
+
+/* Whether hmoe_grouped_gemm_fwd_mxfp8 (panel_values 64) / hmoe_grouped_gemm_fwd_mxfp4 (panel_values 128) can address
+ * operands of these sizes: the scaled-MFMA kernel bases its descriptors at the arrays' starts, so the quantised
+ * activations (a_rows rows), one expert's quantised weights and the output (total_rows x ldo) must each stay below
+ * 2 GiB; beyond that the entry points return HMOE_UNSUPPORTED and a caller multiplies the round-tripped operands on the
+ * bf16 kernels, which have no such limit (what halo_amd.kernels.expert_gemm does).  1 or 0; launches nothing. */
+int hmoe_grouped_gemm_mx_fits(int64_t a_rows, int64_t total_rows, int64_t k, int64_t n, int64_t ldo, int panel_values);
 
 /* ------------------------------------------------------------------------------------------------------- MXFP4
  * The reference's "mxfp4" quant_format (halo/kernels/lowp/spec.py:11): e2m1 elements (magnitudes 0, 0.5, 1, 1.5, 2, 3,
