@@ -11,7 +11,6 @@ from __future__ import annotations
 from typing import Literal
 
 QuantFormat = Literal["mxfp8", "mxfp4", "nvfp4"]
-IMPLEMENTED_FORMATS: tuple[str, ...] = ("mxfp8", "mxfp4", "nvfp4")
 
 # Elements per shared scale along the contraction axis (``halo/kernels/lowp/quantization.py:47``).
 FORMAT_BLOCK_SIZE: dict[str, int] = {"mxfp8": 32, "mxfp4": 32, "nvfp4": 16}
@@ -20,5 +19,3 @@ FORMAT_BLOCK_SIZE: dict[str, int] = {"mxfp8": 32, "mxfp4": 32, "nvfp4": 16}
 def require_implemented(fmt: str) -> None:
     if fmt not in FORMAT_BLOCK_SIZE:
         raise ValueError(f"unknown block-scaled format {fmt!r} (expected one of {sorted(FORMAT_BLOCK_SIZE)})")
-    if fmt not in IMPLEMENTED_FORMATS:
-        raise NotImplementedError(f"quant_format={fmt!r}: only {', '.join(IMPLEMENTED_FORMATS)} are built on this path")
