@@ -37,8 +37,8 @@ SIGNATURES = {
     "hmoe_expert_colsum": (I, [P, P, L, L, I, I, P, P, P]),
     "hmoe_glu_fwd": (I, [P, P, L, L, L, L, I, I, F, F, I, I, P, P]),
     "hmoe_glu_bwd": (I, [P, P, L, L, P, L, L, I, I, F, F, I, I, P, P, L, L, P]),
-    "hmoe_glu_fwd_weighted": (I, [P, P, L, L, P, L, L, I, I, F, F, I, I, P, P]),
-    "hmoe_glu_bwd_weighted": (I, [P, P, L, L, P, P, L, L, I, I, F, F, I, I, P, P, L, L, P, P]),
+    "hmoe_glu_fwd_weighted": (I, [P, P, L, L, P, I, L, L, I, I, F, F, I, I, P, P]),
+    "hmoe_glu_bwd_weighted": (I, [P, P, L, L, P, P, I, L, L, I, I, F, F, I, I, P, P, L, L, P, P]),
     "hmoe_router_topk_fwd": (I, [P, I, L, I, I, I, I, F, P, P, P]),
     "hmoe_router_topk_bwd": (I, [P, I, P, P, L, I, I, I, I, F, P, P]),
     "hmoe_probe_mfma_bf16": (L, [L, P, P]),

@@ -152,18 +152,26 @@ glu_bwd_kernel(const T* __restrict__ gate, const T* __restrict__ up, const T* __
   du.store(dup + row * stride_dup + col);
 }
 
+// A row's gate weight: in the operands' dtype, or fp32 rounded to it here (what a cast of the weights would give,
+// without the cast's launch).
+template <typename T>
+__device__ __forceinline__ float load_row_weight(const void* row_weight, bool weight_f32, int64_t row) {
+  if (weight_f32) return Elem<T>::round(static_cast<const float*>(row_weight)[row]);
+  return Elem<T>::load(static_cast<const T*>(row_weight) + row);
+}
+
 // The combine with the row's gate weight folded in: out[r] = round(w[r] * glu(gate[r], up[r])), the product taken in
 // fp32, so the down projection runs on weighted rows and the combine behind it is a plain sum.
 template <typename T, int W, int kAct, bool kClampAct, bool kPlusOne>
 __global__ void __launch_bounds__(kThreads)
-glu_fwd_weighted_kernel(const T* __restrict__ gate, const T* __restrict__ up, const T* __restrict__ row_weight,
-                        T* __restrict__ out, int64_t stride_gate, int64_t stride_up, int64_t n_rows,
+glu_fwd_weighted_kernel(const T* __restrict__ gate, const T* __restrict__ up, const void* __restrict__ row_weight,
+                        bool weight_f32, T* __restrict__ out, int64_t stride_gate, int64_t stride_up, int64_t n_rows,
                         int64_t chunks_per_row, int64_t width, GluParams p) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   const int64_t row = i / chunks_per_row;
   if (row >= n_rows) return;
   const int64_t col = (i - row * chunks_per_row) * W;
-  const float w = Elem<T>::load(row_weight + row);
+  const float w = load_row_weight<T>(row_weight, weight_f32, row);
   Chunk<T, W> g, u, o;
   g.load(gate + row * stride_gate + col);
   u.load(up + row * stride_up + col);
@@ -176,19 +184,20 @@ glu_fwd_weighted_kernel(const T* __restrict__ gate, const T* __restrict__ up, co
 //   (dgate, dup) = glu_grad(gate, up, w[r] * grad_out[r]),   grad_weight[r] = <grad_out[r], act[r]>.
 // kLanes lanes share a row (a power of two up to the wavefront), each taking every kLanes-th 16-byte chunk; the dot
 // product is summed in fp32 in a fixed order (per lane in chunk order, then a butterfly over the lanes) and stored as
-// fp32.
+// fp32; with fp32 weights the stored value is rounded to the operands' dtype first (the gradient of weights that were
+// cast to it arrives through that dtype).
 template <typename T, int W, int kLanes, int kAct, bool kClampAct, bool kPlusOne>
 __global__ void __launch_bounds__(kThreads)
 glu_bwd_weighted_kernel(const T* __restrict__ gate, const T* __restrict__ up, const T* __restrict__ grad_out,
-                        const T* __restrict__ row_weight, T* __restrict__ dgate, T* __restrict__ dup,
-                        float* __restrict__ grad_weight, int64_t stride_gate, int64_t stride_up, int64_t stride_dgate,
+                        const void* __restrict__ row_weight, bool weight_f32, T* __restrict__ dgate,
+                        T* __restrict__ dup, float* __restrict__ grad_weight, int64_t stride_gate, int64_t stride_up, int64_t stride_dgate,
                         int64_t stride_dup, int64_t n_rows, int chunks_per_row, int64_t width, GluParams p) {
   const int64_t thread = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   const int64_t row = thread / kLanes;
   const int sub = static_cast<int>(thread % kLanes);
   float dot = 0.f;
   if (row < n_rows) {
-    const float w = Elem<T>::load(row_weight + row);
+    const float w = load_row_weight<T>(row_weight, weight_f32, row);
     // kPer chunks per pass, their loads issued together ahead of the arithmetic (a row of 768 values on 32 lanes is
     // one pass of three)
     constexpr int kPer = 3;
@@ -223,7 +232,7 @@ glu_bwd_weighted_kernel(const T* __restrict__ gate, const T* __restrict__ up, co
   }
 #pragma unroll
   for (int off = kLanes / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off, HMOE_WAVE);
-  if (row < n_rows && sub == 0) grad_weight[row] = dot;
+  if (row < n_rows && sub == 0) grad_weight[row] = weight_f32 ? Elem<T>::round(dot) : dot;
 }
 
 struct GluArgs {
@@ -237,6 +246,7 @@ struct GluArgs {
   uint8_t* scale = nullptr;
   int64_t out_rows = 0;
   const void* row_weight = nullptr;  // the weighted forms: one gate weight per row, in the operands' dtype
+  bool weight_f32 = false;           // ... or fp32, rounded to the operands' dtype by the kernel
   float* grad_weight = nullptr;      // backward: its gradient, fp32 [n_rows]
 };
 
@@ -252,7 +262,7 @@ void launch(const GluArgs& a) {
           a.stride_gate, a.stride_up, a.n_rows, chunks, a.p);
   } else if (a.row_weight && !a.backward) {
     glu_fwd_weighted_kernel<T, W, kAct, kClampAct, kPlusOne><<<grid, block, 0, a.stream>>>(
-        static_cast<const T*>(a.gate), static_cast<const T*>(a.up), static_cast<const T*>(a.row_weight),
+        static_cast<const T*>(a.gate), static_cast<const T*>(a.up), a.row_weight, a.weight_f32,
         static_cast<T*>(a.out), a.stride_gate, a.stride_up, a.n_rows, chunks, a.width, a.p);
   } else if (a.row_weight) {
     // lanes per row: the power of two (16, 32 or 64) that leaves the fewest idle lane-iterations, larger on a tie
@@ -267,7 +277,7 @@ void launch(const GluArgs& a) {
 #define HMOE_GLU_BWD_W(L)                                                                                        \
   glu_bwd_weighted_kernel<T, W, L, kAct, kClampAct, kPlusOne><<<row_grid, block, 0, a.stream>>>(                 \
       static_cast<const T*>(a.gate), static_cast<const T*>(a.up), static_cast<const T*>(a.grad_out),             \
-      static_cast<const T*>(a.row_weight), static_cast<T*>(a.dgate), static_cast<T*>(a.dup), a.grad_weight,      \
+      a.row_weight, a.weight_f32, static_cast<T*>(a.dgate), static_cast<T*>(a.dup), a.grad_weight,               \
       a.stride_gate, a.stride_up, a.stride_dgate, a.stride_dup, a.n_rows, static_cast<int>(chunks), a.width, a.p)
     if (lanes == 64) HMOE_GLU_BWD_W(64);
     else if (lanes == 32) HMOE_GLU_BWD_W(32);
@@ -363,10 +373,13 @@ int hmoe_glu_fwd_quant_fp8(const void* gate, const void* up, int64_t stride_gate
 }
 
 int hmoe_glu_fwd_weighted(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up,
-                          const void* row_weight, int64_t n_rows, int64_t width, int dtype, int activation,
-                          float alpha, float limit, int clamp_activated, int up_plus_one, void* out, void* stream) {
+                          const void* row_weight, int weight_dtype, int64_t n_rows, int64_t width, int dtype,
+                          int activation, float alpha, float limit, int clamp_activated, int up_plus_one, void* out,
+                          void* stream) {
+  if (weight_dtype != dtype && weight_dtype != HMOE_F32) return HMOE_UNSUPPORTED;
   hmoe::GluArgs a{};
   a.gate = gate; a.up = up; a.out = out; a.row_weight = row_weight;
+  a.weight_f32 = weight_dtype == HMOE_F32 && dtype != HMOE_F32;
   a.stride_gate = stride_gate; a.stride_up = stride_up; a.n_rows = n_rows; a.width = width;
   a.p = {alpha, limit};
   a.backward = false;
@@ -376,10 +389,13 @@ int hmoe_glu_fwd_weighted(const void* gate, const void* up, int64_t stride_gate,
 }
 
 int hmoe_glu_bwd_weighted(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up,
-                          const void* grad_out, const void* row_weight, int64_t n_rows, int64_t width, int dtype,
-                          int activation, float alpha, float limit, int clamp_activated, int up_plus_one, void* dgate,
-                          void* dup, int64_t stride_dgate, int64_t stride_dup, float* grad_weight, void* stream) {
+                          const void* grad_out, const void* row_weight, int weight_dtype, int64_t n_rows,
+                          int64_t width, int dtype, int activation, float alpha, float limit, int clamp_activated,
+                          int up_plus_one, void* dgate, void* dup, int64_t stride_dgate, int64_t stride_dup,
+                          float* grad_weight, void* stream) {
+  if (weight_dtype != dtype && weight_dtype != HMOE_F32) return HMOE_UNSUPPORTED;
   hmoe::GluArgs a{};
+  a.weight_f32 = weight_dtype == HMOE_F32 && dtype != HMOE_F32;
   a.gate = gate; a.up = up; a.grad_out = grad_out; a.dgate = dgate; a.dup = dup;
   a.row_weight = row_weight; a.grad_weight = grad_weight;
   a.stride_gate = stride_gate; a.stride_up = stride_up; a.stride_dgate = stride_dgate; a.stride_dup = stride_dup;

@@ -180,7 +180,10 @@ class _WeightedPackedGLU(torch.autograd.Function):
         device = _lib.require_device(gate_up, row_weight)
         packed = _as_rows(gate_up)
         rows, half = packed.shape[0], packed.shape[1] // 2
-        weight = row_weight.to(packed.dtype).contiguous()
+        # fp32 weights beside bf16 rows go in as they are: the kernel rounds them to bf16 on the way in and their
+        # gradient on the way out, the bits of casting first, without the cast launches (one forward, two backward)
+        ctx.weight_f32 = row_weight.dtype == torch.float32 and packed.dtype == torch.bfloat16
+        weight = row_weight.contiguous() if ctx.weight_f32 else row_weight.to(packed.dtype).contiguous()
         ctx.combine, ctx.shape, ctx.weight_dtype = combine, gate_up.shape, row_weight.dtype
         ctx.save_for_backward(packed, weight)
         out = packed.new_empty((rows, half))
@@ -188,8 +191,8 @@ class _WeightedPackedGLU(torch.autograd.Function):
             gate, up = packed[:, :half], packed[:, half:]
             with _lib.on_device(device):
                 _lib.call("hmoe_glu_fwd_weighted", _lib.ptr(gate), _lib.ptr(up), gate.stride(0), up.stride(0),
-                          _lib.ptr(weight), rows, half, _lib.dtype_id(packed.dtype), *_kernel_args(combine),
-                          _lib.ptr(out), _lib.stream_ptr(device))
+                          _lib.ptr(weight), _lib.dtype_id(weight.dtype), rows, half, _lib.dtype_id(packed.dtype),
+                          *_kernel_args(combine), _lib.ptr(out), _lib.stream_ptr(device))
         return out
 
     @staticmethod
@@ -205,7 +208,8 @@ class _WeightedPackedGLU(torch.autograd.Function):
             dgate, dup = grad[:, :half], grad[:, half:]
             with _lib.on_device(device):
                 _lib.call("hmoe_glu_bwd_weighted", _lib.ptr(gate), _lib.ptr(up), gate.stride(0), up.stride(0),
-                          _lib.ptr(grad_out), _lib.ptr(weight), rows, half, _lib.dtype_id(packed.dtype),
+                          _lib.ptr(grad_out), _lib.ptr(weight), _lib.dtype_id(weight.dtype), rows, half,
+                          _lib.dtype_id(packed.dtype),
                           *_kernel_args(ctx.combine), _lib.ptr(dgate), _lib.ptr(dup), dgate.stride(0), dup.stride(0),
                           _lib.ptr(grad_weight), _lib.stream_ptr(device))
         else:
@@ -271,7 +275,8 @@ class GluCombine:
         if _FUSED_GLU_ENABLED and gate_up.is_cuda:
             return _WeightedPackedGLU.apply(gate_up, row_weight, self)
         gate, up = gate_up.chunk(2, dim=-1)
-        return (self._eager(gate, up).float() * row_weight.float().unsqueeze(-1)).to(gate_up.dtype)
+        weight = row_weight.to(gate_up.dtype).float()  # the rounding the kernel gives fp32 weights beside bf16 rows
+        return (self._eager(gate, up).float() * weight.unsqueeze(-1)).to(gate_up.dtype)
 
     def packed_quantized(self, gate_up: torch.Tensor):
         """``packed`` with its output as e4m3 panels and scale exponents for the fp8 expert GEMM

@@ -388,7 +388,9 @@ class EPMoELayerBase(ExpertLoadMixin, nn.Module, ABC):
         expert outputs are not kept, and the gate weights' gradient ``<grad_out[token], y_row>`` comes out of the
         GLU's backward as ``<grad_out[token] @ W_down^T, act_row>``, the same number."""
         gate_up = self._expert_proj(sorted_tokens.to(output_dtype), "gate_up_proj", offs, output_dtype)
-        weighted = self._fused_glu_mul.packed_weighted(gate_up, sorted_weights.to(output_dtype))
+        # the fp32 gate weights go in uncast: the kernel rounds them to the output dtype (sorted_weights.to(dt) of
+        # compute.py:241) and their gradient back through it
+        weighted = self._fused_glu_mul.packed_weighted(gate_up, sorted_weights)
         rows, scale = addend if addend is not None else (None, None)
         if addend_ready is not None:
             # the join: the down projection runs ahead of the sum in the same node, so it waits with it (the gate_up

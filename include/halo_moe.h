@@ -148,14 +148,20 @@ int hmoe_glu_bwd(const void* gate, const void* up, int64_t stride_gate, int64_t 
  * _gather_reduce_kernel (halo/kernels/moe_permute.py:33-41) and all of _weighted_unpermute_bwd_kernel (:44-72): since
  * sum_k w_k (act_k @ W) = sum_k (w_k act_k) @ W, the down projection runs on weighted rows, the combine is a plain
  * sum, and its backward needs neither the [R, H] gradient of the expert outputs nor the expert outputs themselves
- * (grad_weight[r] = <grad_out[tok r], y[r]> = <grad_out[tok r] @ W^T, act[r]>). */
+ * (grad_weight[r] = <grad_out[tok r], y[r]> = <grad_out[tok r] @ W^T, act[r]>).
+ * row_weight is [n_rows] of weight_dtype: `dtype`, or HMOE_F32 with bf16 operands, in which case each weight is rounded
+ * to bf16 on the way in and each grad_weight value on the way out: the bits of casting the weights first
+ * (sorted_weights.to(dtype), moe_layer/compute.py:241) and of the gradient that cast hands back, without the three
+ * small cast launches. */
 int hmoe_glu_fwd_weighted(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up,
-                          const void* row_weight, int64_t n_rows, int64_t width, int dtype, int activation,
-                          float alpha, float limit, int clamp_activated, int up_plus_one, void* out, void* stream);
+                          const void* row_weight, int weight_dtype, int64_t n_rows, int64_t width, int dtype,
+                          int activation, float alpha, float limit, int clamp_activated, int up_plus_one, void* out,
+                          void* stream);
 int hmoe_glu_bwd_weighted(const void* gate, const void* up, int64_t stride_gate, int64_t stride_up,
-                          const void* grad_out, const void* row_weight, int64_t n_rows, int64_t width, int dtype,
-                          int activation, float alpha, float limit, int clamp_activated, int up_plus_one, void* dgate,
-                          void* dup, int64_t stride_dgate, int64_t stride_dup, float* grad_weight, void* stream);
+                          const void* grad_out, const void* row_weight, int weight_dtype, int64_t n_rows,
+                          int64_t width, int dtype, int activation, float alpha, float limit, int clamp_activated,
+                          int up_plus_one, void* dgate, void* dup, int64_t stride_dgate, int64_t stride_dup,
+                          float* grad_weight, void* stream);
 
 /* ------------------------------------------------------------------------------------------------------ router
  * Replaces the softmax / top-k / renormalise / cast sequence of the family routers the layer calls
