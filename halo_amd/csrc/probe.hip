@@ -1,6 +1,9 @@
-// What the matrix pipe of this device sustains with nothing else to do: a loop of independent
-// v_mfma_f32_32x32x16_bf16 on register operands, two wavefronts per SIMD on every compute unit (the occupancy of the
-// grouped GEMM kernels).  A measuring stick for the benchmark's roofline figures; no counterpart in the reference.
+// What the matrix pipe of this device sustains with nothing else to do: a loop of independent bf16 MFMAs on register
+// operands, two wavefronts per SIMD on every compute unit (the occupancy of the grouped GEMM kernels).  Two shapes
+// (v_mfma_f32_32x32x16_bf16, the one the GEMM kernels use, and v_mfma_f32_16x16x32_bf16) and two kinds of operands:
+// small integers, which toggle few bits, and pseudo-random values with random signs, which load the multipliers the
+// way real activations and weights do -- the clock this part holds depends on the power the pipe draws.  A measuring
+// stick for the benchmark's roofline figures; no counterpart in the reference.
 #include "common.h"
 
 namespace hmoe {
@@ -8,31 +11,65 @@ namespace {
 
 typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
+typedef float probe_f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kProbeChains = 8;  // independent accumulators per wavefront: no MFMA waits for the one before it
 
-__global__ void __launch_bounds__(512) mfma_probe_kernel(int64_t iterations, float* sink) {
-  probe_f32x16 acc[kProbeChains];
-#pragma unroll
-  for (int c = 0; c < kProbeChains; ++c)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[c][v] = 0.f;
-  probe_bf16x8 a, b;
+// operand values of one lane: kRandom false = integers 0..3 and 0..1; true = a hash of (lane, element) mapped to
+// [-2, 2) with 8 significant bits, signs mixed so that the accumulators random-walk instead of growing
+template <bool kRandom>
+__device__ __forceinline__ void probe_operands(probe_bf16x8& a, probe_bf16x8& b) {
 #pragma unroll
   for (int v = 0; v < 8; ++v) {
-    a[v] = static_cast<__bf16>(static_cast<float>((threadIdx.x + v) & 3));
-    b[v] = static_cast<__bf16>(static_cast<float>((threadIdx.x ^ v) & 1));
+    if (kRandom) {
+      uint32_t h = (threadIdx.x * 8u + v + blockIdx.x * 4099u) * 2654435761u;
+      h ^= h >> 15;
+      h *= 2246822519u;
+      h ^= h >> 13;
+      a[v] = static_cast<__bf16>((static_cast<int>(h & 0x1ff) - 256) * (1.0f / 128));
+      b[v] = static_cast<__bf16>((static_cast<int>(h >> 16 & 0x1ff) - 256) * (1.0f / 128));
+    } else {
+      a[v] = static_cast<__bf16>(static_cast<float>((threadIdx.x + v) & 3));
+      b[v] = static_cast<__bf16>(static_cast<float>((threadIdx.x ^ v) & 1));
+    }
   }
-  for (int64_t i = 0; i < iterations; ++i) {
-#pragma unroll
-    for (int c = 0; c < kProbeChains; ++c) acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[c], 0, 0, 0);
-  }
+}
+
+template <bool kSmallShape, bool kRandom>
+__global__ void __launch_bounds__(512) mfma_probe_kernel(int64_t iterations, float* sink) {
+  probe_bf16x8 a, b;
+  probe_operands<kRandom>(a, b);
   float total = 0.f;
+  if (kSmallShape) {  // 16x16x32: four accumulator registers per chain, half the flops per instruction
+    probe_f32x4 acc[kProbeChains];
 #pragma unroll
-  for (int c = 0; c < kProbeChains; ++c)
+    for (int c = 0; c < kProbeChains; ++c) acc[c] = probe_f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int64_t i = 0; i < iterations; ++i) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) total += acc[c][v];
-  if (total == -1.f) sink[blockIdx.x] = total;  // never true (the sums are non-negative): keeps the loop alive
+      for (int c = 0; c < kProbeChains; ++c) acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[c], 0, 0, 0);
+    }
+#pragma unroll
+    for (int c = 0; c < kProbeChains; ++c)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) total += acc[c][v];
+  } else {
+    probe_f32x16 acc[kProbeChains];
+#pragma unroll
+    for (int c = 0; c < kProbeChains; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[c][v] = 0.f;
+    for (int64_t i = 0; i < iterations; ++i) {
+#pragma unroll
+      for (int c = 0; c < kProbeChains; ++c) acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[c], 0, 0, 0);
+    }
+#pragma unroll
+    for (int c = 0; c < kProbeChains; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) total += acc[c][v];
+  }
+  // never true for the integer operands (their sums are non-negative) and as good as never for the random ones: the
+  // store keeps the loop alive
+  if (total == -1.25f) sink[blockIdx.x] = total;
 }
 
 }  // namespace
@@ -40,17 +77,23 @@ __global__ void __launch_bounds__(512) mfma_probe_kernel(int64_t iterations, flo
 
 extern "C" {
 
-int64_t hmoe_probe_mfma_bf16(int64_t iterations, void* sink, void* stream) {
-  if (iterations <= 0 || sink == nullptr) return HMOE_INVALID_ARGUMENT;
+int64_t hmoe_probe_mfma_bf16(int64_t iterations, int shape, int operands, void* sink, void* stream) {
+  if (iterations <= 0 || sink == nullptr || shape < 0 || shape > 1 || operands < 0 || operands > 1)
+    return HMOE_INVALID_ARGUMENT;
   int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess ||
       hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
     return HMOE_LAUNCH_FAILED;
-  hmoe::mfma_probe_kernel<<<dim3(cus), dim3(512), 0, static_cast<hipStream_t>(stream)>>>(
-      iterations, static_cast<float*>(sink));
+  const dim3 grid(cus), block(512);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* out = static_cast<float*>(sink);
+  if (shape == 0 && operands == 0) hmoe::mfma_probe_kernel<false, false><<<grid, block, 0, s>>>(iterations, out);
+  if (shape == 0 && operands == 1) hmoe::mfma_probe_kernel<false, true><<<grid, block, 0, s>>>(iterations, out);
+  if (shape == 1 && operands == 0) hmoe::mfma_probe_kernel<true, false><<<grid, block, 0, s>>>(iterations, out);
+  if (shape == 1 && operands == 1) hmoe::mfma_probe_kernel<true, true><<<grid, block, 0, s>>>(iterations, out);
   if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
-  // multiply-adds counted twice: workgroups x wavefronts x iterations x chains x (32 x 32 x 16 x 2)
-  return static_cast<int64_t>(cus) * 8 * iterations * hmoe::kProbeChains * 32768;
+  // multiply-adds counted twice: workgroups x wavefronts x iterations x chains x (32 x 32 x 16 x 2 or 16 x 16 x 32 x 2)
+  return static_cast<int64_t>(cus) * 8 * iterations * hmoe::kProbeChains * (shape == 0 ? 32768 : 16384);
 }
 
 }  // extern "C"

@@ -178,10 +178,13 @@ int hmoe_router_topk_bwd(const void* logits, int dtype, const int64_t* indices, 
 
 /* ------------------------------------------------------------------------------------------------ device probe
  * No counterpart in the reference: a measuring stick for benchmarks.  Runs `iterations` rounds of eight independent
- * v_mfma_f32_32x32x16_bf16 per wavefront on register operands, two wavefronts per SIMD on every compute unit, and
- * returns the floating-point operations the launch performs (time it with events on `stream`), or a negative
- * hmoe_status.  `sink` is a device buffer of at least one float per compute unit (never written in practice). */
-int64_t hmoe_probe_mfma_bf16(int64_t iterations, void* sink, void* stream);
+ * bf16 MFMAs per wavefront on register operands, two wavefronts per SIMD on every compute unit, and returns the
+ * floating-point operations the launch performs (time it with events on `stream`), or a negative hmoe_status.
+ * shape 0 = v_mfma_f32_32x32x16_bf16 (what the GEMM kernels issue), 1 = v_mfma_f32_16x16x32_bf16; operands 0 = small
+ * integers (few bits toggle), 1 = pseudo-random values of mixed sign (the power real operands draw: the clock the part
+ * holds, and so the rate, depends on it).  `sink` is a device buffer of at least one float per compute unit (never
+ * written in practice). */
+int64_t hmoe_probe_mfma_bf16(int64_t iterations, int shape, int operands, void* sink, void* stream);
 
 /* ------------------------------------------------------------------------------------------------ grouped GEMM
  * Replace F.grouped_mm as called by halo/kernels/grouped_mm.py:16-47 (forward :39, dgrad :25, wgrad :26).
