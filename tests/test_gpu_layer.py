@@ -473,6 +473,48 @@ def test_dense_projection_weight_gradient_in_token_slices(device, tokens, width,
     assert all(torch.equal(a, b) for a, b in zip(results[0], results[1]))
 
 
+def test_sliced_weight_gradient_rounding_against_the_fp32_accumulated_gradient(device):
+    """The token slices' partial gradients are rounded to bf16 before they are summed (fp32 accumulation, one more
+    rounding), where a dense product accumulates every token in fp32 and rounds once.  On ordinary data the partials
+    add in quadrature and the result stays at the single-rounding floor (Frobenius error within 1.5x of rounding the
+    fp32-accumulated gradient once).  When the slices cancel (the second half of the tokens repeats the first with the
+    output gradient negated, plus a small remainder) the error is bounded by the partials, not by the result: at most
+    splits x 2^-9 x the largest partial magnitude per element."""
+    from halo_amd.moe_layer.layer import _DenseLinear, dense_mm
+
+    tokens, width, hidden = 8192, 512, 2048
+    g = torch.Generator().manual_seed(23)
+    x = torch.randn(tokens, hidden, generator=g).bfloat16()
+    w = (torch.randn(width, hidden, generator=g) * hidden ** -0.5).bfloat16()
+    dout = torch.randn(tokens, width, generator=g).bfloat16()
+    splits = _DenseLinear._splits_for(dout.to(device), x.to(device))
+    assert _DenseLinear._sliced_wgrad_usable(dout.to(device), x.to(device)) and splits >= 4
+
+    def sliced_gradient(rows, grads):
+        wd = w.to(device).requires_grad_(True)
+        dense_mm(rows.to(device), wd).backward(grads.to(device))
+        return wd.grad.double().cpu()
+
+    # ordinary data: at the floor of one bf16 rounding of the exact gradient
+    exact = dout.double().t() @ x.double()
+    floor = (exact.float().bfloat16().double() - exact).norm()
+    err = (sliced_gradient(x, dout) - exact).norm()
+    assert err <= 1.5 * floor, f"Frobenius error {err:.4e} against a rounding floor of {floor:.4e}"
+
+    # cancelling slices: tokens [half:] repeat tokens [:half] with the gradient negated, plus a remainder 2^-6 the size
+    half = tokens // 2
+    x2 = torch.cat([x[:half], x[:half]])
+    small = (torch.randn(half, width, generator=g) * 2.0 ** -6).bfloat16()
+    dout2 = torch.cat([dout[:half], (-dout[:half].float() + small.float()).bfloat16()])
+    exact2 = dout2.double().t() @ x2.double()
+    step = tokens // splits
+    largest_partial = max((dout2[i:i + step].double().t() @ x2[i:i + step].double()).abs().max().item()
+                          for i in range(0, tokens, step))
+    worst = (sliced_gradient(x2, dout2) - exact2).abs().max().item()
+    bound = splits * 2.0 ** -9 * largest_partial + 2.0 ** -8 * exact2.abs().max().item()
+    assert worst <= bound, f"largest error {worst:.4e} against the bound {bound:.4e}"
+
+
 class _SharedMlp(torch.nn.Module):
     def __init__(self, hidden, width, dtype, generator):
         super().__init__()
