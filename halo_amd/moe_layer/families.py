@@ -16,7 +16,7 @@ from halo_amd.kernels.grouped_mm import bias_fusable, grouped_mm_bias
 from halo_amd.kernels.moe_permute import MoEExpertBiasGather
 from halo_amd.kernels.router import SOFTMAX_TOPK, fused_topk_gate
 from halo_amd.moe_layer.config import GEMMA4, GPT_OSS, QWEN3, QWEN3_5
-from halo_amd.moe_layer.layer import EPMoELayerBase, EPSharedExpertsMoELayerBase
+from halo_amd.moe_layer.layer import EPMoELayerBase, EPSharedExpertsMoELayerBase, sigmoid_row_gate
 
 
 def split_interleaved_gate_up(interleaved: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
@@ -55,8 +55,8 @@ class EPQwen3_5MoELayer(EPSharedExpertsMoELayerBase):
         if gate is None:
             return rows, None
         x = hidden_states.reshape(-1, hidden_states.shape[-1])
-        # a [T, 1] projection is below the GEMM kernels' 16-byte row granularity: a matrix-vector product in torch
-        return rows, torch.sigmoid(torch.nn.functional.linear(x, gate.weight.to(x.dtype))).view(-1)
+        # a [T, 1] projection is below the GEMM kernels' 16-byte row granularity: a kernel of its own
+        return rows, sigmoid_row_gate(x, gate.weight)
 
     def replicated_named_params(self) -> list:
         extra = [] if getattr(self, "shared_expert_gate", None) is None else [

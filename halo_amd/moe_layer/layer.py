@@ -21,6 +21,7 @@ from typing import ClassVar
 import torch
 import torch.nn as nn
 
+from halo_amd import _lib
 from halo_amd.kernels.expert_gemm import BlockFp8Weight, expert_gemm, fp8_mfma_usable
 from halo_amd.kernels.fused_glu import GluCombine, fused_glu_enabled, resolve_fused_glu_mul
 from halo_amd.kernels.grouped_mm import (GatheredRows, addto_fusable, grouped_mm_addto, grouped_mm_combine,
@@ -130,6 +131,57 @@ def dense_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     if x.dim() == 2 and weight.dim() == 2 and x.dtype == weight.dtype == torch.bfloat16:
         return _DenseLinear.apply(x, weight)
     return torch.nn.functional.linear(x, weight)
+
+
+class _SigmoidRowGate(torch.autograd.Function):
+    """``sigmoid(x @ weight^T).view(-1)`` for ``weight [1, H]``: the shared expert's per-token output gate
+    (``families/qwen3_5.py:41-42`` of the reference: ``torch.sigmoid(self.shared_expert_gate(hidden_states))``), one
+    kernel forward and one (plus a small reduction) backward in place of the library's matrix-vector products, the
+    sigmoid and their autograd; rounded where those tensor operations round (``csrc/row_gate.hip``)."""
+
+    @staticmethod
+    def forward(ctx, x, weight):
+        device = _lib.require_device(x, weight)
+        gate = torch.empty(x.shape[0], dtype=x.dtype, device=device)
+        with _lib.on_device(device):
+            _lib.call("hmoe_row_gate_fwd", _lib.ptr(x), x.stride(0), _lib.ptr(weight), x.shape[0], x.shape[1],
+                      _lib.dtype_id(x.dtype), _lib.ptr(gate), _lib.stream_ptr(device))
+        ctx.save_for_backward(x, weight, gate)
+        return gate
+
+    @staticmethod
+    def backward(ctx, grad_gate):
+        x, weight, gate = ctx.saved_tensors
+        device = x.device
+        need_x, need_w = ctx.needs_input_grad
+        if not (need_x or need_w):
+            return None, None
+        grad_gate = grad_gate.to(x.dtype).contiguous()
+        grad_x = torch.empty_like(x, memory_format=torch.contiguous_format) if need_x else None
+        grad_w = torch.empty_like(weight, memory_format=torch.contiguous_format) if need_w else None
+        workspace = None
+        if need_w:
+            nbytes = _lib.load().hmoe_row_gate_bwd_workspace_bytes(x.shape[0], x.shape[1])
+            workspace = torch.empty(max(int(nbytes), 4) // 4, dtype=torch.float32, device=device)
+        with _lib.on_device(device):
+            _lib.call("hmoe_row_gate_bwd", _lib.ptr(x), x.stride(0), _lib.ptr(weight), _lib.ptr(gate),
+                      _lib.ptr(grad_gate), x.shape[0], x.shape[1], _lib.dtype_id(x.dtype), _lib.ptr(grad_x),
+                      grad_x.stride(0) if need_x else 0, _lib.ptr(grad_w), _lib.ptr(workspace),
+                      _lib.stream_ptr(device))
+        return grad_x, grad_w
+
+
+def sigmoid_row_gate(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``sigmoid(F.linear(x, weight)).view(-1)`` for ``x [T, H]`` and an ``nn.Linear(H, 1)`` weight ``[1, H]``;
+    differentiable in both.  Device tensors whose rows are 16-byte multiples take :class:`_SigmoidRowGate`; CPU
+    tensors and other shapes the tensor operations."""
+    weight = weight.to(x.dtype)
+    row_bytes_ok = x.dim() == 2 and (x.shape[1] * x.element_size()) % 16 == 0 and x.stride(1) == 1 \
+        and (x.stride(0) * x.element_size()) % 16 == 0 and x.data_ptr() % 16 == 0
+    if (x.is_cuda and row_bytes_ok and x.dtype in (torch.bfloat16, torch.float32) and weight.shape == (1, x.shape[1])
+            and weight.is_contiguous() and weight.data_ptr() % 16 == 0 and x.shape[0] > 0):
+        return _SigmoidRowGate.apply(x, weight)
+    return torch.sigmoid(torch.nn.functional.linear(x, weight)).view(-1)
 
 
 class EPMoELayerBase(ExpertLoadMixin, nn.Module, ABC):

@@ -176,6 +176,22 @@ int hmoe_router_topk_bwd(const void* logits, int dtype, const int64_t* indices, 
                          int64_t n_tokens, int num_experts, int top_k, int mode, int normalize, float eps,
                          void* grad_logits, void* stream);
 
+/* ------------------------------------------------------------------------------------------------ shared-expert gate
+ * Replace the sigmoid output gate of a shared expert, torch.sigmoid(self.shared_expert_gate(hidden_states)) with
+ * shared_expert_gate = nn.Linear(H, 1, bias=False) (halo/distributed/expert_parallel/families/qwen3_5.py:41-42), and
+ * its autograd.  gate[t] = sigmoid(<x[t], w>) for x [n_rows, hidden] (row stride ldx) and w [hidden], in the operands'
+ * dtype, rounded where the tensor operations round (the dot product in fp32 then rounded, the sigmoid in fp32 then
+ * rounded).  hidden and ldx multiples of 16 bytes, x and w 16-byte aligned (HMOE_UNSUPPORTED otherwise). */
+int hmoe_row_gate_fwd(const void* x, int64_t ldx, const void* w, int64_t n_rows, int hidden, int dtype, void* gate,
+                      void* stream);
+/* Backward: gs[t] = round(grad_gate[t] * (1 - gate[t]) * gate[t]); grad_x[t] = gs[t] * w (row stride ld_grad_x; may be
+ * NULL) and grad_w = sum_t gs[t] * x[t] (may be NULL), the sum in fp32 in a fixed order through `workspace`
+ * (hmoe_row_gate_bwd_workspace_bytes(n_rows, hidden) bytes, caller-owned; needed when grad_w is given). */
+int64_t hmoe_row_gate_bwd_workspace_bytes(int64_t n_rows, int hidden);
+int hmoe_row_gate_bwd(const void* x, int64_t ldx, const void* w, const void* gate, const void* grad_gate,
+                      int64_t n_rows, int hidden, int dtype, void* grad_x, int64_t ld_grad_x, void* grad_w,
+                      void* workspace, void* stream);
+
 /* ------------------------------------------------------------------------------------------------ device probe
  * No counterpart in the reference: a measuring stick for benchmarks.  Runs `iterations` rounds of eight independent
  * bf16 MFMAs per wavefront on register operands, two wavefronts per SIMD on every compute unit, and returns the

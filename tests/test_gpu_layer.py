@@ -515,6 +515,59 @@ def test_sliced_weight_gradient_rounding_against_the_fp32_accumulated_gradient(d
     assert worst <= bound, f"largest error {worst:.4e} against the bound {bound:.4e}"
 
 
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float32), ids=("bf16", "fp32"))
+@pytest.mark.parametrize(("tokens", "hidden", "pitch"), ((8192, 2048, 2048), (1027, 264, 264), (45, 512, 640), (3, 64, 64)))
+def test_sigmoid_row_gate_against_the_tensor_operations(device, dtype, tokens, hidden, pitch):
+    """``sigmoid_row_gate`` (the shared expert's per-token output gate, one kernel per direction) against
+    ``sigmoid(x @ w^T)`` and its autograd in fp64 over the same inputs: the gate within one rounding of the dtype, the
+    gradients within the BASELINE tolerance (fp32: 1e-5); row counts that do not fill a workgroup's share, a hidden
+    size of 33 chunks, rows read from a wider buffer; two runs bit-equal."""
+    from halo_amd.moe_layer.layer import _SigmoidRowGate, sigmoid_row_gate
+
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(tokens, pitch, generator=g).to(dtype)
+    w = (torch.randn(1, hidden, generator=g) * hidden ** -0.5 * 2).to(dtype)
+    grad = torch.randn(tokens, generator=g).to(dtype)
+    results = []
+    for _ in range(2):
+        xd = x.to(device)[:, :hidden].requires_grad_(True)
+        wd = w.to(device).requires_grad_(True)
+        gate = sigmoid_row_gate(xd, wd)
+        assert isinstance(gate.grad_fn, _SigmoidRowGate._backward_cls)
+        gate.backward(grad.to(device))
+        results.append((gate.detach().clone(), xd.grad.clone(), wd.grad.clone()))
+    assert all(torch.equal(a, b) for a, b in zip(results[0], results[1]))
+    gate, gx, gw = (t.double().cpu() for t in results[0])
+    xr = x[:, :hidden].double().requires_grad_(True)
+    wr = w.double().requires_grad_(True)
+    want = torch.sigmoid(xr @ wr.t()).view(-1)
+    want.backward(grad.double())
+    # the logit is rounded to the dtype before the sigmoid (the linear's output): |d sigmoid| <= |d logit| / 4; in fp32
+    # the dot product's own accumulation error (hidden terms) is what is left
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -23 * hidden ** 0.5
+    logit = (xr @ wr.t()).view(-1).detach()
+    assert ((gate - want.detach()).abs() <= ulp * (want.detach() + logit.abs() / 4 + 1e-3)).all()
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
+    _check("grad x", gx, xr.grad, tol)
+    _check("grad w", gw, wr.grad, tol)
+
+
+def test_sigmoid_row_gate_roundings_are_the_tensor_operations(device):
+    """Given the same gate values, ``grad_x`` is the tensor operations' bit for bit: sigmoid's backward in fp32 rounded
+    to bf16, then one product per element rounded once (an outer product has no summation order)."""
+    from halo_amd.moe_layer.layer import sigmoid_row_gate
+
+    g = torch.Generator().manual_seed(33)
+    x = torch.randn(4096, 1024, generator=g).bfloat16().to(device).requires_grad_(True)
+    w = (torch.randn(1, 1024, generator=g) * 0.05).bfloat16().to(device).requires_grad_(True)
+    grad = torch.randn(4096, generator=g).bfloat16().to(device)
+    gate = sigmoid_row_gate(x, w)
+    gate.backward(grad)
+    y = gate.detach().float()
+    scaled = (grad.float() * (1.0 - y) * y).bfloat16()
+    assert torch.equal(x.grad, (scaled.float()[:, None] * w.detach().float()).bfloat16())
+
+
 class _SharedMlp(torch.nn.Module):
     def __init__(self, hidden, width, dtype, generator):
         super().__init__()
