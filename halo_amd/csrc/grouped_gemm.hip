@@ -1426,7 +1426,8 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
   sched.init(p, grp_s, grp_e, tile_start);
   // the same for every tile; an e2m1 panel holds 128 values, its last one zeros past K
   const int steps = kFp4 ? static_cast<int>((p.k + 127) / 128) : static_cast<int>(p.k / kF8K);
-  const uint32_t a_panel = static_cast<uint32_t>(p.a_scale_rows) * kF8K, b_panel = static_cast<uint32_t>(p.n) * kF8K;
+  const int64_t a_panel = p.a_scale_rows * kF8K;  // bytes of one panel of the activations
+  const uint32_t b_panel = static_cast<uint32_t>(p.n) * kF8K;
   const int64_t w_bytes = static_cast<int64_t>(steps) * kF8K * p.n;
 
   // ---- the loading wavefronts' view of a tile
@@ -1437,12 +1438,20 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
   // expert's rows, or zeros past the array's end): they reach only output rows and columns that are not stored.
   const uint32_t lane_off =
       static_cast<uint32_t>(lane >> 2) * kF8K + (((lane & 3) ^ ((lane >> 3) & 3) ^ ((lane >> 5) & 1)) << 4);
-  u32x4 rsrc_a, rsrc_b, rsrc_sa, rsrc_sb;
-  uint32_t voff_a = 0, voff_b = 0, voff_sa = 0, voff_sb = 0;
+  // The activations' descriptor is rebased every stage: it starts at the tile's first row in the stage's panel and
+  // spans the tile's rows there (or what the panel holds past them), so the offsets inside it are a tile's 16 KB
+  // whatever the number of rows or panels (the panels of a long batch exceed 32 bits of bytes).
+  u32x4 rsrc_b, rsrc_sa, rsrc_sb;
+  const uint8_t* a_tile = nullptr;  // the tile's first row in panel 0
+  uint32_t a_extent = 0;            // bytes from there to the tile's last row, or to the panel's end
+  const uint32_t voff_a = static_cast<uint32_t>(slot * 64) * kF8K + lane_off;
+  uint32_t voff_b = 0, voff_sa = 0, voff_sb = 0;
   auto describe = [&](const TileInfo& tile) __attribute__((always_inline)) {
     if (load_wave) {
-      const uint8_t* a = static_cast<const uint8_t*>(p.a) + static_cast<int64_t>(tile.row_start) * kF8K;
-      rsrc_a = make_rsrc_words(a, static_cast<uint32_t>(steps) * a_panel - static_cast<uint32_t>(tile.row_start) * kF8K);
+      const int64_t row0 = static_cast<int64_t>(tile.row_start) + tile.a_out0;
+      a_tile = static_cast<const uint8_t*>(p.a) + row0 * kF8K;
+      const int64_t rows_left = p.a_scale_rows - row0;
+      a_extent = static_cast<uint32_t>(rows_left < BM ? rows_left : BM) * kF8K;
       rsrc_b = make_rsrc_words(static_cast<const uint8_t*>(p.b) + tile.g * w_bytes, static_cast<uint32_t>(w_bytes));
       rsrc_sa = make_rsrc_words(p.a_scale, static_cast<uint32_t>(p.k_blocks) * static_cast<uint32_t>(p.a_scale_rows));
       if constexpr (kMx)  // k_blocks counts the exponent bytes per row or column (MXFP4: four per panel)
@@ -1450,7 +1459,6 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
                                   static_cast<uint32_t>(p.k_blocks) * static_cast<uint32_t>(p.n));
       else
         rsrc_sb = make_rsrc_words(p.b_scale, static_cast<uint32_t>(p.groups) * p.k_blocks * p.n_blocks * 4u);
-      voff_a = static_cast<uint32_t>(tile.a_out0 + slot * 64) * kF8K + lane_off;
       voff_b = static_cast<uint32_t>(tile.b_out0 + slot * 64) * kF8K + lane_off;
       // the dword this lane's byte lands in is d = 64 slot + lane; it takes the scale of tile row
       // (d >> 7) * 128 + (d & 3) * 32 + ((d & 127) >> 2), so that the four row blocks of a wavefront's lane lie in
@@ -1476,9 +1484,10 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
   auto issue = [&](int step) __attribute__((always_inline)) {
     const int buf = step & (kF8Stages - 1);
     lds_bytes_ptr ta = lds + buf * kF8Stage + slot * 4096;
-    const uint32_t soff_a = static_cast<uint32_t>(step) * a_panel, soff_b = static_cast<uint32_t>(step) * b_panel;
+    const uint32_t soff_b = static_cast<uint32_t>(step) * b_panel;
+    const u32x4 rsrc_a = make_rsrc_words(a_tile + static_cast<int64_t>(step) * a_panel, a_extent);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) lds_load16(rsrc_a, ta + t * 1024, voff_a + t * 1024, soff_a);
+    for (int t = 0; t < 4; ++t) lds_load16(rsrc_a, ta + t * 1024, voff_a + t * 1024, 0u);
 #pragma unroll
     for (int t = 0; t < 4; ++t) lds_load16(rsrc_b, ta + kF8Tile + t * 1024, voff_b + t * 1024, soff_b);
     lds_bytes_ptr sc = lds + kF8ScaleBase + buf * (kF8ScaleA + kF8ScaleB);
@@ -1733,8 +1742,11 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
         for (int st = 0; st < 3 && st < steps; ++st) issue(st);
     }
 
-    bf16_t* c_base = c + done.row_start * p.ldc;
-    const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(c_base, static_cast<uint32_t>(done.a_out_lim * p.ldc * 2));
+    // the output descriptor spans this tile's rows only, so its 32-bit offsets hold whatever the batch's size
+    const int c_row_lim = done.a_out_lim - done.a_out0;
+    bf16_t* c_base = c + (static_cast<int64_t>(done.row_start) + done.a_out0) * p.ldc;
+    const __amdgpu_buffer_rsrc_t c_rsrc =
+        make_rsrc(c_base, static_cast<uint32_t>((c_row_lim < BM ? c_row_lim : BM) * p.ldc * 2));
     stores_out = 4 * live;
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
@@ -1754,11 +1766,11 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
           for (int pass = 0; pass < 2; ++pass) {
             const int rr = pass * 16 + (lane >> 2);
             const int cc = (lane & 3) << 3;
-            const int row = done.a_out0 + row_a + i * 32 + rr;
+            const int row = row_a + i * 32 + rr;  // from the descriptor's first row
             const int col = done.b_out0 + row_b + j * 32 + cc;
             u32x4 v = *reinterpret_cast<const u32x4*>(stage_rows + (rr * kEpiPitch + cc) * 2);
             if constexpr (kBias) v = add_bf16x8(v, bias_chunk[j]);
-            const uint32_t off = row < done.a_out_lim && col < done.b_out_lim
+            const uint32_t off = row < c_row_lim && col < done.b_out_lim
                                      ? static_cast<uint32_t>(row) * static_cast<uint32_t>(p.ldc) * 2u + col * 2u
                                      : kOutOfRange;
             __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, off, 0, 0);
@@ -2038,15 +2050,17 @@ int launch_fp8(const GemmArgs& p, int64_t workers, void* stream) {
   return HMOE_OK;
 }
 
-// Whether the scaled-MFMA kernel can address the operands of an MX product: it bases its buffer descriptors at the
-// arrays' starts, so every array must stay below 2 GiB (the bf16 kernels rebase theirs per tile and have no such
-// limit; a caller with larger operands multiplies the round-tripped operands there).
+// Whether the scaled-MFMA kernel can address the operands of an MX product.  The quantised activations and the output
+// may be of any size (their descriptors are rebased per stage and per tile); what must stay below 2 GiB is one
+// expert's weight panels, the rows' exponent bytes and a tile's 256 output rows.  A caller whose operands do not fit
+// multiplies the round-tripped operands on the bf16 kernels.
 bool mx_product_fits(int64_t a_rows, int64_t total_rows, int64_t k, int64_t n, int64_t ldo, int panel_values) {
   if (a_rows < 0 || total_rows < 0 || k < 0 || n < 0 || ldo < 0 || (panel_values != 64 && panel_values != 128)) return false;
   const int64_t lim = int64_t(1) << 31, panels = (k + panel_values - 1) / panel_values;
   // products of two values below 2^31 each stay inside int64
   if (a_rows >= lim || total_rows >= lim || panels >= lim || n >= lim || ldo >= lim) return false;
-  return a_rows * panels < lim / 64 && panels * n < lim / 64 && total_rows * ldo < lim / 2;
+  // one expert's weight panels, the rows' exponent bytes (a dword per row and panel for e2m1) and 256 output rows
+  return panels * n < lim / 64 && a_rows * panels * 4 < lim && 256 * ldo < lim / 2;
 }
 
 // The MX products' arguments, checked: `panel_values` contraction values lie in a panel's 64 bytes (64 for e4m3, 128 for
@@ -2251,7 +2265,10 @@ int hmoe_grouped_gemm_fwd_fp8(const uint8_t* a_q, const uint8_t* a_scale, int64_
     return HMOE_UNSUPPORTED;
   const int64_t lim = int64_t(1) << 31;
   const int64_t k_blocks = k / 128, n_blocks = (n + 127) / 128;
-  if (a_rows * k >= lim || k * n >= lim || total_rows * ldo * 2 >= lim || num_groups * k_blocks * n_blocks * 4 >= lim)
+  // activations and output of any size (descriptors rebased per stage and per tile); below 2 GiB: one expert's weight,
+  // the rows' exponent bytes, the weight scales, a tile's 256 output rows
+  if (a_rows >= lim || total_rows >= lim || a_rows * k_blocks >= lim || k * n >= lim || 256 * ldo * 2 >= lim ||
+      num_groups * k_blocks * n_blocks * 4 >= lim)
     return HMOE_UNSUPPORTED;
   GemmArgs p{};
   p.a = a_q;

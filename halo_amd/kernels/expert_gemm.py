@@ -110,8 +110,9 @@ def expert_gemm(
 
 def mxfp8_mfma_usable(mat_a_dtype: torch.dtype, mat_b_dtype: torch.dtype, k: int, n: int, rows: int = 0) -> bool:
     """Whether the scaled e4m3 MFMA kernel takes the product: bf16 operands, whole panels of 64 values along K,
-    16-byte output rows, and ``rows`` activation rows whose quantised panels and output the kernel can address (each
-    array below 2 GiB: the library's own check, ``hmoe_grouped_gemm_mx_fits``).  Anything else multiplies the two
+    16-byte output rows, and ``rows`` activation rows whose operands the kernel can address (activations and output of
+    any size; one expert's weights and the rows' exponent bytes below 2 GiB: the library's own check,
+    ``hmoe_grouped_gemm_mx_fits``).  Anything else multiplies the two
     round-tripped operands on the bf16 / fp32 kernel, which is the reference's own formulation."""
     return (mat_a_dtype == torch.bfloat16 and mat_b_dtype == torch.bfloat16 and k > 0 and k % 64 == 0
             and n % 8 == 0 and bool(_lib.load().hmoe_grouped_gemm_mx_fits(rows, rows, k, n, n, 64)))

@@ -369,10 +369,11 @@ int hmoe_grouped_gemm_fwd_mxfp8(const uint8_t* a_q, const uint8_t* a_scale, int6
                                 int64_t k, int64_t n, void* out, int64_t ldo, void* stream);
 
 /* Whether hmoe_grouped_gemm_fwd_mxfp8 (panel_values 64) / hmoe_grouped_gemm_fwd_mxfp4 (panel_values 128) can address
- * operands of these sizes: the scaled-MFMA kernel bases its descriptors at the arrays' starts, so the quantised
- * activations (a_rows rows), one expert's quantised weights and the output (total_rows x ldo) must each stay below
- * 2 GiB; beyond that the entry points return HMOE_UNSUPPORTED and a caller multiplies the round-tripped operands on the
- * bf16 kernels, which have no such limit (what halo_amd.kernels.expert_gemm does).  1 or 0; launches nothing. */
+ * operands of these sizes.  The quantised activations and the output may be of any size (the kernel rebases their
+ * descriptors per pipeline stage and per tile); one expert's quantised weights, the rows' exponent bytes (counted as
+ * four per row and panel) and 256 output rows (256 x ldo x 2 bytes) must each stay below 2 GiB; beyond that the entry
+ * points return HMOE_UNSUPPORTED and a caller multiplies the round-tripped operands on the bf16 kernels (what
+ * halo_amd.kernels.expert_gemm does).  1 or 0; launches nothing. */
 int hmoe_grouped_gemm_mx_fits(int64_t a_rows, int64_t total_rows, int64_t k, int64_t n, int64_t ldo, int panel_values);
 
 /* ------------------------------------------------------------------------------------------------------- MXFP4

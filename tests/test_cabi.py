@@ -231,8 +231,9 @@ def test_bad_arguments_come_back_as_status_codes_before_any_launch():
 
 
 def test_mx_size_check_is_the_entry_points_own_and_the_predicates_follow_it():
-    """The MX products' scaled-MFMA kernel addresses each array from its start: quantised activations, one expert's
-    quantised weights and the output must stay below 2 GiB.  ``hmoe_grouped_gemm_mx_fits`` is the check the entry
+    """The MX products' scaled-MFMA kernel rebases the activations' descriptor per stage and the output's per tile, so
+    neither has a size limit; one expert's quantised weights, the rows' exponent bytes (counted as four per row and
+    panel) and a tile's 256 output rows must stay below 2 GiB.  ``hmoe_grouped_gemm_mx_fits`` is the check the entry
     points run; the Python predicates that route an oversized product to the round trip on the bf16 kernels call it,
     so the two cannot disagree.  Both sides of each boundary."""
     from halo_amd.kernels.expert_gemm import mxfp4_mfma_usable, mxfp8_mfma_usable
@@ -240,23 +241,24 @@ def test_mx_size_check_is_the_entry_points_own_and_the_predicates_follow_it():
     lib = _lib.load()
     two_gib = 2**31
     k, n = 2048, 1536
-    out_limit = -(-two_gib // (2 * n))      # rows at which the bf16 output reaches 2 GiB
-    assert lib.hmoe_grouped_gemm_mx_fits(out_limit - 1, out_limit - 1, k, n, n, 64) == 1
-    assert lib.hmoe_grouped_gemm_mx_fits(out_limit, out_limit, k, n, n, 64) == 0
-    act_limit = two_gib // k                # rows at which the e4m3 panels reach 2 GiB (narrow output)
-    assert lib.hmoe_grouped_gemm_mx_fits(act_limit - 1, act_limit - 1, k, 8, 8, 64) == 1
-    assert lib.hmoe_grouped_gemm_mx_fits(act_limit, act_limit, k, 8, 8, 64) == 0
-    assert lib.hmoe_grouped_gemm_mx_fits(2 * act_limit - 1, 2 * act_limit - 1, k, 8, 8, 128) == 1  # e2m1: half the bytes
-    assert lib.hmoe_grouped_gemm_mx_fits(2 * act_limit, 2 * act_limit, k, 8, 8, 128) == 0
+    assert lib.hmoe_grouped_gemm_mx_fits(4_000_000, 4_000_000, k, n, n, 64) == 1  # 12 GB of output, 8 GB of panels
+    scale_limit = -(-two_gib // (4 * (k // 64)))  # rows at which the exponent bytes reach 2 GiB
+    assert lib.hmoe_grouped_gemm_mx_fits(scale_limit - 1, scale_limit - 1, k, 8, 8, 64) == 1
+    assert lib.hmoe_grouped_gemm_mx_fits(scale_limit, scale_limit, k, 8, 8, 64) == 0
+    assert lib.hmoe_grouped_gemm_mx_fits(2 * scale_limit - 1, 2 * scale_limit - 1, k, 8, 8, 128) == 1  # half the panels
+    assert lib.hmoe_grouped_gemm_mx_fits(2 * scale_limit, 2 * scale_limit, k, 8, 8, 128) == 0
     assert lib.hmoe_grouped_gemm_mx_fits(16, 16, 32768, 65536, 65536, 64) == 0  # one expert's weights at 2 GiB
     assert lib.hmoe_grouped_gemm_mx_fits(16, 16, 32768, 65528, 65528, 64) == 1
+    wide = two_gib // (2 * 256)             # an output pitch at which 256 rows reach 2 GiB
+    assert lib.hmoe_grouped_gemm_mx_fits(16, 16, 64, 8, wide - 8, 64) == 1
+    assert lib.hmoe_grouped_gemm_mx_fits(16, 16, 64, 8, wide, 64) == 0
     assert lib.hmoe_grouped_gemm_mx_fits(-1, 0, k, n, n, 64) == 0 and lib.hmoe_grouped_gemm_mx_fits(1, 1, k, n, n, 32) == 0
     bf16 = torch.bfloat16
-    for rows in (out_limit - 1, out_limit, 10 * out_limit):
-        fits = rows < out_limit
+    for rows in (scale_limit - 1, scale_limit, 10 * scale_limit):
+        fits = rows < scale_limit
         assert mxfp8_mfma_usable(bf16, bf16, k, n, rows) == fits
-        assert mxfp4_mfma_usable(bf16, bf16, k, n, rows) == fits
+        assert mxfp4_mfma_usable(bf16, bf16, k, n, rows) == (rows < 2 * scale_limit)
     # the entry point itself refuses what the check refuses, before any launch
     fake = 4096  # a non-null, 16-byte aligned address that is never dereferenced on the host
-    rc = lib.hmoe_grouped_gemm_fwd_mxfp8(fake, fake, out_limit, fake, fake, None, out_limit, 1, k, n, fake, n, None)
+    rc = lib.hmoe_grouped_gemm_fwd_mxfp8(fake, fake, scale_limit, fake, fake, None, scale_limit, 1, k, n, fake, n, None)
     assert rc == -2
