@@ -42,6 +42,7 @@ SIGNATURES = {
     "hmoe_router_topk_fwd": (I, [P, I, L, I, I, I, I, F, P, P, P]),
     "hmoe_router_topk_bwd": (I, [P, I, P, P, L, I, I, I, I, F, P, P]),
     "hmoe_probe_mfma_bf16": (L, [L, I, I, P, P]),
+    "hmoe_probe_hbm_read": (L, [P, L, P, P]),
     "hmoe_row_gate_fwd": (I, [P, L, P, L, I, I, P, P]),
     "hmoe_row_gate_bwd_workspace_bytes": (L, [L, I]),
     "hmoe_row_gate_bwd": (I, [P, L, P, P, P, L, I, I, P, L, P, P, P]),

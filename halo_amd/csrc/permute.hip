@@ -154,15 +154,17 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
       constexpr bool kDense = decltype(dense_tag)::value;
       int64_t c = static_cast<int64_t>(lane_id()) * W;
       if constexpr (kDense && kTopK <= 8) {
-        // two column chunks per pass while the row has them: 2 * kTopK row fetches in flight per lane
-        for (; c + step < hidden; c += 2 * step) {
-          Pack<T, W> x[2][kTopK], acc[2], extra_chunk[2];
+        // four column chunks per pass while the row has them (a whole row of 2048 bf16), then two: 4 * kTopK row
+        // fetches in flight per lane at two wavefronts per SIMD (two chunks per pass at three wavefronts: 6 % slower)
+        auto pass = [&](auto width_tag) __attribute__((always_inline)) {
+          constexpr int kWide = decltype(width_tag)::value;
+          Pack<T, W> x[kWide][kTopK], acc[kWide], extra_chunk[kWide];
 #pragma unroll
-          for (int h = 0; h < 2; ++h)
+          for (int h = 0; h < kWide; ++h)
 #pragma unroll
             for (int k = 0; k < kTopK; ++k) x[h][k].load_once(from[k] + c + h * step);
 #pragma unroll
-          for (int h = 0; h < 2; ++h) {
+          for (int h = 0; h < kWide; ++h) {
             if (extra) extra_chunk[h].load(extra + c + h * step);
 #pragma unroll
             for (int i = 0; i < W; ++i) acc[h].v[i] = 0.f;
@@ -174,7 +176,9 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
             finish(acc[h], extra_chunk[h]);
             acc[h].store(to + c + h * step);
           }
-        }
+        };
+        for (; c + 3 * step < hidden; c += 4 * step) pass(std::integral_constant<int, 4>{});
+        for (; c + step < hidden; c += 2 * step) pass(std::integral_constant<int, 2>{});
       }
       for (; c < hidden; c += step) {
         Pack<T, W> x[kTopK], acc, extra_chunk;
@@ -209,8 +213,8 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
     // Some slots are not this rank's (most of them on one GPU's share of an expert-parallel layer).  The valid ones are
     // moved to the front, in slot order (the sum keeps its order; a slot left out adds the +0.0f it added before), and
     // the row is reduced by the loop written for that many sources: every fetch of a pass goes out before the first is
-    // used, and a row with few sources takes more column chunks per pass, so that 8 to 12 fetches are in flight per
-    // lane whatever the count.  Everything here is the same for the whole wavefront (scalar registers, one branch).
+    // used, four column chunks per pass while the row has them, so that 4 to 28 fetches are in flight per lane.
+    // Everything here is the same for the whole wavefront (scalar registers, one branch).
     const T* live_from[kTopK];
     float live_w[kTopK];
     int n_live = 0;
@@ -268,10 +272,10 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
       case 1: reduce_live(integral_constant<int, 1>{}, integral_constant<int, 4>{}); break;
       case 2: reduce_live(integral_constant<int, 2>{}, integral_constant<int, 4>{}); break;
       case 3: reduce_live(integral_constant<int, (kTopK >= 3 ? 3 : 1)>{}, integral_constant<int, 4>{}); break;
-      case 4: reduce_live(integral_constant<int, (kTopK >= 4 ? 4 : 1)>{}, integral_constant<int, 2>{}); break;
-      case 5: reduce_live(integral_constant<int, (kTopK >= 5 ? 5 : 1)>{}, integral_constant<int, 2>{}); break;
-      case 6: reduce_live(integral_constant<int, (kTopK >= 6 ? 6 : 1)>{}, integral_constant<int, 2>{}); break;
-      case 7: reduce_live(integral_constant<int, (kTopK >= 7 ? 7 : 1)>{}, integral_constant<int, 2>{}); break;
+      case 4: reduce_live(integral_constant<int, (kTopK >= 4 ? 4 : 1)>{}, integral_constant<int, 4>{}); break;
+      case 5: reduce_live(integral_constant<int, (kTopK >= 5 ? 5 : 1)>{}, integral_constant<int, 4>{}); break;
+      case 6: reduce_live(integral_constant<int, (kTopK >= 6 ? 6 : 1)>{}, integral_constant<int, 4>{}); break;
+      case 7: reduce_live(integral_constant<int, (kTopK >= 7 ? 7 : 1)>{}, integral_constant<int, 4>{}); break;
       default: reduce_row(std::false_type{}); break;
     }
   } else {

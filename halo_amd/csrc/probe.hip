@@ -72,10 +72,39 @@ __global__ void __launch_bounds__(512) mfma_probe_kernel(int64_t iterations, flo
   if (total == -1.25f) sink[blockIdx.x] = total;
 }
 
+// A read-only stream: every 16 bytes of `src` fetched once (non-temporal, eight fetches in flight per lane), folded
+// into a value that is never stored.  What the memory system delivers to a kernel that only reads.
+typedef unsigned int probe_u32x4 __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(256) hbm_read_probe_kernel(const probe_u32x4* __restrict__ src, int64_t n16,
+                                                             probe_u32x4* sink) {
+  probe_u32x4 acc = {0u, 0u, 0u, 0u};
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+  int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  for (; i + 7 * stride < n16; i += 8 * stride) {
+    probe_u32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= v[u];
+  }
+  for (; i < n16; i += stride) acc ^= __builtin_nontemporal_load(src + i);
+  if (acc[0] == 0x12345678u && acc[1] == 77u && acc[2] == 5u) sink[0] = acc;  // keeps the loads alive
+}
+
 }  // namespace
 }  // namespace hmoe
 
 extern "C" {
+
+int64_t hmoe_probe_hbm_read(const void* src, int64_t bytes, void* sink, void* stream) {
+  if (bytes < 0 || bytes % 16 || (bytes > 0 && (!src || !sink))) return HMOE_INVALID_ARGUMENT;
+  if (!hmoe::aligned16(src) || !hmoe::aligned16(sink)) return HMOE_UNSUPPORTED;
+  if (bytes == 0) return 0;
+  hmoe::hbm_read_probe_kernel<<<dim3(8192), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const hmoe::probe_u32x4*>(src), bytes / 16, static_cast<hmoe::probe_u32x4*>(sink));
+  if (hipGetLastError() != hipSuccess) return HMOE_LAUNCH_FAILED;
+  return bytes;
+}
 
 int64_t hmoe_probe_mfma_bf16(int64_t iterations, int shape, int operands, void* sink, void* stream) {
   if (iterations <= 0 || sink == nullptr || shape < 0 || shape > 1 || operands < 0 || operands > 1)

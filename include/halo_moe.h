@@ -201,6 +201,10 @@ int hmoe_row_gate_bwd(const void* x, int64_t ldx, const void* w, const void* gat
  * holds, and so the rate, depends on it).  `sink` is a device buffer of at least one float per compute unit (never
  * written in practice). */
 int64_t hmoe_probe_mfma_bf16(int64_t iterations, int shape, int operands, void* sink, void* stream);
+/* The same kind of stick for the memory side: reads `bytes` (a multiple of 16, 16-byte aligned) from `src` once with
+ * non-temporal 16-byte fetches and stores nothing; returns the bytes read, or a negative hmoe_status.  `sink` is 16
+ * bytes of device memory (never written in practice). */
+int64_t hmoe_probe_hbm_read(const void* src, int64_t bytes, void* sink, void* stream);
 
 /* ------------------------------------------------------------------------------------------------ grouped GEMM
  * Replace F.grouped_mm as called by halo/kernels/grouped_mm.py:16-47 (forward :39, dgrad :25, wgrad :26).
