@@ -86,11 +86,13 @@ dequantize_kernel(const uint8_t* __restrict__ q, const float* __restrict__ scale
 __global__ void __launch_bounds__(256)
 quantize_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const int64_t* __restrict__ row_index, int64_t x_rows,
                      int64_t rows, int k, uint8_t* __restrict__ q, uint8_t* __restrict__ scale, int64_t out_rows) {
-  const int chunks = k >> 3;
-  const int64_t unit = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  const int64_t row = unit / chunks;
-  const int chunk = static_cast<int>(unit - row * chunks);
-  if (row >= rows) return;  // whole groups of sixteen lanes leave together (chunks is a multiple of 16)
+  // A workgroup takes sixteen consecutive rows of one scale block (128 values, two panels): a row's sixteen lanes read
+  // its 256 bytes (two whole lines) and the sixteen rows' halves land side by side in each panel, 1 KB in one piece.
+  // (With a workgroup walking along one row, every row's 64 bytes of a panel were a write of their own.)
+  const int row_in = threadIdx.x >> 4, lane16 = threadIdx.x & 15;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 16 + row_in;
+  const int chunk = static_cast<int>(blockIdx.y) * 16 + lane16;
+  if (row >= rows) return;  // whole groups of sixteen lanes leave together
   Vec16<bf16_t> in;
   const int64_t from = row_index ? row_index[row] : row;
   if (from >= 0 && from < x_rows) {
@@ -116,11 +118,10 @@ int hmoe_quantize_rows_fp8(const void* x, int64_t ldx, const int64_t* row_index,
   if (rows == 0 || k == 0) return HMOE_OK;
   if (!q || !scale || (!x && x_rows > 0)) return HMOE_INVALID_ARGUMENT;
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(q) % 8) return HMOE_UNSUPPORTED;
-  const int64_t units = rows * (k / 8);
-  const int64_t blocks = (units + 255) / 256;
-  if (blocks >= (int64_t(1) << 31) || k >= (int64_t(1) << 31)) return HMOE_UNSUPPORTED;
+  const int64_t row_groups = (rows + 15) / 16, col_blocks = k / kBlock;
+  if (row_groups >= (int64_t(1) << 31) || col_blocks > 65535) return HMOE_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  quantize_rows_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(
+  quantize_rows_kernel<<<dim3(static_cast<unsigned>(row_groups), static_cast<unsigned>(col_blocks)), dim3(256), 0, s>>>(
       static_cast<const bf16_t*>(x), ldx, row_index, x_rows, rows, static_cast<int>(k), q, scale, out_rows);
   HMOE_CHECK_LAUNCH();
   return HMOE_OK;
