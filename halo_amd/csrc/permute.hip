@@ -104,7 +104,12 @@ gather_rows_kernel(const T* __restrict__ src, int64_t src_stride, const int64_t*
 // a lane keeps kTopK loads in flight instead of one (with one in flight the kernel reached half of the HBM rate).  An
 // invalid slot contributes +0.0f, which leaves the fp32 sum exactly as skipping it does: the accumulator starts at
 // +0.0f and a sum that started there is never -0.0f.
-template <typename T, int W, bool kWeighted, int kTopK>
+// kAllValid: the launch is expected to hold valid slots only (there are as many sources as slots: the inverse of a
+// permutation), so the kernel is built around the all-valid form, four column chunks per pass at two wavefronts per
+// SIMD; a row with an invalid slot is still reduced correctly, one chunk at a time.  Without it such rows take the
+// compacted form, and the register budget stays at four wavefronts per SIMD: they have few fetches in flight per
+// lane and need the wavefronts.
+template <typename T, int W, bool kWeighted, int kTopK, bool kAllValid>
 __global__ void __launch_bounds__(kThreads)
 gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, const int64_t* __restrict__ inv_map,
                      T* __restrict__ out, int64_t n_out, int top_k, int64_t n_src, int64_t hidden,
@@ -154,8 +159,8 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
       constexpr bool kDense = decltype(dense_tag)::value;
       int64_t c = static_cast<int64_t>(lane_id()) * W;
       if constexpr (kDense && kTopK <= 8) {
-        // four column chunks per pass while the row has them (a whole row of 2048 bf16), then two: 4 * kTopK row
-        // fetches in flight per lane at two wavefronts per SIMD (two chunks per pass at three wavefronts: 6 % slower)
+        // kAllValid: four column chunks per pass while the row has them (a whole row of 2048 bf16), then two: 4 * kTopK
+        // row fetches in flight per lane at two wavefronts per SIMD (two chunks per pass at three wavefronts: 6 % slower)
         auto pass = [&](auto width_tag) __attribute__((always_inline)) {
           constexpr int kWide = decltype(width_tag)::value;
           Pack<T, W> x[kWide][kTopK], acc[kWide], extra_chunk[kWide];
@@ -177,7 +182,9 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
             acc[h].store(to + c + h * step);
           }
         };
-        for (; c + 3 * step < hidden; c += 4 * step) pass(std::integral_constant<int, 4>{});
+        if constexpr (kAllValid) {
+          for (; c + 3 * step < hidden; c += 4 * step) pass(std::integral_constant<int, 4>{});
+        }
         for (; c + step < hidden; c += 2 * step) pass(std::integral_constant<int, 2>{});
       }
       for (; c < hidden; c += step) {
@@ -210,10 +217,15 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
       reduce_row(std::true_type{});
       return;
     }
+    if constexpr (kAllValid) {  // the launch was expected to hold valid slots only: a row that does not, the plain way
+      reduce_row(std::false_type{});
+      return;
+    }
     // Some slots are not this rank's (most of them on one GPU's share of an expert-parallel layer).  The valid ones are
     // moved to the front, in slot order (the sum keeps its order; a slot left out adds the +0.0f it added before), and
     // the row is reduced by the loop written for that many sources: every fetch of a pass goes out before the first is
-    // used, four column chunks per pass while the row has them, so that 4 to 28 fetches are in flight per lane.
+    // used, and a row with few sources takes more column chunks per pass (four for one to three sources, two from
+    // four up), so that 4 to 14 fetches are in flight per lane.
     // Everything here is the same for the whole wavefront (scalar registers, one branch).
     const T* live_from[kTopK];
     float live_w[kTopK];
@@ -272,10 +284,10 @@ gather_reduce_kernel(const T* __restrict__ src, const T* __restrict__ weight, co
       case 1: reduce_live(integral_constant<int, 1>{}, integral_constant<int, 4>{}); break;
       case 2: reduce_live(integral_constant<int, 2>{}, integral_constant<int, 4>{}); break;
       case 3: reduce_live(integral_constant<int, (kTopK >= 3 ? 3 : 1)>{}, integral_constant<int, 4>{}); break;
-      case 4: reduce_live(integral_constant<int, (kTopK >= 4 ? 4 : 1)>{}, integral_constant<int, 4>{}); break;
-      case 5: reduce_live(integral_constant<int, (kTopK >= 5 ? 5 : 1)>{}, integral_constant<int, 4>{}); break;
-      case 6: reduce_live(integral_constant<int, (kTopK >= 6 ? 6 : 1)>{}, integral_constant<int, 4>{}); break;
-      case 7: reduce_live(integral_constant<int, (kTopK >= 7 ? 7 : 1)>{}, integral_constant<int, 4>{}); break;
+      case 4: reduce_live(integral_constant<int, (kTopK >= 4 ? 4 : 1)>{}, integral_constant<int, 2>{}); break;
+      case 5: reduce_live(integral_constant<int, (kTopK >= 5 ? 5 : 1)>{}, integral_constant<int, 2>{}); break;
+      case 6: reduce_live(integral_constant<int, (kTopK >= 6 ? 6 : 1)>{}, integral_constant<int, 2>{}); break;
+      case 7: reduce_live(integral_constant<int, (kTopK >= 7 ? 7 : 1)>{}, integral_constant<int, 2>{}); break;
       default: reduce_row(std::false_type{}); break;
     }
   } else {
@@ -612,12 +624,21 @@ int hmoe_gather_reduce_add(const void* src, const void* weight, const int64_t* i
                                       : rows_vectorizable<float>(hidden, {addend_row_stride}, {src, out, addend});
   // n_src == 0: every slot is invalid and the rows come out as zeros; the generic kernel never touches src then
   const int fixed = n_src > 0 && (top_k == 8 || top_k == 4 || top_k == 2) ? top_k : 0;
-#define HMOE_GATHER_REDUCE(WEIGHTED, TOPK)                                                                        \
+  // as many sources as slots: the inverse of a permutation, every slot valid (a hint: either kernel is correct for
+  // any inv_map)
+  const bool wide = fixed > 0 && n_src == n_out * top_k;
+#define HMOE_GATHER_REDUCE_AS(WEIGHTED, TOPK, WIDE)                                                               \
   HMOE_DISPATCH_ROWS(dtype, vec,                                                                                  \
-                     (gather_reduce_kernel<T, W, WEIGHTED, TOPK><<<row_grid(n_out), dim3(kThreads), 0, s>>>(      \
+                     (gather_reduce_kernel<T, W, WEIGHTED, TOPK, WIDE><<<row_grid(n_out), dim3(kThreads), 0, s>>>( \
                          static_cast<const T*>(src), static_cast<const T*>(weight), inv_map, static_cast<T*>(out), \
                          n_out, top_k, n_src, hidden, static_cast<const T*>(addend), addend_row_stride,           \
                          static_cast<const T*>(addend_scale))))
+#define HMOE_GATHER_REDUCE(WEIGHTED, TOPK)                    \
+  if (wide && TOPK > 0) {                                     \
+    HMOE_GATHER_REDUCE_AS(WEIGHTED, TOPK, (TOPK > 0));        \
+  } else {                                                    \
+    HMOE_GATHER_REDUCE_AS(WEIGHTED, TOPK, false);             \
+  }
   if (weight) {
     if (fixed == 8) { HMOE_GATHER_REDUCE(true, 8); }
     else if (fixed == 4) { HMOE_GATHER_REDUCE(true, 4); }
@@ -630,6 +651,7 @@ int hmoe_gather_reduce_add(const void* src, const void* weight, const int64_t* i
     else { HMOE_GATHER_REDUCE(false, 0); }
   }
 #undef HMOE_GATHER_REDUCE
+#undef HMOE_GATHER_REDUCE_AS
   HMOE_CHECK_LAUNCH();
   return HMOE_OK;
 }

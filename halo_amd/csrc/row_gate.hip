@@ -111,15 +111,29 @@ __global__ void __launch_bounds__(kGateThreads) row_gate_bwd_kernel(const T* __r
   }
 }
 
-// grad_w[c] = the partial rows' column c added in row order, rounded once
+// grad_w[c] = the partial rows' column c, rounded once.  Sixteen threads share a column: thread s adds the partial rows
+// s, s + 16, ... in that order and the sixteen sums are added in the order of s, so the result does not depend on
+// timing (one thread per column walking every partial row took 64 us for 256 rows: a chain of dependent loads).
+constexpr int kFinalCols = 16, kFinalSlices = kGateThreads / kFinalCols;
 template <typename T>
 __global__ void __launch_bounds__(kGateThreads) row_gate_bwd_final_kernel(const float* __restrict__ partial, int blocks,
                                                                           int hidden, T* __restrict__ grad_w) {
-  const int c = blockIdx.x * kGateThreads + threadIdx.x;
-  if (c >= hidden) return;
+  __shared__ float sums[kFinalSlices][kFinalCols];
+  const int col_in = threadIdx.x % kFinalCols, slice = threadIdx.x / kFinalCols;
+  const int c = blockIdx.x * kFinalCols + col_in;
   float sum = 0.f;
-  for (int b = 0; b < blocks; ++b) sum += partial[static_cast<int64_t>(b) * hidden + c];
-  Elem<T>::store(grad_w + c, sum);
+  if (c < hidden) {
+#pragma unroll 4
+    for (int b = slice; b < blocks; b += kFinalSlices) sum += partial[static_cast<int64_t>(b) * hidden + c];
+  }
+  sums[slice][col_in] = sum;
+  __syncthreads();
+  if (slice == 0 && c < hidden) {
+    float total = 0.f;
+#pragma unroll
+    for (int s = 0; s < kFinalSlices; ++s) total += sums[s][col_in];
+    Elem<T>::store(grad_w + c, total);
+  }
 }
 
 inline int64_t gate_rows_per_block(int64_t n_rows) {
@@ -158,7 +172,7 @@ int launch_bwd(const void* x, int64_t ldx, const void* w, const void* gate, cons
 #undef HMOE_GATE_BWD
   HMOE_CHECK_LAUNCH();
   if (grad_w) {
-    row_gate_bwd_final_kernel<T><<<dim3((hidden + kGateThreads - 1) / kGateThreads), block, 0, s>>>(
+    row_gate_bwd_final_kernel<T><<<dim3((hidden + kFinalCols - 1) / kFinalCols), block, 0, s>>>(
         part, blocks, hidden, static_cast<T*>(grad_w));
     HMOE_CHECK_LAUNCH();
   }
@@ -199,7 +213,7 @@ int hmoe_row_gate_bwd(const void* x, int64_t ldx, const void* w, const void* gat
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (n_rows == 0) {  // no tokens: the weight gradient is zero (the sum over no partial rows)
     if (grad_w) {
-      const dim3 grid((hidden + hmoe::kGateThreads - 1) / hmoe::kGateThreads), block(hmoe::kGateThreads);
+      const dim3 grid((hidden + hmoe::kFinalCols - 1) / hmoe::kFinalCols), block(hmoe::kGateThreads);
       if (dtype == HMOE_BF16)
         hmoe::row_gate_bwd_final_kernel<hmoe::bf16_t><<<grid, block, 0, s>>>(nullptr, 0, hidden,
                                                                             static_cast<hmoe::bf16_t*>(grad_w));

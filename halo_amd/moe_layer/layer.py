@@ -286,6 +286,7 @@ class EPMoELayerBase(ExpertLoadMixin, nn.Module, ABC):
         self.fuse_permute_into_gemm = True
         # the shared expert's output joins the routed one in the combine kernel instead of a tensor addition
         self.fuse_shared_into_combine = True
+        self.fuse_shared_gate_up = True
         # an adapted projection adds its low-rank delta in the second adapter product's epilogue
         self.fuse_lora_into_gemm = True
         # the gate weights multiply the GLU's output instead of the down projection's: the combine becomes a plain
@@ -769,6 +770,14 @@ class EPSharedExpertsMoELayerBase(EPMoELayerBase):
         shared = getattr(self, self._shared_expert_attr)
         x = hidden_states.reshape(-1, hidden_states.shape[-1])
         dtype = x.dtype
-        gate = dense_mm(x, shared.gate_proj.weight.to(dtype))
-        up = dense_mm(x, shared.up_proj.weight.to(dtype))
+        gate_w, up_w = shared.gate_proj.weight.to(dtype), shared.up_proj.weight.to(dtype)
+        packable = getattr(self._fused_glu_mul, "packed", None)
+        if getattr(self, "fuse_shared_gate_up", True) and packable is not None and gate_w.shape == up_w.shape:
+            # gate and up as one product over the two weights side by side (HF keeps them apart): one launch per
+            # direction, the input gradient summed over both in fp32 instead of two rounded products and an addition,
+            # and the SwiGLU in its packed form.  The same dot products: the forward's bits do not change.
+            gate_up = dense_mm(x, torch.cat((gate_w, up_w), dim=0))
+            return dense_mm(packable(gate_up), shared.down_proj.weight.to(dtype)), None
+        gate = dense_mm(x, gate_w)
+        up = dense_mm(x, up_w)
         return dense_mm(self._fused_glu_mul(gate, up), shared.down_proj.weight.to(dtype)), None
