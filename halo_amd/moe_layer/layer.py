@@ -171,6 +171,28 @@ class _SigmoidRowGate(torch.autograd.Function):
         return grad_x, grad_w
 
 
+class _ScaleRows(torch.autograd.Function):
+    """``rows * scale[:, None]`` (the shared expert's output times its per-token gate, where the sum with the routed
+    output is not taken by the combine kernel: under expert parallelism the routed rows come back through the
+    exchange first).  Forward is the tensor multiplication; backward is one pass of the combine-backward kernel with
+    every row its own token, ``scale * grad`` and ``<grad, rows>`` together, in place of two multiplications and a row
+    sum (the dot product accumulated in fp32 and rounded once, where autograd rounds every product first)."""
+
+    @staticmethod
+    def forward(ctx, rows, scale):
+        ctx.save_for_backward(rows, scale)
+        return rows * scale.unsqueeze(-1)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from halo_amd.kernels.moe_permute import _unpermute_backward
+
+        rows, scale = ctx.saved_tensors
+        own = torch.arange(rows.shape[0], device=rows.device)
+        grad_rows, grad_scale = _unpermute_backward(grad_out, rows, scale, own, ctx.needs_input_grad[1])
+        return (grad_rows if ctx.needs_input_grad[0] else None), grad_scale
+
+
 def sigmoid_row_gate(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``sigmoid(F.linear(x, weight)).view(-1)`` for ``x [T, H]`` and an ``nn.Linear(H, 1)`` weight ``[1, H]``;
     differentiable in both.  Device tensors whose rows are 16-byte multiples take :class:`_SigmoidRowGate`; CPU
@@ -761,8 +783,11 @@ class EPSharedExpertsMoELayerBase(EPMoELayerBase):
     def _shared_expert_output(self, hidden_states: torch.Tensor) -> torch.Tensor:
         """Dense GLU MLP ``down(act(gate(x)) * up(x))`` through the same GEMM and GLU kernels."""
         rows, scale = self._shared_expert_parts(hidden_states)
-        out = rows.view(hidden_states.shape)
-        return out if scale is None else out * scale.view(*hidden_states.shape[:-1], 1)
+        if scale is None:
+            return rows.view(hidden_states.shape)
+        if rows.is_cuda and rows.dim() == 2 and rows.dtype == scale.dtype and rows.shape[0] > 0:
+            return _ScaleRows.apply(rows, scale.reshape(-1)).view(hidden_states.shape)
+        return rows.view(hidden_states.shape) * scale.view(*hidden_states.shape[:-1], 1)
 
     def _shared_expert_parts(self, hidden_states: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor | None]:
         """The shared expert's output as ``(rows [T, H], scale [T] or None)``: ``rows`` the MLP's output, ``scale`` a
