@@ -205,6 +205,47 @@ def test_cpu_layer_forward_backward_matches_the_per_expert_loop(cfg_name):
         _check(f"grad {name}", getattr(layer, attr).grad, want_grads[name], tol)
 
 
+@pytest.mark.parametrize("fuse_gate_up", (True, False), ids=("gate_up_as_one_product", "gate_and_up_apart"))
+def test_cpu_layer_with_a_gated_shared_expert_matches_the_oracle(fuse_gate_up):
+    """Qwen3.5's block with its sigmoid-gated shared expert on CPU tensors: the shared expert's gate and up projections
+    as one product over the two weights side by side (the default) or as two, the gate through ``sigmoid_row_gate``'s
+    tensor-operation form; output and gradients against the oracle's loop with the same selection."""
+    import tests.cases as cases
+    from halo_amd.kernels.router import fused_topk_gate
+    from halo_amd.moe_layer.layer import sigmoid_row_gate
+    from oracle import moe_layer as oracle
+    from tests.test_gpu_layer import _check, _layer_with_shared_expert
+
+    cfg = cases.CONFIG2_SMALL
+    inputs = cases.make_layer_inputs(cfg)
+    cpu = torch.device("cpu")
+    layer = _layer_with_shared_expert(cfg, inputs, cpu, gated=True, fuse=True)
+    layer.fuse_shared_gate_up = fuse_gate_up
+    x = inputs["x"].clone().requires_grad_(True)
+    out = layer(x)
+    out.backward(inputs["grad_out"])
+    with torch.no_grad():
+        idx, _ = fused_topk_gate(layer._linear_router_logits(x.detach()), cfg.top_k, normalize=True, eps=0.0)
+    f = lambda t: t.detach().float().requires_grad_(True)
+    xs, wr = f(inputs["x"]), f(inputs["router_weight"])
+    params = {k: f(v) for k, v in inputs["params"].items()}
+    shared = {n: f(getattr(layer.shared_expert, n).weight) for n in ("gate_proj", "up_proj", "down_proj")}
+    shared["shared_expert_gate"] = f(layer.shared_expert_gate.weight)
+    want, _, _, _ = oracle.moe_layer_forward(xs, wr, params, oracle.Glu(cfg.glu), cfg.top_k, normalize=True, eps=0.0,
+                                             indices=idx, shared=shared)
+    want.backward(inputs["grad_out"].float())
+    tol = 1e-4 if cfg.dtype == torch.float32 else 2e-2
+    _check("out", out, want.detach(), tol)
+    _check("grad x", x.grad, xs.grad, tol)
+    for name in ("gate_proj", "up_proj", "down_proj"):
+        _check(f"grad shared {name}", getattr(layer.shared_expert, name).weight.grad, shared[name].grad, tol)
+    _check("grad shared gate", layer.shared_expert_gate.weight.grad, shared["shared_expert_gate"].grad, tol)
+    # the gate helper on CPU tensors is the tensor operations themselves
+    g = torch.Generator().manual_seed(5)
+    rows, w = torch.randn(33, 24, generator=g), torch.randn(1, 24, generator=g)
+    assert torch.equal(sigmoid_row_gate(rows, w), torch.sigmoid(rows @ w.t()).view(-1))
+
+
 def test_cpu_gemma4_experts_drop_in_matches_the_hf_module():
     """``EPGemma4MoELayer`` wraps transformers' ``Gemma4TextExperts`` (experts only, routing handed in) and returns its
     output and gradients, the gate weights' included, in fp32 on the CPU."""
