@@ -645,6 +645,32 @@ def test_shared_expert_added_in_the_combine_kernel(device, cfg, gated):
     _check("grad shared down_proj", grads_b["shared_expert.down_proj.weight"], shared["down_proj"].grad, check_tol)
 
 
+def test_shared_expert_gate_and_up_as_one_product_keeps_the_forward_bits(device):
+    """The shared expert's gate and up projections as one product over the two weights side by side against two
+    products: the same dot products, so the layer's output is equal bit for bit; the input gradient is summed over both
+    in fp32 instead of two rounded products and an addition, so gradients agree within the bf16 tolerance."""
+    cfg = CONFIG2_SMALL
+    inputs = make_layer_inputs(cfg)
+    results = []
+    for one_product in (False, True):
+        layer = _layer_with_shared_expert(cfg, inputs, device, gated=True, fuse=True)
+        layer.fuse_shared_gate_up = one_product
+        x = inputs["x"].to(device).requires_grad_(True)
+        out = layer(x)
+        out.backward(inputs["grad_out"].to(device))
+        grads = {n: p.grad.clone() for n, p in layer.named_parameters() if p.grad is not None}
+        results.append((out.detach(), x.grad.clone(), grads))
+    (out_a, gx_a, grads_a), (out_b, gx_b, grads_b) = results
+    assert torch.equal(out_a, out_b)
+    assert max_rel(gx_b, gx_a) < 2e-2
+    assert set(grads_a) == set(grads_b)
+    for name in grads_a:
+        assert max_rel(grads_b[name], grads_a[name]) < 2e-2, name
+        # the same contraction per element (at this size the weight gradient is one product, not token slices)
+        if name.startswith(("shared_expert.gate_proj", "shared_expert.up_proj")):
+            assert torch.equal(grads_a[name], grads_b[name]), name
+
+
 @pytest.mark.parametrize("fuse", (False, True), ids=("tensor_add", "in_combine"))
 def test_shared_expert_on_a_side_stream_changes_no_bit(device, fuse, monkeypatch):
     """``HALO_EP_SHARED_OVERLAP``: the shared expert runs on a second stream beside the routed path and is joined
