@@ -1160,6 +1160,9 @@ __global__ void __launch_bounds__(Cfg::kThreads) grouped_gemm_bf16_kernel(GemmAr
     const int steps = (tile.con_lim + BK - 1) / BK;
     int live = (tile.a_out_lim - (tile.a_out0 + row_a) + 31) >> 5;
     live = live < 0 ? 0 : (live > WM ? WM : live);
+    // a wavefront whose columns all lie past the operand's edge (the last column tile of a width that is no multiple
+    // of 256) has nothing to multiply either: its blocks would be products with zeros that are never stored
+    if (tile.b_out0 + row_b >= tile.b_out_lim) live = 0;
     // The expert's bias for this lane's eight output columns (the same columns in every store of the epilogue).  It
     // is fetched here, where the tile's first loads are waited for anyway, and pinned as arrived right behind that
     // wait: a wait placed by the compiler at its first use, in the epilogue, would be for every load in flight, the
@@ -1564,6 +1567,7 @@ __global__ void __launch_bounds__(512) grouped_gemm_fp8_kernel(GemmArgs p) {
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
     int live = (tile.a_out_lim - (tile.a_out0 + row_a) + 31) >> 5;
     live = live < 0 ? 0 : (live > WM ? WM : live);
+    if (tile.b_out0 + row_b >= tile.b_out_lim) live = 0;  // this wavefront's columns lie past the operand's edge
     // The tile's first three stages (issued before the previous tile's epilogue) must be in; that epilogue's stores,
     // issued after them, need not be (vector memory operations complete in issue order, so "all but the youngest n"
     // leaves exactly the stores out): they drain under this tile's first steps.
