@@ -874,3 +874,24 @@ def test_expert_lora_rank_must_span_whole_rows(device):
         ep_config=EPConfig(expert_lora=ExpertLoraSpec(8, 16.0, projections=frozenset({"down"}), use_rslora=True)))
     assert only_down._expert_lora_attrs == frozenset({"down_proj"}) and only_down.gate_up_proj.requires_grad
     assert abs(only_down.expert_lora_scaling - 16.0 / 8 ** 0.5) < 1e-12
+
+
+@pytest.mark.parametrize("frozen", ("weight", "x"))
+def test_sigmoid_row_gate_with_one_side_frozen(device, frozen):
+    """A frozen gate weight (adapter fine-tuning) or a frozen input: the gradient that is asked for keeps the bits of
+    the run that asks for both, and the other one is not produced."""
+    from halo_amd.moe_layer.layer import sigmoid_row_gate
+
+    g = torch.Generator().manual_seed(35)
+    x = torch.randn(777, 512, generator=g).bfloat16().to(device)
+    w = (torch.randn(1, 512, generator=g) * 0.05).bfloat16().to(device)
+    grad = torch.randn(777, generator=g).bfloat16().to(device)
+    xa, wa = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    sigmoid_row_gate(xa, wa).backward(grad)
+    xb, wb = x.clone().requires_grad_(frozen != "x"), w.clone().requires_grad_(frozen != "weight")
+    gate = sigmoid_row_gate(xb, wb)
+    gate.backward(grad)
+    if frozen == "weight":
+        assert wb.grad is None and torch.equal(xb.grad, xa.grad)
+    else:
+        assert xb.grad is None and torch.equal(wb.grad, wa.grad)
