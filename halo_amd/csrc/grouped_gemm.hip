@@ -1943,8 +1943,9 @@ int launch_direct(const GemmArgs& p, hipStream_t stream) {
 // tile of which the product has at least one per compute unit, since a larger tile moves fewer operand bytes per
 // multiply-add (the 256 x 256 tile is 10-25 % faster than the 128 x 256 one at the expert products of every benchmark
 // configuration) and a launch with fewer tiles than compute units leaves some idle (a dense projection of a few
-// thousand rows, a narrow output).  hmoe_set_gemm_tile() or HALO_GEMM_TILE=mono|duo|small forces one configuration
-// for every product.
+// thousand rows, a narrow output); an output of at most 128 columns takes the 128 x 128 tile whatever its tile count
+// (the logits of 32 768 tokens over 128 experts: 39 against 53 us).  hmoe_set_gemm_tile() or
+// HALO_GEMM_TILE=mono|duo|small forces one configuration for every product.
 enum TilePolicy { kTileBySize = 0, kTileMono = 1, kTileDuo = 2, kTileSmall = 3 };
 std::atomic<int> g_gemm_tile{-1};  // a TilePolicy; -1: not yet read from the environment
 
@@ -1972,6 +1973,8 @@ int tile_for(const GemmArgs& p) {
   const int forced = gemm_tile_policy();
   if (forced != kTileBySize) return forced;
   const int cus = device_cus();
+  // an output of at most 128 columns (a router's logits) would leave half of every 256-wide tile empty
+  if ((kMode == kDgrad ? p.k : p.n) <= 128) return kTileSmall;
   if (tile_bound<kMode>(p, 256, 256) >= cus) return kTileMono;
   if (tile_bound<kMode>(p, 128, 256) >= cus) return kTileDuo;
   return kTileSmall;
